@@ -1,0 +1,270 @@
+"""The cache manager: pages of keys and values with a block table for each
+request, and slots for per-request state of fixed size.
+
+A model's cache *streams* (one per schedule entry that caches, or shared
+between entries) each declare a spec.  Streams whose spec is :class:`PagedKV`
+are put into *groups* by their window: all streams that keep every key share
+one page pool and one block table per request; streams with a window of W
+tokens share another, whose pages are given back once a request's window has
+passed them.  Within a group one page index stands for the same ``page_tokens``
+tokens in every stream of the group, each stream having storage of its own
+shape ``[pages, kv_heads, page_tokens, head_dim]`` for keys and for values.
+Streams whose spec is :class:`FixedState` get a tensor ``[max_requests,
+*shape]``; a request's row is its slot, zeroed at admission.
+
+(Reference: KVCache, engine/include/llm/kv_cache.h:14-88 and
+engine/src/kv_cache.cpp:17-153 -- one group, 64-token pages, one page table row
+per slot, pages acquired lazily by reserve() and given back by reset().  Pages
+are never cleared on reuse; masks never read past a request's length.)
+
+The bookkeeping is host-side and does not touch the device except to zero a
+state slot and, when asked, to poison pages.
+"""
+from __future__ import annotations
+
+import dataclasses
+from typing import Any, Dict, Hashable, Iterable, List, Optional, Sequence, Tuple
+
+import torch
+
+from ..errors import EngineError, OutOfPages
+from .page_pool import PagePool
+from .specs import FixedState, PagedKV
+
+_STATE_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "int32": torch.int32}
+
+
+@dataclasses.dataclass
+class PagedView:
+    """What a mixer sees of its paged stream."""
+    k: torch.Tensor            # [pages, kv_heads, page_tokens, head_dim]
+    v: torch.Tensor
+    group: Hashable            # key of the group whose block table addresses it
+    page_tokens: int
+    window: int
+
+
+@dataclasses.dataclass
+class StateView:
+    """What a mixer sees of its fixed-size state stream: row = request slot."""
+    state: torch.Tensor        # [max_requests, *shape]
+
+
+class _Group:
+    def __init__(self, window: int, num_pages: int):
+        self.window = window
+        self.pool = PagePool(num_pages)
+        self.streams: List[Hashable] = []
+
+
+class _Request:
+    def __init__(self, slot: int, groups: Iterable[Hashable]):
+        self.slot = slot
+        self.length = 0
+        # group -> page of every page index so far; -1 where the window has passed
+        self.tables: Dict[Hashable, List[int]] = {g: [] for g in groups}
+        self.released: Dict[Hashable, int] = {g: 0 for g in groups}  # leading pages given back
+
+
+class CacheManager:
+    def __init__(self, streams: Dict[Hashable, Any], *, page_tokens: int, num_pages: int,
+                 max_requests: int, max_tokens: int, dtype: torch.dtype, device: Any,
+                 poison: bool = False):
+        if page_tokens <= 0 or num_pages < 0 or max_requests <= 0 or max_tokens <= 0:
+            raise EngineError(f"cache: bad sizes page_tokens={page_tokens} num_pages={num_pages} "
+                              f"max_requests={max_requests} max_tokens={max_tokens}")
+        self.page_tokens = page_tokens
+        self.max_requests = max_requests
+        self.max_tokens = max_tokens
+        self.max_pages_per_request = -(-max_tokens // page_tokens)
+        self.dtype = dtype
+        self.device = torch.device(device)
+        self.poison = poison
+        self.specs = dict(streams)
+        self.groups: Dict[Hashable, _Group] = {}
+        self._views: Dict[Hashable, Any] = {}
+        for sid, spec in self.specs.items():
+            if isinstance(spec, PagedKV):
+                key = ("window", spec.window)
+                group = self.groups.get(key)
+                if group is None:
+                    group = self.groups[key] = _Group(spec.window, num_pages)
+                group.streams.append(sid)
+                shape = (num_pages, spec.num_kv_heads, page_tokens, spec.head_dim)
+                k = torch.empty(shape, dtype=dtype, device=self.device)
+                v = torch.empty(shape, dtype=dtype, device=self.device)
+                if poison:
+                    k.fill_(float("nan"))
+                    v.fill_(float("nan"))
+                self._views[sid] = PagedView(k=k, v=v, group=key, page_tokens=page_tokens, window=spec.window)
+            elif isinstance(spec, FixedState):
+                sdt = _STATE_DTYPES.get(spec.dtype)
+                if sdt is None:
+                    raise EngineError(f"cache: state dtype {spec.dtype!r} is not one of {sorted(_STATE_DTYPES)}")
+                self._views[sid] = StateView(state=torch.zeros((max_requests, *spec.shape), dtype=sdt,
+                                                               device=self.device))
+            elif spec is not None:
+                raise EngineError(f"cache: stream {sid!r} has an unknown spec {spec!r}")
+        self._requests: Dict[Hashable, _Request] = {}
+        self._free_slots: List[int] = list(range(max_requests - 1, -1, -1))
+
+    # ---- requests ---------------------------------------------------------
+    def has(self, request: Hashable) -> bool:
+        return request in self._requests
+
+    def live_requests(self) -> List[Hashable]:
+        return list(self._requests)
+
+    @property
+    def free_slots(self) -> int:
+        return len(self._free_slots)
+
+    def admit(self, request: Hashable) -> int:
+        """Give the request a slot (zeroing its state); returns the slot."""
+        if request in self._requests:
+            raise EngineError(f"cache: request {request!r} is already live")
+        if not self._free_slots:
+            raise EngineError(f"cache: all {self.max_requests} request slots are taken")
+        slot = self._free_slots.pop()
+        self._requests[request] = _Request(slot, self.groups)
+        for view in self._views.values():
+            if isinstance(view, StateView):
+                view.state[slot].zero_()
+        return slot
+
+    def _req(self, request: Hashable) -> _Request:
+        try:
+            return self._requests[request]
+        except KeyError:
+            raise EngineError(f"cache: unknown request {request!r}") from None
+
+    def slot(self, request: Hashable) -> int:
+        return self._req(request).slot
+
+    def length(self, request: Hashable) -> int:
+        return self._req(request).length
+
+    def table(self, group: Hashable, request: Hashable) -> List[int]:
+        """The request's pages in token order (-1 where the window has passed)."""
+        return self._req(request).tables[group]
+
+    # ---- pages ------------------------------------------------------------
+    def pages_for(self, n_tokens: int) -> int:
+        return -(-n_tokens // self.page_tokens)
+
+    def new_pages_needed(self, request: Hashable, n_new: int) -> Dict[Hashable, int]:
+        r = self._req(request)
+        want = self.pages_for(r.length + n_new)
+        return {g: max(0, want - len(t)) for g, t in r.tables.items()}
+
+    def can_reserve(self, asks: Sequence[Tuple[Hashable, int]]) -> bool:
+        need: Dict[Hashable, int] = {g: 0 for g in self.groups}
+        for request, n_new in asks:
+            for g, n in self.new_pages_needed(request, n_new).items():
+                need[g] += n
+        return all(need[g] <= self.groups[g].pool.free_count for g in need)
+
+    def reserve(self, asks: Sequence[Tuple[Hashable, int]]) -> None:
+        """Make sure every (request, n_new) has pages for its next n_new tokens.
+
+        All or nothing: if any group lacks pages, OutOfPages is raised and no
+        page has been taken.  A request may appear once.
+        """
+        seen = set()
+        need: Dict[Hashable, int] = {g: 0 for g in self.groups}
+        for request, n_new in asks:
+            if request in seen:
+                raise EngineError(f"cache: request {request!r} appears twice in one reservation")
+            seen.add(request)
+            r = self._req(request)
+            if n_new < 0:
+                raise EngineError(f"cache: negative token count {n_new} for request {request!r}")
+            if r.length + n_new > self.max_tokens:
+                raise EngineError(f"cache: request {request!r} would hold {r.length + n_new} tokens, "
+                                  f"the cache is sized for {self.max_tokens} per request")
+            for g, n in self.new_pages_needed(request, n_new).items():
+                need[g] += n
+        for g, n in need.items():
+            free = self.groups[g].pool.free_count
+            if n > free:
+                raise OutOfPages(f"out of pages: group {g} needs {n} more, {free} of "
+                                 f"{self.groups[g].pool.num_pages} are free")
+        for request, n_new in asks:
+            r = self._requests[request]
+            want = self.pages_for(r.length + n_new)
+            for g, t in r.tables.items():
+                while len(t) < want:
+                    page = self.groups[g].pool.acquire()
+                    assert page >= 0
+                    t.append(page)
+
+    def advance(self, request: Hashable, n_new: int) -> None:
+        """The request's next n_new tokens are now cached.  Pages that every
+        later query's window has passed go back to their pool."""
+        r = self._req(request)
+        if n_new < 0 or (r.tables and
+                         r.length + n_new > min(len(t) for t in r.tables.values()) * self.page_tokens):
+            raise EngineError(f"cache: request {request!r} advanced past its reserved pages")
+        r.length += n_new
+        for g, t in r.tables.items():
+            window = self.groups[g].window
+            if window <= 0:
+                continue
+            # the next query sits at position r.length and reads keys from r.length - window + 1
+            first_needed = max(0, r.length - window + 1) // self.page_tokens
+            for idx in range(r.released[g], min(first_needed, len(t))):
+                self._give_back(g, t[idx])
+                t[idx] = -1
+            r.released[g] = max(r.released[g], min(first_needed, len(t)))
+
+    def _give_back(self, group: Hashable, page: int) -> None:
+        if not self.groups[group].pool.release(page):
+            raise EngineError(f"cache: page {page} of group {group} was freed twice or never held")
+        if self.poison:
+            for sid in self.groups[group].streams:
+                view = self._views[sid]
+                if view.k.is_floating_point():
+                    view.k[page].fill_(float("nan"))
+                    view.v[page].fill_(float("nan"))
+
+    def release(self, request: Hashable) -> None:
+        """The request has ended: its pages and its slot are given back."""
+        r = self._req(request)
+        for g, t in r.tables.items():
+            for page in t:
+                if page >= 0:
+                    self._give_back(g, page)
+        self._free_slots.append(r.slot)
+        del self._requests[request]
+
+    def release_all(self) -> None:
+        for request in list(self._requests):
+            self.release(request)
+
+    # ---- views and numbers ---------------------------------------------------
+    def view(self, stream: Hashable):
+        return self._views.get(stream)
+
+    def pages_in_use(self, group: Optional[Hashable] = None) -> int:
+        if group is not None:
+            return self.groups[group].pool.pages_in_use
+        return sum(g.pool.pages_in_use for g in self.groups.values())
+
+    def pages_total(self) -> int:
+        return sum(g.pool.num_pages for g in self.groups.values())
+
+    def free_pages(self, group: Hashable) -> int:
+        return self.groups[group].pool.free_count
+
+    def shuffle_free_pages(self, seed: int) -> None:
+        for i, g in enumerate(self.groups.values()):
+            g.pool.shuffle_free_list(seed + i)
+
+    def storage_bytes(self) -> int:
+        total = 0
+        for view in self._views.values():
+            if isinstance(view, PagedView):
+                total += view.k.numel() * view.k.element_size() * 2
+            else:
+                total += view.state.numel() * view.state.element_size()
+        return total

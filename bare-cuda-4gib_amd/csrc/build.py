@@ -1,0 +1,104 @@
+"""Compiles the HIP kernels for gfx950 into ``libbc4g.so`` beside this file.
+
+Objects go to ``_build/`` under this folder.  Sources are compiled in parallel
+and a line is printed as each one finishes, so a first call that has to
+compile shows that it is alive.
+"""
+from __future__ import annotations
+
+import concurrent.futures
+import hashlib
+import os
+import shutil
+import subprocess
+import sys
+import time
+from typing import List
+
+from ..errors import KernelError
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+SRC_DIR = os.path.join(HERE, "kernels")
+BUILD_DIR = os.path.join(HERE, "_build")
+LIB_PATH = os.path.join(HERE, "libbc4g.so")
+HASH_PATH = LIB_PATH + ".sources"
+
+ARCH = "gfx950"
+# -packed-fp32-ops is switched off: the compiler must not form packed float32
+# instructions from ordinary float code on this hardware.
+HIPCC_FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC",
+               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+               "-Wno-unused-command-line-argument"]
+
+
+def _hipcc() -> str:
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.exists(cand):
+            return cand
+    raise KernelError("hipcc not found: the kernel library cannot be compiled")
+
+
+def sources() -> List[str]:
+    return sorted(f for f in os.listdir(SRC_DIR) if f.endswith(".hip"))
+
+
+def sources_digest() -> str:
+    h = hashlib.sha256()
+    for name in sorted(os.listdir(SRC_DIR)):
+        if name.endswith((".hip", ".h")):
+            h.update(name.encode())
+            with open(os.path.join(SRC_DIR, name), "rb") as fh:
+                h.update(fh.read())
+    h.update(" ".join(HIPCC_FLAGS).encode())
+    return h.hexdigest()
+
+
+def is_built() -> bool:
+    return os.path.exists(LIB_PATH)
+
+
+def is_stale() -> bool:
+    try:
+        with open(HASH_PATH, "r") as fh:
+            return fh.read().strip() != sources_digest()
+    except OSError:
+        return True
+
+
+def _compile_one(hipcc: str, name: str) -> str:
+    obj = os.path.join(BUILD_DIR, name[:-4] + ".o")
+    cmd = [hipcc, *HIPCC_FLAGS, "-I", SRC_DIR, "-c", os.path.join(SRC_DIR, name), "-o", obj]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise KernelError(f"hipcc failed on {name}:\n{proc.stderr[-4000:]}")
+    return obj
+
+
+def build(verbose: bool = True, jobs: int = 0) -> str:
+    """Compile every kernel source and link the library; returns its path."""
+    hipcc = _hipcc()
+    os.makedirs(BUILD_DIR, exist_ok=True)
+    names = sources()
+    jobs = jobs or min(len(names), max(1, min(16, os.cpu_count() or 1)))
+    t0 = time.time()
+    out = sys.stderr
+    if verbose:
+        print(f"[bc4g] compiling {len(names)} kernel sources for {ARCH} with {jobs} jobs ...", file=out, flush=True)
+    objs = []
+    with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
+        futs = {pool.submit(_compile_one, hipcc, n): n for n in names}
+        for fut in concurrent.futures.as_completed(futs):
+            objs.append(fut.result())
+            if verbose:
+                print(f"[bc4g]   {futs[fut]} done ({time.time() - t0:.0f} s)", file=out, flush=True)
+    tmp = LIB_PATH + f".tmp{os.getpid()}"
+    proc = subprocess.run([hipcc, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", tmp, *sorted(objs)],
+                          capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise KernelError(f"linking libbc4g.so failed:\n{proc.stderr[-4000:]}")
+    os.replace(tmp, LIB_PATH)
+    with open(HASH_PATH, "w") as fh:
+        fh.write(sources_digest())
+    if verbose:
+        print(f"[bc4g] built {LIB_PATH} in {time.time() - t0:.0f} s", file=out, flush=True)
+    return LIB_PATH

@@ -1,0 +1,61 @@
+// C entry points of the kernel library (loaded through ctypes).
+//
+// Every function returns 0 on success; otherwise bc4g_last_error() holds the
+// reason (sizes a kernel refuses, a failed launch).  Pointers are device
+// pointers; `stream` is a hipStream_t.  dtype codes: 0 = float32, 1 = bfloat16.
+// Shapes are checked here, on the host, before anything is launched.
+#pragma once
+
+#include <stdint.h>
+
+extern "C" {
+
+const char* bc4g_last_error();
+int bc4g_version();
+
+// x[t, :] = float(table[ids[t], :])            (reference: embedding_lookup.cu:16-31)
+int bc4g_embed_gather(const void* table, int table_dtype, const int32_t* ids, float* out,
+                      int n_tokens, int hidden, int vocab, void* stream);
+
+// out[r, :] = x[rows ? rows[r] : r, :] * rsqrt(mean(x^2) + eps) * w      (rmsnorm.cu:16-41)
+// x is the float residual stream; out has out_dtype; w has w_dtype.
+int bc4g_rmsnorm(const float* x, const int32_t* rows, const void* w, int w_dtype, void* out,
+                 int out_dtype, int n_rows, int hidden, float eps, void* stream);
+
+// out[m, n] (+)= sum_k a[m, k] * w[n, k]        (gemm_tiled.cuh:36-96, plain float FMA)
+// accumulate != 0 adds into a float `out` (the residual stream).
+int bc4g_gemm_generic(const void* a, int a_dtype, const void* w, int w_dtype, void* out,
+                      int out_dtype, int accumulate, int m, int n, int k, void* stream);
+
+// out[t, i] = silu(gu[t, i]) * gu[t, inter + i]                          (swiglu.cu:17-25)
+int bc4g_swiglu(const void* gu, void* out, int dtype, int n_tokens, int inter, void* stream);
+
+// Rotates q (in place) and k by each row's position, and writes k and v into
+// their cache pages (rope.cu:18-55, kv_cache_write.cu:10-20).
+// qkv: [n_tokens, (n_heads + 2 n_kv_heads) * head_dim]; slot_map[t] = page * page_tokens +
+// offset of the row's token; k_cache/v_cache: [pages, n_kv_heads, page_tokens, head_dim].
+// rotary_dim 0 switches the rotation off; write_kv 0 leaves the cache alone.
+int bc4g_rope_kv_write(void* qkv, int dtype, const int32_t* positions, const int32_t* slot_map,
+                       void* k_cache, void* v_cache, int n_tokens, int n_heads, int n_kv_heads,
+                       int head_dim, int rotary_dim, float theta, int page_tokens, int num_pages,
+                       int write_kv, void* stream);
+
+// Causal softmax attention of every row over its request's cached keys
+// (attention_qk.cu:17-70, softmax.cu:22-43, attention_av.cu:18-46, fused).
+// Row t of request s = row_seq[t] at position p = positions[t] sees keys
+// max(0, p - window + 1) .. p (window 0 = all); key j lies in page
+// block_table[s, j / page_tokens].  q is read from the qkv rows; out: [n_tokens, n_heads*head_dim].
+int bc4g_attention_generic(const void* qkv, void* out, int dtype, const void* k_cache,
+                           const void* v_cache, const int32_t* block_table, int table_stride,
+                           const int32_t* row_seq, const int32_t* positions, int n_tokens,
+                           int n_heads, int n_kv_heads, int head_dim, int page_tokens,
+                           int num_pages, int window, float scale, void* stream);
+
+// out[r] = lowest index of the row's maximum                      (logits_argmax.cu:22-65)
+int bc4g_argmax(const float* logits, int32_t* out, int n_rows, int vocab, void* stream);
+
+// out[r] = first i with cumsum(exp((l - max) / temperature[r]))[i] > u[r] * total, walking the
+// vocabulary in order (engine/src/sampler.cpp:39-61); temperature <= 0 gives the argmax.
+int bc4g_sample(const float* logits, const float* temperature, const double* u, int32_t* out,
+                int n_rows, int vocab, void* stream);
+}

@@ -1,0 +1,97 @@
+// Shared device helpers for the gfx950 kernels: storage types, wave64
+// reductions, error reporting of the C entry points.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace bc4g {
+
+constexpr int kWave = 64;  // CDNA wavefront width
+
+// ---- storage types ---------------------------------------------------------
+// Activations, weights and cache are float or bfloat16; bfloat16 is handled as
+// its 16-bit pattern and widened/rounded by hand so that every kernel states
+// where it rounds.  All arithmetic is float.
+struct bf16_t {
+  uint16_t bits;
+};
+
+__host__ __device__ inline float to_float(float v) { return v; }
+__host__ __device__ inline float to_float(bf16_t v) {
+  union { uint32_t u; float f; } c;
+  c.u = static_cast<uint32_t>(v.bits) << 16;
+  return c.f;
+}
+
+// Round to nearest, ties to even; NaN stays NaN.
+__host__ __device__ inline uint16_t bf16_bits_from_float(float f) {
+  union { uint32_t u; float f; } c;
+  c.f = f;
+  if ((c.u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((c.u >> 16) | 0x0040u);
+  const uint32_t lsb = (c.u >> 16) & 1u;
+  c.u += 0x7fffu + lsb;
+  return static_cast<uint16_t>(c.u >> 16);
+}
+
+template <typename T> __host__ __device__ inline T from_float(float f);
+template <> __host__ __device__ inline float from_float<float>(float f) { return f; }
+template <> __host__ __device__ inline bf16_t from_float<bf16_t>(float f) {
+  bf16_t r;
+  r.bits = bf16_bits_from_float(f);
+  return r;
+}
+
+// ---- wave64 / block reductions --------------------------------------------
+__device__ inline float wave_sum(float v) {
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+  return v;
+}
+__device__ inline float wave_max(float v) {
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+  return v;
+}
+
+// Sum over a block of up to 1024 threads; `scratch` holds at least 16 floats.
+// Every thread gets the result.  The order of additions depends only on the
+// block size, so a row's result does not depend on what else is in the batch.
+__device__ inline float block_sum(float v, float* scratch) {
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int nwaves = (blockDim.x + kWave - 1) / kWave;
+  v = wave_sum(v);
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float total = 0.f;
+  for (int w = 0; w < nwaves; ++w) total += scratch[w];
+  return total;
+}
+__device__ inline float block_max(float v, float* scratch) {
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int nwaves = (blockDim.x + kWave - 1) / kWave;
+  v = wave_max(v);
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float m = scratch[0];
+  for (int w = 1; w < nwaves; ++w) m = fmaxf(m, scratch[w]);
+  return m;
+}
+
+// ---- host side --------------------------------------------------------------
+enum DType : int { kF32 = 0, kBF16 = 1 };
+
+// Records a message for bc4g_last_error() and returns a non-zero status.
+int fail(const char* fmt, ...);
+int check_launch(const char* what);
+
+inline int ceil_div(long a, long b) { return static_cast<int>((a + b - 1) / b); }
+
+}  // namespace bc4g
+
+#define BC4G_REQUIRE(cond, ...)                  \
+  do {                                           \
+    if (!(cond)) return bc4g::fail(__VA_ARGS__); \
+  } while (0)

@@ -1,0 +1,29 @@
+#include "common.h"
+
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "api.h"
+
+namespace bc4g {
+
+static thread_local char g_error[512] = "";
+
+int fail(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return 1;
+}
+
+int check_launch(const char* what) {
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail("%s: launch failed: %s", what, hipGetErrorString(e));
+  return 0;
+}
+
+}  // namespace bc4g
+
+extern "C" const char* bc4g_last_error() { return bc4g::g_error; }
+extern "C" int bc4g_version() { return 1; }

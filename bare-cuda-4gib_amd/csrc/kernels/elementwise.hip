@@ -1,0 +1,325 @@
+// Embedding gather, RMSNorm, SwiGLU, rotary positions + cache write, argmax
+// and sampling.  One instantiation per storage type; all arithmetic in float.
+#include <float.h>
+#include <math.h>
+
+#include "api.h"
+#include "common.h"
+
+namespace bc4g {
+namespace {
+
+constexpr int kBlock = 256;
+
+// ---- embedding -------------------------------------------------------------
+template <typename TT>
+__global__ void embed_gather_kernel(const TT* __restrict__ table, const int32_t* __restrict__ ids,
+                                    float* __restrict__ out, int hidden) {
+  const size_t row = blockIdx.x;
+  const TT* src = table + static_cast<size_t>(ids[row]) * hidden;
+  float* dst = out + row * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_float(src[i]);
+}
+
+// ---- RMSNorm ---------------------------------------------------------------
+// eps is added to the mean square; sum and rsqrt in float.
+template <typename TW, typename TO>
+__global__ void rmsnorm_kernel(const float* __restrict__ x, const int32_t* __restrict__ rows,
+                               const TW* __restrict__ w, TO* __restrict__ out, int hidden, float eps) {
+  __shared__ float scratch[16];
+  const size_t src_row = rows ? static_cast<size_t>(rows[blockIdx.x]) : blockIdx.x;
+  const float* xr = x + src_row * hidden;
+  TO* orow = out + static_cast<size_t>(blockIdx.x) * hidden;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    const float v = xr[i];
+    ss += v * v;
+  }
+  const float mean_sq = block_sum(ss, scratch) / static_cast<float>(hidden);
+  const float scale = 1.0f / sqrtf(mean_sq + eps);
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    orow[i] = from_float<TO>(xr[i] * scale * to_float(w[i]));
+  }
+}
+
+// ---- SwiGLU ----------------------------------------------------------------
+template <typename T>
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, long total, int inter) {
+  const long stride = static_cast<long>(blockDim.x) * gridDim.x;
+  for (long idx = blockIdx.x * static_cast<long>(blockDim.x) + threadIdx.x; idx < total; idx += stride) {
+    const long t = idx / inter;
+    const int i = static_cast<int>(idx - t * inter);
+    const float g = to_float(gu[t * 2 * inter + i]);
+    const float u = to_float(gu[t * 2 * inter + inter + i]);
+    out[idx] = from_float<T>((g / (1.0f + expf(-g))) * u);
+  }
+}
+
+// ---- rotary positions + cache write -----------------------------------------
+// One thread per (token, head among q|k|v, pair).  A pair is (i, i + rotary_dim/2)
+// for i < rotary_dim/2; dimensions at or beyond rotary_dim pass through, handled
+// by the threads with pair >= rotary_dim/2 as (lo = rotary_dim/2 + i .. ) below.
+template <typename T>
+__global__ void rope_kv_write_kernel(T* __restrict__ qkv, const int32_t* __restrict__ positions,
+                                     const int32_t* __restrict__ slot_map, T* __restrict__ k_cache,
+                                     T* __restrict__ v_cache, long total, int n_heads, int n_kv_heads,
+                                     int head_dim, int rotary_dim, float theta, int page_tokens,
+                                     int write_kv) {
+  const int half = head_dim / 2;          // threads per head: each moves two elements
+  const int rhalf = rotary_dim / 2;
+  const int heads_total = n_heads + 2 * n_kv_heads;
+  const long stride = static_cast<long>(blockDim.x) * gridDim.x;
+  for (long idx = blockIdx.x * static_cast<long>(blockDim.x) + threadIdx.x; idx < total; idx += stride) {
+    const int j = static_cast<int>(idx % half);
+    const long rest = idx / half;
+    const int head = static_cast<int>(rest % heads_total);
+    const long token = rest / heads_total;
+    T* base = qkv + (token * heads_total + head) * head_dim;
+
+    // Which two elements this thread owns: a rotated pair, or two pass-through elements.
+    int i0, i1;
+    bool rotate;
+    if (j < rhalf) {
+      i0 = j;
+      i1 = j + rhalf;
+      rotate = true;
+    } else {
+      i0 = rotary_dim + 2 * (j - rhalf);
+      i1 = i0 + 1;
+      rotate = false;
+    }
+    float a = to_float(base[i0]);
+    float b = to_float(base[i1]);
+    const bool is_v = head >= n_heads + n_kv_heads;
+    if (rotate && !is_v) {
+      const float inv_freq = 1.0f / powf(theta, (2.0f * static_cast<float>(j)) / static_cast<float>(rotary_dim));
+      const float angle = static_cast<float>(positions[token]) * inv_freq;
+      float s, c;
+      sincosf(angle, &s, &c);
+      const float lo = a, hi = b;
+      a = lo * c - hi * s;
+      b = hi * c + lo * s;
+    }
+    if (head < n_heads) {
+      base[i0] = from_float<T>(a);
+      base[i1] = from_float<T>(b);
+    } else if (write_kv) {
+      const int kvh = is_v ? head - n_heads - n_kv_heads : head - n_heads;
+      const int slot = slot_map[token];
+      const long page = slot / page_tokens, off = slot % page_tokens;
+      T* dst = (is_v ? v_cache : k_cache) + ((page * n_kv_heads + kvh) * page_tokens + off) * head_dim;
+      dst[i0] = from_float<T>(a);
+      dst[i1] = from_float<T>(b);
+    }
+  }
+}
+
+// ---- argmax ----------------------------------------------------------------
+__global__ void argmax_kernel(const float* __restrict__ logits, int32_t* __restrict__ out, int vocab) {
+  __shared__ float best_v[kBlock];
+  __shared__ int best_i[kBlock];
+  const float* row = logits + static_cast<size_t>(blockIdx.x) * vocab;
+  float v = -FLT_MAX;
+  int idx = vocab;  // empty marker: loses every tie against a real index
+  for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
+    const float x = row[i];
+    if (x > v) {
+      v = x;
+      idx = i;
+    }
+  }
+  best_v[threadIdx.x] = v;
+  best_i[threadIdx.x] = idx;
+  __syncthreads();
+  for (int h = blockDim.x / 2; h > 0; h >>= 1) {
+    if (threadIdx.x < h) {
+      const float ov = best_v[threadIdx.x + h];
+      const int oi = best_i[threadIdx.x + h];
+      if (ov > best_v[threadIdx.x] || (ov == best_v[threadIdx.x] && oi < best_i[threadIdx.x])) {
+        best_v[threadIdx.x] = ov;
+        best_i[threadIdx.x] = oi;
+      }
+    }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) out[blockIdx.x] = best_i[0] < vocab ? best_i[0] : 0;
+}
+
+// ---- temperature sampling --------------------------------------------------
+// Thread t owns the contiguous slice [t*chunk, (t+1)*chunk) of the vocabulary, so that the
+// walk "subtract weights in vocabulary order until the target goes negative" can be done
+// as: per-slice sums, a serial scan over the 256 slice sums, then a walk inside one slice.
+__global__ void sample_kernel(const float* __restrict__ logits, const float* __restrict__ temperature,
+                              const double* __restrict__ u, int32_t* __restrict__ out, int vocab) {
+  __shared__ float fscratch[16];
+  __shared__ double slice_sum[kBlock];
+  __shared__ float best_v[kBlock];
+  __shared__ int best_i[kBlock];
+  const float* row = logits + static_cast<size_t>(blockIdx.x) * vocab;
+  const int chunk = (vocab + kBlock - 1) / kBlock;
+  const int begin = min(vocab, static_cast<int>(threadIdx.x) * chunk);
+  const int end = min(vocab, begin + chunk);
+
+  float v = -FLT_MAX;
+  int idx = vocab;
+  for (int i = begin; i < end; ++i) {
+    if (row[i] > v) {
+      v = row[i];
+      idx = i;
+    }
+  }
+  best_v[threadIdx.x] = v;
+  best_i[threadIdx.x] = idx;
+  __syncthreads();
+  for (int h = kBlock / 2; h > 0; h >>= 1) {
+    if (threadIdx.x < h) {
+      const float ov = best_v[threadIdx.x + h];
+      const int oi = best_i[threadIdx.x + h];
+      if (ov > best_v[threadIdx.x] || (ov == best_v[threadIdx.x] && oi < best_i[threadIdx.x])) {
+        best_v[threadIdx.x] = ov;
+        best_i[threadIdx.x] = oi;
+      }
+    }
+    __syncthreads();
+  }
+  const float row_max = best_v[0];
+  const int arg = best_i[0] < vocab ? best_i[0] : 0;
+  (void)fscratch;
+  const float temp = temperature[blockIdx.x];
+  if (!(temp > 0.f)) {
+    if (threadIdx.x == 0) out[blockIdx.x] = arg;
+    return;
+  }
+  const float inv_t = 1.0f / temp;
+  double s = 0.0;
+  for (int i = begin; i < end; ++i) s += static_cast<double>(expf((row[i] - row_max) * inv_t));
+  slice_sum[threadIdx.x] = s;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    double total = 0.0;
+    for (int t = 0; t < kBlock; ++t) total += slice_sum[t];
+    double target = u[blockIdx.x] * total;
+    int result = arg;  // rounding may leave the target a hair above zero after the last token
+    for (int t = 0; t < kBlock; ++t) {
+      if (target - slice_sum[t] < 0.0) {
+        const int b = min(vocab, t * chunk), e = min(vocab, b + chunk);
+        for (int i = b; i < e; ++i) {
+          target -= static_cast<double>(expf((row[i] - row_max) * inv_t));
+          if (target < 0.0) {
+            result = i;
+            break;
+          }
+        }
+        break;
+      }
+      target -= slice_sum[t];
+    }
+    out[blockIdx.x] = result;
+  }
+}
+
+int grid_for(long total) {
+  long g = (total + kBlock - 1) / kBlock;
+  if (g < 1) g = 1;
+  if (g > 65535L * 16) g = 65535L * 16;
+  return static_cast<int>(g);
+}
+
+}  // namespace
+}  // namespace bc4g
+
+using namespace bc4g;
+
+extern "C" int bc4g_embed_gather(const void* table, int table_dtype, const int32_t* ids, float* out,
+                                 int n_tokens, int hidden, int vocab, void* stream) {
+  BC4G_REQUIRE(n_tokens >= 0 && hidden > 0 && vocab > 0, "embed_gather: bad sizes T=%d H=%d V=%d",
+               n_tokens, hidden, vocab);
+  if (n_tokens == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (table_dtype == kF32) {
+    embed_gather_kernel<float><<<n_tokens, kBlock, 0, s>>>(static_cast<const float*>(table), ids, out, hidden);
+  } else if (table_dtype == kBF16) {
+    embed_gather_kernel<bf16_t><<<n_tokens, kBlock, 0, s>>>(static_cast<const bf16_t*>(table), ids, out, hidden);
+  } else {
+    return fail("embed_gather: unknown table dtype %d", table_dtype);
+  }
+  return check_launch("embed_gather");
+}
+
+extern "C" int bc4g_rmsnorm(const float* x, const int32_t* rows, const void* w, int w_dtype, void* out,
+                            int out_dtype, int n_rows, int hidden, float eps, void* stream) {
+  BC4G_REQUIRE(n_rows >= 0 && hidden > 0, "rmsnorm: bad sizes rows=%d H=%d", n_rows, hidden);
+  if (n_rows == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+#define BC4G_RMS(TW, TO)                                                                         \
+  rmsnorm_kernel<TW, TO><<<n_rows, kBlock, 0, s>>>(x, rows, static_cast<const TW*>(w),           \
+                                                   static_cast<TO*>(out), hidden, eps)
+  if (w_dtype == kF32 && out_dtype == kF32) BC4G_RMS(float, float);
+  else if (w_dtype == kF32 && out_dtype == kBF16) BC4G_RMS(float, bf16_t);
+  else if (w_dtype == kBF16 && out_dtype == kF32) BC4G_RMS(bf16_t, float);
+  else if (w_dtype == kBF16 && out_dtype == kBF16) BC4G_RMS(bf16_t, bf16_t);
+  else return fail("rmsnorm: unknown dtypes w=%d out=%d", w_dtype, out_dtype);
+#undef BC4G_RMS
+  return check_launch("rmsnorm");
+}
+
+extern "C" int bc4g_swiglu(const void* gu, void* out, int dtype, int n_tokens, int inter, void* stream) {
+  BC4G_REQUIRE(n_tokens >= 0 && inter > 0, "swiglu: bad sizes T=%d I=%d", n_tokens, inter);
+  if (n_tokens == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const long total = static_cast<long>(n_tokens) * inter;
+  if (dtype == kF32) {
+    swiglu_kernel<float><<<grid_for(total), kBlock, 0, s>>>(static_cast<const float*>(gu),
+                                                            static_cast<float*>(out), total, inter);
+  } else if (dtype == kBF16) {
+    swiglu_kernel<bf16_t><<<grid_for(total), kBlock, 0, s>>>(static_cast<const bf16_t*>(gu),
+                                                             static_cast<bf16_t*>(out), total, inter);
+  } else {
+    return fail("swiglu: unknown dtype %d", dtype);
+  }
+  return check_launch("swiglu");
+}
+
+extern "C" int bc4g_rope_kv_write(void* qkv, int dtype, const int32_t* positions, const int32_t* slot_map,
+                                  void* k_cache, void* v_cache, int n_tokens, int n_heads, int n_kv_heads,
+                                  int head_dim, int rotary_dim, float theta, int page_tokens, int num_pages,
+                                  int write_kv, void* stream) {
+  BC4G_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads > 0, "rope_kv_write: bad sizes T=%d heads=%d/%d",
+               n_tokens, n_heads, n_kv_heads);
+  BC4G_REQUIRE(head_dim > 0 && head_dim % 2 == 0, "rope_kv_write: head_dim %d must be even", head_dim);
+  BC4G_REQUIRE(rotary_dim >= 0 && rotary_dim <= head_dim && rotary_dim % 2 == 0,
+               "rope_kv_write: rotary_dim %d must be even and at most head_dim %d", rotary_dim, head_dim);
+  BC4G_REQUIRE(!write_kv || (page_tokens > 0 && num_pages > 0 && k_cache && v_cache && slot_map),
+               "rope_kv_write: cache write asked for without a cache");
+  BC4G_REQUIRE(rotary_dim == 0 || (positions && theta > 0.f), "rope_kv_write: rotation needs positions and theta > 0");
+  if (n_tokens == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const long total = static_cast<long>(n_tokens) * (n_heads + 2 * n_kv_heads) * (head_dim / 2);
+  if (dtype == kF32) {
+    rope_kv_write_kernel<float><<<grid_for(total), kBlock, 0, s>>>(
+        static_cast<float*>(qkv), positions, slot_map, static_cast<float*>(k_cache),
+        static_cast<float*>(v_cache), total, n_heads, n_kv_heads, head_dim, rotary_dim, theta, page_tokens, write_kv);
+  } else if (dtype == kBF16) {
+    rope_kv_write_kernel<bf16_t><<<grid_for(total), kBlock, 0, s>>>(
+        static_cast<bf16_t*>(qkv), positions, slot_map, static_cast<bf16_t*>(k_cache),
+        static_cast<bf16_t*>(v_cache), total, n_heads, n_kv_heads, head_dim, rotary_dim, theta, page_tokens, write_kv);
+  } else {
+    return fail("rope_kv_write: unknown dtype %d", dtype);
+  }
+  return check_launch("rope_kv_write");
+}
+
+extern "C" int bc4g_argmax(const float* logits, int32_t* out, int n_rows, int vocab, void* stream) {
+  BC4G_REQUIRE(n_rows >= 0 && vocab > 0, "argmax: bad sizes rows=%d V=%d", n_rows, vocab);
+  if (n_rows == 0) return 0;
+  argmax_kernel<<<n_rows, kBlock, 0, static_cast<hipStream_t>(stream)>>>(logits, out, vocab);
+  return check_launch("argmax");
+}
+
+extern "C" int bc4g_sample(const float* logits, const float* temperature, const double* u, int32_t* out,
+                           int n_rows, int vocab, void* stream) {
+  BC4G_REQUIRE(n_rows >= 0 && vocab > 0, "sample: bad sizes rows=%d V=%d", n_rows, vocab);
+  if (n_rows == 0) return 0;
+  sample_kernel<<<n_rows, kBlock, 0, static_cast<hipStream_t>(stream)>>>(logits, temperature, u, out, vocab);
+  return check_launch("sample");
+}

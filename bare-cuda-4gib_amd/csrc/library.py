@@ -1,0 +1,70 @@
+"""Loads ``libbc4g.so`` through ctypes and declares its entry points."""
+from __future__ import annotations
+
+import ctypes
+import sys
+from ctypes import c_char_p, c_double, c_float, c_int, c_void_p
+from typing import Optional
+
+from ..errors import KernelError
+from . import build as _build
+
+_P = c_void_p
+_I = c_int
+_F = c_float
+
+# name -> argument types (every function returns int status, except where noted)
+_SIGNATURES = {
+    "bc4g_embed_gather": [_P, _I, _P, _P, _I, _I, _I, _P],
+    "bc4g_rmsnorm": [_P, _P, _P, _I, _P, _I, _I, _I, _F, _P],
+    "bc4g_gemm_generic": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _P],
+    "bc4g_swiglu": [_P, _P, _I, _I, _I, _P],
+    "bc4g_rope_kv_write": [_P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P],
+    "bc4g_attention_generic": [_P, _P, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _P],
+    "bc4g_argmax": [_P, _P, _I, _I, _P],
+    "bc4g_sample": [_P, _P, _P, _P, _I, _I, _P],
+}
+
+_lib: Optional[ctypes.CDLL] = None
+
+
+def load(build_if_missing: bool = True) -> ctypes.CDLL:
+    """The kernel library; compiled first if it has never been built.
+
+    Fails loudly (KernelError) if it cannot be had: there is no other
+    implementation of the kernels to fall back to.
+    """
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not _build.is_built():
+        if not build_if_missing:
+            raise KernelError(f"{_build.LIB_PATH} is not built; run __graft_entry__.build()")
+        _build.build(verbose=True)
+    elif _build.is_stale():
+        print(f"[bc4g] warning: {_build.LIB_PATH} is older than its sources; "
+              "run __graft_entry__.build() to rebuild", file=sys.stderr, flush=True)
+    try:
+        lib = ctypes.CDLL(_build.LIB_PATH)
+    except OSError as e:
+        raise KernelError(f"cannot load {_build.LIB_PATH}: {e}") from None
+    lib.bc4g_last_error.restype = c_char_p
+    lib.bc4g_last_error.argtypes = []
+    lib.bc4g_version.restype = c_int
+    for name, args in _SIGNATURES.items():
+        try:
+            fn = getattr(lib, name)
+        except AttributeError:
+            raise KernelError(f"{_build.LIB_PATH} lacks {name}; rebuild it with "
+                              "__graft_entry__.build()") from None
+        fn.argtypes = args
+        fn.restype = c_int
+    _lib = lib
+    return lib
+
+
+def call(name: str, *args) -> None:
+    lib = load()
+    status = getattr(lib, name)(*args)
+    if status != 0:
+        raise KernelError(lib.bc4g_last_error().decode("utf-8", "replace"))

@@ -1,0 +1,211 @@
+"""The kernels as functions of torch tensors.
+
+Each wrapper checks on the host that shapes, dtypes, devices and strides are
+what the kernel and its grid assume, then launches on torch's current stream.
+There is no other implementation behind these functions: without the kernel
+library, or on a CPU tensor, they raise.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+
+from ..errors import KernelError
+from . import library
+
+F32, BF16 = 0, 1
+_CODE = {torch.float32: F32, torch.bfloat16: BF16}
+
+
+def _code(t: torch.Tensor, what: str) -> int:
+    try:
+        return _CODE[t.dtype]
+    except KeyError:
+        raise KernelError(f"{what}: dtype {t.dtype} is not supported (float32 or bfloat16)") from None
+
+
+def _dev(what: str, *tensors: Optional[torch.Tensor]) -> None:
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise KernelError(f"{what}: tensors must be on the GPU (got {t.device}); there is no CPU path")
+        if not t.is_contiguous():
+            raise KernelError(f"{what}: tensors must be contiguous (got strides {t.stride()} for shape {tuple(t.shape)})")
+
+
+def _i32(what: str, name: str, t: torch.Tensor, n: int) -> None:
+    if t.dtype != torch.int32 or t.numel() < n:
+        raise KernelError(f"{what}: {name} must be int32 with at least {n} elements, got {t.dtype} x {t.numel()}")
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def embed_gather(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[t, :] = float(table[ids[t], :]); ids must already be known to lie in [0, vocab)."""
+    _dev("embed_gather", table, ids, out)
+    vocab, hidden = table.shape
+    n = ids.numel()
+    _i32("embed_gather", "ids", ids, n)
+    if out is None:
+        out = torch.empty((n, hidden), dtype=torch.float32, device=table.device)
+    elif out.dtype != torch.float32 or tuple(out.shape) != (n, hidden):
+        raise KernelError(f"embed_gather: out must be float32 [{n}, {hidden}]")
+    library.call("bc4g_embed_gather", _ptr(table), _code(table, "embed_gather"), _ptr(ids), _ptr(out),
+                 n, hidden, vocab, _stream())
+    return out
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
+            rows: Optional[torch.Tensor] = None, n_rows: Optional[int] = None) -> torch.Tensor:
+    """RMSNorm of rows of the float residual stream x [T, H]; with ``rows`` (int32
+    indices, the first n_rows are used) only those rows are normed."""
+    _dev("rmsnorm", x, weight, rows)
+    if x.dtype != torch.float32 or x.dim() != 2:
+        raise KernelError(f"rmsnorm: x must be float32 [T, H], got {x.dtype} {tuple(x.shape)}")
+    hidden = x.shape[1]
+    if tuple(weight.shape) != (hidden,):
+        raise KernelError(f"rmsnorm: weight must be [{hidden}], got {tuple(weight.shape)}")
+    if rows is None:
+        n = x.shape[0]
+    else:
+        n = rows.numel() if n_rows is None else n_rows
+        _i32("rmsnorm", "rows", rows, n)
+    out = torch.empty((n, hidden), dtype=out_dtype, device=x.device)
+    library.call("bc4g_rmsnorm", _ptr(x), _ptr(rows), _ptr(weight), _code(weight, "rmsnorm"), _ptr(out),
+                 _code(out, "rmsnorm"), n, hidden, float(eps), _stream())
+    return out
+
+
+def gemm_generic(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = None,
+                 accumulate_into: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """a [M, K] times w [N, K] transposed, in plain float arithmetic.  With
+    ``accumulate_into`` (float32 [M, N]) the product is added to it in place."""
+    _dev("gemm", a, w, accumulate_into)
+    if a.dim() != 2 or w.dim() != 2 or a.shape[1] != w.shape[1]:
+        raise KernelError(f"gemm: shapes {tuple(a.shape)} x {tuple(w.shape)}^T do not match")
+    m, k = a.shape
+    n = w.shape[0]
+    if accumulate_into is not None:
+        out = accumulate_into
+        if out.dtype != torch.float32 or tuple(out.shape) != (m, n):
+            raise KernelError(f"gemm: accumulate_into must be float32 [{m}, {n}], got {out.dtype} {tuple(out.shape)}")
+    else:
+        out = torch.empty((m, n), dtype=out_dtype or a.dtype, device=a.device)
+    library.call("bc4g_gemm_generic", _ptr(a), _code(a, "gemm"), _ptr(w), _code(w, "gemm"), _ptr(out),
+                 _code(out, "gemm"), 1 if accumulate_into is not None else 0, m, n, k, _stream())
+    return out
+
+
+def swiglu(gu: torch.Tensor) -> torch.Tensor:
+    """gu [T, 2I] = gate | up  ->  silu(gate) * up, [T, I]."""
+    _dev("swiglu", gu)
+    if gu.dim() != 2 or gu.shape[1] % 2:
+        raise KernelError(f"swiglu: input must be [T, 2I], got {tuple(gu.shape)}")
+    t, inter = gu.shape[0], gu.shape[1] // 2
+    out = torch.empty((t, inter), dtype=gu.dtype, device=gu.device)
+    library.call("bc4g_swiglu", _ptr(gu), _ptr(out), _code(gu, "swiglu"), t, inter, _stream())
+    return out
+
+
+def _check_cache(what: str, cache: torch.Tensor, n_kv_heads: int, head_dim: int, dtype: torch.dtype):
+    if cache.dim() != 4 or cache.shape[1] != n_kv_heads or cache.shape[3] != head_dim or cache.dtype != dtype:
+        raise KernelError(f"{what}: cache must be {dtype} [pages, {n_kv_heads}, page_tokens, {head_dim}], "
+                          f"got {cache.dtype} {tuple(cache.shape)}")
+
+
+def rope_kv_write(qkv: torch.Tensor, positions: Optional[torch.Tensor], slot_map: Optional[torch.Tensor],
+                  k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor], n_heads: int,
+                  n_kv_heads: int, head_dim: int, rotary_dim: int, theta: float, write_kv: bool = True) -> None:
+    """Rotate q (in place) and k, write k and v into their pages."""
+    _dev("rope_kv_write", qkv, positions, slot_map, k_cache, v_cache)
+    t = qkv.shape[0]
+    width = (n_heads + 2 * n_kv_heads) * head_dim
+    if qkv.dim() != 2 or qkv.shape[1] != width:
+        raise KernelError(f"rope_kv_write: qkv must be [T, {width}], got {tuple(qkv.shape)}")
+    if positions is not None:
+        _i32("rope_kv_write", "positions", positions, t)
+    page_tokens = num_pages = 0
+    if write_kv:
+        _check_cache("rope_kv_write", k_cache, n_kv_heads, head_dim, qkv.dtype)
+        _check_cache("rope_kv_write", v_cache, n_kv_heads, head_dim, qkv.dtype)
+        if k_cache.shape != v_cache.shape:
+            raise KernelError("rope_kv_write: k and v caches differ in shape")
+        _i32("rope_kv_write", "slot_map", slot_map, t)
+        num_pages, page_tokens = k_cache.shape[0], k_cache.shape[2]
+    library.call("bc4g_rope_kv_write", _ptr(qkv), _code(qkv, "rope_kv_write"), _ptr(positions), _ptr(slot_map),
+                 _ptr(k_cache), _ptr(v_cache), t, n_heads, n_kv_heads, head_dim, rotary_dim, float(theta),
+                 page_tokens, num_pages, 1 if write_kv else 0, _stream())
+
+
+def attention_generic(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                      block_table: torch.Tensor, row_seq: torch.Tensor, positions: torch.Tensor,
+                      n_heads: int, n_kv_heads: int, head_dim: int, window: int = 0,
+                      scale: Optional[float] = None) -> torch.Tensor:
+    """Causal attention of every row over its request's cache; returns [T, n_heads*head_dim]."""
+    _dev("attention", qkv, k_cache, v_cache, block_table, row_seq, positions)
+    t = qkv.shape[0]
+    width = (n_heads + 2 * n_kv_heads) * head_dim
+    if qkv.dim() != 2 or qkv.shape[1] != width:
+        raise KernelError(f"attention: qkv must be [T, {width}], got {tuple(qkv.shape)}")
+    _check_cache("attention", k_cache, n_kv_heads, head_dim, qkv.dtype)
+    _check_cache("attention", v_cache, n_kv_heads, head_dim, qkv.dtype)
+    if block_table.dim() != 2 or block_table.dtype != torch.int32:
+        raise KernelError("attention: block_table must be int32 [requests, pages]")
+    _i32("attention", "row_seq", row_seq, t)
+    _i32("attention", "positions", positions, t)
+    out = torch.empty((t, n_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
+    library.call("bc4g_attention_generic", _ptr(qkv), _ptr(out), _code(qkv, "attention"), _ptr(k_cache),
+                 _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(row_seq), _ptr(positions), t,
+                 n_heads, n_kv_heads, head_dim, k_cache.shape[2], k_cache.shape[0], int(window),
+                 float(scale if scale is not None else 1.0 / math.sqrt(head_dim)), _stream())
+    return out
+
+
+def argmax(logits: torch.Tensor) -> torch.Tensor:
+    """Lowest index of each row's maximum, int32 [rows]."""
+    _dev("argmax", logits)
+    if logits.dtype != torch.float32 or logits.dim() != 2:
+        raise KernelError("argmax: logits must be float32 [rows, vocab]")
+    out = torch.empty((logits.shape[0],), dtype=torch.int32, device=logits.device)
+    library.call("bc4g_argmax", _ptr(logits), _ptr(out), logits.shape[0], logits.shape[1], _stream())
+    return out
+
+
+def sample(logits: torch.Tensor, temperature: torch.Tensor, u: torch.Tensor) -> torch.Tensor:
+    """One draw per row from softmax(logits / temperature) by inverse CDF with the given
+    uniform u in [0, 1); rows with temperature <= 0 get the argmax."""
+    _dev("sample", logits, temperature, u)
+    rows = logits.shape[0]
+    if logits.dtype != torch.float32 or logits.dim() != 2:
+        raise KernelError("sample: logits must be float32 [rows, vocab]")
+    if temperature.dtype != torch.float32 or temperature.numel() != rows:
+        raise KernelError("sample: temperature must be float32 [rows]")
+    if u.dtype != torch.float64 or u.numel() != rows:
+        raise KernelError("sample: u must be float64 [rows]")
+    out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    library.call("bc4g_sample", _ptr(logits), _ptr(temperature), _ptr(u), _ptr(out), rows, logits.shape[1], _stream())
+    return out
+
+
+def gemm_fast(a: torch.Tensor, w: torch.Tensor, out_dtype=None,
+              accumulate_into: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """The matrix-core product where a kernel takes these operands, else None
+    (the caller then uses the plain float kernel)."""
+    return None
+
+
+def attention(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
+              ctx, n_heads: int, n_kv_heads: int, head_dim: int, window: int, scale: float) -> torch.Tensor:
+    """Attention of a step's rows over the cache: picks the kernel for the
+    batch's shape (prompt portions, decoded tokens, or both)."""
+    return attention_generic(qkv, k_cache, v_cache, block_table, ctx.row_seq, ctx.positions,
+                             n_heads, n_kv_heads, head_dim, window, scale)

@@ -1,0 +1,147 @@
+"""A model: parts built from a ModelSpec, weights bound to them, and the
+forward pass over one step's batch.  Nothing here names an architecture."""
+from __future__ import annotations
+
+from typing import Dict, Hashable, List, Optional, Tuple
+
+import torch
+
+from ..config.registry import load_config
+from ..errors import ConfigError
+from ..parts.base import Part, build_part
+from ..weights.loader import WeightSpec, load_weights
+from .batch import StepContext
+from .runtime import Runtime
+from .spec import ModelSpec, PartSpec
+
+
+def _walk(part: Part):
+    yield part
+    for child in part.children():
+        yield from _walk(child)
+
+
+class _Bound:
+    """A built part with the file names of its tensors."""
+    def __init__(self, part: Part, spec: PartSpec):
+        self.part, self.spec = part, spec
+
+    def names(self) -> Dict[str, Tuple[str, WeightSpec]]:
+        return {local: (self.spec.prefix + self.spec.rename.get(local, local), ws)
+                for local, ws in self.part.weight_specs().items()}
+
+
+class Model:
+    def __init__(self, spec: ModelSpec):
+        self.spec = spec
+        self.embedding = _Bound(build_part("embedding", spec.embedding), spec.embedding)
+        self.final_norm = _Bound(build_part("norm", spec.final_norm), spec.final_norm)
+        self.head = _Bound(build_part("head", spec.head), spec.head)
+        self.layers: List[Part] = []
+        self._layer_bound: List[List[_Bound]] = []
+        for ls in spec.layers:
+            mixer = _Bound(build_part("mixer", ls.mixer), ls.mixer)
+            ffn = _Bound(build_part("feedforward", ls.ffn), ls.ffn)
+            n1 = _Bound(build_part("norm", ls.mixer_norm), ls.mixer_norm)
+            n2 = _Bound(build_part("norm", ls.ffn_norm), ls.ffn_norm)
+            block = build_part("block", PartSpec(ls.block, dict(
+                mixer=mixer.part, ffn=ffn.part, mixer_norm=n1.part, ffn_norm=n2.part)))
+            self.layers.append(block)
+            self._layer_bound.append([n1, mixer, n2, ffn])
+        self.schedule = list(spec.schedule)
+        for e in self.schedule:
+            if not (0 <= e.layer < len(self.layers)):
+                raise ConfigError(f"schedule names layer {e.layer}, the model has {len(self.layers)}")
+        self.vocab_size = spec.vocab_size
+        self.hidden_size = spec.hidden_size
+        self.max_seq_len = spec.max_seq_len
+        self.rt: Optional[Runtime] = None
+
+    # ---- weights ------------------------------------------------------------
+    def _all_bound(self) -> List[_Bound]:
+        out = [self.embedding]
+        for group in self._layer_bound:
+            out.extend(group)
+        out.extend([self.final_norm, self.head])
+        return out
+
+    def expected_weights(self) -> Dict[str, WeightSpec]:
+        """File tensor name -> what the configuration needs of it."""
+        out: Dict[str, WeightSpec] = {}
+        for b in self._all_bound():
+            for local, (name, ws) in b.names().items():
+                if name in out and out[name].shape != ws.shape:
+                    raise ConfigError(f"tensor '{name}' is wanted in two shapes")
+                out[name] = ws
+        return out
+
+    def bind(self, tensors: Dict[str, torch.Tensor], rt: Runtime) -> None:
+        """Place the loaded tensors on the device and hand each part its own."""
+        self.rt = rt
+        placed: Dict[str, torch.Tensor] = {}
+
+        def get(name: str) -> Optional[torch.Tensor]:
+            if name not in placed and name in tensors:
+                placed[name] = rt.place_weight(tensors[name])
+            return placed.get(name)
+
+        for b in self._all_bound():
+            mine = {}
+            for local, (name, ws) in b.names().items():
+                t = get(name)
+                if t is None:
+                    tied = getattr(b.part, "tied_to", None)
+                    t = get(tied) if tied else None
+                    if t is None:
+                        raise ConfigError(f"tensor '{name}' was not loaded")
+                mine[local] = t
+            b.part.bind(mine, rt)
+        self.weight_bytes = sum(t.numel() * t.element_size() for t in placed.values())
+
+    # ---- cache --------------------------------------------------------------
+    def cache_streams(self) -> Dict[Hashable, object]:
+        """Cache stream id -> spec, from the schedule: the entry that writes a
+        stream decides its spec; an entry may only read a stream that some
+        entry writes."""
+        streams: Dict[Hashable, object] = {}
+        for e in self.schedule:
+            if e.cache is None or not e.writes:
+                continue
+            spec = self.layers[e.layer].mixer.cache_spec()
+            if e.cache in streams and streams[e.cache] != spec:
+                raise ConfigError(f"cache stream {e.cache!r} is written with two different specs")
+            streams[e.cache] = spec
+        for e in self.schedule:
+            if e.cache is not None and e.cache not in streams:
+                raise ConfigError(f"schedule entry for layer {e.layer} reads cache stream {e.cache!r}, "
+                                  "which no entry writes")
+        return streams
+
+    # ---- forward ------------------------------------------------------------
+    def forward(self, ctx: StepContext) -> Optional[torch.Tensor]:
+        """Run the batch through every schedule entry; float32 logits at the
+        wanted rows ([n_logits, vocab]), or None if none are wanted."""
+        x = self.embedding.part.forward(ctx)
+        for e in self.schedule:
+            self.layers[e.layer].forward(x, ctx, ctx.cache(e.cache), e.writes)
+        if ctx.n_logits == 0:
+            return None
+        h = self.final_norm.part.forward(x, ctx, rows=ctx.logit_rows, n_rows=ctx.n_logits)
+        return self.head.part.forward(h)
+
+
+def expected_weights(spec: ModelSpec) -> Dict[str, WeightSpec]:
+    return Model(spec).expected_weights()
+
+
+IGNORED_TENSORS = ("*.rotary_emb.inv_freq",)   # a buffer some checkpoints carry; recomputed here
+
+
+def load_model(model_dir: str, dtype, device="cuda:0") -> Tuple[Model, object]:
+    """(model with weights on the device, typed configuration) of a model folder."""
+    from .runtime import parse_dtype
+    arch, cfg = load_config(model_dir)
+    model = Model(arch.describe(cfg))
+    tensors = load_weights(model_dir, model.expected_weights(), ignore=IGNORED_TENSORS)
+    model.bind(tensors, Runtime(torch.device(device), parse_dtype(dtype)))
+    return model, cfg

@@ -1,0 +1,66 @@
+"""Parts and their registry.
+
+A part is built from its sizes and constants alone (``PartSpec.params``); it
+declares the tensors it needs, receives them once they are on the device, and
+runs on whatever batch it is handed.  No part knows which model it is in.
+
+Interfaces, by category (``ctx`` is the step's StepContext, ``x`` the float32
+residual stream [T, hidden], ``h`` an activation [T, hidden] in the runtime's
+activation dtype):
+
+norm         forward(x, ctx, rows=None, n_rows=None) -> h       (rows: int32 row indices)
+position     fused() -> (rotary_dim, theta) for the fused rotate-and-store kernel, or
+             None, in which case apply(qkv, ctx, n_heads, n_kv_heads, head_dim) rotates
+             q and k in place
+mixer        cache_spec() -> PagedKV | FixedState | None
+             forward(h, ctx, cache_view, residual, writes) -- adds its output to residual
+feedforward  forward(h, ctx, residual) -- adds its output to residual
+block        built from (mixer, ffn, mixer_norm, ffn_norm); forward(x, ctx, cache_view, writes)
+embedding    forward(ctx) -> x
+head         forward(h) -> float32 logits [rows, vocab]
+"""
+from __future__ import annotations
+
+from typing import Any, Callable, Dict, List
+
+import torch
+
+from ..errors import ConfigError
+from ..weights.loader import WeightSpec
+
+_REGISTRY: Dict[str, Dict[str, Callable[..., "Part"]]] = {}
+
+
+class Part:
+    """Base of every part.  Subclasses set ``category``."""
+    category = ""
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        """Own tensor name (e.g. ``q_proj.weight``) -> what is expected of it."""
+        return {}
+
+    def bind(self, tensors: Dict[str, torch.Tensor], rt) -> None:
+        """Receive the tensors (on the device) and pack them for the kernels."""
+
+    def children(self) -> List["Part"]:
+        return []
+
+
+def register_part(category: str, kind: str, factory: Callable[..., Part], *, replace: bool = False) -> None:
+    """Make ``kind`` buildable: ``factory(**params)`` returns the part."""
+    table = _REGISTRY.setdefault(category, {})
+    if kind in table and not replace:
+        raise ConfigError(f"{category} part '{kind}' is already registered")
+    table[kind] = factory
+
+
+def registered_parts(category: str) -> List[str]:
+    return sorted(_REGISTRY.get(category, {}))
+
+
+def build_part(category: str, spec) -> Part:
+    table = _REGISTRY.get(category, {})
+    if spec.kind not in table:
+        raise ConfigError(f"no {category} part named '{spec.kind}'; registered: "
+                          f"{', '.join(sorted(table)) or 'none'}")
+    return table[spec.kind](**spec.params)
