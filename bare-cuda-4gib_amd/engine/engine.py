@@ -1,0 +1,199 @@
+"""The Python entry point, in the manner of the reference's ``llm_engine_py.Engine``
+(server/bindings.cc:70-107 over engine/src/async_engine.cpp): the same
+constructor arguments, ``submit / cancel / poll / stop / stats`` and the same
+properties, events as ``(id, token, index, finish)`` tuples and submit results as
+``(status, message)`` with status ``ok | invalid | busy | unavailable``.
+
+The reference runs the scheduler on a worker thread; here ``poll`` runs one
+scheduler step on the caller's thread when there is work, so the GPU is only
+ever touched by the thread that polls.
+"""
+from __future__ import annotations
+
+import collections
+import dataclasses
+from typing import Deque, Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+from ..errors import EngineError
+from ..sampling.device import DevicePicker
+from ..sampling.params import SamplingParams
+from .executor import Executor, StepEntry
+from .model import load_model
+from .scheduler import (FINISH_CANCELLED, FINISH_ERROR, Request, Scheduler, TokenEvent)
+
+Event = Tuple[int, int, int, str]
+
+
+def fit_kv_pages(model, max_tokens: int, max_seqs: int, page_tokens: int, dtype: torch.dtype,
+                 device, headroom_bytes: int = 1 << 30) -> int:
+    """Pages for every request to reach max_tokens, or as many as free memory
+    (less a headroom) holds (reference: fit_kv_pages, engine/src/model.cpp:259-277)."""
+    per_request = -(-max_tokens // page_tokens)
+    want = per_request * max_seqs
+    elem = 2 if dtype == torch.bfloat16 else 4
+    per_page = 0
+    for spec in model.cache_streams().values():
+        if hasattr(spec, "num_kv_heads"):
+            per_page += 2 * spec.num_kv_heads * spec.head_dim * page_tokens * elem
+    if per_page == 0:
+        return want
+    free, _ = torch.cuda.mem_get_info(device)
+    fit = max(0, (free - headroom_bytes)) // per_page
+    if fit < per_request:
+        raise EngineError(f"free GPU memory holds {fit} cache pages, one request of {max_tokens} tokens "
+                          f"needs {per_request}")
+    return int(min(want, fit))
+
+
+class Engine:
+    def __init__(self, model_path: str, max_tokens: int = 1024, max_seqs: int = 8, kv_pages: int = 0,
+                 max_waiting: int = 64, *, dtype: str = "bfloat16", device: str = "cuda:0",
+                 page_tokens: int = 64, max_batch_tokens: int = 2048, prefill_chunk: int = 512):
+        if max_tokens <= 0 or max_seqs <= 0:
+            raise EngineError("max_tokens and max_seqs must be positive")
+        self.model, self.config = load_model(model_path, dtype, device)
+        if max_tokens > self.model.max_seq_len:
+            raise EngineError(f"max_tokens {max_tokens} is beyond the model's {self.model.max_seq_len} positions")
+        rt = self.model.rt
+        if kv_pages <= 0:
+            kv_pages = fit_kv_pages(self.model, max_tokens, max_seqs, page_tokens, rt.act_dtype, rt.device)
+        self.executor = Executor(self.model, num_pages=kv_pages, max_requests=max_seqs,
+                                 max_tokens=max_tokens, page_tokens=page_tokens,
+                                 max_batch_tokens=max_batch_tokens)
+        self.scheduler = Scheduler(self.executor, DevicePicker(), max_batch_tokens=max_batch_tokens,
+                                   prefill_chunk=prefill_chunk)
+        self._max_waiting = max_waiting
+        self._outbox: Deque[Event] = collections.deque()
+        self._live = set()
+        self._failure = ""
+        self._stopped = False
+        self._injected = ""
+
+    # ---- properties ---------------------------------------------------------
+    @property
+    def healthy(self) -> bool:
+        return not self._failure
+
+    @property
+    def failure(self) -> str:
+        return self._failure
+
+    @property
+    def max_tokens(self) -> int:
+        return self.scheduler.limits.max_tokens
+
+    @property
+    def max_seqs(self) -> int:
+        return self.scheduler.limits.max_seqs
+
+    @property
+    def kv_pages(self) -> int:
+        return self.scheduler.limits.kv_pages
+
+    @property
+    def vocab_size(self) -> int:
+        return self.model.vocab_size
+
+    # ---- requests -----------------------------------------------------------
+    def submit(self, id: int, prompt: Sequence[int], max_new_tokens: int, stop_ids: Sequence[int] = (),
+               temperature: float = 0.0, top_p: float = 1.0, top_k: int = 0, seed: int = -1,
+               timeout_ms: int = 0) -> Tuple[str, str]:
+        """Queues a request; returns (status, message).  temperature 0 is greedy."""
+        request = Request(id=id, prompt=list(prompt), max_new_tokens=max_new_tokens, stop_ids=list(stop_ids),
+                          sampling=SamplingParams(temperature, top_p, top_k, seed), timeout_ms=timeout_ms)
+        error = self.scheduler.check(request)
+        if error:
+            return "invalid", error
+        if self._failure:
+            return "unavailable", "engine failed: " + self._failure
+        if self._stopped:
+            return "unavailable", "engine is stopping"
+        if self._max_waiting > 0 and len(self._live) >= self.max_seqs + self._max_waiting:
+            return "busy", "too many requests waiting"
+        if id in self._live:
+            return "invalid", "request id is already in use"
+        self._live.add(id)
+        self.scheduler.submit(request)
+        return "ok", ""
+
+    def cancel(self, id: int) -> None:
+        """Ends a request early; it then gets one last event with finish 'cancelled'."""
+        if id in self._live and self.scheduler.cancel(id):
+            self._publish([TokenEvent(id, -1, -1, FINISH_CANCELLED)])
+
+    def poll(self, timeout_ms: int = 100) -> List[Event]:
+        """Runs scheduler steps until there are events (or nothing is left to do) and returns
+        them: a list of (id, token, index, finish) tuples."""
+        while not self._outbox and not self._failure and not self._stopped and not self.scheduler.idle():
+            try:
+                if self._injected:
+                    raise EngineError(self._injected)
+                self._publish(self.scheduler.step())
+            except Exception as e:   # every live request ends with 'error'; the engine refuses new work
+                self._fail_all(str(e))
+        out = list(self._outbox)
+        self._outbox.clear()
+        return out
+
+    def stop(self) -> None:
+        """Waiting and running requests are dropped."""
+        self._stopped = True
+        for r in list(self.scheduler.running) + list(self.scheduler.waiting):
+            self.scheduler.cancel(r.id)
+        self._live.clear()
+
+    def stats(self) -> Dict[str, object]:
+        return dataclasses.asdict(self.scheduler.stats())
+
+    def _fail_for_test(self, message: str) -> None:
+        """Makes the next poll fail, to exercise the failure path."""
+        self._injected = message
+
+    # ---- the step function, for programs that bring their own tokens ------------
+    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        for e in entries:
+            if not self.executor.has(e.request):
+                self.executor.admit(e.request)
+        return self.executor.step(entries)
+
+    def release(self, request) -> None:
+        self.executor.release(request)
+
+    # ---- internals -----------------------------------------------------------
+    def _publish(self, events: List[TokenEvent]) -> None:
+        for e in events:
+            if e.finish:
+                self._live.discard(e.id)
+            self._outbox.append((e.id, e.token, e.index, e.finish))
+
+    def _fail_all(self, message: str) -> None:
+        self._failure = message
+        for id in sorted(self._live):
+            self._outbox.append((id, -1, -1, FINISH_ERROR))
+        self._live.clear()
+
+
+def generate_batch(engine: Engine, prompts: Sequence[Sequence[int]], max_new_tokens: int,
+                   **sampling) -> List[List[int]]:
+    """All prompts through the scheduler, ids 0..n-1 (reference: Model::generate_batch,
+    engine/src/model.cpp:693-717)."""
+    out: List[List[int]] = [[] for _ in prompts]
+    for i, p in enumerate(prompts):
+        status, message = engine.submit(i, p, max_new_tokens, **sampling)
+        if status != "ok":
+            raise EngineError(f"prompt {i}: {message}")
+    done = 0
+    while done < len(prompts):
+        events = engine.poll()
+        if not events and engine.scheduler.idle():
+            break
+        for id, token, index, finish in events:
+            if token >= 0:
+                out[id].append(token)
+            if finish:
+                if finish == "error":
+                    raise EngineError(engine.failure)
+                done += 1
+    return out

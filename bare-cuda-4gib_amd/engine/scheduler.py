@@ -1,0 +1,308 @@
+"""Continuous batching above the step function.
+
+What it keeps of the reference's scheduler (engine/include/llm/scheduler.h:15-129,
+engine/src/scheduler.cpp:28-208): requests with ``id, prompt, max_new_tokens,
+stop_ids, sampling, timeout_ms``; the same refusals in ``check``; FIFO admission
+in which a request that does not fit blocks the ones behind it; a stop id ends a
+request and *is* emitted; ``target = min(max_new_tokens, max_tokens - prompt + 1)``
+(the last generated token is never run through the model); per-request random
+generators; TokenEvent and the stats' names.
+
+What it does differently: the reference runs each admitted prompt whole and
+alone and then one decode pass; here every step is ONE batch under a token
+budget -- one token for every request that is decoding, then portions of
+prompts (at most ``prefill_chunk`` tokens of a request a step) in admission
+order.  And pages are not promised for a request's whole run at admission:
+they are taken as tokens arrive.  When a step's tokens do not fit the pool,
+the request admitted last is preempted: its pages are given back and it goes to
+the front of the waiting line with the tokens it has generated so far appended
+to its prompt, to be recomputed later (its generator state and its count of
+generated tokens are kept, so its output is unchanged).  A request that could
+never fit the pool alone is refused at ``check``.
+"""
+from __future__ import annotations
+
+import collections
+import dataclasses
+import time
+from typing import Deque, Dict, Hashable, List, Optional, Sequence
+
+from ..errors import EngineError, OutOfPages
+from ..sampling.mt19937_64 import MT19937_64
+from ..sampling.params import SamplingParams, check_sampling, seed_for
+from .executor import StepEntry
+
+FINISH_NONE, FINISH_STOP, FINISH_LENGTH = "", "stop", "length"
+FINISH_CANCELLED, FINISH_TIMEOUT, FINISH_ERROR = "cancelled", "timeout", "error"
+
+
+@dataclasses.dataclass
+class Request:
+    id: int = 0
+    prompt: Sequence[int] = ()
+    max_new_tokens: int = 16
+    stop_ids: Sequence[int] = ()          # generating any of these ends the request, e.g. EOS
+    sampling: SamplingParams = dataclasses.field(default_factory=SamplingParams)
+    timeout_ms: int = 0                   # from submit, waiting plus running; 0 never times out
+
+
+@dataclasses.dataclass
+class TokenEvent:
+    """One generated token, or a request ending without one (token -1)."""
+    id: int = 0
+    token: int = -1
+    index: int = -1                       # position among this request's generated tokens
+    finish: str = FINISH_NONE
+
+
+@dataclasses.dataclass
+class EngineLimits:
+    max_tokens: int = 0                   # per request, prompt plus generated
+    max_seqs: int = 0
+    kv_pages: int = 0
+    page_tokens: int = 64
+
+
+@dataclasses.dataclass
+class SchedulerStats:
+    running: int = 0
+    waiting: int = 0
+    kv_pages_used: int = 0
+    kv_pages_total: int = 0
+    steps: int = 0                        # batches run
+    prefill_tokens: int = 0               # prompt tokens run through the model (recomputed ones included)
+    decode_tokens: int = 0                # rows decoded, one per decoding request per step
+    preemptions: int = 0
+    busy_seconds: float = 0.0
+
+
+class _Live:
+    """A request that has been submitted: waiting, or running with a cache slot."""
+    def __init__(self, request: Request, deadline: float):
+        self.id = request.id
+        self.tokens: List[int] = [int(t) for t in request.prompt]   # prompt + generated so far
+        self.prompt_len = len(self.tokens)
+        self.computed = 0                 # tokens whose keys are in the cache
+        self.generated = 0
+        self.target = 0
+        self.stop_ids = set(int(s) for s in request.stop_ids)
+        self.sampling = request.sampling
+        self.rng = MT19937_64(seed_for(request.sampling))
+        self.deadline = deadline
+        self.admitted_at = -1             # admission counter; the largest is preempted first
+
+
+def target_tokens(limits: EngineLimits, prompt_len: int, max_new_tokens: int) -> int:
+    return min(max_new_tokens, limits.max_tokens - prompt_len + 1)
+
+
+def pages_needed(limits: EngineLimits, prompt_len: int, max_new_tokens: int) -> int:
+    cached = prompt_len + target_tokens(limits, prompt_len, max_new_tokens) - 1
+    return -(-cached // limits.page_tokens)
+
+
+def check_request(limits: EngineLimits, request: Request) -> str:
+    """Empty if the request can ever run, else why not."""
+    n = len(request.prompt)
+    if n == 0:
+        return "empty prompt"
+    if request.max_new_tokens <= 0:
+        return "max_new_tokens must be positive"
+    if n > limits.max_tokens:
+        return f"prompt has {n} tokens, the engine holds {limits.max_tokens} per sequence"
+    pages = pages_needed(limits, n, request.max_new_tokens)
+    if pages > limits.kv_pages:
+        return f"request needs {pages} KV pages, the pool holds {limits.kv_pages}"
+    return check_sampling(request.sampling)
+
+
+class Scheduler:
+    """Not thread-safe; one thread calls everything.
+
+    executor: the step function and its cache (``step, admit, release, has,
+    cache``).  picker: chooses tokens from logits rows (``pick(logits, params,
+    rngs) -> ids``).  max_batch_tokens: rows a step may hold.  prefill_chunk:
+    the most prompt tokens of one request in one step.
+    """
+
+    def __init__(self, executor, picker, *, max_batch_tokens: int = 2048, prefill_chunk: int = 512,
+                 clock=time.monotonic):
+        if max_batch_tokens <= 0 or prefill_chunk <= 0:
+            raise EngineError("scheduler: max_batch_tokens and prefill_chunk must be positive")
+        self.executor = executor
+        self.picker = picker
+        self.max_batch_tokens = max_batch_tokens
+        self.prefill_chunk = prefill_chunk
+        self._clock = clock
+        cache = executor.cache
+        pools = [g.pool.num_pages for g in cache.groups.values()]
+        self.limits = EngineLimits(max_tokens=cache.max_tokens, max_seqs=cache.max_requests,
+                                   kv_pages=min(pools) if pools else 1 << 30, page_tokens=cache.page_tokens)
+        self.waiting: Deque[_Live] = collections.deque()
+        self.running: List[_Live] = []
+        self._admissions = 0
+        self._totals = SchedulerStats()
+        self.vocab_size = getattr(getattr(executor, "model", None), "vocab_size", None)
+
+    # ---- submitting and cancelling ---------------------------------------------
+    def check(self, request: Request) -> str:
+        error = check_request(self.limits, request)
+        if error:
+            return error
+        if self.vocab_size is not None:
+            for t in request.prompt:
+                if not (0 <= int(t) < self.vocab_size):
+                    return f"token id {t} is outside the vocabulary [0, {self.vocab_size})"
+        return ""
+
+    def submit(self, request: Request) -> None:
+        error = self.check(request)
+        if error:
+            raise EngineError(f"scheduler: request {request.id}: {error}")
+        if any(r.id == request.id for r in self.waiting) or any(r.id == request.id for r in self.running):
+            raise EngineError(f"scheduler: request {request.id}: id is already live")
+        deadline = self._clock() + request.timeout_ms / 1000.0 if request.timeout_ms > 0 else float("inf")
+        live = _Live(request, deadline)
+        live.target = target_tokens(self.limits, live.prompt_len, request.max_new_tokens)
+        self.waiting.append(live)
+
+    def cancel(self, request_id) -> bool:
+        """Drops a waiting or running request and frees what it holds.  False if unknown."""
+        for r in self.waiting:
+            if r.id == request_id:
+                self.waiting.remove(r)
+                return True
+        for r in self.running:
+            if r.id == request_id:
+                self._retire(r)
+                self.running.remove(r)
+                return True
+        return False
+
+    def idle(self) -> bool:
+        return not self.waiting and not self.running
+
+    def stats(self) -> SchedulerStats:
+        s = dataclasses.replace(self._totals)
+        s.running, s.waiting = len(self.running), len(self.waiting)
+        s.kv_pages_used = self.executor.cache.pages_in_use()
+        s.kv_pages_total = self.executor.cache.pages_total()
+        return s
+
+    # ---- one step ---------------------------------------------------------------
+    def step(self) -> List[TokenEvent]:
+        start = self._clock()
+        try:
+            return self._run_step()
+        finally:
+            self._totals.busy_seconds += self._clock() - start
+
+    def _retire(self, r: _Live) -> None:
+        if self.executor.has(r.id):
+            self.executor.release(r.id)
+
+    def _expire(self, events: List[TokenEvent]) -> None:
+        now = self._clock()
+        for r in [r for r in self.waiting if r.deadline <= now]:
+            self.waiting.remove(r)
+            events.append(TokenEvent(r.id, -1, -1, FINISH_TIMEOUT))
+        for r in [r for r in self.running if r.deadline <= now]:
+            self._retire(r)
+            self.running.remove(r)
+            events.append(TokenEvent(r.id, -1, -1, FINISH_TIMEOUT))
+
+    def _preempt_latest(self) -> bool:
+        """Give back everything the request admitted last holds and put it at the front of
+        the waiting line, to be recomputed.  False if at most one request is running (a lone
+        request always fits: check() saw to that)."""
+        if len(self.running) <= 1:
+            return False
+        victim = max(self.running, key=lambda r: r.admitted_at)
+        self.running.remove(victim)
+        self._retire(victim)
+        victim.computed = 0
+        self.waiting.appendleft(victim)
+        self._totals.preemptions += 1
+        return True
+
+    def plan(self) -> List[tuple]:
+        """Decide this step's batch: [(live request, number of its next tokens)].  Admits
+        waiting requests (taking their slot) and preempts running ones as needed; touches no
+        pages."""
+        cache = self.executor.cache
+        preempted = False
+        while True:
+            budget = self.max_batch_tokens
+            batch: List[tuple] = []
+            # 1. one token for every request that is decoding
+            for r in self.running:
+                if len(r.tokens) - r.computed == 1 and budget > 0:
+                    batch.append((r, 1))
+                    budget -= 1
+            # 2. portions of the prompts of running requests, in admission order
+            for r in sorted(self.running, key=lambda r: r.admitted_at):
+                left = len(r.tokens) - r.computed
+                if left > 1 and budget > 0:
+                    n = min(left, self.prefill_chunk, budget)
+                    batch.append((r, n))
+                    budget -= n
+            if cache.can_reserve([(r.id, n) for r, n in batch]):
+                break
+            if not self._preempt_latest():
+                raise OutOfPages("scheduler: a lone request does not fit the page pool")
+            preempted = True
+        # 3. admit waiting requests in order; one that does not fit blocks those behind it
+        #    (not in a step that had to preempt: the pool is full)
+        while not preempted and self.waiting and budget > 0 and cache.free_slots > 0:
+            r = self.waiting[0]
+            n = min(len(r.tokens) - r.computed, self.prefill_chunk, budget)
+            self.executor.admit(r.id)
+            if not cache.can_reserve([(q.id, m) for q, m in batch] + [(r.id, n)]):
+                self.executor.release(r.id)
+                break
+            self.waiting.popleft()
+            r.admitted_at = self._admissions
+            self._admissions += 1
+            self.running.append(r)
+            batch.append((r, n))
+            budget -= n
+        return batch
+
+    def _run_step(self) -> List[TokenEvent]:
+        events: List[TokenEvent] = []
+        self._expire(events)
+        batch = self.plan()
+        if not batch:
+            return events
+        entries, wanted = [], []
+        for r, n in batch:
+            last = r.computed + n == len(r.tokens)
+            entries.append(StepEntry(r.id, r.tokens[r.computed:r.computed + n], [n - 1] if last else []))
+            if last:
+                wanted.append(r)
+            if n == 1 and r.computed >= r.prompt_len:
+                self._totals.decode_tokens += 1
+            else:
+                self._totals.prefill_tokens += n
+        logits = self.executor.step(entries)
+        self._totals.steps += 1
+        for r, n in batch:
+            r.computed += n
+        if wanted:
+            tokens = self.picker.pick(logits, [r.sampling for r in wanted], [r.rng for r in wanted])
+            for r, token in zip(wanted, tokens):
+                self._emit(r, int(token), events)
+        return events
+
+    def _emit(self, r: _Live, token: int, events: List[TokenEvent]) -> None:
+        e = TokenEvent(r.id, token, r.generated)
+        r.generated += 1
+        r.tokens.append(token)
+        if token in r.stop_ids:
+            e.finish = FINISH_STOP
+        elif r.generated == r.target:
+            e.finish = FINISH_LENGTH
+        events.append(e)
+        if e.finish != FINISH_NONE:
+            self._retire(r)
+            self.running.remove(r)

@@ -141,11 +141,11 @@ class PlainLlama:
             assert self.tied, "no lm_head.weight and embeddings are not tied"
             self.w["lm_head.weight"] = self.w["model.embed_tokens.weight"]
 
-    def hidden_states(self, ids: Sequence[int]) -> torch.Tensor:
+    def hidden_states(self, ids: Sequence[int], position_offset: int = 0) -> torch.Tensor:
         w = self.w
         ids_t = torch.tensor(list(ids), dtype=torch.long)
         t = len(ids)
-        positions = torch.arange(t)
+        positions = torch.arange(t) + position_offset
         x = embedding(w["model.embed_tokens.weight"], ids_t)
         for i in range(self.layers):
             p = f"model.layers.{i}."
@@ -162,9 +162,9 @@ class PlainLlama:
             x = x + a @ w[p + "mlp.down_proj.weight"].T
         return x
 
-    def logits(self, ids: Sequence[int]) -> torch.Tensor:
+    def logits(self, ids: Sequence[int], position_offset: int = 0) -> torch.Tensor:
         """[T, vocab] logits at every position of the sequence."""
-        x = self.hidden_states(ids)
+        x = self.hidden_states(ids, position_offset)
         return rmsnorm(x, self.w["model.norm.weight"], self.eps) @ self.w["lm_head.weight"].T
 
     def greedy(self, prompt: Sequence[int], steps: int) -> List[int]:

@@ -1,0 +1,228 @@
+"""The scheduler's decisions, on the host, with a stand-in for the step function whose logits
+depend only on a request's own tokens (so outputs must not depend on batching, portions or
+preemption).  Scenarios after engine/tests/test_scheduler.cu:122-255."""
+import hashlib
+
+import numpy as np
+import pytest
+import torch
+
+from bare_cuda_4gib_amd.cache import CacheManager, PagedKV
+from bare_cuda_4gib_amd.engine.scheduler import Request, Scheduler, check_request, EngineLimits
+from bare_cuda_4gib_amd.errors import EngineError
+from bare_cuda_4gib_amd.sampling import SamplingParams, sample_token
+
+VOCAB = 50
+
+
+def fake_logits(tokens):
+    digest = hashlib.sha256(np.asarray(tokens, dtype=np.int64).tobytes()).digest()
+    rng = np.random.default_rng(int.from_bytes(digest[:8], "little"))
+    return rng.normal(size=VOCAB).astype(np.float32) * 3.0
+
+
+class FakeExecutor:
+    """Keeps a real cache manager (so pages run out for real) and checks that tokens arrive in
+    order, each exactly once per (re)computation."""
+    def __init__(self, num_pages=8, page_tokens=4, max_requests=3, max_tokens=32):
+        self.cache = CacheManager({0: PagedKV(1, 2)}, page_tokens=page_tokens, num_pages=num_pages,
+                                  max_requests=max_requests, max_tokens=max_tokens, dtype=torch.float32, device="cpu")
+        self.history = {}
+        self.batches = []
+
+    def admit(self, rid):
+        self.history[rid] = []
+        return self.cache.admit(rid)
+
+    def release(self, rid):
+        self.cache.release(rid)
+        del self.history[rid]
+
+    def has(self, rid):
+        return self.cache.has(rid)
+
+    def step(self, entries):
+        self.cache.reserve([(e.request, len(e.tokens)) for e in entries])
+        self.batches.append([(e.request, len(e.tokens)) for e in entries])
+        rows = []
+        for e in entries:
+            assert len(self.history[e.request]) == self.cache.length(e.request)
+            self.history[e.request].extend(e.tokens)
+            self.cache.advance(e.request, len(e.tokens))
+            for w in e.want:
+                rows.append(fake_logits(self.history[e.request][:self.cache.length(e.request) - len(e.tokens) + w + 1]))
+        return torch.tensor(np.stack(rows)) if rows else None
+
+
+class HostPicker:
+    def pick(self, logits, params, rngs):
+        return [sample_token(logits[i].numpy(), p, r) for i, (p, r) in enumerate(zip(params, rngs))]
+
+
+def expected_greedy(prompt, n, stop=()):
+    tokens, out = list(prompt), []
+    for _ in range(n):
+        t = int(np.argmax(fake_logits(tokens)))
+        out.append(t)
+        tokens.append(t)
+        if t in stop:
+            break
+    return out
+
+
+def run(sched, max_steps=500):
+    out, finish = {}, {}
+    for _ in range(max_steps):
+        if sched.idle():
+            break
+        for e in sched.step():
+            if e.token >= 0:
+                assert e.index == len(out.setdefault(e.id, []))
+                out[e.id].append(e.token)
+            if e.finish:
+                finish[e.id] = e.finish
+    assert sched.idle()
+    return out, finish
+
+
+def make(**kw):
+    sched_kw = {k: kw.pop(k) for k in ("max_batch_tokens", "prefill_chunk", "clock") if k in kw}
+    ex = FakeExecutor(**kw)
+    return Scheduler(ex, HostPicker(), **{"max_batch_tokens": 16, "prefill_chunk": 6, **sched_kw}), ex
+
+
+def prompt(n, seed):
+    return [int(x) for x in np.random.default_rng(seed).integers(0, VOCAB, n)]
+
+
+def test_outputs_do_not_depend_on_batching_and_budget_is_kept():
+    sched, ex = make(num_pages=24)
+    prompts = {i: prompt(n, i) for i, n in enumerate([5, 13, 1, 9, 7])}
+    for i, p in prompts.items():
+        sched.submit(Request(id=i, prompt=p, max_new_tokens=6))
+    out, finish = run(sched)
+    for i, p in prompts.items():
+        assert out[i] == expected_greedy(p, 6) and finish[i] == "length"
+    for batch in ex.batches:
+        assert sum(n for _, n in batch) <= 16 and all(n <= 6 for _, n in batch)
+        assert len(batch) <= 3                                         # slots
+    assert any(len(b) > 1 and any(n > 1 for _, n in b) and any(n == 1 for _, n in b) for b in ex.batches), \
+        "portions of prompts beside decoded tokens were expected in one batch"
+    s = sched.stats()
+    assert s.prefill_tokens == sum(len(p) for p in prompts.values()) and s.decode_tokens == 5 * 5
+    assert s.kv_pages_used == 0 and s.running == 0 and s.waiting == 0 and s.preemptions == 0
+    assert ex.cache.free_slots == 3
+
+
+def test_admission_is_in_order_and_the_head_blocks():
+    sched, ex = make(num_pages=4, max_tokens=16, prefill_chunk=16, max_batch_tokens=32)   # 16 tokens of pool
+    sched.submit(Request(id=0, prompt=prompt(9, 0), max_new_tokens=2))    # 3 pages
+    sched.submit(Request(id=1, prompt=prompt(9, 1), max_new_tokens=2))    # 3 pages: must wait for 0 to end
+    sched.submit(Request(id=2, prompt=prompt(2, 2), max_new_tokens=2))    # would fit beside 0, but waits behind 1
+    first_seen = []
+    while not sched.idle():
+        sched.step()
+        for rid, _ in ex.batches[-1]:
+            if rid not in first_seen:
+                first_seen.append(rid)
+    assert first_seen == [0, 1, 2]
+    assert all(0 not in [r for r, _ in b] or 1 not in [r for r, _ in b] for b in ex.batches)
+
+
+def test_stop_ids_budgets_and_prefill_only():
+    sched, _ = make()
+    p = prompt(7, 3)
+    free_run = expected_greedy(p, 7)
+    stop = free_run[3]
+    sched.submit(Request(id=0, prompt=p, max_new_tokens=7))
+    sched.submit(Request(id=1, prompt=p, max_new_tokens=7, stop_ids=[stop]))
+    sched.submit(Request(id=2, prompt=p, max_new_tokens=1))
+    out, finish = run(sched)
+    assert out[0] == free_run and finish[0] == "length"
+    first = free_run.index(stop)
+    assert out[1] == free_run[:first + 1] and finish[1] == "stop"         # the stop token is emitted
+    assert out[2] == free_run[:1] and finish[2] == "length"
+
+
+def test_target_is_capped_by_max_tokens():
+    sched, _ = make(num_pages=8, max_tokens=12)
+    p = prompt(10, 4)
+    sched.submit(Request(id=0, prompt=p, max_new_tokens=50))
+    out, finish = run(sched)
+    assert len(out[0]) == 12 - 10 + 1 and finish[0] == "length"           # the last token is never cached
+
+
+def test_check_refusals():
+    limits = EngineLimits(max_tokens=32, max_seqs=3, kv_pages=4, page_tokens=4)
+    assert check_request(limits, Request(prompt=[], max_new_tokens=1)) == "empty prompt"
+    assert "positive" in check_request(limits, Request(prompt=[1], max_new_tokens=0))
+    assert "holds 32 per sequence" in check_request(limits, Request(prompt=[1] * 33, max_new_tokens=1))
+    assert "KV pages" in check_request(limits, Request(prompt=[1] * 10, max_new_tokens=8))
+    assert check_request(limits, Request(prompt=[1] * 10, max_new_tokens=7)) == ""
+    assert "top_p" in check_request(limits, Request(prompt=[1], max_new_tokens=1, sampling=SamplingParams(top_p=0.0)))
+    sched, _ = make()
+    with pytest.raises(EngineError):
+        sched.submit(Request(id=0, prompt=[], max_new_tokens=1))
+    sched.submit(Request(id=0, prompt=[1], max_new_tokens=1))
+    with pytest.raises(EngineError):
+        sched.submit(Request(id=0, prompt=[1], max_new_tokens=1))          # id already live
+
+
+def test_cancel_running_and_waiting():
+    sched, ex = make(max_requests=1)
+    sched.submit(Request(id=0, prompt=prompt(4, 0), max_new_tokens=20))
+    sched.submit(Request(id=1, prompt=prompt(4, 1), max_new_tokens=3))
+    sched.step(), sched.step()
+    assert sched.cancel(1) and sched.cancel(0) and not sched.cancel(5)
+    assert sched.idle() and ex.cache.pages_in_use() == 0 and ex.cache.free_slots == 1
+
+
+def test_sampling_seeds():
+    def sample_run(seed, others=0, temperature=0.9, top_p=1.0):
+        sched, _ = make(num_pages=24)
+        sched.submit(Request(id=0, prompt=prompt(5, 9), max_new_tokens=8,
+                             sampling=SamplingParams(temperature=temperature, top_p=top_p, seed=seed)))
+        for j in range(others):
+            sched.submit(Request(id=10 + j, prompt=prompt(6, 20 + j), max_new_tokens=8,
+                                 sampling=SamplingParams(temperature=1.3, seed=99 + j)))
+        return run(sched)[0][0]
+    assert sample_run(7) == sample_run(7, others=2)                       # alone == batched
+    assert sample_run(7) != sample_run(8)
+    assert sample_run(7, top_p=1e-6) == expected_greedy(prompt(5, 9), 8)  # a vanishing nucleus is greedy
+
+
+def test_timeouts_with_a_stepped_clock():
+    now = [0.0]
+    sched, ex = make(max_requests=1, clock=lambda: now[0])
+    sched.submit(Request(id=0, prompt=prompt(4, 0), max_new_tokens=30, timeout_ms=50))
+    sched.submit(Request(id=1, prompt=prompt(4, 1), max_new_tokens=2, timeout_ms=20))   # expires while waiting
+    sched.submit(Request(id=2, prompt=prompt(4, 2), max_new_tokens=2))
+    sched.step()
+    now[0] = 0.03
+    events = sched.step()
+    assert [(e.id, e.token, e.finish) for e in events if e.finish] == [(1, -1, "timeout")]
+    now[0] = 0.06
+    events = sched.step()
+    assert (0, -1, "timeout") in [(e.id, e.token, e.finish) for e in events]
+    tokens = [e.token for e in events if e.id == 2]
+    while not sched.idle():
+        tokens += [e.token for e in sched.step() if e.id == 2]
+    assert tokens == expected_greedy(prompt(4, 2), 2) and ex.cache.pages_in_use() == 0
+
+
+def test_when_pages_run_out_the_latest_request_is_recomputed():
+    # 3 requests of 6 + 10 tokens each need 4 pages each at the end; the pool has 9.
+    sched, ex = make(num_pages=9, max_tokens=32)
+    prompts = {i: prompt(6, 30 + i) for i in range(3)}
+    for i, p in prompts.items():
+        sched.submit(Request(id=i, prompt=p, max_new_tokens=10, sampling=SamplingParams(temperature=0.7, seed=i)))
+    out, finish = run(sched)
+    assert sched.stats().preemptions >= 1
+    ref_sched, _ = make(num_pages=24, max_tokens=32)
+    for i, p in prompts.items():
+        ref_sched.submit(Request(id=i, prompt=p, max_new_tokens=10, sampling=SamplingParams(temperature=0.7, seed=i)))
+    ref_out, _ = run(ref_sched)
+    assert out == ref_out and set(finish.values()) == {"length"}
+    assert ex.cache.pages_in_use() == 0 and ex.cache.free_slots == 3
+    assert max(g.pool.high_water_mark for g in ex.cache.groups.values()) <= 9
+    assert sched.stats().prefill_tokens > 18                              # recomputed tokens are counted
