@@ -1,0 +1,194 @@
+"""Decode and prefill throughput of the engine on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--dtype bf16]
+
+The default run has the layer sizes of TinyLlama-1.1B (22 layers, hidden 2048, 32 query heads /
+4 key-value heads, head size 64, feed-forward 5632, vocabulary 32000, context 2048) with random
+weights, a batch of 8 requests with 512-token prompts, and times K decode steps (each step: one
+token for every request through the engine's step function, greedy choice on the device, the
+chosen ids read back).  It prints ONE JSON line: decoded tokens a second, the prefill of one
+2,048-token prompt, the decode step against the HBM roofline, and decoding at batch 1 and 64.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0                       # MI355X: 8 TB/s
+PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3}
+TINYLLAMA = dict(architectures=["LlamaForCausalLM"], model_type="llama", vocab_size=32000, hidden_size=2048,
+                 num_hidden_layers=22, num_attention_heads=32, num_key_value_heads=4, head_dim=64,
+                 intermediate_size=5632, rope_theta=10000.0, rms_norm_eps=1e-5,
+                 max_position_embeddings=2048, tie_word_embeddings=False)
+FULL_LAYERS = 22
+BASELINE_DECODE_B1 = 77.3                   # the reference's only FP16 decode number (batch 1, RTX 3050)
+
+
+def build_model(layers, dtype, seed=0):
+    import torch
+    from bare_cuda_4gib_amd.config import architecture_for
+    from bare_cuda_4gib_amd.engine import Model, Runtime, parse_dtype
+    from bare_cuda_4gib_amd.weights.random_device import random_tensors_on_device
+    raw = dict(TINYLLAMA, num_hidden_layers=layers)
+    arch = architecture_for(raw)
+    cfg = arch.config_class.from_dict(raw)
+    model = Model(arch.describe(cfg))
+    tdtype = parse_dtype(dtype)
+    tensors = random_tensors_on_device(model.expected_weights(), seed, tdtype, "cuda:0")
+    model.bind(tensors, Runtime(torch.device("cuda:0"), tdtype))
+    return model, cfg
+
+
+def linear_params(cfg):
+    """Weights of the linear maps of one layer, and of the output head."""
+    h, q, kv, i = cfg.hidden_size, cfg.num_heads * cfg.head_dim, cfg.num_kv_heads * cfg.head_dim, cfg.intermediate_size
+    return h * (q + 2 * kv) + q * h + 3 * h * i, cfg.vocab_size * h
+
+
+def decode_bytes(cfg, elem, contexts):
+    """Bytes one decode step has to read: every weight it uses once (linear maps, norms, the
+    embedding rows of the batch) and the cached keys and values of the live requests."""
+    per_layer, head = linear_params(cfg)
+    weights = (cfg.num_layers * (per_layer + 2 * cfg.hidden_size) + head + cfg.hidden_size) * elem
+    weights += len(contexts) * cfg.hidden_size * elem
+    kv = sum(contexts) * cfg.num_layers * 2 * cfg.num_kv_heads * cfg.head_dim * elem
+    return weights + kv
+
+
+def prefill_flops(cfg, t):
+    per_layer, head = linear_params(cfg)
+    linear = 2.0 * t * cfg.num_layers * per_layer + 2.0 * head       # logits at the last place only
+    attn = cfg.num_layers * 4.0 * cfg.num_heads * cfg.head_dim * (t * (t + 1) / 2.0)
+    return linear + attn
+
+
+def run_decode(model, cfg, batch, prompt_len, steps, warmup, seed=1):
+    """(seconds for `steps` decode steps, context lengths at the middle of the timed region)."""
+    import torch
+    from bare_cuda_4gib_amd.csrc import ops
+    from bare_cuda_4gib_amd.engine import Executor, StepEntry
+    total = prompt_len + warmup + steps + 1
+    page = 64
+    pages_each = -(-total // page)
+    ex = Executor(model, num_pages=pages_each * batch, max_requests=batch, max_tokens=pages_each * page,
+                  page_tokens=page)
+    gen = torch.Generator().manual_seed(seed)
+    last = []
+    for b in range(batch):
+        ex.admit(b)
+        prompt = torch.randint(0, cfg.vocab_size, (prompt_len,), generator=gen).tolist()
+        logits = ex.step([StepEntry(b, prompt, [prompt_len - 1])])
+        last.append(int(ops.argmax(logits)[0]))
+
+    def one_step(tokens):
+        logits = ex.step([StepEntry(b, [tokens[b]], [0]) for b in range(batch)])
+        return ops.argmax(logits).tolist()
+
+    for _ in range(warmup):
+        last = one_step(last)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        last = one_step(last)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    mid = prompt_len + warmup + steps // 2
+    for b in range(batch):
+        ex.release(b)
+    del ex
+    torch.cuda.empty_cache()
+    return dt, [mid] * batch
+
+
+def run_prefill(model, cfg, tokens, runs=3, seed=2):
+    import torch
+    from bare_cuda_4gib_amd.engine import Executor, StepEntry
+    page = 64
+    ex = Executor(model, num_pages=-(-tokens // page), max_requests=1, max_tokens=-(-tokens // page) * page,
+                  page_tokens=page)
+    gen = torch.Generator().manual_seed(seed)
+    prompt = torch.randint(0, cfg.vocab_size, (tokens,), generator=gen).tolist()
+    best = float("inf")
+    for i in range(runs + 1):
+        ex.admit("p")
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        ex.step([StepEntry("p", prompt, [tokens - 1])])
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        ex.release("p")
+        if i > 0:
+            best = min(best, dt)
+    del ex
+    torch.cuda.empty_cache()
+    return best
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--prompt-len", type=int, default=512)
+    ap.add_argument("--prefill-tokens", type=int, default=2048)
+    ap.add_argument("--layers", type=int, default=FULL_LAYERS, help="fewer than 22 only where time needs it")
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
+    ap.add_argument("--no-points", action="store_true", help="skip decoding at batch 1 and 64")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+
+    import torch
+    from bare_cuda_4gib_amd.csrc import library
+    library.load()
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dtype = "bfloat16" if args.dtype == "bf16" else "float32"
+    elem = 2 if args.dtype == "bf16" else 4
+    model, cfg = build_model(args.layers, dtype)
+
+    dt, contexts = run_decode(model, cfg, args.batch, args.prompt_len, args.steps, args.warmup)
+    ms_per_step = dt / args.steps * 1e3
+    value = args.batch * args.steps / dt
+    achieved = decode_bytes(cfg, elem, contexts) / (dt / args.steps) / 1e9
+
+    pre_s = run_prefill(model, cfg, args.prefill_tokens)
+    pre_frac = prefill_flops(cfg, args.prefill_tokens) / pre_s / (PEAK_TFLOPS[args.dtype] * 1e12)
+
+    points = {}
+    if not args.no_points:
+        for b in (1, 64):
+            steps_b = max(16, args.steps // 2)
+            dtb, _ = run_decode(model, cfg, b, args.prompt_len, steps_b, max(4, args.warmup // 2))
+            points[f"decode_b{b}"] = round(b * steps_b / dtb, 1)
+
+    line = {
+        "metric": "decode tok/s at batch 1/8/64; prefill tok/s at 2,048 tokens",
+        "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": round(points.get("decode_b1", 0.0) / BASELINE_DECODE_B1, 2) if points else None,
+        "dtype": args.dtype, "data": "synthetic: random weights N(0, 0.02), uniform random token ids",
+        "config": {"model": "TinyLlama-1.1B shape", "layers": args.layers, "layers_full": FULL_LAYERS,
+                   "hidden": cfg.hidden_size, "heads": cfg.num_heads, "kv_heads": cfg.num_kv_heads,
+                   "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
+                   "global_batch": args.batch, "seq_len": cfg.max_seq_len, "prompt_len": args.prompt_len,
+                   "page_tokens": 64, "parallelism": "single GPU",
+                   "vs_baseline_is": "decode_b1 / 77.3 tok/s (reference, FP16, batch 1, RTX 3050)"},
+        "prefill": {"value": round(args.prefill_tokens / pre_s, 1), "tokens": args.prefill_tokens,
+                    "ms": round(pre_s * 1e3, 3), "frac": round(pre_frac, 4)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4)},
+        "points": points,
+    }
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
