@@ -8,7 +8,8 @@ one page pool and one block table per request; streams with a window of W
 tokens share another, whose pages are given back once a request's window has
 passed them.  Within a group one page index stands for the same ``page_tokens``
 tokens in every stream of the group, each stream having storage of its own
-shape ``[pages, kv_heads, page_tokens, head_dim]`` for keys and for values.
+shape ``[pages, kv_heads, page_tokens, head_dim]`` for keys and, transposed,
+``[pages, kv_heads, head_dim, page_tokens]`` for values.
 Streams whose spec is :class:`FixedState` get a tensor ``[max_requests,
 *shape]``; a request's row is its slot, zeroed at admission.
 
@@ -38,7 +39,7 @@ _STATE_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "int32": 
 class PagedView:
     """What a mixer sees of its paged stream."""
     k: torch.Tensor            # [pages, kv_heads, page_tokens, head_dim]
-    v: torch.Tensor
+    v: torch.Tensor            # [pages, kv_heads, head_dim, page_tokens]
     group: Hashable            # key of the group whose block table addresses it
     page_tokens: int
     window: int
@@ -90,9 +91,11 @@ class CacheManager:
                 if group is None:
                     group = self.groups[key] = _Group(spec.window, num_pages)
                 group.streams.append(sid)
-                shape = (num_pages, spec.num_kv_heads, page_tokens, spec.head_dim)
-                k = torch.empty(shape, dtype=dtype, device=self.device)
-                v = torch.empty(shape, dtype=dtype, device=self.device)
+                k = torch.empty((num_pages, spec.num_kv_heads, page_tokens, spec.head_dim),
+                                dtype=dtype, device=self.device)
+                # values are kept transposed (consecutive tokens of one dimension lie together)
+                v = torch.empty((num_pages, spec.num_kv_heads, spec.head_dim, page_tokens),
+                                dtype=dtype, device=self.device)
                 if poison:
                     k.fill_(float("nan"))
                     v.fill_(float("nan"))

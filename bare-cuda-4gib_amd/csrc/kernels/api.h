@@ -33,7 +33,9 @@ int bc4g_swiglu(const void* gu, void* out, int dtype, int n_tokens, int inter, v
 // Rotates q (in place) and k by each row's position, and writes k and v into
 // their cache pages (rope.cu:18-55, kv_cache_write.cu:10-20).
 // qkv: [n_tokens, (n_heads + 2 n_kv_heads) * head_dim]; slot_map[t] = page * page_tokens +
-// offset of the row's token; k_cache/v_cache: [pages, n_kv_heads, page_tokens, head_dim].
+// offset of the row's token; k_cache: [pages, n_kv_heads, page_tokens, head_dim]; v_cache is kept
+// transposed, [pages, n_kv_heads, head_dim, page_tokens], so that the matrix-core kernels can load
+// consecutive tokens of one dimension.
 // rotary_dim 0 switches the rotation off; write_kv 0 leaves the cache alone.
 int bc4g_rope_kv_write(void* qkv, int dtype, const int32_t* positions, const int32_t* slot_map,
                        void* k_cache, void* v_cache, int n_tokens, int n_heads, int n_kv_heads,
@@ -58,4 +60,31 @@ int bc4g_argmax(const float* logits, int32_t* out, int n_rows, int vocab, void* 
 // vocabulary in order (engine/src/sampler.cpp:39-61); temperature <= 0 gives the argmax.
 int bc4g_sample(const float* logits, const float* temperature, const double* u, int32_t* out,
                 int n_rows, int vocab, void* stream);
+}
+
+extern "C" {
+// bfloat16 x [m, k] (m <= 64) times bfloat16 w [n, k] transposed, weights streamed once through
+// the matrix cores.  epilogue: 0 store bfloat16 [m, n]; 1 store float32; 2 add into float32;
+// 3 SwiGLU: w = gate rows then up rows (n = 2 * inter), out bfloat16 [m, inter] = silu(gate) * up.
+int bc4g_gemm_skinny(const void* x, const void* w, void* out, int epilogue, int m, int n, int k, void* stream);
+}
+
+extern "C" {
+// Attention on the matrix cores (bfloat16): see attention_mfma.hip.  tile_start[s] is the first
+// 16-row tile of request s when every request's rows are cut into tiles of tokens_per_tile tokens
+// (times the query heads of one key/value head); n_tiles their total.  With n_splits > 1 the keys
+// are cut into that many parts whose float partials (part_o [n_splits, T, heads, d], part_ml
+// [n_splits, T, heads, 2]) are merged into out.
+int bc4g_attention_mfma(const void* qkv, void* out, float* part_o, float* part_ml, const void* k_cache,
+                        const void* v_cache, const int32_t* block_table, int table_stride,
+                        const int32_t* seq_start, const int32_t* seq_ctx, const int32_t* tile_start,
+                        int n_seqs, int n_tiles, int n_tokens, int n_heads, int n_kv_heads, int head_dim,
+                        int page_tokens, int window, float scale, int tokens_per_tile, int n_splits,
+                        void* stream);
+}
+
+extern "C" {
+// bfloat16 a [m, k] times bfloat16 w [n, k] transposed on the matrix cores, any m.
+// epilogue: 0 store bfloat16; 1 store float32; 2 add into float32.
+int bc4g_gemm_mfma(const void* a, const void* w, void* out, int epilogue, int m, int n, int k, void* stream);
 }

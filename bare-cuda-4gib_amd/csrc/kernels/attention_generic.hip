@@ -66,12 +66,12 @@ __global__ __launch_bounds__(kWave) void attention_generic_kernel(
     for (int jj = 0; jj < n_here; ++jj) {
       const int jk = j0 + jj;
       const long page = table[jk / page_tokens];
-      const T* vrow = v_cache + ((page * n_kv_heads + kvh) * page_tokens + jk % page_tokens) * head_dim;
+      const T* vcol = v_cache + (page * n_kv_heads + kvh) * head_dim * page_tokens + jk % page_tokens;
       const float pj = p_s[jj];
 #pragma unroll
       for (int i = 0; i < kDimsPerLane; ++i) {
         const int c = lane + i * kWave;
-        if (c < head_dim) acc[i] = fmaf(pj, to_float(vrow[c]), acc[i]);
+        if (c < head_dim) acc[i] = fmaf(pj, to_float(vcol[static_cast<long>(c) * page_tokens]), acc[i]);
       }
     }
     __syncthreads();

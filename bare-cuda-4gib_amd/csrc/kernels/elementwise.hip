@@ -107,9 +107,15 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const int32_t* __restr
       const int kvh = is_v ? head - n_heads - n_kv_heads : head - n_heads;
       const int slot = slot_map[token];
       const long page = slot / page_tokens, off = slot % page_tokens;
-      T* dst = (is_v ? v_cache : k_cache) + ((page * n_kv_heads + kvh) * page_tokens + off) * head_dim;
-      dst[i0] = from_float<T>(a);
-      dst[i1] = from_float<T>(b);
+      if (is_v) {  // values are kept transposed: [page][kv head][dim][token]
+        T* dst = v_cache + (page * n_kv_heads + kvh) * head_dim * page_tokens + off;
+        dst[static_cast<long>(i0) * page_tokens] = from_float<T>(a);
+        dst[static_cast<long>(i1) * page_tokens] = from_float<T>(b);
+      } else {     // keys: [page][kv head][token][dim]
+        T* dst = k_cache + ((page * n_kv_heads + kvh) * page_tokens + off) * head_dim;
+        dst[i0] = from_float<T>(a);
+        dst[i1] = from_float<T>(b);
+      }
     }
   }
 }

@@ -1,0 +1,143 @@
+// out[m, n] (+)= sum_k a[m, k] * w[n, k], bfloat16 operands, float accumulation on the matrix
+// cores: the product of prompt portions (many rows).
+//
+// A workgroup of 4 waves computes a 128 x 128 tile of the output in k-steps of 64.  Both operands
+// are contiguous in k, so a tile of each is staged through LDS as [128 rows][64 k] with rows padded
+// to 144 bytes (which makes the 16-byte fragment reads of 8 consecutive lanes cover all banks), in
+// two buffers: while the waves feed 32x32x16 MFMAs from one, the next k-step's global loads are in
+// flight and are written to the other.  Each wave owns a 64 x 64 quarter (2 x 2 MFMA blocks).
+// Rows and columns beyond the matrix are read as zero and not stored; k must be a multiple of 8.
+// Every output element is accumulated over k in ascending order, whatever the number of rows.
+//
+// Workgroups are numbered so that those sharing a tile of w run on the same XCD (workgroups are
+// dealt to the 8 XCDs in turn, each with an L2 of its own).
+#include "api.h"
+#include "mfma.h"
+
+namespace bc4g {
+namespace {
+
+constexpr int kBM = 128, kBN = 128, kBK = 64;
+constexpr int kLdsStride = kBK + 8;   // elements; 144 bytes
+constexpr int kXcds = 8;
+
+enum Epilogue : int { kStoreBf16 = 0, kStoreF32 = 1, kAccumF32 = 2 };
+
+struct Tile {
+  bf16_t a[kBM][kLdsStride];
+  bf16_t w[kBN][kLdsStride];
+};
+
+template <int EPI>
+__global__ __launch_bounds__(256) void gemm_mfma_kernel(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
+                                                        void* __restrict__ out, int m, int n, int k,
+                                                        int m_blocks, int n_blocks) {
+  __shared__ Tile tiles[2];
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const int wm = wave / 2, wn = wave % 2;   // this wave's 64 x 64 quarter
+
+  // XCD-aware numbering: consecutive logical ids stay on one XCD; m runs fastest so that
+  // neighbours share a tile of w.
+  const int total = m_blocks * n_blocks;
+  int logical = blockIdx.x;
+  if (total % kXcds == 0) logical = (blockIdx.x % kXcds) * (total / kXcds) + blockIdx.x / kXcds;
+  const int bm = logical % m_blocks, bn = logical / m_blocks;
+  const long m0 = static_cast<long>(bm) * kBM, n0 = static_cast<long>(bn) * kBN;
+
+  // global -> LDS: a tile is 128 rows x 8 segments of 16 bytes; thread t moves segment t%8 of rows t/8 + 32 i
+  const int seg = tid % 8, lrow = tid / 8;
+  uint4 ra[4], rw[4];
+  auto load_tiles = [&](int k0) {
+    const int kk = k0 + seg * 8;
+    const bool k_ok = kk < k;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const long gm = m0 + lrow + 32 * i, gn = n0 + lrow + 32 * i;
+      ra[i] = (k_ok && gm < m) ? load16(a + gm * k + kk) : zero16();
+      rw[i] = (k_ok && gn < n) ? load16(w + gn * k + kk) : zero16();
+    }
+  };
+  auto store_tiles = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      *reinterpret_cast<uint4*>(&tiles[buf].a[lrow + 32 * i][seg * 8]) = ra[i];
+      *reinterpret_cast<uint4*>(&tiles[buf].w[lrow + 32 * i][seg * 8]) = rw[i];
+    }
+  };
+
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  const int nk = (k + kBK - 1) / kBK;
+  load_tiles(0);
+  store_tiles(0);
+  __syncthreads();
+  const int frow = lane % 32, fk = (lane / 32) * 8;
+  for (int kt = 0; kt < nk; ++kt) {
+    const int buf = kt & 1;
+    if (kt + 1 < nk) load_tiles((kt + 1) * kBK);
+#pragma unroll
+    for (int ks = 0; ks < kBK / 16; ++ks) {
+      uint4 fa[2], fw[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        fa[i] = *reinterpret_cast<const uint4*>(&tiles[buf].a[wm * 64 + i * 32 + frow][ks * 16 + fk]);
+        fw[i] = *reinterpret_cast<const uint4*>(&tiles[buf].w[wn * 64 + i * 32 + frow][ks * 16 + fk]);
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = mfma_32x32x16(fa[i], fw[j], acc[i][j]);
+    }
+    if (kt + 1 < nk) store_tiles(buf ^ 1);
+    __syncthreads();
+  }
+
+  // acc[i][j][r]: row m0 + wm*64 + i*32 + 8*(r/4) + 4*(lane/32) + r%4, column n0 + wn*64 + j*32 + lane%32
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const long gn = n0 + wn * 64 + j * 32 + lane % 32;
+      if (gn >= n) continue;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const long gm = m0 + wm * 64 + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + r % 4;
+        if (gm >= m) continue;
+        const long o = gm * n + gn;
+        if constexpr (EPI == kStoreBf16) static_cast<bf16_t*>(out)[o] = from_float<bf16_t>(acc[i][j][r]);
+        else if constexpr (EPI == kStoreF32) static_cast<float*>(out)[o] = acc[i][j][r];
+        else static_cast<float*>(out)[o] += acc[i][j][r];
+      }
+    }
+}
+
+}  // namespace
+}  // namespace bc4g
+
+using namespace bc4g;
+
+extern "C" int bc4g_gemm_mfma(const void* a, const void* w, void* out, int epilogue, int m, int n, int k,
+                              void* stream) {
+  BC4G_REQUIRE(m >= 0 && n > 0 && k > 0 && k % 8 == 0, "gemm_mfma: K=%d must be a positive multiple of 8 (M=%d N=%d)",
+               k, m, n);
+  if (m == 0) return 0;
+  const long m_blocks = (m + kBM - 1) / kBM, n_blocks = (n + kBN - 1) / kBN;
+  BC4G_REQUIRE(m_blocks * n_blocks <= 2147483647L, "gemm_mfma: too many tiles");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  dim3 grid(static_cast<unsigned>(m_blocks * n_blocks)), block(256);
+  const bf16_t* ap = static_cast<const bf16_t*>(a);
+  const bf16_t* wp = static_cast<const bf16_t*>(w);
+  switch (epilogue) {
+    case kStoreBf16: gemm_mfma_kernel<kStoreBf16><<<grid, block, 0, s>>>(ap, wp, out, m, n, k, m_blocks, n_blocks); break;
+    case kStoreF32: gemm_mfma_kernel<kStoreF32><<<grid, block, 0, s>>>(ap, wp, out, m, n, k, m_blocks, n_blocks); break;
+    case kAccumF32: gemm_mfma_kernel<kAccumF32><<<grid, block, 0, s>>>(ap, wp, out, m, n, k, m_blocks, n_blocks); break;
+    default: return fail("gemm_mfma: unknown epilogue %d", epilogue);
+  }
+  return check_launch("gemm_mfma");
+}

@@ -23,6 +23,9 @@ _SIGNATURES = {
     "bc4g_attention_generic": [_P, _P, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _P],
     "bc4g_argmax": [_P, _P, _I, _I, _P],
     "bc4g_sample": [_P, _P, _P, _P, _I, _I, _P],
+    "bc4g_gemm_skinny": [_P, _P, _P, _I, _I, _I, _I, _P],
+    "bc4g_gemm_mfma": [_P, _P, _P, _I, _I, _I, _I, _P],
+    "bc4g_attention_mfma": [_P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P],
 }
 
 _lib: Optional[ctypes.CDLL] = None

@@ -116,10 +116,15 @@ def swiglu(gu: torch.Tensor) -> torch.Tensor:
     return out
 
 
-def _check_cache(what: str, cache: torch.Tensor, n_kv_heads: int, head_dim: int, dtype: torch.dtype):
-    if cache.dim() != 4 or cache.shape[1] != n_kv_heads or cache.shape[3] != head_dim or cache.dtype != dtype:
-        raise KernelError(f"{what}: cache must be {dtype} [pages, {n_kv_heads}, page_tokens, {head_dim}], "
-                          f"got {cache.dtype} {tuple(cache.shape)}")
+def _check_cache(what: str, k: torch.Tensor, v: torch.Tensor, n_kv_heads: int, head_dim: int, dtype: torch.dtype):
+    """k: [pages, kv_heads, page_tokens, head_dim]; v transposed: [pages, kv_heads, head_dim, page_tokens]."""
+    ok = (k.dim() == 4 and v.dim() == 4 and k.shape[1] == n_kv_heads and k.shape[3] == head_dim
+          and k.dtype == dtype and v.dtype == dtype
+          and tuple(v.shape) == (k.shape[0], n_kv_heads, head_dim, k.shape[2]))
+    if not ok:
+        raise KernelError(f"{what}: caches must be {dtype}, keys [pages, {n_kv_heads}, page_tokens, {head_dim}] and "
+                          f"values [pages, {n_kv_heads}, {head_dim}, page_tokens]; got {k.dtype} {tuple(k.shape)} "
+                          f"and {v.dtype} {tuple(v.shape)}")
 
 
 def rope_kv_write(qkv: torch.Tensor, positions: Optional[torch.Tensor], slot_map: Optional[torch.Tensor],
@@ -135,10 +140,7 @@ def rope_kv_write(qkv: torch.Tensor, positions: Optional[torch.Tensor], slot_map
         _i32("rope_kv_write", "positions", positions, t)
     page_tokens = num_pages = 0
     if write_kv:
-        _check_cache("rope_kv_write", k_cache, n_kv_heads, head_dim, qkv.dtype)
-        _check_cache("rope_kv_write", v_cache, n_kv_heads, head_dim, qkv.dtype)
-        if k_cache.shape != v_cache.shape:
-            raise KernelError("rope_kv_write: k and v caches differ in shape")
+        _check_cache("rope_kv_write", k_cache, v_cache, n_kv_heads, head_dim, qkv.dtype)
         _i32("rope_kv_write", "slot_map", slot_map, t)
         num_pages, page_tokens = k_cache.shape[0], k_cache.shape[2]
     library.call("bc4g_rope_kv_write", _ptr(qkv), _code(qkv, "rope_kv_write"), _ptr(positions), _ptr(slot_map),
@@ -156,8 +158,7 @@ def attention_generic(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.T
     width = (n_heads + 2 * n_kv_heads) * head_dim
     if qkv.dim() != 2 or qkv.shape[1] != width:
         raise KernelError(f"attention: qkv must be [T, {width}], got {tuple(qkv.shape)}")
-    _check_cache("attention", k_cache, n_kv_heads, head_dim, qkv.dtype)
-    _check_cache("attention", v_cache, n_kv_heads, head_dim, qkv.dtype)
+    _check_cache("attention", k_cache, v_cache, n_kv_heads, head_dim, qkv.dtype)
     if block_table.dim() != 2 or block_table.dtype != torch.int32:
         raise KernelError("attention: block_table must be int32 [requests, pages]")
     _i32("attention", "row_seq", row_seq, t)
@@ -196,16 +197,117 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, u: torch.Tensor) -> 
     return out
 
 
+SKINNY_MAX_ROWS = 64
+EPI_STORE_BF16, EPI_STORE_F32, EPI_ACCUM_F32, EPI_SWIGLU = 0, 1, 2, 3
+
+
+def _fast_operands(a: torch.Tensor, w: torch.Tensor) -> bool:
+    return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.dim() == 2 and w.dim() == 2
+            and a.shape[1] == w.shape[1] and a.shape[1] % 8 == 0 and a.shape[0] > 0)
+
+
 def gemm_fast(a: torch.Tensor, w: torch.Tensor, out_dtype=None,
               accumulate_into: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
-    """The matrix-core product where a kernel takes these operands, else None
-    (the caller then uses the plain float kernel)."""
-    return None
+    """The matrix-core product where a kernel takes these operands (bfloat16, k a multiple of
+    8), else None (the caller then uses the plain float kernel).  Up to 64 rows the weights
+    are streamed once (a decode step); beyond that the tiled kernel runs."""
+    if not _fast_operands(a, w):
+        return None
+    _dev("gemm", a, w, accumulate_into)
+    m, k = a.shape
+    n = w.shape[0]
+    if accumulate_into is not None:
+        out, epi = accumulate_into, EPI_ACCUM_F32
+        if out.dtype != torch.float32 or tuple(out.shape) != (m, n):
+            raise KernelError(f"gemm: accumulate_into must be float32 [{m}, {n}], got {out.dtype} {tuple(out.shape)}")
+    else:
+        out_dtype = out_dtype or a.dtype
+        if out_dtype not in (torch.bfloat16, torch.float32):
+            return None
+        out = torch.empty((m, n), dtype=out_dtype, device=a.device)
+        epi = EPI_STORE_BF16 if out_dtype == torch.bfloat16 else EPI_STORE_F32
+    name = "bc4g_gemm_skinny" if m <= SKINNY_MAX_ROWS else "bc4g_gemm_mfma"
+    library.call(name, _ptr(a), _ptr(w), _ptr(out), epi, m, n, k, _stream())
+    return out
+
+
+def gemm_swiglu(a: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
+    """silu(a Wg^T) * (a Wu^T) for w_gate_up = gate rows followed by up rows, [2I, K] -> [M, I].
+    For a few rows the activation is applied to the float sums inside the product's kernel;
+    otherwise the product is stored and the activation kernel follows."""
+    if _fast_operands(a, w_gate_up) and a.shape[0] <= SKINNY_MAX_ROWS and w_gate_up.shape[0] % 2 == 0:
+        _dev("gemm_swiglu", a, w_gate_up)
+        m, k = a.shape
+        n = w_gate_up.shape[0]
+        out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=a.device)
+        library.call("bc4g_gemm_skinny", _ptr(a), _ptr(w_gate_up), _ptr(out), EPI_SWIGLU, m, n, k, _stream())
+        return out
+    gu = gemm_fast(a, w_gate_up, a.dtype)
+    if gu is None:
+        gu = gemm_generic(a, w_gate_up, a.dtype)
+    return swiglu(gu)
+
+
+def attention_mfma_supported(qkv: torch.Tensor, k_cache: torch.Tensor, head_dim: int) -> bool:
+    return (qkv.dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= 256
+            and k_cache.shape[2] % 16 == 0)
+
+
+def attention_tile_tokens(n_heads: int, n_kv_heads: int) -> int:
+    """Tokens of one request per 16-row tile of the matrix-core attention kernel."""
+    return 16 // min(n_heads // n_kv_heads, 16)
+
+
+ATTENTION_TARGET_WAVES = 2048
+
+
+def attention_splits(n_tiles: int, n_heads: int, n_kv_heads: int, max_kv_len: int) -> int:
+    """Into how many parts the keys are cut so that the GPU has enough waves: none if the rows
+    alone fill it, else towards ATTENTION_TARGET_WAVES waves with at least one 32-key tile each."""
+    group = n_heads // n_kv_heads
+    waves = n_tiles * n_kv_heads * (-(-group // 16))
+    key_tiles = max(1, -(-max_kv_len // 32))
+    return max(1, min(ATTENTION_TARGET_WAVES // max(waves, 1), key_tiles))
+
+
+def attention_mfma(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
+                   seq_start: torch.Tensor, seq_ctx: torch.Tensor, tile_start: torch.Tensor, n_tiles: int,
+                   n_heads: int, n_kv_heads: int, head_dim: int, window: int, scale: float,
+                   n_splits: int) -> torch.Tensor:
+    _dev("attention_mfma", qkv, k_cache, v_cache, block_table, seq_start, seq_ctx, tile_start)
+    t = qkv.shape[0]
+    width = (n_heads + 2 * n_kv_heads) * head_dim
+    if qkv.dim() != 2 or qkv.shape[1] != width or qkv.dtype != torch.bfloat16:
+        raise KernelError(f"attention_mfma: qkv must be bfloat16 [T, {width}], got {qkv.dtype} {tuple(qkv.shape)}")
+    _check_cache("attention_mfma", k_cache, v_cache, n_kv_heads, head_dim, qkv.dtype)
+    if block_table.dim() != 2 or block_table.dtype != torch.int32:
+        raise KernelError("attention_mfma: block_table must be int32 [requests, pages]")
+    n_seqs = block_table.shape[0]
+    _i32("attention_mfma", "seq_start", seq_start, n_seqs + 1)
+    _i32("attention_mfma", "seq_ctx", seq_ctx, n_seqs)
+    _i32("attention_mfma", "tile_start", tile_start, n_seqs + 1)
+    out = torch.empty((t, n_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
+    part_o = part_ml = None
+    if n_splits > 1:
+        part_o = torch.empty((n_splits, t, n_heads, head_dim), dtype=torch.float32, device=qkv.device)
+        part_ml = torch.empty((n_splits, t, n_heads, 2), dtype=torch.float32, device=qkv.device)
+    library.call("bc4g_attention_mfma", _ptr(qkv), _ptr(out), _ptr(part_o), _ptr(part_ml), _ptr(k_cache),
+                 _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(seq_start), _ptr(seq_ctx),
+                 _ptr(tile_start), n_seqs, n_tiles, t, n_heads, n_kv_heads, head_dim, k_cache.shape[2],
+                 int(window), float(scale), attention_tile_tokens(n_heads, n_kv_heads), int(n_splits), _stream())
+    return out
 
 
 def attention(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
               ctx, n_heads: int, n_kv_heads: int, head_dim: int, window: int, scale: float) -> torch.Tensor:
-    """Attention of a step's rows over the cache: picks the kernel for the
-    batch's shape (prompt portions, decoded tokens, or both)."""
+    """Attention of a step's rows over the cache: the matrix-core kernel where it takes the
+    sizes (bfloat16, head size a multiple of 16 up to 256, pages of a multiple of 16 tokens),
+    else the plain float kernel."""
+    if attention_mfma_supported(qkv, k_cache, head_dim):
+        tpt = attention_tile_tokens(n_heads, n_kv_heads)
+        tile_start, n_tiles = ctx.attention_tiles(tpt)
+        n_splits = ctx.fixed_attention_splits or attention_splits(n_tiles, n_heads, n_kv_heads, ctx.max_kv_len)
+        return attention_mfma(qkv, k_cache, v_cache, block_table, ctx.seq_start_dev, ctx.seq_ctx_dev,
+                              tile_start, n_tiles, n_heads, n_kv_heads, head_dim, window, scale, n_splits)
     return attention_generic(qkv, k_cache, v_cache, block_table, ctx.row_seq, ctx.positions,
                              n_heads, n_kv_heads, head_dim, window, scale)

@@ -35,6 +35,21 @@ class StepContext:
     max_q_len: int
     max_kv_len: int
     cache_views: Dict[Hashable, Any] = dataclasses.field(default_factory=dict)
+    # tokens per attention tile -> (device int32 [S+1] first tile of each request, number of tiles)
+    tiles: Dict[int, Any] = dataclasses.field(default_factory=dict)
+    fixed_attention_splits: int = 0      # non-zero: the key split count is fixed (a captured step)
 
     def cache(self, stream: Optional[Hashable]):
         return None if stream is None else self.cache_views.get(stream)
+
+    def attention_tiles(self, tokens_per_tile: int):
+        """Each request's rows cut into tiles of ``tokens_per_tile`` tokens: (first tile of each
+        request as a device tensor, total).  Made once per step and tile size."""
+        if tokens_per_tile not in self.tiles:
+            starts = [0]
+            for s in range(self.n_seqs):
+                n = self.seq_start[s + 1] - self.seq_start[s]
+                starts.append(starts[-1] + -(-n // tokens_per_tile))
+            dev = torch.tensor(starts, dtype=torch.int32).to(self.token_ids.device, non_blocking=True)
+            self.tiles[tokens_per_tile] = (dev, starts[-1])
+        return self.tiles[tokens_per_tile]

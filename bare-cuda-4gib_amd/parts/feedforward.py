@@ -34,8 +34,7 @@ class SwiGLU(Part):
         self.act_dtype = rt.act_dtype
 
     def forward(self, h, ctx, residual) -> None:
-        gu = linear(h, self.w_gu, out_dtype=self.act_dtype)
-        act = ops.swiglu(gu)
+        act = ops.gemm_swiglu(h, self.w_gu)
         linear(act, self.w_down, accumulate_into=residual)
 
 

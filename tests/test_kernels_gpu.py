@@ -1,0 +1,315 @@
+"""Each kernel alone against a plain float64 reference, at other sizes than the engine's: ragged
+widths (300, 130, 17, 61, 48 -- the reference's own test shapes), head sizes 16..256, groups of
+1, 2, 3, 8 and 32 query heads, pages that are shuffled and poisoned with NaN where nobody owns
+them."""
+import math
+import random
+
+import numpy as np
+import pytest
+import torch
+
+import plain_llama as P
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from bare_cuda_4gib_amd.csrc import ops
+    return ops
+
+
+def rnd(*shape, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(*shape, generator=g, dtype=torch.float64) * scale
+
+
+def close(got, want, rtol, atol, what=""):
+    got, want = got.double().cpu(), want.double().cpu()
+    assert torch.isfinite(got).all(), f"{what}: non-finite values"
+    err = (got - want).abs()
+    bound = atol + rtol * want.abs()
+    assert bool((err <= bound).all()), f"{what}: max error {float(err.max()):.3g} at {int(err.argmax())}, bound {float(bound.flatten()[int(err.argmax())]):.3g}"
+
+
+def bf(x):
+    return x.to(torch.bfloat16)
+
+
+def test_embed_gather_is_exact(ops):
+    table = rnd(61, 48, seed=1)
+    ids = torch.tensor([0, 60, 5, 5, 17, 33, 2, 59, 1], dtype=torch.int32)
+    for t in (table.float(), bf(table)):
+        out = ops.embed_gather(t.to(DEV), ids.to(DEV))
+        assert out.dtype == torch.float32 and torch.equal(out.cpu(), t.float()[ids.long()])
+
+
+@pytest.mark.parametrize("wdt,odt", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16),
+                                     (torch.float32, torch.bfloat16), (torch.bfloat16, torch.float32)])
+def test_rmsnorm(ops, wdt, odt):
+    x, w = rnd(5, 300, seed=2), 1.0 + 0.1 * rnd(300, seed=3)
+    w = w.to(wdt)
+    want = P.rmsnorm(x.float().double(), w.double(), 1e-5)
+    tol = dict(rtol=1e-5, atol=1e-5) if odt == torch.float32 else dict(rtol=8e-3, atol=1e-3)
+    close(ops.rmsnorm(x.float().to(DEV), w.to(DEV), 1e-5, odt), want, what="rmsnorm", **tol)
+    rows = torch.tensor([4, 0, 4], dtype=torch.int32, device=DEV)
+    close(ops.rmsnorm(x.float().to(DEV), w.to(DEV), 1e-5, odt, rows=rows), want[[4, 0, 4]], what="rmsnorm rows", **tol)
+    short = torch.tensor([[3.0, 4.0]])                       # eps on the mean, not on the sum
+    got = ops.rmsnorm(short.to(DEV), torch.ones(2, device=DEV), 1.0, torch.float32)
+    close(got, short.double() / math.sqrt(13.5), 1e-6, 1e-6, "rmsnorm eps")
+
+
+@pytest.mark.parametrize("m,n,k", [(17, 130, 300), (1, 130, 300), (150, 61, 48), (64, 64, 64), (3, 5, 7)])
+def test_gemm_generic(ops, m, n, k):
+    a, w = rnd(m, k, seed=4), rnd(n, k, seed=5)
+    want = a.float().double() @ w.float().double().T
+    close(ops.gemm_generic(a.float().to(DEV), w.float().to(DEV)), want, 1e-5, 1e-4, "f32")
+    base = rnd(m, n, seed=6).float()
+    acc = base.clone().to(DEV)
+    ops.gemm_generic(a.float().to(DEV), w.float().to(DEV), accumulate_into=acc)
+    close(acc, want + base.double(), 1e-5, 1e-4, "f32 accumulate")
+    ab, wb = bf(a), bf(w)
+    wantb = ab.double() @ wb.double().T
+    close(ops.gemm_generic(ab.to(DEV), wb.to(DEV), torch.float32), wantb, 1e-5, 1e-4, "bf16 -> f32")
+    close(ops.gemm_generic(ab.to(DEV), wb.to(DEV), torch.bfloat16), wantb, 8e-3, 1e-2, "bf16 -> bf16")
+    close(ops.gemm_generic(ab.to(DEV), w.float().to(DEV), torch.float32), ab.double() @ w.float().double().T, 1e-5, 1e-4,
+          "bf16 x f32")
+
+
+@pytest.mark.parametrize("m", [1, 2, 3, 5, 8, 16, 17, 33, 48, 64])
+@pytest.mark.parametrize("n,k", [(130, 304), (16, 8), (2560, 2048), (301, 80)])
+def test_gemm_skinny(ops, m, n, k):
+    a, w = bf(rnd(m, k, seed=7)), bf(rnd(n, k, seed=8))
+    want = a.double() @ w.double().T
+    scale = math.sqrt(k)
+    got = ops.gemm_fast(a.to(DEV), w.to(DEV), torch.float32)
+    close(got, want, 1e-4, 1e-4 * scale, "skinny -> f32")
+    close(ops.gemm_fast(a.to(DEV), w.to(DEV), torch.bfloat16), want, 8e-3, 1e-3 * scale, "skinny -> bf16")
+    base = rnd(m, n, seed=9).float()
+    acc = base.clone().to(DEV)
+    assert ops.gemm_fast(a.to(DEV), w.to(DEV), accumulate_into=acc) is acc
+    close(acc, want + base.double(), 1e-4, 1e-4 * scale, "skinny accumulate")
+    # a row's result must not depend on the other rows of the call
+    alone = ops.gemm_fast(a[:1].contiguous().to(DEV), w.to(DEV), torch.float32)
+    assert torch.equal(alone[0], got[0])
+
+
+@pytest.mark.parametrize("m", [1, 7, 64])
+@pytest.mark.parametrize("inter,k", [(176, 64), (112, 80), (5632, 256)])
+def test_gemm_swiglu_fused(ops, m, inter, k):
+    a, w = bf(rnd(m, k, seed=10)), bf(rnd(2 * inter, k, seed=11, scale=0.3))
+    gu = a.double() @ w.double().T
+    want = P.swiglu(gu[:, :inter], gu[:, inter:])
+    close(ops.gemm_swiglu(a.to(DEV), w.to(DEV)), want, 8e-3, 2e-2, "fused swiglu")
+
+
+@pytest.mark.parametrize("m,n,k", [(65, 130, 304), (150, 257, 64), (300, 128, 2048), (128, 384, 96), (129, 61, 8)])
+def test_gemm_mfma(ops, m, n, k):
+    a, w = bf(rnd(m, k, seed=12)), bf(rnd(n, k, seed=13))
+    want = a.double() @ w.double().T
+    scale = math.sqrt(k)
+    got = ops.gemm_fast(a.to(DEV), w.to(DEV), torch.float32)
+    close(got, want, 1e-4, 1e-4 * scale, "mfma -> f32")
+    close(ops.gemm_fast(a.to(DEV), w.to(DEV), torch.bfloat16), want, 8e-3, 1e-3 * scale, "mfma -> bf16")
+    base = rnd(m, n, seed=14).float()
+    acc = base.clone().to(DEV)
+    ops.gemm_fast(a.to(DEV), w.to(DEV), accumulate_into=acc)
+    close(acc, want + base.double(), 1e-4, 1e-4 * scale, "mfma accumulate")
+    fewer = ops.gemm_fast(a[:70].contiguous().to(DEV), w.to(DEV), torch.float32)   # rows do not depend on M
+    assert torch.equal(fewer, got[:70])
+    assert ops.gemm_fast(a.float().to(DEV), w.to(DEV)) is None                      # float operands: not taken
+
+
+def test_gemm_mfma_xcd_numbering_covers_every_tile(ops):
+    a, w = bf(rnd(1024, 64, seed=15)), bf(rnd(1024, 64, seed=16))                    # 8 x 8 tiles: remapped ids
+    close(ops.gemm_fast(a.to(DEV), w.to(DEV), torch.float32), a.double() @ w.double().T, 1e-4, 1e-3, "xcd")
+
+
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
+def test_swiglu(ops, dt):
+    gu = rnd(9, 2 * 176, seed=17).to(dt)
+    want = P.swiglu(gu.double()[:, :176], gu.double()[:, 176:])
+    close(ops.swiglu(gu.to(DEV)), want, 1e-5 if dt == torch.float32 else 8e-3, 1e-6 if dt == torch.float32 else 1e-3)
+
+
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rotary_dim", [16, 8, 0])
+def test_rope_kv_write(ops, dt, rotary_dim):
+    nh, nkv, d, page, pages = 4, 2, 16, 4, 9
+    positions = [0, 1, 2, 5, 8, 13, 21]                                 # reference_forward.py:163
+    t = len(positions)
+    qkv = rnd(t, (nh + 2 * nkv) * d, seed=18).to(dt)
+    slots = [5 * page + 1, 5 * page + 2, 2 * page + 0, 0, 8 * page + 3, 7 * page + 2, 3 * page + 1]
+    sentinel = -7.5                                                       # test_kv_cache_write.cu:25-41
+    kc = torch.full((pages, nkv, page, d), sentinel, dtype=dt, device=DEV)
+    vc = torch.full((pages, nkv, d, page), sentinel, dtype=dt, device=DEV)
+    buf = qkv.clone().to(DEV)
+    ops.rope_kv_write(buf, torch.tensor(positions, dtype=torch.int32, device=DEV),
+                      torch.tensor(slots, dtype=torch.int32, device=DEV), kc, vc, nh, nkv, d, rotary_dim, 10000.0)
+    x = qkv.double().view(t, nh + 2 * nkv, d)
+    pos = torch.tensor(positions)
+    q_want = P.rope(x[:, :nh], pos, 10000.0, rotary_dim) if rotary_dim else x[:, :nh]
+    k_want = P.rope(x[:, nh:nh + nkv], pos, 10000.0, rotary_dim) if rotary_dim else x[:, nh:nh + nkv]
+    v_want = x[:, nh + nkv:]
+    tol = dict(rtol=1e-5, atol=1e-5) if dt == torch.float32 else dict(rtol=8e-3, atol=8e-3)
+    out = buf.cpu().double().view(t, nh + 2 * nkv, d)
+    close(out[:, :nh], q_want, what="q", **tol)
+    assert torch.equal(out[:, nh:], x[:, nh:]) or rotary_dim       # k, v in the buffer are not the product
+    kc_c, vc_c = kc.cpu().double(), vc.cpu().double()
+    touched_k = torch.zeros_like(kc_c, dtype=torch.bool)
+    touched_v = torch.zeros_like(vc_c, dtype=torch.bool)
+    for i, s in enumerate(slots):
+        pg, off = divmod(s, page)
+        close(kc_c[pg, :, off, :], k_want[i], what=f"k row {i}", **tol)
+        close(vc_c[pg, :, :, off], v_want[i], what=f"v row {i}", **tol)
+        touched_k[pg, :, off, :] = True
+        touched_v[pg, :, :, off] = True
+    assert bool((kc_c[~touched_k] == sentinel).all()) and bool((vc_c[~touched_v] == sentinel).all()), "spill"
+
+
+# --- attention --------------------------------------------------------------------
+
+def paged_case(seqs, nh, nkv, d, page, dt, seed, poison=True, far=None):
+    """seqs: [(cached tokens, new tokens)].  Builds q for the new tokens, keys and values for all,
+    puts them into shuffled pages (NaN elsewhere) and returns what the kernels need plus the
+    plain result."""
+    rng = random.Random(seed)
+    total_pages = sum(-(-(c + n) // page) for c, n in seqs) + 3
+    free = list(range(total_pages))
+    rng.shuffle(free)
+    fill = float("nan") if poison else 0.0
+    kc = torch.full((total_pages, nkv, page, d), fill, dtype=torch.float64)
+    vc = torch.full((total_pages, nkv, d, page), fill, dtype=torch.float64)
+    width = max(-(-(c + n) // page) for c, n in seqs) + 1
+    table = torch.full((len(seqs), width), -1, dtype=torch.int32)
+    rows_q, row_seq, positions, seq_start, seq_ctx, wants = [], [], [], [0], [], []
+    for s, (c, n) in enumerate(seqs):
+        L = c + n
+        k = rnd(L, nkv, d, seed=seed * 100 + 2 * s)
+        v = rnd(L, nkv, d, seed=seed * 100 + 2 * s + 1)
+        q = rnd(L, nh, d, seed=seed * 100 + 50 + s)
+        if far is not None and L > far[1]:
+            # one query (the last) and one far key made to stand out: a kernel that skips that
+            # key, or reads its neighbour, is off by far more than rounding
+            h, j = far
+            q[L - 1, h] = 0.0
+            q[L - 1, h, 0] = 16.0
+            k[:, h // (nh // nkv), 0] = 0.0
+            k[j, h // (nh // nkv), 0] = 16.0
+        k, v, q = k.to(dt).double(), v.to(dt).double(), q.to(dt).double()
+        for pidx in range(-(-L // page)):
+            pg = free.pop()
+            table[s, pidx] = pg
+            lo, hi = pidx * page, min(L, (pidx + 1) * page)
+            kc[pg, :, :hi - lo, :] = k[lo:hi].transpose(0, 1)
+            vc[pg, :, :, :hi - lo] = v[lo:hi].permute(1, 2, 0)
+        rows_q.append(q[c:])
+        row_seq += [s] * n
+        positions += list(range(c, L))
+        seq_start.append(seq_start[-1] + n)
+        seq_ctx.append(c)
+        wants.append((q, k, v, c))
+    qkv = torch.zeros(seq_start[-1], nh + 2 * nkv, d, dtype=torch.float64)
+    qkv[:, :nh] = torch.cat(rows_q)
+    return dict(qkv=qkv.view(seq_start[-1], -1).to(dt).to(DEV), kc=kc.to(dt).to(DEV), vc=vc.to(dt).to(DEV),
+                table=table.to(DEV), row_seq=torch.tensor(row_seq, dtype=torch.int32, device=DEV),
+                positions=torch.tensor(positions, dtype=torch.int32, device=DEV),
+                seq_start=seq_start, seq_ctx=seq_ctx, wants=wants, nh=nh, nkv=nkv, d=d)
+
+
+def plain_result(case, window=0):
+    outs = []
+    for q, k, v, c in case["wants"]:
+        outs.append(P.attention(q, k, v, window)[c:].reshape(q.shape[0] - c, -1))
+    return torch.cat(outs)
+
+
+SHAPES = [  # nh, nkv, d, page
+    (4, 2, 16, 16), (3, 3, 32, 16), (6, 2, 48, 32), (32, 4, 64, 64), (8, 1, 128, 16), (32, 1, 16, 16), (2, 1, 256, 16),
+]
+SEQS = [(0, 33), (40, 1), (17, 2), (0, 1), (64, 70), (129, 1)]
+
+
+@pytest.mark.parametrize("nh,nkv,d,page", SHAPES)
+@pytest.mark.parametrize("window", [0, 20])
+def test_attention_generic(ops, nh, nkv, d, page, window):
+    for dt, tol in ((torch.float32, dict(rtol=1e-4, atol=1e-5)), (torch.bfloat16, dict(rtol=2e-2, atol=2e-2))):
+        case = paged_case(SEQS, nh, nkv, d, page, dt, seed=3)
+        got = ops.attention_generic(case["qkv"], case["kc"], case["vc"], case["table"], case["row_seq"],
+                                    case["positions"], nh, nkv, d, window)
+        close(got, plain_result(case, window), what=f"generic {dt}", **tol)
+
+
+def run_mfma(ops, case, window, n_splits):
+    nh, nkv, d = case["nh"], case["nkv"], case["d"]
+    tpt = ops.attention_tile_tokens(nh, nkv)
+    starts = [0]
+    for s in range(len(case["seq_ctx"])):
+        starts.append(starts[-1] + -(-(case["seq_start"][s + 1] - case["seq_start"][s]) // tpt))
+    dev = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
+    return ops.attention_mfma(case["qkv"], case["kc"], case["vc"], case["table"], dev(case["seq_start"]),
+                              dev(case["seq_ctx"]), dev(starts), starts[-1], nh, nkv, d, window,
+                              1.0 / math.sqrt(d), n_splits)
+
+
+@pytest.mark.parametrize("nh,nkv,d,page", SHAPES)
+@pytest.mark.parametrize("window", [0, 20])
+@pytest.mark.parametrize("n_splits", [1, 3, 16])
+def test_attention_mfma(ops, nh, nkv, d, page, window, n_splits):
+    case = paged_case(SEQS, nh, nkv, d, page, torch.bfloat16, seed=4)
+    assert ops.attention_mfma_supported(case["qkv"], case["kc"], d)
+    got = run_mfma(ops, case, window, n_splits)
+    close(got, plain_result(case, window), rtol=2e-2, atol=2e-2, what="mfma")
+
+
+@pytest.mark.parametrize("n_splits", [1, 5])
+def test_attention_far_key_among_hundreds(ops, n_splits):
+    """The last query of each request looks at one key far back (position 3 of 400+): softmax puts
+    nearly all weight there, so skipping it or reading a neighbour shows at once."""
+    seqs = [(0, 420), (418, 2), (431, 1)]
+    for dt, fn in ((torch.bfloat16, "mfma"), (torch.float32, "generic")):
+        case = paged_case(seqs, 4, 2, 64, 16, dt, seed=5, far=(1, 3))
+        want = plain_result(case)
+        if fn == "mfma":
+            got = run_mfma(ops, case, 0, n_splits)
+        else:
+            got = ops.attention_generic(case["qkv"], case["kc"], case["vc"], case["table"], case["row_seq"],
+                                        case["positions"], 4, 2, 64, 0)
+        close(got, want, rtol=2e-2, atol=2e-2, what=fn)
+        v_far = case["wants"][0][2][3, 0]                          # the value row the far key carries
+        last = got[419].double().cpu().view(4, 64)[1]
+        assert float((last - v_far).abs().max()) < 0.05, "the far key's value must dominate"
+
+
+def test_attention_window_edge(ops):
+    """Keys exactly at the window's edge: position p sees p - window + 1 but not p - window."""
+    case = paged_case([(0, 50)], 2, 1, 32, 16, torch.bfloat16, seed=6, poison=False)
+    for window in (1, 16, 17, 31, 32, 33):
+        close(run_mfma(ops, case, window, 1), plain_result(case, window), rtol=2e-2, atol=2e-2, what=f"window {window}")
+
+
+def test_argmax_ties_and_sampling(ops):
+    logits = torch.full((3, 1000), -1.0)
+    logits[0, 7] = logits[0, 500] = logits[0, 999] = 5.0             # tie: lowest index
+    logits[1, 999] = 2.0                                              # maximum in the last place
+    logits[2] = torch.linspace(0, 1, 1000)
+    assert ops.argmax(logits.to(DEV)).tolist() == [7, 999, 999]
+    from bare_cuda_4gib_amd.sampling import MT19937_64, SamplingParams, sample_token
+    row = rnd(1, 32000, seed=20, scale=2.0).float()
+    us = [MT19937_64(s).uniform() for s in range(64)]
+    temps = [0.0 if i % 8 == 0 else 0.5 + 0.05 * i for i in range(64)]
+    got = ops.sample(row.expand(64, -1).contiguous().to(DEV), torch.tensor(temps, device=DEV),
+                     torch.tensor(us, dtype=torch.float64, device=DEV)).tolist()
+
+    class Fixed:
+        def __init__(self, u): self.u = u
+        def uniform(self): return self.u
+    for i in range(64):
+        want = sample_token(row[0].numpy(), SamplingParams(temperature=temps[i]), Fixed(us[i]))
+        if got[i] != want:   # float sums in another order may move a boundary by one token at most
+            w = np.exp((row[0].numpy() - row[0].numpy().max()) / temps[i])
+            cum = np.cumsum(w.astype(np.float64))
+            edge = abs(us[i] * cum[-1] - cum[min(got[i], want)])
+            assert abs(got[i] - want) == 1 and edge < 1e-3 * cum[-1], (i, got[i], want)
