@@ -20,6 +20,12 @@ from .batch import StepContext
 from .model import Model
 
 
+def _walk_parts(part):
+    yield part
+    for child in part.children():
+        yield from _walk_parts(child)
+
+
 @dataclasses.dataclass
 class StepEntry:
     """A request's next tokens, and the places among them (0-based) whose
@@ -39,7 +45,8 @@ class Executor:
     """
 
     def __init__(self, model: Model, *, num_pages: int, max_requests: int, max_tokens: int,
-                 page_tokens: int = 64, max_batch_tokens: int = 0, poison: bool = False):
+                 page_tokens: int = 64, max_batch_tokens: int = 0, poison: bool = False,
+                 use_graphs: bool = True, graph_max_batch: int = 64):
         if model.rt is None:
             raise EngineError("executor: the model has no weights bound")
         self.model = model
@@ -49,6 +56,15 @@ class Executor:
                                   max_requests=max_requests, max_tokens=max_tokens,
                                   dtype=self.rt.act_dtype, device=self.rt.device, poison=poison)
         self._views = {sid: self.cache.view(sid) for sid in self.cache.specs}
+        # attention tile sizes the model's mixers ask for (made once per step, with the batch)
+        parts = [p for layer in model.layers for p in _walk_parts(layer)]
+        self._attention_parts = [p for p in parts if hasattr(p, "attention_tile_tokens")]
+        self._tile_sizes = sorted({p.attention_tile_tokens() for p in self._attention_parts})
+        # decode steps are replayed from captured graphs if every part of the model allows it
+        self.use_graphs = bool(use_graphs) and all(getattr(p, "graph_safe", False) for p in parts) \
+            and self.rt.device.type == "cuda"
+        self.graph_max_batch = graph_max_batch
+        self._graphs = {}
 
     # ---- requests -----------------------------------------------------------
     def admit(self, request: Hashable) -> int:
@@ -90,8 +106,9 @@ class Executor:
             raise EngineError(f"step: {total} rows are more than max_batch_tokens={self.max_batch_tokens}")
         return total
 
-    def build_context(self, entries: Sequence[StepEntry]) -> StepContext:
-        """Host arrays of the batch, uploaded in one copy."""
+    def _host_arrays(self, entries: Sequence[StepEntry], table_width: int = 0, all_logits: bool = False):
+        """The batch as one flat list of int32 and the layout of its parts.  ``table_width`` 0
+        makes block tables as wide as the batch needs; ``all_logits`` asks for every row."""
         cache, P = self.cache, self.cache.page_tokens
         token_ids: List[int] = []
         positions: List[int] = []
@@ -107,44 +124,113 @@ class Executor:
             seq_start.append(base + n)
             seq_ctx.append(ctx_len)
             seq_slots.append(cache.slot(e.request))
-            logit_rows.extend(base + int(w) for w in e.want)
+            logit_rows.extend(range(base, base + n) if all_logits else (base + int(w) for w in e.want))
             max_q, max_kv = max(max_q, n), max(max_kv, ctx_len + n)
         T, S = len(token_ids), len(entries)
         flat = token_ids + positions + row_seq + seq_start + seq_ctx + seq_slots + logit_rows
-        layout = {"token_ids": T, "positions": T, "row_seq": T, "seq_start": S + 1, "seq_ctx": S,
-                  "seq_slots": S, "logit_rows": len(logit_rows)}
+        layout = [("token_ids", T), ("positions", T), ("row_seq", T), ("seq_start", S + 1), ("seq_ctx", S),
+                  ("seq_slots", S), ("logit_rows", len(logit_rows))]
+        tiles = {}
+        for tpt in self._tile_sizes:
+            starts = [0]
+            for s in range(S):
+                starts.append(starts[-1] + -(-(seq_start[s + 1] - seq_start[s]) // tpt))
+            flat.extend(starts)
+            layout.append((("tiles", tpt), S + 1))
+            tiles[tpt] = starts[-1]
         group_layout = []
         for g in cache.groups:
             tables = [cache.table(g, e.request) for e in entries]
-            width = max(1, max(len(t) for t in tables))
+            width = table_width or max(1, max(len(t) for t in tables))
             for t in tables:
                 flat.extend(t)
                 flat.extend([-1] * (width - len(t)))
-            slot_map = []
             for e, t in zip(entries, tables):
                 ctx_len = cache.length(e.request)
-                for p in range(ctx_len, ctx_len + len(e.tokens)):
-                    slot_map.append(t[p // P] * P + p % P)
-            flat.extend(slot_map)
+                flat.extend(t[p // P] * P + p % P for p in range(ctx_len, ctx_len + len(e.tokens)))
             group_layout.append((g, width))
-        dev = torch.tensor(flat, dtype=torch.int32).to(self.rt.device, non_blocking=True)
+        host = dict(seq_start=seq_start, seq_ctx=seq_ctx, seq_slots=seq_slots, n_logits=len(logit_rows),
+                    max_q=max_q, max_kv=max_kv, tiles=tiles, T=T, S=S)
+        return flat, layout, group_layout, host
+
+    def _context_from(self, dev: torch.Tensor, layout, group_layout, host, fixed_splits: int = 0) -> StepContext:
         off = 0
         parts = {}
-        for name, n in layout.items():
+        for name, n in layout:
             parts[name] = dev[off:off + n]
             off += n
+        T, S = host["T"], host["S"]
         block_tables, slot_maps = {}, {}
         for g, width in group_layout:
             block_tables[g] = dev[off:off + S * width].view(S, width)
             off += S * width
             slot_maps[g] = dev[off:off + T]
             off += T
+        tiles = {tpt: (parts[("tiles", tpt)], n) for tpt, n in host["tiles"].items()}
         return StepContext(
             rt=self.rt, n_tokens=T, n_seqs=S, token_ids=parts["token_ids"], positions=parts["positions"],
-            row_seq=parts["row_seq"], seq_start=seq_start, seq_ctx=seq_ctx, seq_slots=seq_slots,
-            seq_start_dev=parts["seq_start"], seq_ctx_dev=parts["seq_ctx"], seq_slots_dev=parts["seq_slots"],
-            logit_rows=parts["logit_rows"], n_logits=len(logit_rows), block_tables=block_tables,
-            slot_maps=slot_maps, max_q_len=max_q, max_kv_len=max_kv, cache_views=self._views)
+            row_seq=parts["row_seq"], seq_start=host["seq_start"], seq_ctx=host["seq_ctx"],
+            seq_slots=host["seq_slots"], seq_start_dev=parts["seq_start"], seq_ctx_dev=parts["seq_ctx"],
+            seq_slots_dev=parts["seq_slots"], logit_rows=parts["logit_rows"], n_logits=host["n_logits"],
+            block_tables=block_tables, slot_maps=slot_maps, max_q_len=host["max_q"], max_kv_len=host["max_kv"],
+            cache_views=self._views, tiles=tiles, fixed_attention_splits=fixed_splits)
+
+    def build_context(self, entries: Sequence[StepEntry]) -> StepContext:
+        """Host arrays of the batch, uploaded in one copy."""
+        flat, layout, group_layout, host = self._host_arrays(entries)
+        dev = torch.tensor(flat, dtype=torch.int32).to(self.rt.device, non_blocking=True)
+        return self._context_from(dev, layout, group_layout, host)
+
+    # ---- decode steps as captured graphs ------------------------------------------
+    def _graph_eligible(self, entries: Sequence[StepEntry]) -> bool:
+        return (self.use_graphs and len(entries) <= self.graph_max_batch
+                and all(len(e.tokens) == 1 for e in entries))
+
+    def _graph_step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """A step in which every request brings one token, replayed from a HIP graph captured
+        for this batch size and context bucket.  Only the int32 batch description changes
+        between replays; it is copied into the graph's own buffer first.  Logits of every row
+        come back ([S, vocab]); the buffer is the graph's and is overwritten by its next replay."""
+        S = len(entries)
+        width = self.cache.max_pages_per_request
+        flat, layout, group_layout, host = self._host_arrays(entries, table_width=width, all_logits=True)
+        bucket = 256
+        while bucket < host["max_kv"]:
+            bucket *= 2
+        key = (S, bucket)
+        slot = self._graphs.get(key)
+        if slot is None:
+            slot = self._capture(key, flat, layout, group_layout, host, bucket)
+        ring = slot["ring"]
+        buf, event = ring[slot["next"] % len(ring)]
+        slot["next"] += 1
+        if event is not None:
+            event.synchronize()
+        buf.numpy()[:] = flat
+        slot["dev"].copy_(buf, non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record()
+        ring[(slot["next"] - 1) % len(ring)] = (buf, ev)
+        slot["graph"].replay()
+        return slot["logits"]
+
+    def _capture(self, key, flat, layout, group_layout, host, bucket):
+        from ..csrc import ops
+        S = key[0]
+        dev = torch.tensor(flat, dtype=torch.int32).to(self.rt.device)
+        # the key split count is frozen into the graph: chosen for the bucket's longest context
+        splits = max((ops.attention_splits(S, m.num_heads, m.num_kv_heads, bucket)
+                      for m in self._attention_parts), default=1)
+        ctx = self._context_from(dev, layout, group_layout, dict(host, max_kv=bucket), fixed_splits=splits)
+        self.model.forward(ctx)                      # once outside the graph: first-use work happens here
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            logits = self.model.forward(ctx)
+        ring = [(torch.empty(len(flat), dtype=torch.int32).pin_memory(), None) for _ in range(4)]
+        slot = dict(graph=graph, dev=dev, logits=logits, ring=ring, next=0)
+        self._graphs[key] = slot
+        return slot
 
     def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
         """Run the entries as one batch.  Returns float32 logits
@@ -155,8 +241,17 @@ class Executor:
         batch's tokens."""
         self._validate(entries)
         self.cache.reserve([(e.request, len(e.tokens)) for e in entries])
-        ctx = self.build_context(entries)
-        logits = self.model.forward(ctx)
+        if self._graph_eligible(entries):
+            every = self._graph_step(entries)
+            wanted = [i for i, e in enumerate(entries) if len(e.want)]
+            if not wanted:
+                logits = None
+            elif len(wanted) == len(entries):
+                logits = every
+            else:
+                logits = every[torch.tensor(wanted, device=every.device)]
+        else:
+            logits = self.model.forward(self.build_context(entries))
         for e in entries:
             self.cache.advance(e.request, len(e.tokens))
         return logits

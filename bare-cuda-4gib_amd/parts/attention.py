@@ -22,6 +22,7 @@ class CausalAttention(Part):
     softmax; output projection added to the residual stream.
     (Reference: engine/src/model.cpp:540-577, engine/kernels/attention_qk.cu:25-68.)"""
     category = "mixer"
+    graph_safe = True     # launches kernels only: may run inside a captured graph
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  window: int = 0, position=None):
@@ -40,6 +41,10 @@ class CausalAttention(Part):
 
     def cache_spec(self):
         return PagedKV(self.num_kv_heads, self.head_dim, self.window)
+
+    def attention_tile_tokens(self) -> int:
+        """Tokens per 16-row tile the matrix-core kernel wants the batch cut into."""
+        return ops.attention_tile_tokens(self.num_heads, self.num_kv_heads)
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
         q, kv, h = self.num_heads * self.head_dim, self.num_kv_heads * self.head_dim, self.hidden_size

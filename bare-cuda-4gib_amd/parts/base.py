@@ -32,8 +32,11 @@ _REGISTRY: Dict[str, Dict[str, Callable[..., "Part"]]] = {}
 
 
 class Part:
-    """Base of every part.  Subclasses set ``category``."""
+    """Base of every part.  Subclasses set ``category``; a part whose forward only launches
+    kernels on the current stream (no host reads of device data, no host-side decisions that
+    depend on the batch's values) may set ``graph_safe`` so that decode steps can be captured."""
     category = ""
+    graph_safe = False
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
         """Own tensor name (e.g. ``q_proj.weight``) -> what is expected of it."""

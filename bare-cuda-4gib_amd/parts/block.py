@@ -8,6 +8,7 @@ class PreNormBlock(Part):
     """x += mixer(norm(x)); x += ffn(norm(x))  (reference: engine/src/model.cpp:526-604).
     The residual stream x is float32 and is updated in place."""
     category = "block"
+    graph_safe = True     # launches kernels only: may run inside a captured graph
 
     def __init__(self, mixer, ffn, mixer_norm, ffn_norm):
         self.mixer, self.ffn, self.mixer_norm, self.ffn_norm = mixer, ffn, mixer_norm, ffn_norm

@@ -15,6 +15,7 @@ class SwiGLU(Part):
     """x += (silu(h Wg^T) * (h Wu^T)) Wd^T with silu(g) = g / (1 + exp(-g)), no
     biases (reference: engine/src/model.cpp:579-603, engine/kernels/swiglu.cu:17-25)."""
     category = "feedforward"
+    graph_safe = True     # launches kernels only: may run inside a captured graph
 
     def __init__(self, hidden_size: int, intermediate_size: int):
         self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)

@@ -13,6 +13,7 @@ from .base import Part, register_part
 
 class RMSNorm(Part):
     category = "norm"
+    graph_safe = True
 
     def __init__(self, size: int, eps: float):
         self.size, self.eps = int(size), float(eps)

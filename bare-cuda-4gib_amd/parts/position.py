@@ -12,6 +12,7 @@ class Rotary(Part):
     (reference: engine/kernels/rope.cu:44-53).  ``dim`` may be smaller than the
     head size; the remaining elements pass through."""
     category = "position"
+    graph_safe = True     # launches kernels only: may run inside a captured graph
 
     def __init__(self, theta: float, dim: int):
         if dim <= 0 or dim % 2:
@@ -27,6 +28,7 @@ class Rotary(Part):
 class NoPosition(Part):
     """No position encoding: queries and keys are used as projected."""
     category = "position"
+    graph_safe = True     # launches kernels only: may run inside a captured graph
 
     def fused(self):
         return 0, 1.0
