@@ -88,3 +88,12 @@ extern "C" {
 // epilogue: 0 store bfloat16; 1 store float32; 2 add into float32.
 int bc4g_gemm_mfma(const void* a, const void* w, void* out, int epilogue, int m, int n, int k, void* stream);
 }
+
+extern "C" {
+// RMSNorm fused into the skinny product (m <= 16): x is the float residual stream (row m reads
+// x[rows[m]] if rows is given), g the norm's scale (g_dtype 0 float32, 1 bfloat16); the result is
+// rsqrt(mean(x^2) + eps) * sum_k bf16(x[k] g[k]) w[n, k], with the epilogues of bc4g_gemm_skinny
+// except adding into a float output.
+int bc4g_gemm_skinny_normed(const float* x, const int32_t* rows, const void* g, int g_dtype, float eps,
+                            const void* w, void* out, int epilogue, int m, int n, int k, void* stream);
+}

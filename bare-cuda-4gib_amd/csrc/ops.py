@@ -231,6 +231,41 @@ def gemm_fast(a: torch.Tensor, w: torch.Tensor, out_dtype=None,
     return out
 
 
+NORMED_MAX_ROWS = 16
+
+
+def gemm_normed_supported(x: torch.Tensor, n_rows: int, g: torch.Tensor, w: torch.Tensor) -> bool:
+    """Whether RMSNorm can be fused into the product: few rows, bfloat16 weights, k a multiple of 8."""
+    staged = (-(-n_rows // 4) * 4) * (x.shape[1] + 8) * 2          # bytes of LDS the normed rows take
+    return (x.is_cuda and x.dtype == torch.float32 and w.dtype == torch.bfloat16 and 0 < n_rows <= NORMED_MAX_ROWS
+            and x.shape[1] == w.shape[1] and x.shape[1] % 8 == 0 and g.dtype in _CODE and staged <= 96 * 1024)
+
+
+def gemm_normed(x: torch.Tensor, rows: Optional[torch.Tensor], n_rows: int, g: torch.Tensor, eps: float,
+                w: torch.Tensor, epilogue: int) -> torch.Tensor:
+    """rmsnorm(x[rows]) W^T with the norm fused into the product (see gemm_skinny.hip): epilogue
+    EPI_STORE_BF16, EPI_STORE_F32 or EPI_SWIGLU (w = gate rows then up rows)."""
+    _dev("gemm_normed", x, rows, g, w)
+    k, n = x.shape[1], w.shape[0]
+    if tuple(g.shape) != (k,):
+        raise KernelError(f"gemm_normed: norm scale must be [{k}], got {tuple(g.shape)}")
+    if rows is not None:
+        _i32("gemm_normed", "rows", rows, n_rows)
+    elif n_rows != x.shape[0]:
+        raise KernelError("gemm_normed: without row indices every row of x is used")
+    if epilogue == EPI_SWIGLU:
+        out = torch.empty((n_rows, n // 2), dtype=torch.bfloat16, device=x.device)
+    elif epilogue == EPI_STORE_BF16:
+        out = torch.empty((n_rows, n), dtype=torch.bfloat16, device=x.device)
+    elif epilogue == EPI_STORE_F32:
+        out = torch.empty((n_rows, n), dtype=torch.float32, device=x.device)
+    else:
+        raise KernelError(f"gemm_normed: epilogue {epilogue} is not supported")
+    library.call("bc4g_gemm_skinny_normed", _ptr(x), _ptr(rows), _ptr(g), _code(g, "gemm_normed"), float(eps),
+                 _ptr(w), _ptr(out), epilogue, n_rows, n, k, _stream())
+    return out
+
+
 def gemm_swiglu(a: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
     """silu(a Wg^T) * (a Wu^T) for w_gate_up = gate rows followed by up rows, [2I, K] -> [M, I].
     For a few rows the activation is applied to the float sums inside the product's kernel;

@@ -9,6 +9,7 @@ import torch
 from ..config.registry import load_config
 from ..errors import ConfigError
 from ..parts.base import Part, build_part
+from ..parts.lazy import Normed
 from ..weights.loader import WeightSpec, load_weights
 from .batch import StepContext
 from .runtime import Runtime
@@ -126,8 +127,10 @@ class Model:
             self.layers[e.layer].forward(x, ctx, ctx.cache(e.cache), e.writes)
         if ctx.n_logits == 0:
             return None
-        h = self.final_norm.part.forward(x, ctx, rows=ctx.logit_rows, n_rows=ctx.n_logits)
-        return self.head.part.forward(h)
+        norm, head = self.final_norm.part, self.head.part
+        if getattr(head, "accepts_lazy_norm", False):
+            return head.forward(Normed(x, norm, ctx, rows=ctx.logit_rows, n_rows=ctx.n_logits))
+        return head.forward(norm.forward(x, ctx, rows=ctx.logit_rows, n_rows=ctx.n_logits))
 
 
 def expected_weights(spec: ModelSpec) -> Dict[str, WeightSpec]:

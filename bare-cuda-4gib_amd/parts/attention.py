@@ -23,6 +23,7 @@ class CausalAttention(Part):
     (Reference: engine/src/model.cpp:540-577, engine/kernels/attention_qk.cu:25-68.)"""
     category = "mixer"
     graph_safe = True     # launches kernels only: may run inside a captured graph
+    accepts_lazy_norm = True
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  window: int = 0, position=None):

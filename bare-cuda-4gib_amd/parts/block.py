@@ -2,6 +2,7 @@
 from __future__ import annotations
 
 from .base import Part, register_part
+from .lazy import Normed
 
 
 class PreNormBlock(Part):
@@ -17,10 +18,16 @@ class PreNormBlock(Part):
         return [self.mixer_norm, self.mixer, self.ffn_norm, self.ffn]
 
     def forward(self, x, ctx, cache, writes: bool = True) -> None:
-        h = self.mixer_norm.forward(x, ctx)
-        self.mixer.forward(h, ctx, cache, x, writes)
-        h = self.ffn_norm.forward(x, ctx)
-        self.ffn.forward(h, ctx, x)
+        self.mixer.forward(self._normed(self.mixer, self.mixer_norm, x, ctx), ctx, cache, x, writes)
+        self.ffn.forward(self._normed(self.ffn, self.ffn_norm, x, ctx), ctx, x)
+
+    @staticmethod
+    def _normed(part, norm, x, ctx):
+        """The part's input: the norm's result, or -- for a part that says it takes one -- the
+        norm not yet computed, so that the part's first product can absorb it."""
+        if getattr(part, "accepts_lazy_norm", False):
+            return Normed(x, norm, ctx)
+        return norm.forward(x, ctx)
 
 
 register_part("block", "prenorm", PreNormBlock)

@@ -46,7 +46,9 @@ class LMHead(Part):
     def bind(self, tensors, rt) -> None:
         self.weight = tensors["weight"]
 
-    def forward(self, h: torch.Tensor) -> torch.Tensor:
+    accepts_lazy_norm = True
+
+    def forward(self, h) -> torch.Tensor:
         return linear(h, self.weight, out_dtype=torch.float32)
 
 

@@ -8,7 +8,7 @@ import torch
 from ..csrc import ops
 from ..weights.loader import WeightSpec
 from .base import Part, register_part
-from .linear import linear
+from .linear import linear, linear_swiglu
 
 
 class SwiGLU(Part):
@@ -16,6 +16,7 @@ class SwiGLU(Part):
     biases (reference: engine/src/model.cpp:579-603, engine/kernels/swiglu.cu:17-25)."""
     category = "feedforward"
     graph_safe = True     # launches kernels only: may run inside a captured graph
+    accepts_lazy_norm = True
 
     def __init__(self, hidden_size: int, intermediate_size: int):
         self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
@@ -35,7 +36,7 @@ class SwiGLU(Part):
         self.act_dtype = rt.act_dtype
 
     def forward(self, h, ctx, residual) -> None:
-        act = ops.gemm_swiglu(h, self.w_gu)
+        act = linear_swiglu(h, self.w_gu)
         linear(act, self.w_down, accumulate_into=residual)
 
 

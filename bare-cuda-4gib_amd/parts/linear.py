@@ -1,20 +1,50 @@
 """y = x W^T for a weight stored [out, in] (the orientation a checkpoint stores
 a linear layer in; reference: engine/include/llm/kernels.h:48-57), and the
-choice of kernel for it (reference: matmul dispatch, engine/src/model.cpp:153-192)."""
+choice of kernel for it (reference: matmul dispatch, engine/src/model.cpp:153-192):
+up to 64 rows the weight-streaming kernel (with RMSNorm fused in up to 16 rows),
+beyond that the tiled matrix-core kernel, and the plain float kernel for
+everything those refuse (float32 operands, k no multiple of 8)."""
 from __future__ import annotations
 
-from typing import Optional
+from typing import Optional, Union
 
 import torch
 
 from ..csrc import ops
+from .lazy import Normed
 
 
-def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
+def _fused_norm(x: Normed, w: torch.Tensor, epilogue: int) -> Optional[torch.Tensor]:
+    if x._tensor is not None:
+        return None
+    scale = x.fusable_scale()
+    if scale is None or not ops.gemm_normed_supported(x.x, x.n_rows, scale[0], w):
+        return None
+    return ops.gemm_normed(x.x, x.rows, x.n_rows, scale[0], scale[1], w, epilogue)
+
+
+def linear(x: Union[torch.Tensor, Normed], w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
            accumulate_into: Optional[torch.Tensor] = None) -> torch.Tensor:
     """x [M, K] times w [N, K] transposed.  With ``accumulate_into`` (the
     float32 residual stream) the product is added to it in place."""
+    if isinstance(x, Normed):
+        if accumulate_into is None and out_dtype in (torch.bfloat16, torch.float32):
+            epi = ops.EPI_STORE_BF16 if out_dtype == torch.bfloat16 else ops.EPI_STORE_F32
+            fused = _fused_norm(x, w, epi)
+            if fused is not None:
+                return fused
+        x = x.tensor()
     fast = ops.gemm_fast(x, w, out_dtype, accumulate_into)
     if fast is not None:
         return fast
     return ops.gemm_generic(x, w, out_dtype, accumulate_into)
+
+
+def linear_swiglu(x: Union[torch.Tensor, Normed], w_gate_up: torch.Tensor) -> torch.Tensor:
+    """silu(x Wg^T) * (x Wu^T) for w_gate_up = gate rows followed by up rows."""
+    if isinstance(x, Normed):
+        fused = _fused_norm(x, w_gate_up, ops.EPI_SWIGLU) if w_gate_up.shape[0] % 2 == 0 else None
+        if fused is not None:
+            return fused
+        x = x.tensor()
+    return ops.gemm_swiglu(x, w_gate_up)

@@ -26,6 +26,10 @@ class RMSNorm(Part):
         self.weight = tensors["weight"]
         self.out_dtype = rt.act_dtype
 
+    def fusable(self):
+        """What a product needs to absorb this norm: (scale vector, eps)."""
+        return self.weight, self.eps
+
     def forward(self, x: torch.Tensor, ctx=None, rows=None, n_rows=None) -> torch.Tensor:
         return ops.rmsnorm(x, self.weight, self.eps, self.out_dtype, rows=rows, n_rows=n_rows)
 

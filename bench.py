@@ -140,6 +140,8 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=FULL_LAYERS, help="fewer than 22 only where time needs it")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--no-points", action="store_true", help="skip decoding at batch 1 and 64")
+    ap.add_argument("--only", choices=["decode", "prefill"], default=None,
+                    help="run one part only and print its own short line (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -152,6 +154,17 @@ def main() -> int:
     dtype = "bfloat16" if args.dtype == "bf16" else "float32"
     elem = 2 if args.dtype == "bf16" else 4
     model, cfg = build_model(args.layers, dtype)
+
+    if args.only == "decode":
+        dt, contexts = run_decode(model, cfg, args.batch, args.prompt_len, args.steps, args.warmup)
+        print(json.dumps({"only": "decode", "batch": args.batch, "ms_per_step": round(dt / args.steps * 1e3, 4),
+                          "tokens_per_s": round(args.batch * args.steps / dt, 1)}), flush=True)
+        return 0
+    if args.only == "prefill":
+        pre_s = run_prefill(model, cfg, args.prefill_tokens)
+        print(json.dumps({"only": "prefill", "tokens": args.prefill_tokens, "ms": round(pre_s * 1e3, 3),
+                          "tokens_per_s": round(args.prefill_tokens / pre_s, 1)}), flush=True)
+        return 0
 
     dt, contexts = run_decode(model, cfg, args.batch, args.prompt_len, args.steps, args.warmup)
     ms_per_step = dt / args.steps * 1e3

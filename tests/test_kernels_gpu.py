@@ -313,3 +313,28 @@ def test_argmax_ties_and_sampling(ops):
             cum = np.cumsum(w.astype(np.float64))
             edge = abs(us[i] * cum[-1] - cum[min(got[i], want)])
             assert abs(got[i] - want) == 1 and edge < 1e-3 * cum[-1], (i, got[i], want)
+
+
+@pytest.mark.parametrize("m", [1, 7, 16])
+@pytest.mark.parametrize("n,k", [(130, 304), (2560, 2048), (301, 80)])
+@pytest.mark.parametrize("gdt", [torch.bfloat16, torch.float32])
+def test_gemm_with_fused_rmsnorm(ops, m, n, k, gdt):
+    x = rnd(m + 3, k, seed=21, scale=3.0).float()
+    g = (1.0 + 0.2 * rnd(k, seed=22)).to(gdt)
+    w = bf(rnd(n, k, seed=23))
+    rows = torch.tensor(list(range(m + 2, 2, -1)), dtype=torch.int32)          # a gather, in another order
+    xs = x[rows.long()]
+    # rounded where the kernel rounds: bf16(x * g) into the matrix cores, the row's scale afterwards
+    hb = (xs * g.float()).to(torch.bfloat16).double()
+    scale = 1.0 / torch.sqrt((xs.double() ** 2).mean(-1, keepdim=True) + 1e-5)
+    exact = scale * (hb @ w.double().T)
+    ideal = P.rmsnorm(xs.double(), g.double(), 1e-5) @ w.double().T
+    mag = math.sqrt(k)
+    got = ops.gemm_normed(x.to(DEV), rows.to(DEV), m, g.to(DEV), 1e-5, w.to(DEV), ops.EPI_STORE_F32)
+    close(got, exact, 1e-4, 1e-4 * mag, "fused norm, same rounding")
+    close(got, ideal, 2e-2, 1e-2 * mag, "fused norm, ideal")
+    whole = ops.gemm_normed(x[:m].contiguous().to(DEV), None, m, g.to(DEV), 1e-5, w.to(DEV), ops.EPI_STORE_BF16)
+    close(whole, P.rmsnorm(x.double()[:m], g.double(), 1e-5) @ w.double().T, 2e-2, 1e-2 * mag, "fused norm bf16")
+    if n % 2 == 0:
+        got = ops.gemm_normed(x.to(DEV), rows.to(DEV), m, g.to(DEV), 1e-5, w.to(DEV), ops.EPI_SWIGLU)
+        close(got, P.swiglu(exact[:, :n // 2], exact[:, n // 2:]), 1e-2, 1e-2 * mag, "fused norm + swiglu")
