@@ -1,0 +1,172 @@
+"""The engine above the step function on the GPU: long decoding, the first tokens of a sequence,
+greedy generation through the entry point and the command line, batching and preemption."""
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import helpers
+from plain_llama import PlainLlama, argmax_lowest
+
+pytestmark = pytest.mark.gpu
+TOL = {"float32": dict(rtol=1e-4, atol=2e-6), "bfloat16": dict(rtol=2e-2, atol=6e-3)}
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    tmp = tmp_path_factory.mktemp("models")
+    return lambda name, dtype: helpers.make_model_dir(tmp, name, dtype)
+
+
+def follow_with_plain(plain, prompt, tokens, margin):
+    """The engine's tokens, checked step by step against the plain logits of the engine's own
+    sequence: each chosen token must be the plain argmax, or within `margin` of it (a near-tie
+    that rounding may turn)."""
+    ids = list(prompt)
+    full = plain.logits(ids + list(tokens))
+    for i, tok in enumerate(tokens):
+        row = full[len(prompt) - 1 + i]
+        gap = float(row.max() - row[tok])
+        assert gap <= margin, f"token {i} ({tok}) lies {gap:.4g} below the plain best {argmax_lowest(row)}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(folders, dtype):
+    """A short prompt, then several hundred tokens one by one (captured graphs, many pages)."""
+    from bare_cuda_4gib_amd.engine import Executor, StepEntry, load_model
+    folder = folders("C", dtype)
+    ids = helpers.random_ids(400, helpers.TINY_C["vocab_size"], 77)
+    plain = PlainLlama(folder).logits(ids).numpy()
+    model, _ = load_model(folder, dtype)
+    ex = Executor(model, num_pages=26, max_requests=2, max_tokens=416, page_tokens=16, poison=True)
+    ex.cache.shuffle_free_pages(3)
+    ex.admit("r")
+    got = {}
+    rows = ex.step([StepEntry("r", ids[:3], [0, 1, 2])]).cpu().numpy()      # the first tokens of a sequence
+    got.update({p: rows[p] for p in range(3)})
+    for p in range(3, 400):
+        got[p] = ex.step([StepEntry("r", [ids[p]], [0])]).cpu().numpy()[0]
+    where = {(0, p): ("r", p) for p in range(400)}
+    helpers.compare_with_plain({(0, p): got[p] for p in range(400)}, where, {"r": plain}, label=f"long {dtype}", **TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_first_tokens_one_by_one(folders, dtype):
+    """Positions 0, 1, 2, ... each as a step of its own: one key, then two, then three."""
+    from bare_cuda_4gib_amd.engine import Executor, StepEntry, load_model
+    folder = folders("A", dtype)
+    ids = helpers.random_ids(6, 256, 5)
+    plain = PlainLlama(folder).logits(ids).numpy()
+    model, _ = load_model(folder, dtype)
+    ex = Executor(model, num_pages=1, max_requests=1, max_tokens=64, page_tokens=64)
+    ex.admit(0)
+    got = {(0, p): ex.step([StepEntry(0, [ids[p]], [0])]).cpu().numpy()[0] for p in range(6)}
+    helpers.compare_with_plain(got, {(0, p): ("r", p) for p in range(6)}, {"r": plain}, label="first", **TOL[dtype])
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_greedy_generation_through_the_entry_point(folders, name, dtype):
+    from bare_cuda_4gib_amd.engine import Engine, generate_batch
+    cfg, _ = helpers.TINY[name]
+    folder = folders(name, dtype)
+    plain = PlainLlama(folder)
+    prompts = [helpers.random_ids(n, cfg["vocab_size"], 10 + n) for n in (1, 7, 33)]   # BASELINE's workload for A
+    engine = Engine(folder, max_tokens=64, max_seqs=3, kv_pages=0, dtype=dtype, page_tokens=16, prefill_chunk=16)
+    assert engine.vocab_size == cfg["vocab_size"] and engine.max_seqs == 3 and engine.healthy
+    together = generate_batch(engine, prompts, 16)
+    margin = 0.0 if dtype == "float32" else 2e-2
+    for p, toks in zip(prompts, together):
+        assert len(toks) == 16
+        follow_with_plain(plain, p, toks, margin + 1e-6)
+    if dtype == "float32":
+        assert together == [plain.greedy(p, 16) for p in prompts]
+    alone = [generate_batch(engine, [p], 16)[0] for p in prompts]
+    assert alone == together, "a request's tokens must not depend on what else is in the batch"
+    stats = engine.stats()
+    assert stats["kv_pages_used"] == 0 and stats["running"] == 0 and stats["prefill_tokens"] == 2 * sum(map(len, prompts))
+
+
+def test_entry_point_statuses_and_failure_path(folders):
+    from bare_cuda_4gib_amd.engine import Engine
+    engine = Engine(folders("A", "bfloat16"), max_tokens=32, max_seqs=1, max_waiting=1, page_tokens=16)
+    assert engine.submit(1, [], 4)[0] == "invalid"
+    assert engine.submit(1, [1] * 40, 4)[0] == "invalid"
+    assert engine.submit(1, [999], 4)[0] == "invalid"                              # outside the vocabulary
+    assert engine.submit(1, [1, 2], 4, temperature=-1.0)[0] == "invalid"
+    assert engine.submit(1, [1, 2, 3], 4) == ("ok", "")
+    assert engine.submit(1, [1, 2, 3], 4)[0] == "invalid"                          # id in use
+    assert engine.submit(2, [4, 5], 4, stop_ids=[7])[0] == "ok"
+    assert engine.submit(3, [4, 5], 4)[0] == "busy"                                # max_seqs + max_waiting live
+    events = engine.poll()
+    assert events and events[0][0] == 1 and events[0][2] == 0 and events[0][3] == ""
+    engine.cancel(2)
+    assert (2, -1, -1, "cancelled") in engine.poll() + engine.poll()
+    engine._fail_for_test("injected")
+    while True:
+        ev = engine.poll()
+        if any(e[3] == "error" for e in ev):
+            assert ev[-1][:3] == (1, -1, -1)
+            break
+        assert ev, "the failure must surface"
+    assert not engine.healthy and "injected" in engine.failure
+    assert engine.submit(9, [1], 1)[0] == "unavailable"
+
+
+def test_sampling_and_preemption_on_the_device(folders):
+    """Temperature sampling on the device: a seed gives the same tokens alone, batched, and when the
+    pool is so small that requests are preempted and recomputed."""
+    from bare_cuda_4gib_amd.engine import Engine, generate_batch
+    folder = folders("B", "float32")
+    prompts = [helpers.random_ids(n, 384, 40 + n) for n in (5, 64, 130)]            # BASELINE's workload for B
+    def run(kv_pages, which):
+        engine = Engine(folder, max_tokens=256, max_seqs=3, kv_pages=kv_pages, dtype="float32", page_tokens=16,
+                        prefill_chunk=32, max_batch_tokens=96)
+        out = {}
+        for i in which:
+            assert engine.submit(i, prompts[i], 24, temperature=0.8, seed=4 + i)[0] == "ok"
+        while len(out) < len(which) or any(len(v) < 24 for v in out.values()):
+            for id, tok, idx, fin in engine.poll():
+                out.setdefault(id, []).append(tok)
+        return out, engine.stats()
+    roomy, _ = run(0, [0, 1, 2])
+    tight, stats = run(13, [0, 1, 2])                                               # 208 tokens of pool for 5+64+130+3*23
+    assert stats["preemptions"] >= 1 and stats["kv_pages_used"] == 0
+    assert tight == roomy
+    assert run(0, [1])[0][1] == roomy[1]
+    again, _ = run(0, [0, 1, 2])
+    assert again == roomy and len(set(roomy[2])) > 3                                # repeatable, and really sampled
+
+
+def test_command_line(folders, tmp_path):
+    folder = folders("A", "float32")
+    prompt = helpers.random_ids(7, 256, 1)
+    proc = subprocess.run([sys.executable, os.path.join(helpers.ROOT, "bin", "llm-infer"), "--model", folder,
+                           "--prompt", ",".join(map(str, prompt)), "--tokens", "5", "--dtype", "float32"],
+                          capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    lines = proc.stdout.strip().splitlines()
+    assert lines[0].startswith("[llm] 2 layers, hidden 64, vocab 256") and lines[1].split() == ["prompt:"] + [str(t) for t in prompt]
+    assert [int(t) for t in lines[2].split()[1:]] == PlainLlama(folder).greedy(prompt, 5)
+    bad = subprocess.run([sys.executable, os.path.join(helpers.ROOT, "bin", "llm-infer"), "--model", str(tmp_path / "none"),
+                          "--prompt", "1,2"], capture_output=True, text=True, timeout=300)
+    assert bad.returncode != 0 and "config.json" in bad.stderr
+
+
+def test_missing_kernel_library_fails_loudly(monkeypatch):
+    from bare_cuda_4gib_amd.csrc import build, library
+    from bare_cuda_4gib_amd.errors import KernelError
+    monkeypatch.setattr(library, "_lib", None)
+    monkeypatch.setattr(build, "LIB_PATH", "/nonexistent/libbc4g.so")
+    with pytest.raises(KernelError):
+        library.load(build_if_missing=False)
+
+
+def test_cpu_tensors_are_refused():
+    from bare_cuda_4gib_amd.csrc import ops
+    from bare_cuda_4gib_amd.errors import KernelError
+    with pytest.raises(KernelError):
+        ops.rmsnorm(torch.zeros(2, 8), torch.ones(8), 1e-5, torch.float32)

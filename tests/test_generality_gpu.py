@@ -1,0 +1,265 @@
+"""That the framework's parts are general: a toy architecture, defined here and registered from
+here without a change to the framework's files, with
+  - a mixer with state of its own (a running mean over the request's tokens, kept in a state slot),
+  - attention with a window (its cache group gives pages back as the window moves on),
+  - a layer that runs twice (own cache each time) and a layer that reads another layer's cache,
+  - attention without any position encoding,
+is built, loaded from a random model folder, and stepped whole, in portions, and mixed with few
+pages -- against a plain implementation of the same toy model written with the plain functions.
+Each part of a layer is also run alone against its plain function."""
+import dataclasses
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import helpers
+import plain_llama as P
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+H, NH, NKV, D, INTER, VOCAB, WINDOW = 48, 4, 2, 16, 80, 97, 24
+
+
+def register_toy():
+    from bare_cuda_4gib_amd.cache import FixedState
+    from bare_cuda_4gib_amd.config import Architecture, ModelConfig, field_from_json, register_architecture
+    from bare_cuda_4gib_amd.config.registry import unregister_architecture
+    from bare_cuda_4gib_amd.engine.spec import LayerSpec, ModelSpec, PartSpec, ScheduleEntry
+    from bare_cuda_4gib_amd.parts import Part, register_part
+    from bare_cuda_4gib_amd.weights import WeightSpec
+
+    class RunningMean(Part):
+        """out[t] = W * mean(h[0..t]) over the request's tokens so far; state = [sum of h, count]."""
+        category = "mixer"
+
+        def __init__(self, hidden_size):
+            self.hidden = hidden_size
+
+        def cache_spec(self):
+            return FixedState((self.hidden + 1,), "float32")
+
+        def weight_specs(self):
+            return {"mix.weight": WeightSpec((self.hidden, self.hidden))}
+
+        def bind(self, tensors, rt):
+            self.w = tensors["mix.weight"].float()
+
+        def forward(self, h, ctx, cache, residual, writes=True):
+            h = h.float()
+            for s in range(ctx.n_seqs):
+                a, b = ctx.seq_start[s], ctx.seq_start[s + 1]
+                state = cache.state[ctx.seq_slots[s]]
+                sums = torch.cumsum(h[a:b], dim=0) + state[:self.hidden]
+                counts = torch.arange(1, b - a + 1, device=h.device, dtype=torch.float32) + state[self.hidden]
+                residual[a:b] += (sums / counts[:, None]) @ self.w.T
+                if writes:
+                    state[:self.hidden] = sums[-1]
+                    state[self.hidden] = counts[-1]
+
+    @dataclasses.dataclass
+    class ToyConfig(ModelConfig):
+        vocab_size: int = field_from_json("vocab_size")
+        hidden_size: int = field_from_json("hidden_size")
+        window: int = field_from_json("window")
+        eps: float = field_from_json("eps")
+
+    def describe(cfg):
+        norm = dict(size=cfg.hidden_size, eps=cfg.eps)
+        def attn(prefix, window, position):
+            return PartSpec("attention", dict(hidden_size=cfg.hidden_size, num_heads=NH, num_kv_heads=NKV, head_dim=D,
+                                              window=window, position=position), prefix=prefix)
+        rot = PartSpec("rotary", dict(theta=100.0, dim=8))              # rotary on half of the head only
+        def layer(i, mixer):
+            p = f"blocks.{i}."
+            return LayerSpec("prenorm", mixer, PartSpec("swiglu", dict(hidden_size=cfg.hidden_size, intermediate_size=INTER),
+                                                        prefix=p + "ffn."),
+                             PartSpec("rmsnorm", dict(norm), prefix=p + "norm1."), PartSpec("rmsnorm", dict(norm), prefix=p + "norm2."))
+        layers = [layer(0, attn("blocks.0.attn.", cfg.window, rot)),
+                  layer(1, PartSpec("toy_running_mean", dict(hidden_size=cfg.hidden_size), prefix="blocks.1.")),
+                  layer(2, attn("blocks.2.attn.", 0, PartSpec("none", {}))),
+                  layer(3, attn("blocks.3.attn.", 0, rot))]
+        schedule = [ScheduleEntry(0, "win"), ScheduleEntry(1, "mean"), ScheduleEntry(2, "full-a"),
+                    ScheduleEntry(2, "full-b"),                           # the same layer again, a cache of its own
+                    ScheduleEntry(3, "full-a", writes=False)]             # reads what layer 2's first run cached
+        return ModelSpec(vocab_size=cfg.vocab_size, hidden_size=cfg.hidden_size, max_seq_len=4096,
+                         embedding=PartSpec("embedding", dict(vocab_size=cfg.vocab_size, hidden_size=cfg.hidden_size), prefix="embed."),
+                         layers=layers, schedule=schedule, final_norm=PartSpec("rmsnorm", dict(norm), prefix="final_norm."),
+                         head=PartSpec("lm_head", dict(vocab_size=cfg.vocab_size, hidden_size=cfg.hidden_size, tied_to="embed.weight"),
+                                       prefix="head."))
+
+    try:
+        register_part("mixer", "toy_running_mean", RunningMean)
+    except Exception:
+        pass
+    unregister_architecture("ToyHybridForTests")
+    register_architecture(Architecture("ToyHybridForTests", "toy_hybrid_for_tests", ToyConfig, describe))
+
+
+TOY_CONFIG = dict(architectures=["ToyHybridForTests"], vocab_size=VOCAB, hidden_size=H, window=WINDOW, eps=1e-4)
+
+
+def plain_toy_logits(folder, ids):
+    """The toy model, whole sequence, float64, from the plain functions."""
+    from safetensors import safe_open
+    with safe_open(os.path.join(folder, "model.safetensors"), "pt") as f:
+        w = {n: f.get_tensor(n).double() for n in f.keys()}
+    t = len(ids)
+    pos = torch.arange(t)
+    x = w["embed.weight"][torch.tensor(ids)]
+
+    def qkv(p, h):
+        q = (h @ w[p + "q_proj.weight"].T).view(t, NH, D)
+        k = (h @ w[p + "k_proj.weight"].T).view(t, NKV, D)
+        v = (h @ w[p + "v_proj.weight"].T).view(t, NKV, D)
+        return q, k, v
+
+    def ffn(i, x):
+        p = f"blocks.{i}."
+        h = P.rmsnorm(x, w[p + "norm2.weight"], 1e-4)
+        return x + P.swiglu(h @ w[p + "ffn.gate_proj.weight"].T, h @ w[p + "ffn.up_proj.weight"].T) @ w[p + "ffn.down_proj.weight"].T
+
+    # layer 0: windowed attention with partial rotary
+    h = P.rmsnorm(x, w["blocks.0.norm1.weight"], 1e-4)
+    q, k, v = qkv("blocks.0.attn.", h)
+    o = P.attention(P.rope(q, pos, 100.0, 8), P.rope(k, pos, 100.0, 8), v, window=WINDOW)
+    x = ffn(0, x + o.reshape(t, -1) @ w["blocks.0.attn.o_proj.weight"].T)
+    # layer 1: running mean
+    h = P.rmsnorm(x, w["blocks.1.norm1.weight"], 1e-4)
+    mean = torch.cumsum(h, 0) / torch.arange(1, t + 1, dtype=torch.float64)[:, None]
+    x = ffn(1, x + mean @ w["blocks.1.mix.weight"].T)
+    # layer 2, twice; the first run's keys and values are kept for layer 3
+    kept = None
+    for run in range(2):
+        h = P.rmsnorm(x, w["blocks.2.norm1.weight"], 1e-4)
+        q, k, v = qkv("blocks.2.attn.", h)
+        if run == 0:
+            kept = (k, v)
+        x = ffn(2, x + P.attention(q, k, v).reshape(t, -1) @ w["blocks.2.attn.o_proj.weight"].T)
+    # layer 3: its own queries (rotated) on layer 2's cached keys (not rotated) and values
+    h = P.rmsnorm(x, w["blocks.3.norm1.weight"], 1e-4)
+    q, _, _ = qkv("blocks.3.attn.", h)
+    x = ffn(3, x + P.attention(P.rope(q, pos, 100.0, 8), kept[0], kept[1]).reshape(t, -1) @ w["blocks.3.attn.o_proj.weight"].T)
+    return P.rmsnorm(x, w["final_norm.weight"], 1e-4) @ w["embed.weight"].T
+
+
+@pytest.fixture(scope="module")
+def toy(tmp_path_factory):
+    register_toy()
+    from bare_cuda_4gib_amd.weights import write_random_model
+    tmp = tmp_path_factory.mktemp("toy")
+    out = {}
+    for dtype in ("float32", "bfloat16"):
+        folder = write_random_model(TOY_CONFIG, 9, str(tmp / dtype), dtype, std=0.08)
+        requests = {f"r{i}": helpers.random_ids(n, VOCAB, 300 + i) for i, n in enumerate([3, 50, 131, 90, 64])}
+        out[dtype] = (folder, requests, {r: plain_toy_logits(folder, ids).numpy() for r, ids in requests.items()})
+    return out
+
+
+TOL = {"float32": dict(rtol=2e-4, atol=2e-5), "bfloat16": dict(rtol=3e-2, atol=3e-2)}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_architecture_whole_portions_and_mixed(toy, dtype):
+    from bare_cuda_4gib_amd.cache import FixedState, PagedKV
+    from bare_cuda_4gib_amd.engine import Executor, load_model
+    folder, requests, plain = toy[dtype]
+    model, cfg = load_model(folder, dtype)
+    streams = model.cache_streams()
+    assert streams["win"] == PagedKV(NKV, D, WINDOW) and streams["full-a"] == PagedKV(NKV, D, 0)
+    assert streams["mean"] == FixedState((H + 1,), "float32") and set(streams) == {"win", "mean", "full-a", "full-b"}
+    page = 16
+    for label, (steps, where), pages in (
+            ("whole", helpers.trace_whole(requests), 12),
+            ("tail", helpers.trace_tail_one_by_one(requests, 32), 12),
+            ("portions", helpers.trace_portions(requests, seed=8), 12)):
+        ex = Executor(model, num_pages=pages, max_requests=4, max_tokens=160, page_tokens=page, poison=True)
+        assert not ex.use_graphs                                      # the toy mixer is not graph-safe
+        ex.cache.shuffle_free_pages(1)
+        got = helpers.replay_in_process(ex, steps)
+        helpers.compare_with_plain(got, where, plain, label=f"toy {label} {dtype}", **TOL[dtype])
+        assert ex.cache.pages_in_use() == 0
+    steps, where, peak = helpers.trace_mixed(requests, seed=2, max_live=4, page_tokens=page)
+    ex = Executor(model, num_pages=peak // page, max_requests=4, max_tokens=160, page_tokens=page, poison=True)
+    ex.cache.shuffle_free_pages(2)
+    got = helpers.replay_in_process(ex, steps)
+    helpers.compare_with_plain(got, where, plain, label=f"toy mixed {dtype}", **TOL[dtype])
+    full, win = ex.cache.groups[("window", 0)].pool, ex.cache.groups[("window", WINDOW)].pool
+    assert full.high_water_mark == full.num_pages                    # the pool of the full group was used up
+    assert win.high_water_mark < full.high_water_mark, "the windowed group must have given pages back early"
+
+
+def test_unknown_part_and_bad_schedule_are_refused(toy):
+    from bare_cuda_4gib_amd.engine import Model
+    from bare_cuda_4gib_amd.engine.spec import PartSpec, ScheduleEntry
+    from bare_cuda_4gib_amd.config import architecture_for
+    from bare_cuda_4gib_amd.errors import ConfigError
+    arch = architecture_for(TOY_CONFIG)
+    spec = arch.describe(arch.config_class.from_dict(TOY_CONFIG))
+    spec.schedule.append(ScheduleEntry(3, "nobody-writes-this", writes=False))
+    with pytest.raises(ConfigError):
+        Model(spec).cache_streams()
+    spec = arch.describe(arch.config_class.from_dict(TOY_CONFIG))
+    spec.layers[0].ffn = PartSpec("no_such_feedforward", {})
+    with pytest.raises(ConfigError) as e:
+        Model(spec)
+    assert "swiglu" in str(e.value)
+
+
+# --- each part of a layer alone -------------------------------------------------------
+
+def _bind(part, tensors, dtype):
+    from bare_cuda_4gib_amd.engine import Runtime
+    rt = Runtime(torch.device(DEV), dtype)
+    part.bind({k: rt.place_weight(v) for k, v in tensors.items()}, rt)
+    return part
+
+
+def _ctx_for(model_like_executor, entries):
+    return model_like_executor.build_context(entries)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_parts_alone(dtype):
+    """Norm, feed-forward, embedding and head, each built from its sizes alone and compared with
+    its plain function; attention (with rotary, cache write and block table) through a one-layer
+    context is covered by the kernel tests and the toy model above."""
+    from bare_cuda_4gib_amd.parts import build_part
+    from bare_cuda_4gib_amd.engine.spec import PartSpec
+    g = torch.Generator().manual_seed(0)
+    tol = dict(rtol=1e-4, atol=1e-5) if dtype == torch.float32 else dict(rtol=3e-2, atol=3e-2)
+    wdt = dtype
+    x = torch.randn(70, 48, generator=g)                                  # 70 rows: beyond the skinny kernels
+    xs = x[:5].contiguous()
+    # norm
+    nw = (1 + 0.1 * torch.randn(48, generator=g)).to(wdt)
+    norm = _bind(build_part("norm", PartSpec("rmsnorm", dict(size=48, eps=1e-3))), {"weight": nw}, dtype)
+    for inp in (x, xs):
+        got = norm.forward(inp.to(DEV)).float().cpu()
+        want = P.rmsnorm(inp.double(), nw.double(), 1e-3)
+        assert torch.allclose(got.double(), want, **tol)
+    # feed-forward: adds into the residual stream
+    wg, wu, wd = (torch.randn(s, generator=g).mul(0.2).to(wdt) for s in ((80, 48), (80, 48), (48, 80)))
+    ffn = _bind(build_part("feedforward", PartSpec("swiglu", dict(hidden_size=48, intermediate_size=80))),
+                {"gate_proj.weight": wg, "up_proj.weight": wu, "down_proj.weight": wd}, dtype)
+    for inp in (x, xs):
+        h = inp.to(dtype)
+        res = torch.ones(inp.shape[0], 48, device=DEV)
+        ffn.forward(h.to(DEV), None, res)
+        want = 1.0 + P.swiglu(h.double() @ wg.double().T, h.double() @ wu.double().T) @ wd.double().T
+        assert torch.allclose(res.cpu().double(), want, **tol)
+    # embedding and head
+    table = torch.randn(61, 48, generator=g).to(wdt)
+    emb = _bind(build_part("embedding", PartSpec("embedding", dict(vocab_size=61, hidden_size=48))), {"weight": table}, dtype)
+
+    class Ids:
+        token_ids = torch.tensor([3, 60, 0, 3], dtype=torch.int32, device=DEV)
+    assert torch.equal(emb.forward(Ids).cpu(), table.float()[[3, 60, 0, 3]])
+    head = _bind(build_part("head", PartSpec("lm_head", dict(vocab_size=61, hidden_size=48))), {"weight": table}, dtype)
+    hrows = x[:9].to(dtype)
+    got = head.forward(hrows.to(DEV).contiguous())
+    assert got.dtype == torch.float32
+    assert torch.allclose(got.cpu().double(), hrows.double() @ table.double().T, **tol)
