@@ -209,23 +209,35 @@ __global__ __launch_bounds__(kWavesPerBlock * kWave) void attention_mfma_kernel(
 }
 
 // out[row, head, :] = sum_z 2^(m_z - M) O_z / sum_z 2^(m_z - M) l_z, parts added in order of z.
-__global__ void attention_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                       bf16_t* __restrict__ out, int n_splits, long n_rows_heads, int d) {
+// One wave per (row, head), up to 64 parts: lane z reads part z's statistics, the weights go
+// through LDS, and every lane then sums its output dimensions over the parts.
+constexpr int kMaxSplits = 64;
+
+__global__ __launch_bounds__(kWave) void attention_merge_kernel(const float* __restrict__ part_o,
+                                                                const float* __restrict__ part_ml,
+                                                                bf16_t* __restrict__ out, int n_splits,
+                                                                long n_rows_heads, int d) {
+  __shared__ float weight[kMaxSplits];
   const long rh = blockIdx.x;
-  float m = -INFINITY;
-  for (int z = 0; z < n_splits; ++z) m = fmaxf(m, part_ml[(z * n_rows_heads + rh) * 2]);
-  float l = 0.f;
-  for (int z = 0; z < n_splits; ++z) {
-    const float mz = part_ml[(z * n_rows_heads + rh) * 2];
-    if (mz != -INFINITY) l += exp2f(mz - m) * part_ml[(z * n_rows_heads + rh) * 2 + 1];
+  const int lane = threadIdx.x;
+  float mz = -INFINITY, lz = 0.f;
+  if (lane < n_splits) {
+    const float2 ml = *reinterpret_cast<const float2*>(part_ml + (lane * n_rows_heads + rh) * 2);
+    mz = ml.x;
+    lz = ml.y;
   }
+  const float m = wave_max(mz);
+  const float wz = (mz == -INFINITY) ? 0.f : exp2f(mz - m);
+  weight[lane] = wz;
+  // the sum over parts in order of z, the same in every lane
+  __syncthreads();
+  float l = 0.f;
+  for (int z = 0; z < n_splits; ++z) l += weight[z] * __shfl(lz, z, kWave);
   const float inv = 1.0f / l;
-  for (int c = threadIdx.x; c < d; c += blockDim.x) {
+  for (int c = lane; c < d; c += kWave) {
     float acc = 0.f;
-    for (int z = 0; z < n_splits; ++z) {
-      const float mz = part_ml[(z * n_rows_heads + rh) * 2];
-      if (mz != -INFINITY) acc += exp2f(mz - m) * part_o[(z * n_rows_heads + rh) * d + c];
-    }
+#pragma unroll 8
+    for (int z = 0; z < n_splits; ++z) acc += weight[z] * part_o[(z * n_rows_heads + rh) * d + c];
     out[rh * d + c] = from_float<bf16_t>(acc * inv);
   }
 }
@@ -247,8 +259,8 @@ extern "C" int bc4g_attention_mfma(const void* qkv, void* out, float* part_o, fl
                "attention_mfma: head_dim %d must be a multiple of 16 up to 256", head_dim);
   BC4G_REQUIRE(page_tokens > 0 && page_tokens % 16 == 0, "attention_mfma: page_tokens %d must be a multiple of 16",
                page_tokens);
-  BC4G_REQUIRE(n_splits >= 1 && n_splits <= 65535 && (n_splits == 1 || (part_o && part_ml)),
-               "attention_mfma: bad split count %d", n_splits);
+  BC4G_REQUIRE(n_splits >= 1 && n_splits <= kMaxSplits && (n_splits == 1 || (part_o && part_ml)),
+               "attention_mfma: the split count %d must lie in 1..64", n_splits);
   BC4G_REQUIRE(window >= 0 && table_stride > 0 && n_seqs > 0, "attention_mfma: bad sizes");
   if (n_tiles == 0 || n_tokens == 0) return 0;
   const int group = n_heads / n_kv_heads;

@@ -294,6 +294,7 @@ def attention_tile_tokens(n_heads: int, n_kv_heads: int) -> int:
 
 
 ATTENTION_TARGET_WAVES = 2048
+ATTENTION_MAX_SPLITS = 64
 
 
 def attention_splits(n_tiles: int, n_heads: int, n_kv_heads: int, max_kv_len: int) -> int:
@@ -302,7 +303,7 @@ def attention_splits(n_tiles: int, n_heads: int, n_kv_heads: int, max_kv_len: in
     group = n_heads // n_kv_heads
     waves = n_tiles * n_kv_heads * (-(-group // 16))
     key_tiles = max(1, -(-max_kv_len // 32))
-    return max(1, min(ATTENTION_TARGET_WAVES // max(waves, 1), key_tiles))
+    return max(1, min(ATTENTION_TARGET_WAVES // max(waves, 1), key_tiles, ATTENTION_MAX_SPLITS))
 
 
 def attention_mfma(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,

@@ -256,7 +256,7 @@ def run_mfma(ops, case, window, n_splits):
 
 @pytest.mark.parametrize("nh,nkv,d,page", SHAPES)
 @pytest.mark.parametrize("window", [0, 20])
-@pytest.mark.parametrize("n_splits", [1, 3, 16])
+@pytest.mark.parametrize("n_splits", [1, 3, 16, 64])
 def test_attention_mfma(ops, nh, nkv, d, page, window, n_splits):
     case = paged_case(SEQS, nh, nkv, d, page, torch.bfloat16, seed=4)
     assert ops.attention_mfma_supported(case["qkv"], case["kc"], d)
