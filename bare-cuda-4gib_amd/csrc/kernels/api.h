@@ -27,8 +27,10 @@ int bc4g_rmsnorm(const float* x, const int32_t* rows, const void* w, int w_dtype
 int bc4g_gemm_generic(const void* a, int a_dtype, const void* w, int w_dtype, void* out,
                       int out_dtype, int accumulate, int m, int n, int k, void* stream);
 
-// out[t, i] = silu(gu[t, i]) * gu[t, inter + i]                          (swiglu.cu:17-25)
-int bc4g_swiglu(const void* gu, void* out, int dtype, int n_tokens, int inter, void* stream);
+// out[t, i] = silu(gate_i) * up_i                                        (swiglu.cu:17-25)
+// interleaved 0: gu[t] = all gates, then all ups.  1: blocks of 16 = eight gates, then the eight
+// ups of the same outputs.
+int bc4g_swiglu(const void* gu, void* out, int dtype, int n_tokens, int inter, int interleaved, void* stream);
 
 // Rotates q (in place) and k by each row's position, and writes k and v into
 // their cache pages (rope.cu:18-55, kv_cache_write.cu:10-20).
@@ -36,18 +38,22 @@ int bc4g_swiglu(const void* gu, void* out, int dtype, int n_tokens, int inter, v
 // offset of the row's token; k_cache: [pages, n_kv_heads, page_tokens, head_dim]; v_cache is kept
 // transposed, [pages, n_kv_heads, head_dim, page_tokens], so that the matrix-core kernels can load
 // consecutive tokens of one dimension.
-// rotary_dim 0 switches the rotation off; write_kv 0 leaves the cache alone.
+// rotary_dim 0 switches the rotation off; write_kv 0 leaves the cache alone.  block_pairs 1: every
+// head's dimensions come reordered in blocks of 16 (dimensions 8b..8b+7, then their rotation
+// partners head_dim/2 + 8b..), the order the fused weight-streaming kernel works in; queries, keys and
+// values then all live in that order (scores and outputs do not care, as long as all agree).
 int bc4g_rope_kv_write(void* qkv, int dtype, const int32_t* positions, const int32_t* slot_map,
                        void* k_cache, void* v_cache, int n_tokens, int n_heads, int n_kv_heads,
                        int head_dim, int rotary_dim, float theta, int page_tokens, int num_pages,
-                       int write_kv, void* stream);
+                       int write_kv, int block_pairs, void* stream);
 
 // Causal softmax attention of every row over its request's cached keys
 // (attention_qk.cu:17-70, softmax.cu:22-43, attention_av.cu:18-46, fused).
 // Row t of request s = row_seq[t] at position p = positions[t] sees keys
 // max(0, p - window + 1) .. p (window 0 = all); key j lies in page
-// block_table[s, j / page_tokens].  q is read from the qkv rows; out: [n_tokens, n_heads*head_dim].
-int bc4g_attention_generic(const void* qkv, void* out, int dtype, const void* k_cache,
+// block_table[s, j / page_tokens].  The query of row t, head h is read at qkv + t * q_stride + h * head_dim
+// (the rows of the fused q|k|v product, or of a buffer of queries alone); out: [n_tokens, n_heads*head_dim].
+int bc4g_attention_generic(const void* qkv, int q_stride, void* out, int dtype, const void* k_cache,
                            const void* v_cache, const int32_t* block_table, int table_stride,
                            const int32_t* row_seq, const int32_t* positions, int n_tokens,
                            int n_heads, int n_kv_heads, int head_dim, int page_tokens,
@@ -65,22 +71,25 @@ int bc4g_sample(const float* logits, const float* temperature, const double* u, 
 extern "C" {
 // bfloat16 x [m, k] (m <= 64) times bfloat16 w [n, k] transposed, weights streamed once through
 // the matrix cores.  epilogue: 0 store bfloat16 [m, n]; 1 store float32; 2 add into float32;
-// 3 SwiGLU: w = gate rows then up rows (n = 2 * inter), out bfloat16 [m, inter] = silu(gate) * up.
+// 3 SwiGLU: every 16 rows of w are eight gate rows and the eight up rows of the same outputs
+// (n = 2 * inter), out bfloat16 [m, inter] = silu(gate) * up.
 int bc4g_gemm_skinny(const void* x, const void* w, void* out, int epilogue, int m, int n, int k, void* stream);
 }
 
 extern "C" {
-// Attention on the matrix cores (bfloat16): see attention_mfma.hip.  tile_start[s] is the first
-// 16-row tile of request s when every request's rows are cut into tiles of tokens_per_tile tokens
-// (times the query heads of one key/value head); n_tiles their total.  With n_splits > 1 the keys
+// Attention on the matrix cores (bfloat16): see attention_mfma.hip.  A wave takes q_tiles tiles of
+// 16 rows, each tokens_per_tile tokens times the query heads of one key/value head; tile_start[s]
+// is the first wave-sized piece of request s when every request's rows are cut into pieces of
+// q_tiles * tokens_per_tile tokens; n_tiles their total.  q_tiles is 1, or 4 for head sizes up to
+// 64 and 2 up to 128.  With n_splits > 1 the keys
 // are cut into that many parts whose float partials (part_o [n_splits, T, heads, d], part_ml
 // [n_splits, T, heads, 2]) are merged into out.
-int bc4g_attention_mfma(const void* qkv, void* out, float* part_o, float* part_ml, const void* k_cache,
+int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, float* part_o, float* part_ml, const void* k_cache,
                         const void* v_cache, const int32_t* block_table, int table_stride,
                         const int32_t* seq_start, const int32_t* seq_ctx, const int32_t* tile_start,
                         int n_seqs, int n_tiles, int n_tokens, int n_heads, int n_kv_heads, int head_dim,
-                        int page_tokens, int window, float scale, int tokens_per_tile, int n_splits,
-                        void* stream);
+                        int page_tokens, int window, float scale, int tokens_per_tile, int q_tiles,
+                        int n_splits, void* stream);
 }
 
 extern "C" {
@@ -96,4 +105,15 @@ extern "C" {
 // except adding into a float output.
 int bc4g_gemm_skinny_normed(const float* x, const int32_t* rows, const void* g, int g_dtype, float eps,
                             const void* w, void* out, int epilogue, int m, int n, int k, void* stream);
+}
+
+extern "C" {
+// The query/key/value product of a decode step with rotary positions and the cache write in its
+// epilogue (see gemm_skinny.hip).  x: bfloat16 [m, k] with g null (m <= 64), or the float32 residual
+// stream with RMSNorm fused (g given, m <= 16).  w: [(heads + 2 kv heads) * head_dim, k] with every
+// head's rows reordered in blocks of 16.  q_out: bfloat16 [m, heads * head_dim].
+int bc4g_gemm_skinny_qkv(const void* x, const void* g, int g_dtype, float eps, const void* w, void* q_out,
+                         const int32_t* positions, const int32_t* slot_map, void* k_cache, void* v_cache,
+                         int m, int k, int n_heads, int n_kv_heads, int head_dim, int rotary_dim, float theta,
+                         int page_tokens, int write_kv, void* stream);
 }

@@ -25,14 +25,14 @@ __global__ __launch_bounds__(kWave) void attention_generic_kernel(
     const T* __restrict__ qkv, T* __restrict__ out, const T* __restrict__ k_cache,
     const T* __restrict__ v_cache, const int32_t* __restrict__ block_table, int table_stride,
     const int32_t* __restrict__ row_seq, const int32_t* __restrict__ positions, int n_heads,
-    int n_kv_heads, int head_dim, int page_tokens, int window, float scale) {
+    int n_kv_heads, int head_dim, int page_tokens, int window, float scale, int q_stride) {
   __shared__ float q_s[kMaxHeadDim];
   __shared__ float p_s[kWave];
   const int row = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   const int kvh = head / (n_heads / n_kv_heads);
   const int pos = positions[row];
   const int32_t* table = block_table + static_cast<long>(row_seq[row]) * table_stride;
-  const long qkv_stride = static_cast<long>(n_heads + 2 * n_kv_heads) * head_dim;
+  const long qkv_stride = q_stride;
   const T* q = qkv + row * qkv_stride + static_cast<long>(head) * head_dim;
   for (int c = lane; c < head_dim; c += kWave) q_s[c] = to_float(q[c]);
   __syncthreads();
@@ -90,7 +90,7 @@ __global__ __launch_bounds__(kWave) void attention_generic_kernel(
 
 using namespace bc4g;
 
-extern "C" int bc4g_attention_generic(const void* qkv, void* out, int dtype, const void* k_cache,
+extern "C" int bc4g_attention_generic(const void* qkv, int q_stride, void* out, int dtype, const void* k_cache,
                                       const void* v_cache, const int32_t* block_table, int table_stride,
                                       const int32_t* row_seq, const int32_t* positions, int n_tokens,
                                       int n_heads, int n_kv_heads, int head_dim, int page_tokens,
@@ -103,6 +103,7 @@ extern "C" int bc4g_attention_generic(const void* qkv, void* out, int dtype, con
                "attention: bad cache sizes page_tokens=%d pages=%d table_stride=%d window=%d", page_tokens,
                num_pages, table_stride, window);
   BC4G_REQUIRE(n_heads <= 65535, "attention: %d heads are beyond the grid limit", n_heads);
+  BC4G_REQUIRE(q_stride >= n_heads * head_dim, "attention: bad query row stride %d", q_stride);
   if (n_tokens == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   dim3 grid(n_tokens, n_heads);
@@ -110,12 +111,12 @@ extern "C" int bc4g_attention_generic(const void* qkv, void* out, int dtype, con
     attention_generic_kernel<float><<<grid, kWave, 0, s>>>(
         static_cast<const float*>(qkv), static_cast<float*>(out), static_cast<const float*>(k_cache),
         static_cast<const float*>(v_cache), block_table, table_stride, row_seq, positions, n_heads,
-        n_kv_heads, head_dim, page_tokens, window, scale);
+        n_kv_heads, head_dim, page_tokens, window, scale, q_stride);
   } else if (dtype == kBF16) {
     attention_generic_kernel<bf16_t><<<grid, kWave, 0, s>>>(
         static_cast<const bf16_t*>(qkv), static_cast<bf16_t*>(out), static_cast<const bf16_t*>(k_cache),
         static_cast<const bf16_t*>(v_cache), block_table, table_stride, row_seq, positions, n_heads,
-        n_kv_heads, head_dim, page_tokens, window, scale);
+        n_kv_heads, head_dim, page_tokens, window, scale, q_stride);
   } else {
     return fail("attention: unknown dtype %d", dtype);
   }

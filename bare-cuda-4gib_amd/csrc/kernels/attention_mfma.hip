@@ -27,8 +27,19 @@ namespace {
 constexpr int kWavesPerBlock = 4;
 constexpr float kLog2e = 1.4426950408889634f;
 
+// 2^x by the hardware instruction (arguments here are <= 0 or -inf; results below the smallest
+// normal number flush to zero, which is what a softmax weight that small may do).
+__device__ inline float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Two floats to two bfloat16 (round to nearest even) in one instruction of gfx950.
+__device__ inline uint32_t pack_bf16x2(float lo, float hi) {
+  uint32_t r;
+  asm volatile("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(r) : "v"(lo), "v"(hi));
+  return r;
+}
+
 struct AttnArgs {
-  const bf16_t* qkv;
+  const bf16_t* qkv;           // queries: row t, head h at qkv + t * q_stride + h * d
   bf16_t* out;                 // [T, n_heads * d]               (n_splits == 1)
   float* part_o;               // [n_splits, T, n_heads, d]      (n_splits > 1), unnormalized
   float* part_ml;              // [n_splits, T, n_heads, 2]      running max (base 2) and sum
@@ -38,16 +49,18 @@ struct AttnArgs {
   const int32_t* seq_start;    // [S + 1] first row of each request in the batch
   const int32_t* seq_ctx;      // [S] tokens cached before this step
   const int32_t* tile_start;   // [S + 1] first tile of each request
-  int table_stride, n_seqs, n_tiles, n_tokens;
+  int table_stride, n_seqs, n_tiles, n_tokens, q_stride;
   int n_heads, n_kv_heads, head_dim, page_tokens, window;
   int hg, tpt, n_sub;          // heads per tile, tokens per tile, head sub-groups per kv head
   int n_splits;
   float scale_log2;            // softmax scale times log2(e)
 };
 
-// DJ: k-steps of 32 over head_dim for the scores; DB: blocks of 16 output dimensions.
-template <int DJ, int DB>
-__global__ __launch_bounds__(kWavesPerBlock * kWave) void attention_mfma_kernel(const AttnArgs a) {
+// DJ: k-steps of 32 over head_dim for the scores; DB: blocks of 16 output dimensions; QT: 16-row
+// query tiles per wave (consecutive tokens), which share every key and value fragment the wave
+// loads -- prompt portions use 4 (or 2 for large heads), decoded tokens 1.
+template <int DJ, int DB, int QT>
+__global__ __launch_bounds__(kWavesPerBlock * kWave, 2) void attention_mfma_kernel(const AttnArgs a) {
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int col = lane % 16, grp = lane / 16;
   const int tile = blockIdx.x * kWavesPerBlock + wave;
@@ -63,28 +76,34 @@ __global__ __launch_bounds__(kWavesPerBlock * kWave) void attention_mfma_kernel(
   const int row0 = a.seq_start[s];
   const int q_len = a.seq_start[s + 1] - row0;
   const int ctx = a.seq_ctx[s];
-  const int tok0 = (tile - a.tile_start[s]) * a.tpt;
-  const int ntok = min(a.tpt, q_len - tok0);
+  const int tok0 = (tile - a.tile_start[s]) * a.tpt * QT;
+  const int ntok = min(a.tpt * QT, q_len - tok0);
   const int kvh = blockIdx.y / a.n_sub, hsub = blockIdx.y % a.n_sub;
   const int group = a.n_heads / a.n_kv_heads;
   const int d = a.head_dim, P = a.page_tokens;
   const int32_t* table = a.block_table + static_cast<long>(s) * a.table_stride;
 
-  // this lane's query row (as B operand and as owner of one row's statistics)
-  const int q_tok = col / a.hg, q_hsub = col % a.hg;
+  // this lane's query row in each tile (as B operand and as owner of one row's statistics)
+  const int q_hsub = col % a.hg;
   const int q_head_in_group = hsub * a.hg + q_hsub;
-  const bool q_ok = q_tok < ntok && q_head_in_group < group;
   const int q_head = kvh * group + q_head_in_group;
-  const int q_pos = ctx + tok0 + q_tok;
-  const int q_lo = (a.window > 0 && q_pos - a.window + 1 > 0) ? q_pos - a.window + 1 : 0;
-  const long qkv_stride = static_cast<long>(a.n_heads + 2 * a.n_kv_heads) * d;
-
-  uint4 qf[DJ];
+  const long qkv_stride = a.q_stride;
+  int q_tok[QT], q_pos[QT], q_lo[QT];
+  bool q_ok[QT];
+  uint4 qf[QT][DJ];
 #pragma unroll
-  for (int j = 0; j < DJ; ++j) {
-    const int c = 32 * j + 8 * grp;
-    qf[j] = (q_ok && c < d) ? load16(a.qkv + (row0 + tok0 + q_tok) * qkv_stride + static_cast<long>(q_head) * d + c)
-                            : zero16();
+  for (int t = 0; t < QT; ++t) {
+    q_tok[t] = t * a.tpt + col / a.hg;
+    q_ok[t] = col / a.hg < a.tpt && q_tok[t] < ntok && q_head_in_group < group;
+    q_pos[t] = ctx + tok0 + q_tok[t];
+    q_lo[t] = (a.window > 0 && q_pos[t] - a.window + 1 > 0) ? q_pos[t] - a.window + 1 : 0;
+#pragma unroll
+    for (int j = 0; j < DJ; ++j) {
+      const int c = 32 * j + 8 * grp;
+      qf[t][j] = (q_ok[t] && c < d)
+                     ? load16(a.qkv + (row0 + tok0 + q_tok[t]) * qkv_stride + static_cast<long>(q_head) * d + c)
+                     : zero16();
+    }
   }
 
   const int pos_min = ctx + tok0, pos_max = ctx + tok0 + ntok - 1;
@@ -95,65 +114,69 @@ __global__ __launch_bounds__(kWavesPerBlock * kWave) void attention_mfma_kernel(
   const int kt_begin = kt_first + blockIdx.z * per_split;
   const int kt_end = min(kt_last + 1, kt_begin + per_split);
 
-  float m_run = -INFINITY, l_run = 0.f;
-  floatx4 o[DB];
+  float m_run[QT], l_run[QT];
+  floatx4 o[QT][DB];
 #pragma unroll
-  for (int b = 0; b < DB; ++b) o[b] = floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int t = 0; t < QT; ++t) {
+    m_run[t] = -INFINITY;
+    l_run[t] = 0.f;
+#pragma unroll
+    for (int b = 0; b < DB; ++b) o[t][b] = floatx4{0.f, 0.f, 0.f, 0.f};
+  }
 
-  for (int kt = kt_begin; kt < kt_end; ++kt) {
-    const int key0 = kt * 32;
-    floatx4 sc[2];
-    long vbase[2];
-    bool sub_ok[2];
+  // The request's block table, held across the wave's lanes (entry i in lane i % 64 of register
+  // i / 64), so that finding a tile's page is a lane read and not a trip to memory.
+  constexpr int kTableRegs = 4;
+  int32_t tbl[kTableRegs];
+  const int pages_needed = pos_max / P + 1;
+#pragma unroll
+  for (int r = 0; r < kTableRegs; ++r) {
+    const int idx = r * kWave + lane;
+    tbl[r] = (idx < pages_needed && idx < a.table_stride) ? table[idx] : 0;
+  }
+  auto page_of = [&](int page_index) -> long {
+    if (page_index >= kTableRegs * kWave) return table[page_index];
+    int32_t v = __shfl(tbl[0], page_index % kWave, kWave);
+#pragma unroll
+    for (int r = 1; r < kTableRegs; ++r) {
+      const int32_t w = __shfl(tbl[r], page_index % kWave, kWave);
+      if (page_index / kWave == r) v = w;
+    }
+    return v;
+  };
+
+  // one tile of 32 keys: key fragments (A operand of the scores) and value fragments (A operand
+  // of the output), fetched one tile ahead of their use
+  struct KeyTile {
+    uint4 k[2][DJ];
+    uint2 v[2][DB];
+    bool ok[2];
+  };
+  auto fetch = [&](KeyTile& t, int kt) {
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-      const int kb = key0 + 16 * h;
-      sub_ok[h] = kb <= pos_max && kb + 15 >= lo_min;
-      sc[h] = floatx4{0.f, 0.f, 0.f, 0.f};
-      vbase[h] = 0;
-      if (sub_ok[h]) {
-        const long page = table[kb / P];
-        const int off = kb % P;
-        const bf16_t* kptr = a.k_cache + ((page * a.n_kv_heads + kvh) * P + off + col) * d + 8 * grp;
-        vbase[h] = (page * a.n_kv_heads + kvh) * static_cast<long>(d) * P + off + 4 * grp;
+      const int kb = kt * 32 + 16 * h;
+      t.ok[h] = kb <= pos_max && kb + 15 >= lo_min;
+      long page = 0;
+      if (t.ok[h]) page = page_of(kb / P);
+      const int off = kb % P;
+      const bf16_t* kptr = a.k_cache + ((page * a.n_kv_heads + kvh) * P + off + col) * d + 8 * grp;
+      const bf16_t* vptr = a.v_cache + (page * a.n_kv_heads + kvh) * static_cast<long>(d) * P + off + 4 * grp +
+                           static_cast<long>(col) * P;
 #pragma unroll
-        for (int j = 0; j < DJ; ++j) {
-          const uint4 kf = (32 * j + 8 * grp < d) ? load16(kptr + 32 * j) : zero16();
-          sc[h] = mfma_16x16x32(kf, qf[j], sc[h]);
-        }
-      }
+      for (int j = 0; j < DJ; ++j) t.k[h][j] = (t.ok[h] && 32 * j + 8 * grp < d) ? load16(kptr + 32 * j) : zero16();
+#pragma unroll
+      for (int b = 0; b < DB; ++b)
+        t.v[h][b] = (t.ok[h] && 16 * b < d) ? *reinterpret_cast<const uint2*>(vptr + static_cast<long>(16 * b) * P)
+                                            : make_uint2(0u, 0u);
     }
-    // mask by position; this lane holds, for its query row, keys key0 + 16h + 4*grp + r
-    float sv[8];
-    float m_tile = -INFINITY;
-#pragma unroll
-    for (int h = 0; h < 2; ++h)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int key = key0 + 16 * h + 4 * grp + r;
-        const bool vis = sub_ok[h] && q_ok && key <= q_pos && key >= q_lo;
-        const float v = vis ? sc[h][r] * a.scale_log2 : -INFINITY;
-        sv[4 * h + r] = v;
-        m_tile = fmaxf(m_tile, v);
-      }
-    m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 16, kWave));
-    m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, kWave));
-    const float m_new = fmaxf(m_run, m_tile);
-    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-    const float alpha = exp2f(m_run - m_safe);   // 0 while nothing has been seen
-    float psum = 0.f;
-    uint32_t pk[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const float p0 = exp2f(sv[2 * i] - m_safe), p1 = exp2f(sv[2 * i + 1] - m_safe);
-      psum += p0 + p1;
-      pk[i] = static_cast<uint32_t>(bf16_bits_from_float(p0)) |
-              (static_cast<uint32_t>(bf16_bits_from_float(p1)) << 16);
-    }
-    l_run = l_run * alpha + psum;
-    m_run = m_new;
-    const uint4 pf = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+  };
 
+  KeyTile cur, nxt;
+  if (kt_begin < kt_end) fetch(cur, kt_begin);
+  for (int kt = kt_begin; kt < kt_end; ++kt) {
+    if (kt + 1 < kt_end) fetch(nxt, kt + 1);
+    const int key0 = kt * 32;
     // values of keys past the tile's last position are replaced by zero
     uint32_t vmask[4];
 #pragma unroll
@@ -163,47 +186,105 @@ __global__ __launch_bounds__(kWavesPerBlock * kWave) void attention_mfma_kernel(
       vmask[2 * h + 1] = (kb + 2 <= pos_max ? 0xffffu : 0u) | (kb + 3 <= pos_max ? 0xffff0000u : 0u);
     }
 #pragma unroll
-    for (int b = 0; b < DB; ++b) {
-      if (16 * b >= d) break;   // DB is the most blocks this instantiation holds
-      uint2 v0 = make_uint2(0u, 0u), v1 = make_uint2(0u, 0u);
-      const long dim_off = static_cast<long>(16 * b + col) * P;
-      if (sub_ok[0]) v0 = *reinterpret_cast<const uint2*>(a.v_cache + vbase[0] + dim_off);
-      if (sub_ok[1]) v1 = *reinterpret_cast<const uint2*>(a.v_cache + vbase[1] + dim_off);
-      const uint4 vf = make_uint4(v0.x & vmask[0], v0.y & vmask[1], v1.x & vmask[2], v1.y & vmask[3]);
+    for (int t = 0; t < QT; ++t) {
+      if (QT > 1 && t * a.tpt >= ntok) continue;          // a tile beyond the request's rows (uniform)
+      floatx4 sc[2];
 #pragma unroll
-      for (int r = 0; r < 4; ++r) o[b][r] *= alpha;
-      o[b] = mfma_16x16x32(vf, pf, o[b]);
+      for (int h = 0; h < 2; ++h) {
+        sc[h] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < DJ; ++j) sc[h] = mfma_16x16x32(cur.k[h][j], qf[t][j], sc[h]);
+      }
+      // This lane holds, for its query row, the scores of keys key0 + 16h + 4*grp + r.  A tile
+      // that every row of the query tile sees whole needs no mask (the usual case away from the
+      // diagonal); otherwise scores are masked by position, window and row validity.
+      const int tile_first_pos = ctx + tok0 + t * a.tpt;
+      const int tile_last_pos = min(tile_first_pos + a.tpt - 1, pos_max);
+      const int tile_lo = (a.window > 0 && tile_last_pos - a.window + 1 > 0) ? tile_last_pos - a.window + 1 : 0;
+      const bool interior = key0 + 31 <= tile_first_pos && key0 >= tile_lo;
+      float sv[8];
+      float m_tile = -INFINITY;
+      if (interior) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            sv[4 * h + r] = sc[h][r] * a.scale_log2;
+            m_tile = fmaxf(m_tile, sv[4 * h + r]);
+          }
+      } else {
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int key = key0 + 16 * h + 4 * grp + r;
+            const bool vis = cur.ok[h] && q_ok[t] && key <= q_pos[t] && key >= q_lo[t];
+            const float v = vis ? sc[h][r] * a.scale_log2 : -INFINITY;
+            sv[4 * h + r] = v;
+            m_tile = fmaxf(m_tile, v);
+          }
+      }
+      m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 16, kWave));
+      m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, kWave));
+      const float m_new = fmaxf(m_run[t], m_tile);
+      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+      const float alpha = fast_exp2(m_run[t] - m_safe);   // 0 while nothing has been seen
+      float psum = 0.f;
+      uint32_t pk[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float p0 = fast_exp2(sv[2 * i] - m_safe), p1 = fast_exp2(sv[2 * i + 1] - m_safe);
+        psum += p0 + p1;
+        pk[i] = pack_bf16x2(p0, p1);
+      }
+      l_run[t] = l_run[t] * alpha + psum;
+      m_run[t] = m_new;
+      const uint4 pf = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+      const bool rescale = __any(alpha != 1.0f);   // the running maximum moved for some row
+#pragma unroll
+      for (int b = 0; b < DB; ++b) {
+        if (16 * b >= d) break;   // DB is the most blocks this instantiation holds
+        const uint4 vf = make_uint4(cur.v[0][b].x & vmask[0], cur.v[0][b].y & vmask[1],
+                                    cur.v[1][b].x & vmask[2], cur.v[1][b].y & vmask[3]);
+        if (rescale) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) o[t][b][r] *= alpha;
+        }
+        o[t][b] = mfma_16x16x32(vf, pf, o[t][b]);
+      }
     }
+    if (kt + 1 < kt_end) cur = nxt;
   }
 
-  float l_tot = l_run + __shfl_xor(l_run, 16, kWave);
-  l_tot += __shfl_xor(l_tot, 32, kWave);
-  if (!q_ok) return;
-  const long row = row0 + tok0 + q_tok;
-  if (a.n_splits == 1) {
-    const float inv = 1.0f / l_tot;
-    bf16_t* dst = a.out + (row * a.n_heads + q_head) * d + 4 * grp;
 #pragma unroll
-    for (int b = 0; b < DB; ++b) {
-      if (16 * b >= d) break;
-      uint2 pack;
-      pack.x = static_cast<uint32_t>(bf16_bits_from_float(o[b][0] * inv)) |
-               (static_cast<uint32_t>(bf16_bits_from_float(o[b][1] * inv)) << 16);
-      pack.y = static_cast<uint32_t>(bf16_bits_from_float(o[b][2] * inv)) |
-               (static_cast<uint32_t>(bf16_bits_from_float(o[b][3] * inv)) << 16);
-      *reinterpret_cast<uint2*>(dst + 16 * b) = pack;
-    }
-  } else {
-    const long slot = (static_cast<long>(blockIdx.z) * a.n_tokens + row) * a.n_heads + q_head;
-    float* dst = a.part_o + slot * d + 4 * grp;
+  for (int t = 0; t < QT; ++t) {
+    float l_tot = l_run[t] + __shfl_xor(l_run[t], 16, kWave);
+    l_tot += __shfl_xor(l_tot, 32, kWave);
+    if (!q_ok[t]) continue;
+    const long row = row0 + tok0 + q_tok[t];
+    if (a.n_splits == 1) {
+      const float inv = 1.0f / l_tot;
+      bf16_t* dst = a.out + (row * a.n_heads + q_head) * d + 4 * grp;
 #pragma unroll
-    for (int b = 0; b < DB; ++b) {
-      if (16 * b >= d) break;
-      *reinterpret_cast<floatx4*>(dst + 16 * b) = o[b];
-    }
-    if (grp == 0) {
-      a.part_ml[slot * 2] = m_run;
-      a.part_ml[slot * 2 + 1] = l_tot;
+      for (int b = 0; b < DB; ++b) {
+        if (16 * b >= d) break;
+        uint2 pack;
+        pack.x = pack_bf16x2(o[t][b][0] * inv, o[t][b][1] * inv);
+        pack.y = pack_bf16x2(o[t][b][2] * inv, o[t][b][3] * inv);
+        *reinterpret_cast<uint2*>(dst + 16 * b) = pack;
+      }
+    } else {
+      const long slot = (static_cast<long>(blockIdx.z) * a.n_tokens + row) * a.n_heads + q_head;
+      float* dst = a.part_o + slot * d + 4 * grp;
+#pragma unroll
+      for (int b = 0; b < DB; ++b) {
+        if (16 * b >= d) break;
+        *reinterpret_cast<floatx4*>(dst + 16 * b) = o[t][b];
+      }
+      if (grp == 0) {
+        a.part_ml[slot * 2] = m_run[t];
+        a.part_ml[slot * 2 + 1] = l_tot;
+      }
     }
   }
 }
@@ -247,12 +328,12 @@ __global__ __launch_bounds__(kWave) void attention_merge_kernel(const float* __r
 
 using namespace bc4g;
 
-extern "C" int bc4g_attention_mfma(const void* qkv, void* out, float* part_o, float* part_ml, const void* k_cache,
+extern "C" int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, float* part_o, float* part_ml, const void* k_cache,
                                    const void* v_cache, const int32_t* block_table, int table_stride,
                                    const int32_t* seq_start, const int32_t* seq_ctx, const int32_t* tile_start,
                                    int n_seqs, int n_tiles, int n_tokens, int n_heads, int n_kv_heads, int head_dim,
-                                   int page_tokens, int window, float scale, int tokens_per_tile, int n_splits,
-                                   void* stream) {
+                                   int page_tokens, int window, float scale, int tokens_per_tile, int q_tiles,
+                                   int n_splits, void* stream) {
   BC4G_REQUIRE(n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0, "attention_mfma: bad heads %d/%d",
                n_heads, n_kv_heads);
   BC4G_REQUIRE(head_dim >= 16 && head_dim <= 256 && head_dim % 16 == 0,
@@ -262,6 +343,7 @@ extern "C" int bc4g_attention_mfma(const void* qkv, void* out, float* part_o, fl
   BC4G_REQUIRE(n_splits >= 1 && n_splits <= kMaxSplits && (n_splits == 1 || (part_o && part_ml)),
                "attention_mfma: the split count %d must lie in 1..64", n_splits);
   BC4G_REQUIRE(window >= 0 && table_stride > 0 && n_seqs > 0, "attention_mfma: bad sizes");
+  BC4G_REQUIRE(q_stride >= n_heads * head_dim && q_stride % 8 == 0, "attention_mfma: bad query row stride %d", q_stride);
   if (n_tiles == 0 || n_tokens == 0) return 0;
   const int group = n_heads / n_kv_heads;
   AttnArgs a;
@@ -279,6 +361,7 @@ extern "C" int bc4g_attention_mfma(const void* qkv, void* out, float* part_o, fl
   a.n_seqs = n_seqs;
   a.n_tiles = n_tiles;
   a.n_tokens = n_tokens;
+  a.q_stride = q_stride;
   a.n_heads = n_heads;
   a.n_kv_heads = n_kv_heads;
   a.head_dim = head_dim;
@@ -291,14 +374,24 @@ extern "C" int bc4g_attention_mfma(const void* qkv, void* out, float* part_o, fl
   a.scale_log2 = scale * kLog2e;
   BC4G_REQUIRE(a.tpt >= 1 && a.tpt * a.hg <= 16, "attention_mfma: %d tokens x %d heads do not fit a 16-row tile",
                a.tpt, a.hg);
+  const int dj = (head_dim + 31) / 32, db = head_dim / 16;
+  const int max_qt = db <= 4 ? 4 : (db <= 8 ? 2 : 1);
+  BC4G_REQUIRE(q_tiles == 1 || (q_tiles == max_qt && (q_tiles == 2 || q_tiles == 4)),
+               "attention_mfma: %d query tiles per wave are not built for head_dim %d (1 or %d)", q_tiles, head_dim,
+               max_qt);
   BC4G_REQUIRE(n_kv_heads * a.n_sub <= 65535, "attention_mfma: too many heads for the grid");
   hipStream_t s = static_cast<hipStream_t>(stream);
   dim3 grid((n_tiles + kWavesPerBlock - 1) / kWavesPerBlock, n_kv_heads * a.n_sub, n_splits);
   dim3 block(kWavesPerBlock * kWave);
-  const int dj = (head_dim + 31) / 32, db = head_dim / 16;
-  if (dj <= 2 && db <= 4) attention_mfma_kernel<2, 4><<<grid, block, 0, s>>>(a);
-  else if (dj <= 4 && db <= 8) attention_mfma_kernel<4, 8><<<grid, block, 0, s>>>(a);
-  else attention_mfma_kernel<8, 16><<<grid, block, 0, s>>>(a);
+  if (dj <= 2 && db <= 4) {
+    if (q_tiles == 4) attention_mfma_kernel<2, 4, 4><<<grid, block, 0, s>>>(a);
+    else attention_mfma_kernel<2, 4, 1><<<grid, block, 0, s>>>(a);
+  } else if (dj <= 4 && db <= 8) {
+    if (q_tiles == 2) attention_mfma_kernel<4, 8, 2><<<grid, block, 0, s>>>(a);
+    else attention_mfma_kernel<4, 8, 1><<<grid, block, 0, s>>>(a);
+  } else {
+    attention_mfma_kernel<8, 16, 1><<<grid, block, 0, s>>>(a);
+  }
   if (int e = check_launch("attention_mfma")) return e;
   if (n_splits > 1) {
     const long rows_heads = static_cast<long>(n_tokens) * n_heads;

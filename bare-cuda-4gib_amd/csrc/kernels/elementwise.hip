@@ -43,14 +43,20 @@ __global__ void rmsnorm_kernel(const float* __restrict__ x, const int32_t* __res
 }
 
 // ---- SwiGLU ----------------------------------------------------------------
+// interleaved 0: a row of gu holds the gate values, then the up values.  1: blocks of 16 -- eight
+// gate values followed by the eight up values of the same outputs (the layout the fused
+// weight-streaming kernel produces and consumes).
 template <typename T>
-__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, long total, int inter) {
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, long total, int inter,
+                              int interleaved) {
   const long stride = static_cast<long>(blockDim.x) * gridDim.x;
   for (long idx = blockIdx.x * static_cast<long>(blockDim.x) + threadIdx.x; idx < total; idx += stride) {
     const long t = idx / inter;
     const int i = static_cast<int>(idx - t * inter);
-    const float g = to_float(gu[t * 2 * inter + i]);
-    const float u = to_float(gu[t * 2 * inter + inter + i]);
+    const long gi = interleaved ? (i / 8) * 16 + i % 8 : i;
+    const long ui = interleaved ? gi + 8 : inter + i;
+    const float g = to_float(gu[t * 2 * inter + gi]);
+    const float u = to_float(gu[t * 2 * inter + ui]);
     out[idx] = from_float<T>((g / (1.0f + expf(-g))) * u);
   }
 }
@@ -59,12 +65,15 @@ __global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, lon
 // One thread per (token, head among q|k|v, pair).  A pair is (i, i + rotary_dim/2)
 // for i < rotary_dim/2; dimensions at or beyond rotary_dim pass through, handled
 // by the threads with pair >= rotary_dim/2 as (lo = rotary_dim/2 + i .. ) below.
+// block_pairs != 0: the head's dimensions were reordered in blocks of 16 (eight "lo" dimensions
+// 8b .. 8b+7 followed by their partners), so pair i = 8b + t lies at 16b + t and 16b + 8 + t;
+// this needs rotary_dim == head_dim or 0.
 template <typename T>
 __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const int32_t* __restrict__ positions,
                                      const int32_t* __restrict__ slot_map, T* __restrict__ k_cache,
                                      T* __restrict__ v_cache, long total, int n_heads, int n_kv_heads,
                                      int head_dim, int rotary_dim, float theta, int page_tokens,
-                                     int write_kv) {
+                                     int write_kv, int block_pairs) {
   const int half = head_dim / 2;          // threads per head: each moves two elements
   const int rhalf = rotary_dim / 2;
   const int heads_total = n_heads + 2 * n_kv_heads;
@@ -79,7 +88,11 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const int32_t* __restr
     // Which two elements this thread owns: a rotated pair, or two pass-through elements.
     int i0, i1;
     bool rotate;
-    if (j < rhalf) {
+    if (block_pairs) {
+      i0 = (j / 8) * 16 + j % 8;
+      i1 = i0 + 8;
+      rotate = rotary_dim > 0;
+    } else if (j < rhalf) {
       i0 = j;
       i1 = j + rhalf;
       rotate = true;
@@ -269,17 +282,19 @@ extern "C" int bc4g_rmsnorm(const float* x, const int32_t* rows, const void* w, 
   return check_launch("rmsnorm");
 }
 
-extern "C" int bc4g_swiglu(const void* gu, void* out, int dtype, int n_tokens, int inter, void* stream) {
+extern "C" int bc4g_swiglu(const void* gu, void* out, int dtype, int n_tokens, int inter, int interleaved,
+                           void* stream) {
   BC4G_REQUIRE(n_tokens >= 0 && inter > 0, "swiglu: bad sizes T=%d I=%d", n_tokens, inter);
+  BC4G_REQUIRE(!interleaved || inter % 8 == 0, "swiglu: the interleaved layout needs I=%d to be a multiple of 8", inter);
   if (n_tokens == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const long total = static_cast<long>(n_tokens) * inter;
   if (dtype == kF32) {
     swiglu_kernel<float><<<grid_for(total), kBlock, 0, s>>>(static_cast<const float*>(gu),
-                                                            static_cast<float*>(out), total, inter);
+                                                            static_cast<float*>(out), total, inter, interleaved);
   } else if (dtype == kBF16) {
     swiglu_kernel<bf16_t><<<grid_for(total), kBlock, 0, s>>>(static_cast<const bf16_t*>(gu),
-                                                             static_cast<bf16_t*>(out), total, inter);
+                                                             static_cast<bf16_t*>(out), total, inter, interleaved);
   } else {
     return fail("swiglu: unknown dtype %d", dtype);
   }
@@ -289,7 +304,7 @@ extern "C" int bc4g_swiglu(const void* gu, void* out, int dtype, int n_tokens, i
 extern "C" int bc4g_rope_kv_write(void* qkv, int dtype, const int32_t* positions, const int32_t* slot_map,
                                   void* k_cache, void* v_cache, int n_tokens, int n_heads, int n_kv_heads,
                                   int head_dim, int rotary_dim, float theta, int page_tokens, int num_pages,
-                                  int write_kv, void* stream) {
+                                  int write_kv, int block_pairs, void* stream) {
   BC4G_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads > 0, "rope_kv_write: bad sizes T=%d heads=%d/%d",
                n_tokens, n_heads, n_kv_heads);
   BC4G_REQUIRE(head_dim > 0 && head_dim % 2 == 0, "rope_kv_write: head_dim %d must be even", head_dim);
@@ -298,17 +313,21 @@ extern "C" int bc4g_rope_kv_write(void* qkv, int dtype, const int32_t* positions
   BC4G_REQUIRE(!write_kv || (page_tokens > 0 && num_pages > 0 && k_cache && v_cache && slot_map),
                "rope_kv_write: cache write asked for without a cache");
   BC4G_REQUIRE(rotary_dim == 0 || (positions && theta > 0.f), "rope_kv_write: rotation needs positions and theta > 0");
+  BC4G_REQUIRE(!block_pairs || (head_dim % 16 == 0 && (rotary_dim == 0 || rotary_dim == head_dim)),
+               "rope_kv_write: the block layout needs head_dim %d to be a multiple of 16 and a full rotation", head_dim);
   if (n_tokens == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const long total = static_cast<long>(n_tokens) * (n_heads + 2 * n_kv_heads) * (head_dim / 2);
   if (dtype == kF32) {
     rope_kv_write_kernel<float><<<grid_for(total), kBlock, 0, s>>>(
         static_cast<float*>(qkv), positions, slot_map, static_cast<float*>(k_cache),
-        static_cast<float*>(v_cache), total, n_heads, n_kv_heads, head_dim, rotary_dim, theta, page_tokens, write_kv);
+        static_cast<float*>(v_cache), total, n_heads, n_kv_heads, head_dim, rotary_dim, theta, page_tokens, write_kv,
+        block_pairs);
   } else if (dtype == kBF16) {
     rope_kv_write_kernel<bf16_t><<<grid_for(total), kBlock, 0, s>>>(
         static_cast<bf16_t*>(qkv), positions, slot_map, static_cast<bf16_t*>(k_cache),
-        static_cast<bf16_t*>(v_cache), total, n_heads, n_kv_heads, head_dim, rotary_dim, theta, page_tokens, write_kv);
+        static_cast<bf16_t*>(v_cache), total, n_heads, n_kv_heads, head_dim, rotary_dim, theta, page_tokens, write_kv,
+        block_pairs);
   } else {
     return fail("rope_kv_write: unknown dtype %d", dtype);
   }

@@ -5,7 +5,7 @@
 // are contiguous in k, so a tile of each is staged through LDS as [128 rows][64 k] with rows padded
 // to 144 bytes (which makes the 16-byte fragment reads of 8 consecutive lanes cover all banks), in
 // two buffers: while the waves feed 32x32x16 MFMAs from one, the next k-step's global loads are in
-// flight and are written to the other.  Each wave owns a 64 x 64 quarter (2 x 2 MFMA blocks).
+// flight (two k-steps ahead, in registers) and the one after the current is written to the other.  Each wave owns a 64 x 64 quarter (2 x 2 MFMA blocks).
 // Rows and columns beyond the matrix are read as zero and not stored; k must be a multiple of 8.
 // Every output element is accumulated over k in ascending order, whatever the number of rows.
 //
@@ -44,24 +44,28 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const bf16_t* __restrict
   const int bm = logical % m_blocks, bn = logical / m_blocks;
   const long m0 = static_cast<long>(bm) * kBM, n0 = static_cast<long>(bn) * kBN;
 
-  // global -> LDS: a tile is 128 rows x 8 segments of 16 bytes; thread t moves segment t%8 of rows t/8 + 32 i
+  // global -> LDS: a tile is 128 rows x 8 segments of 16 bytes; thread t moves segment t%8 of rows t/8 + 32 i.
+  // Two register sets hold the k-steps that are on their way from memory (two steps ahead of the
+  // MFMAs); LDS holds the step being multiplied and the next one.
   const int seg = tid % 8, lrow = tid / 8;
-  uint4 ra[4], rw[4];
-  auto load_tiles = [&](int k0) {
-    const int kk = k0 + seg * 8;
+  struct Staged {
+    uint4 a[4], w[4];
+  };
+  auto load_tiles = [&](Staged& r, int kt) {
+    const int kk = kt * kBK + seg * 8;
     const bool k_ok = kk < k;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const long gm = m0 + lrow + 32 * i, gn = n0 + lrow + 32 * i;
-      ra[i] = (k_ok && gm < m) ? load16(a + gm * k + kk) : zero16();
-      rw[i] = (k_ok && gn < n) ? load16(w + gn * k + kk) : zero16();
+      r.a[i] = (k_ok && gm < m) ? load16(a + gm * k + kk) : zero16();
+      r.w[i] = (k_ok && gn < n) ? load16(w + gn * k + kk) : zero16();
     }
   };
-  auto store_tiles = [&](int buf) {
+  auto store_tiles = [&](const Staged& r, int buf) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      *reinterpret_cast<uint4*>(&tiles[buf].a[lrow + 32 * i][seg * 8]) = ra[i];
-      *reinterpret_cast<uint4*>(&tiles[buf].w[lrow + 32 * i][seg * 8]) = rw[i];
+      *reinterpret_cast<uint4*>(&tiles[buf].a[lrow + 32 * i][seg * 8]) = r.a[i];
+      *reinterpret_cast<uint4*>(&tiles[buf].w[lrow + 32 * i][seg * 8]) = r.w[i];
     }
   };
 
@@ -73,14 +77,8 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const bf16_t* __restrict
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  const int nk = (k + kBK - 1) / kBK;
-  load_tiles(0);
-  store_tiles(0);
-  __syncthreads();
   const int frow = lane % 32, fk = (lane / 32) * 8;
-  for (int kt = 0; kt < nk; ++kt) {
-    const int buf = kt & 1;
-    if (kt + 1 < nk) load_tiles((kt + 1) * kBK);
+  auto multiply = [&](int buf) {
 #pragma unroll
     for (int ks = 0; ks < kBK / 16; ++ks) {
       uint4 fa[2], fw[2];
@@ -94,7 +92,23 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const bf16_t* __restrict
 #pragma unroll
         for (int j = 0; j < 2; ++j) acc[i][j] = mfma_32x32x16(fa[i], fw[j], acc[i][j]);
     }
-    if (kt + 1 < nk) store_tiles(buf ^ 1);
+  };
+
+  const int nk = (k + kBK - 1) / kBK;
+  Staged r0, r1;
+  load_tiles(r0, 0);
+  if (nk > 1) load_tiles(r1, 1);
+  store_tiles(r0, 0);
+  if (nk > 2) load_tiles(r0, 2);
+  __syncthreads();
+  for (int kt = 0; kt < nk; kt += 2) {
+    multiply(0);                                  // k-step kt
+    if (kt + 1 < nk) store_tiles(r1, 1);
+    if (kt + 3 < nk) load_tiles(r1, kt + 3);
+    __syncthreads();
+    if (kt + 1 < nk) multiply(1);                 // k-step kt + 1
+    if (kt + 2 < nk) store_tiles(r0, 0);
+    if (kt + 4 < nk) load_tiles(r0, kt + 4);
     __syncthreads();
   }
 

@@ -14,8 +14,11 @@
 //            workgroup writes bf16(x * g) into LDS and sums x^2 per row; the MFMAs read their B
 //            operand from LDS, and the row's rsqrt(mean(x^2) + eps) -- a factor common to the
 //            whole row -- multiplies the finished sum.
-// What goes out (EPI): bfloat16 or float stored, float added into the residual stream, or, when
-// w holds gate rows followed by up rows, SwiGLU of the pair of sums.
+// What goes out (EPI): bfloat16 or float stored; float added into the residual stream; SwiGLU,
+// when every 16 rows of w are eight gate rows followed by the eight up rows of the same outputs; or
+// rotary positions and the cache write, when w holds query, key and value heads with every head's
+// rows reordered in blocks of 16 (eight dimensions, then their rotation partners): queries are
+// stored rotated, keys rotated into their page, values into theirs.
 #include <math.h>
 
 #include "api.h"
@@ -29,7 +32,16 @@ constexpr int kThreads = kWaves * kWave;
 constexpr int kRedPad = 17;
 constexpr int kStagePad = 8;     // bf16 elements appended to each staged row of x
 
-enum Epilogue : int { kStoreBf16 = 0, kStoreF32 = 1, kAccumF32 = 2, kSwigluBf16 = 3 };
+enum Epilogue : int { kStoreBf16 = 0, kStoreF32 = 1, kAccumF32 = 2, kSwigluBf16 = 3, kRopeKvBf16 = 4 };
+
+struct RopeKvArgs {
+  const int32_t* positions;   // [m]
+  const int32_t* slot_map;    // [m] page * page_tokens + offset
+  bf16_t* k_cache;            // [pages, n_kv, page_tokens, d]
+  bf16_t* v_cache;            // [pages, n_kv, d, page_tokens]
+  int n_heads, n_kv_heads, head_dim, rotary_dim, page_tokens, write_kv;
+  float theta;
+};
 enum XMode : int { kPlain = 0, kNormedG16 = 1, kNormedG32 = 2 };   // norm scale g in bfloat16 / float
 
 struct SkinnyArgs {
@@ -41,6 +53,7 @@ struct SkinnyArgs {
   int m, n, k, n_out;
   int m_stage;              // normed modes: rows of x staged in LDS (m rounded up to 4)
   float eps;
+  RopeKvArgs rope;          // kRopeKvBf16 only
 };
 
 __device__ inline uint32_t pack2(float a, float b) {
@@ -48,8 +61,8 @@ __device__ inline uint32_t pack2(float a, float b) {
 }
 
 template <int MT, int EPI, int XMODE, int U>
-__global__ __launch_bounds__(kThreads) void gemm_skinny_kernel(const SkinnyArgs a) {
-  constexpr int kSets = (EPI == kSwigluBf16) ? 2 : 1;   // gate and up rows
+__global__ __launch_bounds__(kThreads, 4) void gemm_skinny_kernel(const SkinnyArgs a) {
+  constexpr int kSets = 1;
   constexpr bool kNormed = XMODE != kPlain;
   static_assert(!kNormed || MT == 1, "the fused norm handles one tile of rows");
   __shared__ float red[kWaves][kSets][MT][16][kRedPad];
@@ -71,10 +84,10 @@ __global__ __launch_bounds__(kThreads) void gemm_skinny_kernel(const SkinnyArgs 
     for (int t = 0; t < MT; ++t) acc[s][t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
   const int wrow = n0 + col;                           // this lane's row of w (output column)
-  const bool wrow_ok = wrow < a.n_out;
+  const bool wrow_ok = wrow < a.n;
   const bf16_t* wptr[kSets];
 #pragma unroll
-  for (int s = 0; s < kSets; ++s) wptr[s] = a.w + (static_cast<long>(wrow) + static_cast<long>(s) * a.n_out) * k;
+  for (int s = 0; s < kSets; ++s) wptr[s] = a.w + static_cast<long>(wrow) * k;
 
   // where this lane's B operand comes from
   const bf16_t* xptr[MT];
@@ -128,33 +141,55 @@ __global__ __launch_bounds__(kThreads) void gemm_skinny_kernel(const SkinnyArgs 
 
   constexpr int kStep = 32 * U;
   Batch cur, nxt;
-  if (k_begin < k_end) load(cur, k_begin);   // the first weights are on their way
 
   if constexpr (kNormed) {
-    // stage bf16(x * g) for every row: 32 threads walk one row, 8 elements each per pass
+    // Stage bf16(x * g): wave w takes rows w, w + 8; a lane takes 8 elements of each 512.  The
+    // loads of x and g are issued first and the first weights right after them: loads come back
+    // in the order they were issued, so the (cached) x arrives while the weights are on their way.
+    constexpr int kStageIters = 4;                       // 2048 elements of a row per round
     bf16_t* stage = reinterpret_cast<bf16_t*>(stage_raw);
-    const int srow0 = threadIdx.x / 32, sl = threadIdx.x % 32;
-    for (int row = srow0; row < a.m_stage; row += kThreads / 32) {
+    bool first = true;
+    for (int row = wave; row < a.m_stage; row += kWaves) {
       float ss = 0.f;
-      if (row < m) {
-        const long src = a.rows ? a.rows[row] : row;
-        const float* xr = static_cast<const float*>(a.x) + src * k;
-        for (int kk = sl * 8; kk < k; kk += 256) {
-          const uint4 x0 = load16(xr + kk), x1 = load16(xr + kk + 4);
-          float xv[8] = {__uint_as_float(x0.x), __uint_as_float(x0.y), __uint_as_float(x0.z), __uint_as_float(x0.w),
-                         __uint_as_float(x1.x), __uint_as_float(x1.y), __uint_as_float(x1.z), __uint_as_float(x1.w)};
+      const bool live = row < m;
+      const long src = (live && a.rows) ? a.rows[row] : row;
+      const float* xr = static_cast<const float*>(a.x) + src * k;
+      for (int kb = 0; kb < k; kb += 512 * kStageIters) {
+        uint4 x0[kStageIters], x1[kStageIters], g0[kStageIters], g1[kStageIters];
+#pragma unroll
+        for (int it = 0; it < kStageIters; ++it) {
+          const int kk = kb + it * 512 + lane * 8;
+          const bool ok = live && kk < k;
+          x0[it] = ok ? load16(xr + kk) : zero16();
+          x1[it] = ok ? load16(xr + kk + 4) : zero16();
+          if constexpr (XMODE == kNormedG16) {
+            g0[it] = ok ? load16(static_cast<const bf16_t*>(a.g) + kk) : zero16();
+          } else {
+            g0[it] = ok ? load16(static_cast<const float*>(a.g) + kk) : zero16();
+            g1[it] = ok ? load16(static_cast<const float*>(a.g) + kk + 4) : zero16();
+          }
+        }
+        if (first) {                                       // the first weights follow the first x
+          if (k_begin < k_end) load(cur, k_begin);
+          first = false;
+        }
+#pragma unroll
+        for (int it = 0; it < kStageIters; ++it) {
+          const int kk = kb + it * 512 + lane * 8;
+          if (kk >= k) continue;
+          const float xv[8] = {__uint_as_float(x0[it].x), __uint_as_float(x0[it].y), __uint_as_float(x0[it].z),
+                               __uint_as_float(x0[it].w), __uint_as_float(x1[it].x), __uint_as_float(x1[it].y),
+                               __uint_as_float(x1[it].z), __uint_as_float(x1[it].w)};
           float gv[8];
           if constexpr (XMODE == kNormedG16) {
-            const uint4 g0 = load16(static_cast<const bf16_t*>(a.g) + kk);
-            const uint32_t gr[4] = {g0.x, g0.y, g0.z, g0.w};
+            const uint32_t gr[4] = {g0[it].x, g0[it].y, g0[it].z, g0[it].w};
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
               gv[2 * i] = __uint_as_float(gr[i] << 16);
               gv[2 * i + 1] = __uint_as_float(gr[i] & 0xffff0000u);
             }
           } else {
-            const uint4 g0 = load16(static_cast<const float*>(a.g) + kk), g1 = load16(static_cast<const float*>(a.g) + kk + 4);
-            const uint32_t gr[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
+            const uint32_t gr[8] = {g0[it].x, g0[it].y, g0[it].z, g0[it].w, g1[it].x, g1[it].y, g1[it].z, g1[it].w};
 #pragma unroll
             for (int i = 0; i < 8; ++i) gv[i] = __uint_as_float(gr[i]);
           }
@@ -164,15 +199,14 @@ __global__ __launch_bounds__(kThreads) void gemm_skinny_kernel(const SkinnyArgs 
               make_uint4(pack2(xv[0] * gv[0], xv[1] * gv[1]), pack2(xv[2] * gv[2], xv[3] * gv[3]),
                          pack2(xv[4] * gv[4], xv[5] * gv[5]), pack2(xv[6] * gv[6], xv[7] * gv[7]));
         }
-      } else {
-        for (int kk = sl * 8; kk < k; kk += 256)
-          *reinterpret_cast<uint4*>(stage + static_cast<long>(row) * stage_stride + kk) = zero16();
       }
-#pragma unroll
-      for (int off = 16; off > 0; off >>= 1) ss += __shfl_xor(ss, off, kWave);   // the row's 32 threads
-      if (sl == 0 && row < 16) ssq_row[row] = ss;
+      ss = wave_sum(ss);
+      if (lane == 0 && row < 16) ssq_row[row] = ss;
     }
+    if (first && k_begin < k_end) load(cur, k_begin);      // a wave without a row to stage
     __syncthreads();
+  } else {
+    if (k_begin < k_end) load(cur, k_begin);
   }
 
   for (int k0 = k_begin; k0 < k_end; k0 += kStep) {
@@ -191,33 +225,68 @@ __global__ __launch_bounds__(kThreads) void gemm_skinny_kernel(const SkinnyArgs 
       for (int r = 0; r < 4; ++r) red[wave][s][t][4 * grp + r][col] = acc[s][t][r];
   __syncthreads();
 
-  for (int idx = threadIdx.x; idx < MT * 256; idx += kThreads) {
-    const int nl = idx % 16, row = idx / 16;
+  constexpr bool kPaired = EPI == kSwigluBf16 || EPI == kRopeKvBf16;   // columns nl and nl + 8 belong together
+  constexpr int kCols = kPaired ? 8 : 16;
+  for (int idx = threadIdx.x; idx < MT * 16 * kCols; idx += kThreads) {
+    const int nl = idx % kCols, row = idx / kCols;
     const int gn = n0 + nl;
-    if (row >= m || gn >= a.n_out) continue;
-    float sum[kSets];
+    if (row >= m || gn >= a.n) continue;
+    float sum = 0.f, partner = 0.f;
 #pragma unroll
-    for (int s = 0; s < kSets; ++s) {
-      float v = 0.f;
+    for (int wv = 0; wv < kWaves; ++wv) sum += red[wv][0][row / 16][nl][row % 16];
+    if constexpr (kPaired) {
 #pragma unroll
-      for (int wv = 0; wv < kWaves; ++wv) v += red[wv][s][row / 16][nl][row % 16];
-      sum[s] = v;
+      for (int wv = 0; wv < kWaves; ++wv) partner += red[wv][0][row / 16][nl + 8][row % 16];
     }
     if constexpr (kNormed) {
       const float scale = 1.0f / sqrtf(ssq_row[row] / static_cast<float>(k) + a.eps);
-#pragma unroll
-      for (int s = 0; s < kSets; ++s) sum[s] *= scale;
+      sum *= scale;
+      partner *= scale;
     }
-    const long o = static_cast<long>(row) * a.n_out + gn;
     if constexpr (EPI == kStoreBf16) {
-      static_cast<bf16_t*>(a.out)[o] = from_float<bf16_t>(sum[0]);
+      static_cast<bf16_t*>(a.out)[static_cast<long>(row) * a.n + gn] = from_float<bf16_t>(sum);
     } else if constexpr (EPI == kStoreF32) {
-      static_cast<float*>(a.out)[o] = sum[0];
+      static_cast<float*>(a.out)[static_cast<long>(row) * a.n + gn] = sum;
     } else if constexpr (EPI == kAccumF32) {
-      static_cast<float*>(a.out)[o] += sum[0];
+      static_cast<float*>(a.out)[static_cast<long>(row) * a.n + gn] += sum;
+    } else if constexpr (EPI == kSwigluBf16) {
+      // block b = n0 / 16 holds gates and ups of outputs 8b .. 8b + 7
+      const long o = static_cast<long>(row) * (a.n / 2) + (n0 / 2 + nl);
+      static_cast<bf16_t*>(a.out)[o] = from_float<bf16_t>((sum / (1.0f + expf(-sum))) * partner);
     } else {
-      const float gt = sum[0], up = sum[kSets - 1];
-      static_cast<bf16_t*>(a.out)[o] = from_float<bf16_t>((gt / (1.0f + expf(-gt))) * up);
+      const RopeKvArgs& r = a.rope;
+      const int d = r.head_dim;
+      const int head = n0 / d, in_head = n0 % d + nl;         // the pair lies at in_head and in_head + 8
+      const int pair = (n0 % d) / 2 + nl;                     // 8 * block + nl
+      float lo = sum, hi = partner;
+      const bool is_v = head >= r.n_heads + r.n_kv_heads;
+      if (r.rotary_dim > 0 && !is_v) {
+        const float inv_freq = 1.0f / powf(r.theta, (2.0f * static_cast<float>(pair)) / static_cast<float>(d));
+        const float angle = static_cast<float>(r.positions[row]) * inv_freq;
+        float sn, cs;
+        sincosf(angle, &sn, &cs);
+        const float l0 = lo, h0 = hi;
+        lo = l0 * cs - h0 * sn;
+        hi = h0 * cs + l0 * sn;
+      }
+      if (head < r.n_heads) {
+        bf16_t* q = static_cast<bf16_t*>(a.out) + (static_cast<long>(row) * r.n_heads + head) * d + in_head;
+        q[0] = from_float<bf16_t>(lo);
+        q[8] = from_float<bf16_t>(hi);
+      } else if (r.write_kv) {
+        const int kvh = is_v ? head - r.n_heads - r.n_kv_heads : head - r.n_heads;
+        const int slot = r.slot_map[row];
+        const long page = slot / r.page_tokens, off = slot % r.page_tokens;
+        if (is_v) {
+          bf16_t* dst = r.v_cache + ((page * r.n_kv_heads + kvh) * d + in_head) * r.page_tokens + off;
+          dst[0] = from_float<bf16_t>(lo);
+          dst[8L * r.page_tokens] = from_float<bf16_t>(hi);
+        } else {
+          bf16_t* dst = r.k_cache + ((page * r.n_kv_heads + kvh) * r.page_tokens + off) * d + in_head;
+          dst[0] = from_float<bf16_t>(lo);
+          dst[8] = from_float<bf16_t>(hi);
+        }
+      }
     }
   }
 }
@@ -227,12 +296,12 @@ constexpr int kMaxStageBytes = 96 * 1024;
 template <int EPI, int XMODE>
 int launch(const SkinnyArgs& a, hipStream_t s) {
   const int mt = (a.m + 15) / 16;
-  dim3 grid((a.n_out + 15) / 16), block(kThreads);
+  dim3 grid((a.n + 15) / 16), block(kThreads);
   if constexpr (XMODE != kPlain) {
     if (mt != 1) return fail("gemm_skinny: the fused norm takes at most 16 rows, got %d", a.m);
     const size_t stage = static_cast<size_t>(a.m_stage) * (a.k + kStagePad) * 2;
     if (stage > kMaxStageBytes) return fail("gemm_skinny: %d rows of k=%d do not fit the staging buffer", a.m, a.k);
-    auto kernel = gemm_skinny_kernel<1, EPI, XMODE, (EPI == kSwigluBf16 ? 4 : 8)>;
+    auto kernel = gemm_skinny_kernel<1, EPI, XMODE, 8>;
     static bool raised = false;   // per instantiation: allow more than the default dynamic LDS
     if (!raised) {
       if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -243,6 +312,7 @@ int launch(const SkinnyArgs& a, hipStream_t s) {
     kernel<<<grid, block, stage, s>>>(a);
   } else {
     switch (mt) {
+      // k-steps per batch chosen so that two batches of operands fit 128 registers (two workgroups a CU)
       case 1: gemm_skinny_kernel<1, EPI, XMODE, 4><<<grid, block, 0, s>>>(a); break;
       case 2: gemm_skinny_kernel<2, EPI, XMODE, 4><<<grid, block, 0, s>>>(a); break;
       case 3: gemm_skinny_kernel<3, EPI, XMODE, 2><<<grid, block, 0, s>>>(a); break;
@@ -259,10 +329,33 @@ int launch_epilogue(SkinnyArgs& a, int epilogue, hipStream_t s) {
   switch (epilogue) {
     case kStoreBf16: return launch<kStoreBf16, XMODE>(a, s);
     case kStoreF32: return launch<kStoreF32, XMODE>(a, s);
-    case kAccumF32: return launch<kAccumF32, XMODE>(a, s);
-    case kSwigluBf16: a.n_out = a.n / 2; return launch<kSwigluBf16, XMODE>(a, s);
+    case kAccumF32:
+      if constexpr (XMODE == kPlain) return launch<kAccumF32, XMODE>(a, s);
+      else return fail("gemm_skinny: adding into the stream that is being normed is not supported");
+    case kSwigluBf16: return launch<kSwigluBf16, XMODE>(a, s);
+    case kRopeKvBf16: return launch<kRopeKvBf16, XMODE>(a, s);
     default: return fail("gemm_skinny: unknown epilogue %d", epilogue);
   }
+}
+
+int check_common(const char* what, int m, int max_m, int n, int k, int epilogue) {
+  BC4G_REQUIRE(m >= 0 && m <= max_m, "%s: M=%d must be at most %d", what, m, max_m);
+  BC4G_REQUIRE(n > 0 && k > 0 && k % 8 == 0, "%s: K=%d must be a positive multiple of 8 (N=%d)", what, k, n);
+  BC4G_REQUIRE(epilogue != kSwigluBf16 || n % 16 == 0,
+               "%s: SwiGLU needs blocks of eight gate and eight up rows, N=%d is no multiple of 16", what, n);
+  return 0;
+}
+
+int check_rope(const char* what, const RopeKvArgs& r, int n) {
+  BC4G_REQUIRE(r.n_heads > 0 && r.n_kv_heads > 0 && r.head_dim > 0 && r.head_dim % 16 == 0,
+               "%s: bad head sizes %d/%d x %d (head_dim must be a multiple of 16)", what, r.n_heads, r.n_kv_heads,
+               r.head_dim);
+  BC4G_REQUIRE(n == (r.n_heads + 2 * r.n_kv_heads) * r.head_dim, "%s: N=%d is not (heads + 2 kv heads) * head_dim", what, n);
+  BC4G_REQUIRE(r.rotary_dim == 0 || (r.rotary_dim == r.head_dim && r.positions && r.theta > 0.f),
+               "%s: the rotation must cover the whole head (rotary_dim %d, head_dim %d)", what, r.rotary_dim, r.head_dim);
+  BC4G_REQUIRE(!r.write_kv || (r.slot_map && r.k_cache && r.v_cache && r.page_tokens > 0),
+               "%s: cache write asked for without a cache", what);
+  return 0;
 }
 
 }  // namespace
@@ -272,30 +365,44 @@ using namespace bc4g;
 
 extern "C" int bc4g_gemm_skinny(const void* x, const void* w, void* out, int epilogue, int m, int n, int k,
                                 void* stream) {
-  BC4G_REQUIRE(m >= 0 && m <= 64, "gemm_skinny: M=%d must be at most 64", m);
-  BC4G_REQUIRE(n > 0 && k > 0 && k % 8 == 0, "gemm_skinny: K=%d must be a positive multiple of 8 (N=%d)", k, n);
-  BC4G_REQUIRE(epilogue != kSwigluBf16 || n % 2 == 0, "gemm_skinny: SwiGLU needs gate and up rows, N=%d is odd", n);
+  if (int e = check_common("gemm_skinny", m, 64, n, k, epilogue)) return e;
+  BC4G_REQUIRE(epilogue != kRopeKvBf16, "gemm_skinny: use bc4g_gemm_skinny_qkv for the rotary epilogue");
   if (m == 0) return 0;
-  SkinnyArgs a{x, nullptr, nullptr, static_cast<const bf16_t*>(w), out, m, n, k, n, 0, 0.f};
+  SkinnyArgs a{x, nullptr, nullptr, static_cast<const bf16_t*>(w), out, m, n, k, n, 0, 0.f, {}};
   return launch_epilogue<kPlain>(a, epilogue, static_cast<hipStream_t>(stream));
-}
-
-extern "C" int bc4g_gemm_skinny_normed_max_k(int m) {
-  const int m_stage = ((m + 3) / 4) * 4;
-  return m_stage > 0 ? kMaxStageBytes / (2 * m_stage) - kStagePad : 0;
 }
 
 extern "C" int bc4g_gemm_skinny_normed(const float* x, const int32_t* rows, const void* g, int g_dtype,
                                        float eps, const void* w, void* out, int epilogue, int m, int n, int k,
                                        void* stream) {
-  BC4G_REQUIRE(m >= 0 && m <= 16, "gemm_skinny_normed: M=%d must be at most 16", m);
-  BC4G_REQUIRE(n > 0 && k > 0 && k % 8 == 0, "gemm_skinny_normed: K=%d must be a positive multiple of 8 (N=%d)", k, n);
-  BC4G_REQUIRE(epilogue != kSwigluBf16 || n % 2 == 0, "gemm_skinny_normed: SwiGLU needs gate and up rows, N=%d is odd", n);
-  BC4G_REQUIRE(epilogue != kAccumF32, "gemm_skinny_normed: adding into the stream it reads is not supported");
+  if (int e = check_common("gemm_skinny_normed", m, 16, n, k, epilogue)) return e;
+  BC4G_REQUIRE(epilogue != kAccumF32 && epilogue != kRopeKvBf16, "gemm_skinny_normed: epilogue %d is not supported here",
+               epilogue);
   if (m == 0) return 0;
-  SkinnyArgs a{x, rows, g, static_cast<const bf16_t*>(w), out, m, n, k, n, ((m + 3) / 4) * 4, eps};
+  SkinnyArgs a{x, rows, g, static_cast<const bf16_t*>(w), out, m, n, k, n, ((m + 3) / 4) * 4, eps, {}};
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (g_dtype == kBF16) return launch_epilogue<kNormedG16>(a, epilogue, s);
   if (g_dtype == kF32) return launch_epilogue<kNormedG32>(a, epilogue, s);
   return fail("gemm_skinny_normed: unknown norm scale dtype %d", g_dtype);
+}
+
+// The query/key/value product of a decode step with rotary positions and the cache write in its
+// epilogue.  x: bfloat16 [m, k] (g null), or the float residual stream with RMSNorm fused (g given,
+// m <= 16).  q_out: bfloat16 [m, n_heads * head_dim], rotated, in the reordered head layout.
+extern "C" int bc4g_gemm_skinny_qkv(const void* x, const void* g, int g_dtype, float eps, const void* w, void* q_out,
+                                    const int32_t* positions, const int32_t* slot_map, void* k_cache, void* v_cache,
+                                    int m, int k, int n_heads, int n_kv_heads, int head_dim, int rotary_dim,
+                                    float theta, int page_tokens, int write_kv, void* stream) {
+  RopeKvArgs r{positions, slot_map, static_cast<bf16_t*>(k_cache), static_cast<bf16_t*>(v_cache), n_heads, n_kv_heads,
+               head_dim, rotary_dim, page_tokens, write_kv, theta};
+  const int n = (n_heads + 2 * n_kv_heads) * head_dim;
+  if (int e = check_common("gemm_skinny_qkv", m, g ? 16 : 64, n, k, kRopeKvBf16)) return e;
+  if (int e = check_rope("gemm_skinny_qkv", r, n)) return e;
+  if (m == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  SkinnyArgs a{x, nullptr, g, static_cast<const bf16_t*>(w), q_out, m, n, k, n, g ? ((m + 3) / 4) * 4 : 0, eps, r};
+  if (!g) return launch<kRopeKvBf16, kPlain>(a, s);
+  if (g_dtype == kBF16) return launch<kRopeKvBf16, kNormedG16>(a, s);
+  if (g_dtype == kF32) return launch<kRopeKvBf16, kNormedG32>(a, s);
+  return fail("gemm_skinny_qkv: unknown norm scale dtype %d", g_dtype);
 }

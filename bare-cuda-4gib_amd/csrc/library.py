@@ -18,15 +18,16 @@ _SIGNATURES = {
     "bc4g_embed_gather": [_P, _I, _P, _P, _I, _I, _I, _P],
     "bc4g_rmsnorm": [_P, _P, _P, _I, _P, _I, _I, _I, _F, _P],
     "bc4g_gemm_generic": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _P],
-    "bc4g_swiglu": [_P, _P, _I, _I, _I, _P],
-    "bc4g_rope_kv_write": [_P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P],
-    "bc4g_attention_generic": [_P, _P, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _P],
+    "bc4g_swiglu": [_P, _P, _I, _I, _I, _I, _P],
+    "bc4g_rope_kv_write": [_P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _P],
+    "bc4g_attention_generic": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _P],
     "bc4g_argmax": [_P, _P, _I, _I, _P],
     "bc4g_sample": [_P, _P, _P, _P, _I, _I, _P],
     "bc4g_gemm_skinny": [_P, _P, _P, _I, _I, _I, _I, _P],
     "bc4g_gemm_mfma": [_P, _P, _P, _I, _I, _I, _I, _P],
     "bc4g_gemm_skinny_normed": [_P, _P, _P, _I, _F, _P, _P, _I, _I, _I, _I, _P],
-    "bc4g_attention_mfma": [_P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P],
+    "bc4g_attention_mfma": [_P, _I, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P],
+    "bc4g_gemm_skinny_qkv": [_P, _P, _I, _F, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P],
 }
 
 _lib: Optional[ctypes.CDLL] = None

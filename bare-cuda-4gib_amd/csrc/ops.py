@@ -105,14 +105,17 @@ def gemm_generic(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = None
     return out
 
 
-def swiglu(gu: torch.Tensor) -> torch.Tensor:
-    """gu [T, 2I] = gate | up  ->  silu(gate) * up, [T, I]."""
+def swiglu(gu: torch.Tensor, interleaved: bool = False) -> torch.Tensor:
+    """gu [T, 2I] -> silu(gate) * up, [T, I].  gu holds all gates then all ups, or (interleaved)
+    blocks of 16: eight gates and the eight ups of the same outputs."""
     _dev("swiglu", gu)
     if gu.dim() != 2 or gu.shape[1] % 2:
         raise KernelError(f"swiglu: input must be [T, 2I], got {tuple(gu.shape)}")
     t, inter = gu.shape[0], gu.shape[1] // 2
     out = torch.empty((t, inter), dtype=gu.dtype, device=gu.device)
-    library.call("bc4g_swiglu", _ptr(gu), _ptr(out), _code(gu, "swiglu"), t, inter, _stream())
+    if interleaved and inter % 8:
+        raise KernelError(f"swiglu: the interleaved layout needs I={inter} to be a multiple of 8")
+    library.call("bc4g_swiglu", _ptr(gu), _ptr(out), _code(gu, "swiglu"), t, inter, 1 if interleaved else 0, _stream())
     return out
 
 
@@ -129,8 +132,10 @@ def _check_cache(what: str, k: torch.Tensor, v: torch.Tensor, n_kv_heads: int, h
 
 def rope_kv_write(qkv: torch.Tensor, positions: Optional[torch.Tensor], slot_map: Optional[torch.Tensor],
                   k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor], n_heads: int,
-                  n_kv_heads: int, head_dim: int, rotary_dim: int, theta: float, write_kv: bool = True) -> None:
-    """Rotate q (in place) and k, write k and v into their pages."""
+                  n_kv_heads: int, head_dim: int, rotary_dim: int, theta: float, write_kv: bool = True,
+                  block_pairs: bool = False) -> None:
+    """Rotate q (in place) and k, write k and v into their pages.  block_pairs: every head's
+    dimensions come reordered in blocks of 16 (see bc4g_rope_kv_write)."""
     _dev("rope_kv_write", qkv, positions, slot_map, k_cache, v_cache)
     t = qkv.shape[0]
     width = (n_heads + 2 * n_kv_heads) * head_dim
@@ -145,7 +150,14 @@ def rope_kv_write(qkv: torch.Tensor, positions: Optional[torch.Tensor], slot_map
         num_pages, page_tokens = k_cache.shape[0], k_cache.shape[2]
     library.call("bc4g_rope_kv_write", _ptr(qkv), _code(qkv, "rope_kv_write"), _ptr(positions), _ptr(slot_map),
                  _ptr(k_cache), _ptr(v_cache), t, n_heads, n_kv_heads, head_dim, rotary_dim, float(theta),
-                 page_tokens, num_pages, 1 if write_kv else 0, _stream())
+                 page_tokens, num_pages, 1 if write_kv else 0, 1 if block_pairs else 0, _stream())
+
+
+def _check_queries(what: str, q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int) -> None:
+    """Queries come as the rows of the fused q|k|v product or as a buffer of queries alone."""
+    widths = ((n_heads + 2 * n_kv_heads) * head_dim, n_heads * head_dim)
+    if q.dim() != 2 or q.shape[1] not in widths:
+        raise KernelError(f"{what}: queries must be [T, {widths[0]}] or [T, {widths[1]}], got {tuple(q.shape)}")
 
 
 def attention_generic(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
@@ -155,16 +167,14 @@ def attention_generic(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.T
     """Causal attention of every row over its request's cache; returns [T, n_heads*head_dim]."""
     _dev("attention", qkv, k_cache, v_cache, block_table, row_seq, positions)
     t = qkv.shape[0]
-    width = (n_heads + 2 * n_kv_heads) * head_dim
-    if qkv.dim() != 2 or qkv.shape[1] != width:
-        raise KernelError(f"attention: qkv must be [T, {width}], got {tuple(qkv.shape)}")
+    _check_queries("attention", qkv, n_heads, n_kv_heads, head_dim)
     _check_cache("attention", k_cache, v_cache, n_kv_heads, head_dim, qkv.dtype)
     if block_table.dim() != 2 or block_table.dtype != torch.int32:
         raise KernelError("attention: block_table must be int32 [requests, pages]")
     _i32("attention", "row_seq", row_seq, t)
     _i32("attention", "positions", positions, t)
     out = torch.empty((t, n_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
-    library.call("bc4g_attention_generic", _ptr(qkv), _ptr(out), _code(qkv, "attention"), _ptr(k_cache),
+    library.call("bc4g_attention_generic", _ptr(qkv), qkv.shape[1], _ptr(out), _code(qkv, "attention"), _ptr(k_cache),
                  _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(row_seq), _ptr(positions), t,
                  n_heads, n_kv_heads, head_dim, k_cache.shape[2], k_cache.shape[0], int(window),
                  float(scale if scale is not None else 1.0 / math.sqrt(head_dim)), _stream())
@@ -266,11 +276,12 @@ def gemm_normed(x: torch.Tensor, rows: Optional[torch.Tensor], n_rows: int, g: t
     return out
 
 
-def gemm_swiglu(a: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
-    """silu(a Wg^T) * (a Wu^T) for w_gate_up = gate rows followed by up rows, [2I, K] -> [M, I].
-    For a few rows the activation is applied to the float sums inside the product's kernel;
-    otherwise the product is stored and the activation kernel follows."""
-    if _fast_operands(a, w_gate_up) and a.shape[0] <= SKINNY_MAX_ROWS and w_gate_up.shape[0] % 2 == 0:
+def gemm_swiglu(a: torch.Tensor, w_gate_up: torch.Tensor, interleaved: bool = False) -> torch.Tensor:
+    """silu(a Wg^T) * (a Wu^T), [M, I], for w_gate_up [2I, K].  interleaved: every 16 rows of the
+    weight are eight gate rows and the eight up rows of the same outputs -- then, for a few rows,
+    the activation is applied to the float sums inside the product's kernel.  Otherwise (and for
+    many rows) the product is stored and the activation kernel follows."""
+    if interleaved and _fast_operands(a, w_gate_up) and a.shape[0] <= SKINNY_MAX_ROWS and w_gate_up.shape[0] % 16 == 0:
         _dev("gemm_swiglu", a, w_gate_up)
         m, k = a.shape
         n = w_gate_up.shape[0]
@@ -280,7 +291,44 @@ def gemm_swiglu(a: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
     gu = gemm_fast(a, w_gate_up, a.dtype)
     if gu is None:
         gu = gemm_generic(a, w_gate_up, a.dtype)
-    return swiglu(gu)
+    return swiglu(gu, interleaved)
+
+
+def gemm_qkv_rope_supported(x: torch.Tensor, n_rows: int, normed: bool, w: torch.Tensor, head_dim: int,
+                            rotary_dim: int) -> bool:
+    """Whether the q|k|v product of these rows can rotate and write the cache in its epilogue."""
+    rows_ok = n_rows <= (NORMED_MAX_ROWS if normed else SKINNY_MAX_ROWS)
+    return (x.is_cuda and w.dtype == torch.bfloat16 and x.shape[1] % 8 == 0 and 0 < n_rows and rows_ok
+            and head_dim % 16 == 0 and rotary_dim in (0, head_dim)
+            and x.dtype == (torch.float32 if normed else torch.bfloat16))
+
+
+def gemm_qkv_rope(x: torch.Tensor, g: Optional[torch.Tensor], eps: float, w: torch.Tensor,
+                  positions: torch.Tensor, slot_map: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
+                  v_cache: Optional[torch.Tensor], n_heads: int, n_kv_heads: int, head_dim: int, rotary_dim: int,
+                  theta: float, write_kv: bool = True) -> torch.Tensor:
+    """The q|k|v product of a decode step with rotary positions and the cache write in its
+    epilogue (w in the reordered head layout).  With g the input is the float residual stream
+    and RMSNorm is fused.  Returns the rotated queries [M, heads * head_dim]."""
+    _dev("gemm_qkv_rope", x, g, w, positions, slot_map, k_cache, v_cache)
+    m, k = x.shape
+    n = (n_heads + 2 * n_kv_heads) * head_dim
+    if tuple(w.shape) != (n, k):
+        raise KernelError(f"gemm_qkv_rope: weight must be [{n}, {k}], got {tuple(w.shape)}")
+    _i32("gemm_qkv_rope", "positions", positions, m)
+    page_tokens = 0
+    if write_kv:
+        _check_cache("gemm_qkv_rope", k_cache, v_cache, n_kv_heads, head_dim, torch.bfloat16)
+        _i32("gemm_qkv_rope", "slot_map", slot_map, m)
+        page_tokens = k_cache.shape[2]
+    if g is not None and (tuple(g.shape) != (k,) or x.dtype != torch.float32):
+        raise KernelError("gemm_qkv_rope: the fused norm needs a float32 input and a scale of its width")
+    q = torch.empty((m, n_heads * head_dim), dtype=torch.bfloat16, device=x.device)
+    library.call("bc4g_gemm_skinny_qkv", _ptr(x), _ptr(g), _code(g, "gemm_qkv_rope") if g is not None else 0,
+                 float(eps), _ptr(w), _ptr(q), _ptr(positions), _ptr(slot_map), _ptr(k_cache), _ptr(v_cache),
+                 m, k, n_heads, n_kv_heads, head_dim, int(rotary_dim), float(theta), page_tokens,
+                 1 if write_kv else 0, _stream())
+    return q
 
 
 def attention_mfma_supported(qkv: torch.Tensor, k_cache: torch.Tensor, head_dim: int) -> bool:
@@ -293,8 +341,14 @@ def attention_tile_tokens(n_heads: int, n_kv_heads: int) -> int:
     return 16 // min(n_heads // n_kv_heads, 16)
 
 
+def attention_q_tiles(head_dim: int) -> int:
+    """16-row tiles a wave of the matrix-core attention kernel takes for prompt portions."""
+    return 4 if head_dim <= 64 else (2 if head_dim <= 128 else 1)
+
+
 ATTENTION_TARGET_WAVES = 2048
 ATTENTION_MAX_SPLITS = 64
+ATTENTION_ENOUGH_WAVES = 512      # from here on the rows alone occupy the GPU
 
 
 def attention_splits(n_tiles: int, n_heads: int, n_kv_heads: int, max_kv_len: int) -> int:
@@ -302,6 +356,8 @@ def attention_splits(n_tiles: int, n_heads: int, n_kv_heads: int, max_kv_len: in
     alone fill it, else towards ATTENTION_TARGET_WAVES waves with at least one 32-key tile each."""
     group = n_heads // n_kv_heads
     waves = n_tiles * n_kv_heads * (-(-group // 16))
+    if waves >= ATTENTION_ENOUGH_WAVES:
+        return 1
     key_tiles = max(1, -(-max_kv_len // 32))
     return max(1, min(ATTENTION_TARGET_WAVES // max(waves, 1), key_tiles, ATTENTION_MAX_SPLITS))
 
@@ -309,12 +365,12 @@ def attention_splits(n_tiles: int, n_heads: int, n_kv_heads: int, max_kv_len: in
 def attention_mfma(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                    seq_start: torch.Tensor, seq_ctx: torch.Tensor, tile_start: torch.Tensor, n_tiles: int,
                    n_heads: int, n_kv_heads: int, head_dim: int, window: int, scale: float,
-                   n_splits: int) -> torch.Tensor:
+                   n_splits: int, q_tiles: int = 1) -> torch.Tensor:
     _dev("attention_mfma", qkv, k_cache, v_cache, block_table, seq_start, seq_ctx, tile_start)
     t = qkv.shape[0]
-    width = (n_heads + 2 * n_kv_heads) * head_dim
-    if qkv.dim() != 2 or qkv.shape[1] != width or qkv.dtype != torch.bfloat16:
-        raise KernelError(f"attention_mfma: qkv must be bfloat16 [T, {width}], got {qkv.dtype} {tuple(qkv.shape)}")
+    _check_queries("attention_mfma", qkv, n_heads, n_kv_heads, head_dim)
+    if qkv.dtype != torch.bfloat16:
+        raise KernelError(f"attention_mfma: queries must be bfloat16, got {qkv.dtype}")
     _check_cache("attention_mfma", k_cache, v_cache, n_kv_heads, head_dim, qkv.dtype)
     if block_table.dim() != 2 or block_table.dtype != torch.int32:
         raise KernelError("attention_mfma: block_table must be int32 [requests, pages]")
@@ -327,10 +383,11 @@ def attention_mfma(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     if n_splits > 1:
         part_o = torch.empty((n_splits, t, n_heads, head_dim), dtype=torch.float32, device=qkv.device)
         part_ml = torch.empty((n_splits, t, n_heads, 2), dtype=torch.float32, device=qkv.device)
-    library.call("bc4g_attention_mfma", _ptr(qkv), _ptr(out), _ptr(part_o), _ptr(part_ml), _ptr(k_cache),
+    library.call("bc4g_attention_mfma", _ptr(qkv), qkv.shape[1], _ptr(out), _ptr(part_o), _ptr(part_ml), _ptr(k_cache),
                  _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(seq_start), _ptr(seq_ctx),
                  _ptr(tile_start), n_seqs, n_tiles, t, n_heads, n_kv_heads, head_dim, k_cache.shape[2],
-                 int(window), float(scale), attention_tile_tokens(n_heads, n_kv_heads), int(n_splits), _stream())
+                 int(window), float(scale), attention_tile_tokens(n_heads, n_kv_heads), int(q_tiles),
+                 int(n_splits), _stream())
     return out
 
 
@@ -341,9 +398,11 @@ def attention(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, b
     else the plain float kernel."""
     if attention_mfma_supported(qkv, k_cache, head_dim):
         tpt = attention_tile_tokens(n_heads, n_kv_heads)
-        tile_start, n_tiles = ctx.attention_tiles(tpt)
+        # a wave takes several query tiles as soon as some request brings more than one tile of rows
+        q_tiles = attention_q_tiles(head_dim) if ctx.max_q_len > tpt else 1
+        tile_start, n_tiles = ctx.attention_tiles(tpt * q_tiles)
         n_splits = ctx.fixed_attention_splits or attention_splits(n_tiles, n_heads, n_kv_heads, ctx.max_kv_len)
         return attention_mfma(qkv, k_cache, v_cache, block_table, ctx.seq_start_dev, ctx.seq_ctx_dev,
-                              tile_start, n_tiles, n_heads, n_kv_heads, head_dim, window, scale, n_splits)
+                              tile_start, n_tiles, n_heads, n_kv_heads, head_dim, window, scale, n_splits, q_tiles)
     return attention_generic(qkv, k_cache, v_cache, block_table, ctx.row_seq, ctx.positions,
                              n_heads, n_kv_heads, head_dim, window, scale)

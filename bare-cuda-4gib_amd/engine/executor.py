@@ -59,7 +59,7 @@ class Executor:
         # attention tile sizes the model's mixers ask for (made once per step, with the batch)
         parts = [p for layer in model.layers for p in _walk_parts(layer)]
         self._attention_parts = [p for p in parts if hasattr(p, "attention_tile_tokens")]
-        self._tile_sizes = sorted({p.attention_tile_tokens() for p in self._attention_parts})
+        self._tile_sizes = sorted({size for p in self._attention_parts for size in p.attention_tile_tokens()})
         # decode steps are replayed from captured graphs if every part of the model allows it
         self.use_graphs = bool(use_graphs) and all(getattr(p, "graph_safe", False) for p in parts) \
             and self.rt.device.type == "cuda"

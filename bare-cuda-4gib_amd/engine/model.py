@@ -112,10 +112,20 @@ class Model:
             if e.cache in streams and streams[e.cache] != spec:
                 raise ConfigError(f"cache stream {e.cache!r} is written with two different specs")
             streams[e.cache] = spec
+        layouts: Dict[Hashable, object] = {}
         for e in self.schedule:
-            if e.cache is not None and e.cache not in streams:
+            if e.cache is None:
+                continue
+            if e.cache not in streams:
                 raise ConfigError(f"schedule entry for layer {e.layer} reads cache stream {e.cache!r}, "
                                   "which no entry writes")
+            mixer = self.layers[e.layer].mixer
+            if mixer.cache_spec() != streams[e.cache]:
+                raise ConfigError(f"layer {e.layer} uses cache stream {e.cache!r} with another spec than its writer")
+            layout = mixer.cache_layout() if hasattr(mixer, "cache_layout") else None
+            if layouts.setdefault(e.cache, layout) != layout:
+                raise ConfigError(f"layers sharing cache stream {e.cache!r} keep a head's dimensions in "
+                                  "different orders (their position encodings or dtypes differ)")
         return streams
 
     # ---- forward ------------------------------------------------------------

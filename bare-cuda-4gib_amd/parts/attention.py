@@ -11,6 +11,7 @@ from ..csrc import ops
 from ..errors import ConfigError
 from ..weights.loader import WeightSpec
 from .base import Part, build_part, register_part
+from .lazy import Normed
 from .linear import linear
 
 
@@ -43,9 +44,16 @@ class CausalAttention(Part):
     def cache_spec(self):
         return PagedKV(self.num_kv_heads, self.head_dim, self.window)
 
-    def attention_tile_tokens(self) -> int:
-        """Tokens per 16-row tile the matrix-core kernel wants the batch cut into."""
-        return ops.attention_tile_tokens(self.num_heads, self.num_kv_heads)
+    def cache_layout(self):
+        """The order in which a head's dimensions lie in the cache (known once weights are bound):
+        layers that share a cache stream must agree on it."""
+        return getattr(self, "dim_order", None)
+
+    def attention_tile_tokens(self):
+        """The piece sizes (in tokens) the matrix-core kernel wants each request's rows cut into:
+        one 16-row tile for decoded tokens, several for prompt portions."""
+        tpt = ops.attention_tile_tokens(self.num_heads, self.num_kv_heads)
+        return (tpt, tpt * ops.attention_q_tiles(self.head_dim))
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
         q, kv, h = self.num_heads * self.head_dim, self.num_kv_heads * self.head_dim, self.hidden_size
@@ -53,27 +61,62 @@ class CausalAttention(Part):
                 "v_proj.weight": WeightSpec((kv, h)), "o_proj.weight": WeightSpec((h, q))}
 
     def bind(self, tensors, rt) -> None:
-        parts = [tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]]
-        dt = torch.float32 if any(p.dtype == torch.float32 for p in parts) else parts[0].dtype
+        q, k, v, o = (tensors[n] for n in ("q_proj.weight", "k_proj.weight", "v_proj.weight", "o_proj.weight"))
+        dt = torch.float32 if any(p.dtype == torch.float32 for p in (q, k, v)) else q.dtype
+        fused = self.position.fused() if self.position is not None else (0, 1.0)
+        # For the matrix-core kernels every head's dimensions are reordered in blocks of 16 -- eight
+        # dimensions, then their rotation partners -- so that the weight-streaming kernel can rotate and
+        # write the cache in its epilogue.  Queries, keys and values all live in that order (scores and
+        # outputs do not depend on the order, as long as all agree), and the output projection's
+        # columns are reordered to match.
+        self.block_pairs = (dt == torch.bfloat16 and o.dtype == torch.bfloat16 and self.head_dim % 16 == 0
+                            and fused is not None and fused[0] in (0, self.head_dim))
+        self.dim_order = tuple(range(self.head_dim))
+        if self.block_pairs:
+            d, half = self.head_dim, self.head_dim // 2
+            self.dim_order = tuple(8 * b + t if t < 8 else half + 8 * b + (t - 8)
+                                   for b in range(d // 16) for t in range(16))
+            order = torch.tensor(self.dim_order, device=q.device)
+            def rows(w, heads):
+                return w.view(heads, d, -1)[:, order, :].reshape(heads * d, -1)
+            q, k, v = rows(q, self.num_heads), rows(k, self.num_kv_heads), rows(v, self.num_kv_heads)
+            o = o.view(-1, self.num_heads, d)[:, :, order].reshape(-1, self.num_heads * d).contiguous()
         # one product for q, k and v: their rows one after the other
-        self.w_qkv = torch.cat([p.to(dt) for p in parts], dim=0).contiguous()
-        self.w_o = tensors["o_proj.weight"]
+        self.w_qkv = torch.cat([p.to(dt) for p in (q, k, v)], dim=0).contiguous()
+        self.w_o = o
         self.act_dtype = rt.act_dtype
 
     def forward(self, h, ctx, cache, residual, writes: bool = True) -> None:
-        qkv = linear(h, self.w_qkv, out_dtype=self.act_dtype)
         fused = self.position.fused() if self.position is not None else (0, 1.0)
-        if fused is None:
-            self.position.apply(qkv, ctx, self.num_heads, self.num_kv_heads, self.head_dim)
-            fused = (0, 1.0)
-        rotary_dim, theta = fused
-        ops.rope_kv_write(qkv, ctx.positions, ctx.slot_maps[cache.group] if writes else None,
-                          cache.k if writes else None, cache.v if writes else None,
-                          self.num_heads, self.num_kv_heads, self.head_dim, rotary_dim, theta,
-                          write_kv=writes)
-        o = ops.attention(qkv, cache.k, cache.v, ctx.block_tables[cache.group], ctx,
+        rotary_dim, theta = fused if fused is not None else (0, 1.0)
+        slot_map = ctx.slot_maps[cache.group] if writes else None
+        k_cache, v_cache = (cache.k, cache.v) if writes else (None, None)
+        q = None
+        if self.block_pairs and fused is not None:
+            q = self._fused_qkv(h, ctx, slot_map, k_cache, v_cache, rotary_dim, theta, writes)
+        if q is None:
+            q = linear(h, self.w_qkv, out_dtype=self.act_dtype)
+            if fused is None:
+                self.position.apply(q, ctx, self.num_heads, self.num_kv_heads, self.head_dim)
+            ops.rope_kv_write(q, ctx.positions, slot_map, k_cache, v_cache, self.num_heads, self.num_kv_heads,
+                              self.head_dim, rotary_dim, theta, write_kv=writes, block_pairs=self.block_pairs)
+        o = ops.attention(q, cache.k, cache.v, ctx.block_tables[cache.group], ctx,
                           self.num_heads, self.num_kv_heads, self.head_dim, self.window, self.scale)
         linear(o, self.w_o, accumulate_into=residual)
+
+    def _fused_qkv(self, h, ctx, slot_map, k_cache, v_cache, rotary_dim, theta, writes):
+        """The q|k|v product with rotation and cache write in its epilogue, where a kernel takes
+        the rows (a decode step); None otherwise."""
+        args = (ctx.positions, slot_map, k_cache, v_cache, self.num_heads, self.num_kv_heads, self.head_dim,
+                rotary_dim, theta, writes)
+        if isinstance(h, Normed):
+            scale = h.fusable_scale() if h._tensor is None and h.rows is None else None
+            if scale is not None and ops.gemm_qkv_rope_supported(h.x, h.n_rows, True, self.w_qkv, self.head_dim, rotary_dim):
+                return ops.gemm_qkv_rope(h.x, scale[0], scale[1], self.w_qkv, *args)
+            h = h.tensor()
+        if ops.gemm_qkv_rope_supported(h, h.shape[0], False, self.w_qkv, self.head_dim, rotary_dim):
+            return ops.gemm_qkv_rope(h, None, 0.0, self.w_qkv, *args)
+        return None
 
 
 register_part("mixer", "attention", CausalAttention)

@@ -30,13 +30,21 @@ class SwiGLU(Part):
     def bind(self, tensors, rt) -> None:
         g, u = tensors["gate_proj.weight"], tensors["up_proj.weight"]
         dt = torch.float32 if torch.float32 in (g.dtype, u.dtype) else g.dtype
-        # one product for gate and up: gate's rows, then up's
-        self.w_gu = torch.cat([g.to(dt), u.to(dt)], dim=0).contiguous()
+        i, h = self.intermediate_size, self.hidden_size
+        # One product for gate and up.  For the matrix-core kernels (bfloat16, I a multiple of 8) the
+        # rows go in blocks of 16 -- eight gate rows, then the eight up rows of the same outputs -- so
+        # that one workgroup of the weight-streaming kernel holds both halves of its outputs;
+        # otherwise gate's rows, then up's.
+        self.interleaved = dt == torch.bfloat16 and i % 8 == 0
+        if self.interleaved:
+            self.w_gu = torch.stack([g.view(i // 8, 8, h), u.view(i // 8, 8, h)], dim=1).reshape(2 * i, h).contiguous()
+        else:
+            self.w_gu = torch.cat([g.to(dt), u.to(dt)], dim=0).contiguous()
         self.w_down = tensors["down_proj.weight"]
         self.act_dtype = rt.act_dtype
 
     def forward(self, h, ctx, residual) -> None:
-        act = linear_swiglu(h, self.w_gu)
+        act = linear_swiglu(h, self.w_gu, self.interleaved)
         linear(act, self.w_down, accumulate_into=residual)
 
 

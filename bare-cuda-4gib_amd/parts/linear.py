@@ -40,11 +40,12 @@ def linear(x: Union[torch.Tensor, Normed], w: torch.Tensor, out_dtype: Optional[
     return ops.gemm_generic(x, w, out_dtype, accumulate_into)
 
 
-def linear_swiglu(x: Union[torch.Tensor, Normed], w_gate_up: torch.Tensor) -> torch.Tensor:
-    """silu(x Wg^T) * (x Wu^T) for w_gate_up = gate rows followed by up rows."""
+def linear_swiglu(x: Union[torch.Tensor, Normed], w_gate_up: torch.Tensor, interleaved: bool = False) -> torch.Tensor:
+    """silu(x Wg^T) * (x Wu^T) for w_gate_up = gate rows followed by up rows, or (interleaved)
+    blocks of eight gate rows and the eight up rows of the same outputs."""
     if isinstance(x, Normed):
-        fused = _fused_norm(x, w_gate_up, ops.EPI_SWIGLU) if w_gate_up.shape[0] % 2 == 0 else None
+        fused = _fused_norm(x, w_gate_up, ops.EPI_SWIGLU) if interleaved and w_gate_up.shape[0] % 16 == 0 else None
         if fused is not None:
             return fused
         x = x.tensor()
-    return ops.gemm_swiglu(x, w_gate_up)
+    return ops.gemm_swiglu(x, w_gate_up, interleaved)
