@@ -94,7 +94,7 @@ int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, float* part_o,
 
 extern "C" {
 // bfloat16 a [m, k] times bfloat16 w [n, k] transposed on the matrix cores, any m.
-// epilogue: 0 store bfloat16; 1 store float32; 2 add into float32.
+// epilogue: 0 store bfloat16; 1 store float32; 2 add into float32; 3 SwiGLU as in bc4g_gemm_skinny.
 int bc4g_gemm_mfma(const void* a, const void* w, void* out, int epilogue, int m, int n, int k, void* stream);
 }
 

@@ -11,6 +11,8 @@
 //
 // Workgroups are numbered so that those sharing a tile of w run on the same XCD (workgroups are
 // dealt to the 8 XCDs in turn, each with an L2 of its own).
+#include <math.h>
+
 #include "api.h"
 #include "mfma.h"
 
@@ -21,7 +23,9 @@ constexpr int kBM = 128, kBN = 128, kBK = 64;
 constexpr int kLdsStride = kBK + 8;   // elements; 144 bytes
 constexpr int kXcds = 8;
 
-enum Epilogue : int { kStoreBf16 = 0, kStoreF32 = 1, kAccumF32 = 2 };
+// kSwigluBf16: every 16 rows of w are eight gate rows and the eight up rows of the same outputs;
+// out [m, n / 2] = silu(gate) * up.  A gate and its up lie eight lanes apart in the MFMA result.
+enum Epilogue : int { kStoreBf16 = 0, kStoreF32 = 1, kAccumF32 = 2, kSwigluBf16 = 3 };
 
 struct Tile {
   bf16_t a[kBM][kLdsStride];
@@ -118,11 +122,19 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const bf16_t* __restrict
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       const long gn = n0 + wn * 64 + j * 32 + lane % 32;
-      if (gn >= n) continue;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const long gm = m0 + wm * 64 + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + r % 4;
-        if (gm >= m) continue;
+        if constexpr (EPI == kSwigluBf16) {
+          const float mine = acc[i][j][r];
+          const float other = __shfl_xor(mine, 8, kWave);          // every lane takes part
+          if ((lane & 8) == 0 && gm < m && gn < n) {
+            const long oc = (gn / 16) * 8 + gn % 8;
+            static_cast<bf16_t*>(out)[gm * (n / 2) + oc] = from_float<bf16_t>((mine / (1.0f + expf(-mine))) * other);
+          }
+          continue;
+        }
+        if (gm >= m || gn >= n) continue;
         const long o = gm * n + gn;
         if constexpr (EPI == kStoreBf16) static_cast<bf16_t*>(out)[o] = from_float<bf16_t>(acc[i][j][r]);
         else if constexpr (EPI == kStoreF32) static_cast<float*>(out)[o] = acc[i][j][r];
@@ -151,6 +163,10 @@ extern "C" int bc4g_gemm_mfma(const void* a, const void* w, void* out, int epilo
     case kStoreBf16: gemm_mfma_kernel<kStoreBf16><<<grid, block, 0, s>>>(ap, wp, out, m, n, k, m_blocks, n_blocks); break;
     case kStoreF32: gemm_mfma_kernel<kStoreF32><<<grid, block, 0, s>>>(ap, wp, out, m, n, k, m_blocks, n_blocks); break;
     case kAccumF32: gemm_mfma_kernel<kAccumF32><<<grid, block, 0, s>>>(ap, wp, out, m, n, k, m_blocks, n_blocks); break;
+    case kSwigluBf16:
+      BC4G_REQUIRE(n % 16 == 0, "gemm_mfma: SwiGLU needs blocks of eight gate and eight up rows, N=%d is no multiple of 16", n);
+      gemm_mfma_kernel<kSwigluBf16><<<grid, block, 0, s>>>(ap, wp, out, m, n, k, m_blocks, n_blocks);
+      break;
     default: return fail("gemm_mfma: unknown epilogue %d", epilogue);
   }
   return check_launch("gemm_mfma");

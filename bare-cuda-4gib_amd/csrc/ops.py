@@ -278,15 +278,16 @@ def gemm_normed(x: torch.Tensor, rows: Optional[torch.Tensor], n_rows: int, g: t
 
 def gemm_swiglu(a: torch.Tensor, w_gate_up: torch.Tensor, interleaved: bool = False) -> torch.Tensor:
     """silu(a Wg^T) * (a Wu^T), [M, I], for w_gate_up [2I, K].  interleaved: every 16 rows of the
-    weight are eight gate rows and the eight up rows of the same outputs -- then, for a few rows,
-    the activation is applied to the float sums inside the product's kernel.  Otherwise (and for
-    many rows) the product is stored and the activation kernel follows."""
-    if interleaved and _fast_operands(a, w_gate_up) and a.shape[0] <= SKINNY_MAX_ROWS and w_gate_up.shape[0] % 16 == 0:
+    weight are eight gate rows and the eight up rows of the same outputs -- then the activation
+    is applied to the float sums inside the product's kernel.  Otherwise the product is stored
+    and the activation kernel follows."""
+    if interleaved and _fast_operands(a, w_gate_up) and w_gate_up.shape[0] % 16 == 0:
         _dev("gemm_swiglu", a, w_gate_up)
         m, k = a.shape
         n = w_gate_up.shape[0]
         out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=a.device)
-        library.call("bc4g_gemm_skinny", _ptr(a), _ptr(w_gate_up), _ptr(out), EPI_SWIGLU, m, n, k, _stream())
+        name = "bc4g_gemm_skinny" if m <= SKINNY_MAX_ROWS else "bc4g_gemm_mfma"
+        library.call(name, _ptr(a), _ptr(w_gate_up), _ptr(out), EPI_SWIGLU, m, n, k, _stream())
         return out
     gu = gemm_fast(a, w_gate_up, a.dtype)
     if gu is None:
@@ -349,6 +350,8 @@ def attention_q_tiles(head_dim: int) -> int:
 ATTENTION_TARGET_WAVES = 2048
 ATTENTION_MAX_SPLITS = 64
 ATTENTION_ENOUGH_WAVES = 512      # from here on the rows alone occupy the GPU
+ATTENTION_TILES_PER_WALK = 16     # 32-key tiles one wave should walk at most, if parts are to be had
+ATTENTION_MAX_PROMPT_SPLITS = 8
 
 
 def attention_splits(n_tiles: int, n_heads: int, n_kv_heads: int, max_kv_len: int) -> int:
@@ -356,9 +359,11 @@ def attention_splits(n_tiles: int, n_heads: int, n_kv_heads: int, max_kv_len: in
     alone fill it, else towards ATTENTION_TARGET_WAVES waves with at least one 32-key tile each."""
     group = n_heads // n_kv_heads
     waves = n_tiles * n_kv_heads * (-(-group // 16))
-    if waves >= ATTENTION_ENOUGH_WAVES:
-        return 1
     key_tiles = max(1, -(-max_kv_len // 32))
+    if waves >= ATTENTION_ENOUGH_WAVES:
+        # the rows alone occupy the GPU; what is left to shorten is the longest wave's walk over
+        # its keys, which bounds the kernel's time
+        return max(1, min(ATTENTION_MAX_PROMPT_SPLITS, -(-key_tiles // ATTENTION_TILES_PER_WALK)))
     return max(1, min(ATTENTION_TARGET_WAVES // max(waves, 1), key_tiles, ATTENTION_MAX_SPLITS))
 
 
