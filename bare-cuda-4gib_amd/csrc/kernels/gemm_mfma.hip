@@ -143,6 +143,13 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const bf16_t* __restrict
     }
 }
 
+template <int EPI>
+void launch_tiled(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, int k, long m_blocks, long n_blocks,
+                  hipStream_t s) {
+  dim3 grid(static_cast<unsigned>(m_blocks * n_blocks)), block(256);
+  gemm_mfma_kernel<EPI><<<grid, block, 0, s>>>(ap, wp, out, m, n, k, m_blocks, n_blocks);
+}
+
 }  // namespace
 }  // namespace bc4g
 
@@ -156,16 +163,15 @@ extern "C" int bc4g_gemm_mfma(const void* a, const void* w, void* out, int epilo
   const long m_blocks = (m + kBM - 1) / kBM, n_blocks = (n + kBN - 1) / kBN;
   BC4G_REQUIRE(m_blocks * n_blocks <= 2147483647L, "gemm_mfma: too many tiles");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  dim3 grid(static_cast<unsigned>(m_blocks * n_blocks)), block(256);
   const bf16_t* ap = static_cast<const bf16_t*>(a);
   const bf16_t* wp = static_cast<const bf16_t*>(w);
   switch (epilogue) {
-    case kStoreBf16: gemm_mfma_kernel<kStoreBf16><<<grid, block, 0, s>>>(ap, wp, out, m, n, k, m_blocks, n_blocks); break;
-    case kStoreF32: gemm_mfma_kernel<kStoreF32><<<grid, block, 0, s>>>(ap, wp, out, m, n, k, m_blocks, n_blocks); break;
-    case kAccumF32: gemm_mfma_kernel<kAccumF32><<<grid, block, 0, s>>>(ap, wp, out, m, n, k, m_blocks, n_blocks); break;
+    case kStoreBf16: launch_tiled<kStoreBf16>(ap, wp, out, m, n, k, m_blocks, n_blocks, s); break;
+    case kStoreF32: launch_tiled<kStoreF32>(ap, wp, out, m, n, k, m_blocks, n_blocks, s); break;
+    case kAccumF32: launch_tiled<kAccumF32>(ap, wp, out, m, n, k, m_blocks, n_blocks, s); break;
     case kSwigluBf16:
       BC4G_REQUIRE(n % 16 == 0, "gemm_mfma: SwiGLU needs blocks of eight gate and eight up rows, N=%d is no multiple of 16", n);
-      gemm_mfma_kernel<kSwigluBf16><<<grid, block, 0, s>>>(ap, wp, out, m, n, k, m_blocks, n_blocks);
+      launch_tiled<kSwigluBf16>(ap, wp, out, m, n, k, m_blocks, n_blocks, s);
       break;
     default: return fail("gemm_mfma: unknown epilogue %d", epilogue);
   }
