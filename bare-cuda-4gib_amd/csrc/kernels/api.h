@@ -60,7 +60,9 @@ int bc4g_attention_generic(const void* qkv, int q_stride, void* out, int dtype, 
                            int num_pages, int window, float scale, void* stream);
 
 // out[r] = lowest index of the row's maximum                      (logits_argmax.cu:22-65)
-int bc4g_argmax(const float* logits, int32_t* out, int n_rows, int vocab, void* stream);
+// part_v, part_i: scratch [n_rows, 64] each (the best of every slice of a row).
+int bc4g_argmax(const float* logits, int32_t* out, float* part_v, int32_t* part_i, int n_rows, int vocab,
+                void* stream);
 
 // out[r] = first i with cumsum(exp((l - max) / temperature[r]))[i] > u[r] * total, walking the
 // vocabulary in order (engine/src/sampler.cpp:39-61); temperature <= 0 gives the argmax.

@@ -134,34 +134,48 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const int32_t* __restr
 }
 
 // ---- argmax ----------------------------------------------------------------
-__global__ void argmax_kernel(const float* __restrict__ logits, int32_t* __restrict__ out, int vocab) {
+// Two stages so that a few rows still use many CUs: every block takes one slice of one row and
+// writes its best (value, index); one wave per row then picks among the slices.  Equal values
+// keep the lower index at every step.
+constexpr int kArgmaxSlices = 64;
+
+__device__ inline void better(float& v, int& i, float ov, int oi) {
+  if (ov > v || (ov == v && oi < i)) {
+    v = ov;
+    i = oi;
+  }
+}
+
+__global__ void argmax_slices_kernel(const float* __restrict__ logits, float* __restrict__ part_v,
+                                     int32_t* __restrict__ part_i, int vocab) {
   __shared__ float best_v[kBlock];
   __shared__ int best_i[kBlock];
   const float* row = logits + static_cast<size_t>(blockIdx.x) * vocab;
+  const int per = (vocab + kArgmaxSlices - 1) / kArgmaxSlices;
+  const int begin = min(vocab, static_cast<int>(blockIdx.y) * per), end = min(vocab, begin + per);
   float v = -FLT_MAX;
   int idx = vocab;  // empty marker: loses every tie against a real index
-  for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
-    const float x = row[i];
-    if (x > v) {
-      v = x;
-      idx = i;
-    }
-  }
+  for (int i = begin + threadIdx.x; i < end; i += blockDim.x) better(v, idx, row[i], i);
   best_v[threadIdx.x] = v;
   best_i[threadIdx.x] = idx;
   __syncthreads();
   for (int h = blockDim.x / 2; h > 0; h >>= 1) {
-    if (threadIdx.x < h) {
-      const float ov = best_v[threadIdx.x + h];
-      const int oi = best_i[threadIdx.x + h];
-      if (ov > best_v[threadIdx.x] || (ov == best_v[threadIdx.x] && oi < best_i[threadIdx.x])) {
-        best_v[threadIdx.x] = ov;
-        best_i[threadIdx.x] = oi;
-      }
-    }
+    if (threadIdx.x < h) better(best_v[threadIdx.x], best_i[threadIdx.x], best_v[threadIdx.x + h], best_i[threadIdx.x + h]);
     __syncthreads();
   }
-  if (threadIdx.x == 0) out[blockIdx.x] = best_i[0] < vocab ? best_i[0] : 0;
+  if (threadIdx.x == 0) {
+    part_v[blockIdx.x * kArgmaxSlices + blockIdx.y] = best_v[0];
+    part_i[blockIdx.x * kArgmaxSlices + blockIdx.y] = best_i[0];
+  }
+}
+
+__global__ void argmax_pick_kernel(const float* __restrict__ part_v, const int32_t* __restrict__ part_i,
+                                   int32_t* __restrict__ out, int vocab) {
+  float v = part_v[blockIdx.x * kArgmaxSlices + threadIdx.x];
+  int idx = part_i[blockIdx.x * kArgmaxSlices + threadIdx.x];
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) better(v, idx, __shfl_xor(v, off, kWave), __shfl_xor(idx, off, kWave));
+  if (threadIdx.x == 0) out[blockIdx.x] = idx < vocab ? idx : 0;
 }
 
 // ---- temperature sampling --------------------------------------------------
@@ -334,11 +348,17 @@ extern "C" int bc4g_rope_kv_write(void* qkv, int dtype, const int32_t* positions
   return check_launch("rope_kv_write");
 }
 
-extern "C" int bc4g_argmax(const float* logits, int32_t* out, int n_rows, int vocab, void* stream) {
-  BC4G_REQUIRE(n_rows >= 0 && vocab > 0, "argmax: bad sizes rows=%d V=%d", n_rows, vocab);
+extern "C" int bc4g_argmax(const float* logits, int32_t* out, float* part_v, int32_t* part_i, int n_rows, int vocab,
+                           void* stream) {
+  BC4G_REQUIRE(n_rows >= 0 && vocab > 0 && n_rows <= 65535, "argmax: bad sizes rows=%d V=%d", n_rows, vocab);
+  BC4G_REQUIRE(part_v && part_i, "argmax: the slice buffers ([rows, 64] each) are missing");
   if (n_rows == 0) return 0;
-  argmax_kernel<<<n_rows, kBlock, 0, static_cast<hipStream_t>(stream)>>>(logits, out, vocab);
-  return check_launch("argmax");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  static_assert(kArgmaxSlices == kWave, "one lane per slice in the second stage");
+  argmax_slices_kernel<<<dim3(n_rows, kArgmaxSlices), kBlock, 0, s>>>(logits, part_v, part_i, vocab);
+  if (int e = check_launch("argmax_slices")) return e;
+  argmax_pick_kernel<<<n_rows, kWave, 0, s>>>(part_v, part_i, out, vocab);
+  return check_launch("argmax_pick");
 }
 
 extern "C" int bc4g_sample(const float* logits, const float* temperature, const double* u, int32_t* out,

@@ -186,8 +186,11 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
     _dev("argmax", logits)
     if logits.dtype != torch.float32 or logits.dim() != 2:
         raise KernelError("argmax: logits must be float32 [rows, vocab]")
-    out = torch.empty((logits.shape[0],), dtype=torch.int32, device=logits.device)
-    library.call("bc4g_argmax", _ptr(logits), _ptr(out), logits.shape[0], logits.shape[1], _stream())
+    rows = logits.shape[0]
+    out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    part_v = torch.empty((rows, 64), dtype=torch.float32, device=logits.device)
+    part_i = torch.empty((rows, 64), dtype=torch.int32, device=logits.device)
+    library.call("bc4g_argmax", _ptr(logits), _ptr(out), _ptr(part_v), _ptr(part_i), rows, logits.shape[1], _stream())
     return out
 
 

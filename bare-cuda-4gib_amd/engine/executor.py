@@ -201,16 +201,14 @@ class Executor:
         slot = self._graphs.get(key)
         if slot is None:
             slot = self._capture(key, flat, layout, group_layout, host, bucket)
+        # a ring of pinned staging buffers, each with an event that says its copy has been done
         ring = slot["ring"]
-        buf, event = ring[slot["next"] % len(ring)]
+        buf, view, event = ring[slot["next"] % len(ring)]
         slot["next"] += 1
-        if event is not None:
-            event.synchronize()
-        buf.numpy()[:] = flat
+        event.synchronize()
+        view[:] = flat
         slot["dev"].copy_(buf, non_blocking=True)
-        ev = torch.cuda.Event()
-        ev.record()
-        ring[(slot["next"] - 1) % len(ring)] = (buf, ev)
+        event.record()
         slot["graph"].replay()
         return slot["logits"]
 
@@ -227,7 +225,12 @@ class Executor:
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             logits = self.model.forward(ctx)
-        ring = [(torch.empty(len(flat), dtype=torch.int32).pin_memory(), None) for _ in range(4)]
+        ring = []
+        for _ in range(4):
+            buf = torch.empty(len(flat), dtype=torch.int32).pin_memory()
+            event = torch.cuda.Event()
+            event.record()
+            ring.append((buf, buf.numpy(), event))
         slot = dict(graph=graph, dev=dev, logits=logits, ring=ring, next=0)
         self._graphs[key] = slot
         return slot
