@@ -72,7 +72,8 @@ int bc4g_sample(const float* logits, const float* temperature, const double* u, 
 
 extern "C" {
 // bfloat16 x [m, k] (m <= 64) times bfloat16 w [n, k] transposed, weights streamed once through
-// the matrix cores.  epilogue: 0 store bfloat16 [m, n]; 1 store float32; 2 add into float32;
+// the matrix cores.  w comes packed in fragment order: [ceil(n/16)][ceil(k/32)][64][8], where lane l
+// of a k-step holds row l % 16 of the block and k 8 * (l / 16) .. + 7 of the step, zeros past n and k.  epilogue: 0 store bfloat16 [m, n]; 1 store float32; 2 add into float32;
 // 3 SwiGLU: every 16 rows of w are eight gate rows and the eight up rows of the same outputs
 // (n = 2 * inter), out bfloat16 [m, inter] = silu(gate) * up.
 int bc4g_gemm_skinny(const void* x, const void* w, void* out, int epilogue, int m, int n, int k, void* stream);

@@ -2,10 +2,13 @@
 //
 // The weights are read once, straight from memory into matrix-core registers: a workgroup owns
 // 16 output columns n (16 rows of w) and all of k; its 8 waves split k between them, each wave
-// feeding 16x16x32 MFMAs with w as the A operand (16-byte loads, rows of w are contiguous in k)
-// and x as the B operand.  Loads run one batch of k-steps ahead of the MFMAs that use them.  The
-// waves' partial sums meet in LDS and are added in wave order, so a result does not depend on
-// the number of rows or on timing.
+// feeding 16x16x32 MFMAs with w as the A operand and x as the B operand.  The weights come
+// *packed in fragment order*: for every block of 16 rows and every k-step of 32, the 1 KB that a
+// wave's 64 lanes load (lane l: row l % 16, k 8 * (l / 16) .. + 7) lies contiguous, blocks and
+// k-steps in order -- so every load instruction reads eight whole cache lines and a wave walks
+// straight through memory (rows past n and k past the matrix are stored as zeros).  Loads run
+// one batch of k-steps ahead of the MFMAs that use them.  The waves' partial sums meet in LDS
+// and are added in wave order, so a result does not depend on the number of rows or on timing.
 //
 // What comes in (XMODE):
 //   plain    x is bfloat16 [m, k], read from cache as the B operand
@@ -48,7 +51,7 @@ struct SkinnyArgs {
   const void* x;            // bf16 [m, k], or float [*, k] in the normed modes
   const int32_t* rows;      // normed modes: row m of the product reads x[rows[m]] (null: x[m])
   const void* g;            // normed modes: RMSNorm scale [k]
-  const bf16_t* w;          // [n, k]
+  const bf16_t* w;          // packed: [ceil(n / 16)][ceil(k / 32)][64 lanes][8]
   void* out;
   int m, n, k, n_out;
   int m_stage;              // normed modes: rows of x staged in LDS (m rounded up to 4)
@@ -68,7 +71,8 @@ __global__ __launch_bounds__(kThreads, 4) void gemm_skinny_kernel(const SkinnyAr
   __shared__ float red[kWaves][kSets][MT][16][kRedPad];
   __shared__ float ssq_row[16];
   extern __shared__ __align__(16) unsigned char stage_raw[];   // normed: bf16 [m_stage][k + kStagePad]
-  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int lane = threadIdx.x % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);   // uniform: k ranges and bases stay scalar
   const int col = lane % 16, grp = lane / 16;
   const int n0 = blockIdx.x * 16;
   const int k = a.k, m = a.m;
@@ -83,11 +87,11 @@ __global__ __launch_bounds__(kThreads, 4) void gemm_skinny_kernel(const SkinnyAr
 #pragma unroll
     for (int t = 0; t < MT; ++t) acc[s][t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  const int wrow = n0 + col;                           // this lane's row of w (output column)
-  const bool wrow_ok = wrow < a.n;
-  const bf16_t* wptr[kSets];
-#pragma unroll
-  for (int s = 0; s < kSets; ++s) wptr[s] = a.w + static_cast<long>(wrow) * k;
+  // this workgroup's block of 16 rows in the packed weights: k-step ks at wblock + ks * 512 elements
+  // (a scalar base and a 32-bit lane offset, so the loads of a batch differ in their scalar part only)
+  const int ksteps_total = (k + 31) / 32;
+  const bf16_t* wblock = a.w + static_cast<long>(blockIdx.x) * ksteps_total * (kWave * 8);
+  const int wlane = lane * 8;
 
   // where this lane's B operand comes from
   const bf16_t* xptr[MT];
@@ -114,7 +118,8 @@ __global__ __launch_bounds__(kThreads, 4) void gemm_skinny_kernel(const SkinnyAr
       const int kk = k0 + 32 * u + 8 * grp;
       const bool ok = kk < k_end;
 #pragma unroll
-      for (int s = 0; s < kSets; ++s) b.w[s][u] = (ok && wrow_ok) ? load16(wptr[s] + kk) : zero16();
+      for (int s = 0; s < kSets; ++s)
+        b.w[s][u] = k0 + 32 * u < k_end ? load16(wblock + static_cast<long>(k0 / 32 + u) * (kWave * 8) + wlane) : zero16();
       if constexpr (!kNormed) {
 #pragma unroll
         for (int t = 0; t < MT; ++t) b.x[t][u] = (ok && xrow_ok[t]) ? load16(xptr[t] + kk) : zero16();

@@ -89,6 +89,7 @@ def gemm_generic(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = None
                  accumulate_into: Optional[torch.Tensor] = None) -> torch.Tensor:
     """a [M, K] times w [N, K] transposed, in plain float arithmetic.  With
     ``accumulate_into`` (float32 [M, N]) the product is added to it in place."""
+    w, _ = _weight(w)
     _dev("gemm", a, w, accumulate_into)
     if a.dim() != 2 or w.dim() != 2 or a.shape[1] != w.shape[1]:
         raise KernelError(f"gemm: shapes {tuple(a.shape)} x {tuple(w.shape)}^T do not match")
@@ -210,6 +211,38 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, u: torch.Tensor) -> 
     return out
 
 
+def pack_weight(w: torch.Tensor) -> torch.Tensor:
+    """A [n, k] weight in the fragment order the weight-streaming kernel reads:
+    [ceil(n/16)][ceil(k/32)][64 lanes][8], lane l of a k-step holding row l % 16 of the block and
+    k 8 * (l / 16) .. + 7 of the step; rows past n and k past the matrix are zeros."""
+    n, k = w.shape
+    nb, ks = -(-n // 16), -(-k // 32)
+    padded = w
+    if nb * 16 != n or ks * 32 != k:
+        padded = torch.zeros((nb * 16, ks * 32), dtype=w.dtype, device=w.device)
+        padded[:n, :k] = w
+    return padded.view(nb, 16, ks, 4, 8).permute(0, 2, 3, 1, 4).contiguous().view(-1)
+
+
+class StreamedWeight:
+    """A linear map's weight in both orders: by rows (for the tiled and the plain kernels) and
+    packed for the weight-streaming kernel.  The second copy costs memory, not traffic: every
+    step reads one of them."""
+
+    def __init__(self, rows: torch.Tensor):
+        self.rows = rows
+        self.shape, self.dtype, self.device = rows.shape, rows.dtype, rows.device
+        ok = rows.is_cuda and rows.dtype == torch.bfloat16 and rows.dim() == 2 and rows.shape[1] % 8 == 0
+        self.packed = pack_weight(rows) if ok else None
+
+
+def _weight(w):
+    """(rows, packed or None) of a weight given as a tensor or a StreamedWeight."""
+    if isinstance(w, StreamedWeight):
+        return w.rows, w.packed
+    return w, None
+
+
 SKINNY_MAX_ROWS = 64
 EPI_STORE_BF16, EPI_STORE_F32, EPI_ACCUM_F32, EPI_SWIGLU = 0, 1, 2, 3
 
@@ -219,11 +252,12 @@ def _fast_operands(a: torch.Tensor, w: torch.Tensor) -> bool:
             and a.shape[1] == w.shape[1] and a.shape[1] % 8 == 0 and a.shape[0] > 0)
 
 
-def gemm_fast(a: torch.Tensor, w: torch.Tensor, out_dtype=None,
+def gemm_fast(a: torch.Tensor, w, out_dtype=None,
               accumulate_into: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
     """The matrix-core product where a kernel takes these operands (bfloat16, k a multiple of
     8), else None (the caller then uses the plain float kernel).  Up to 64 rows the weights
     are streamed once (a decode step); beyond that the tiled kernel runs."""
+    w, packed = _weight(w)
     if not _fast_operands(a, w):
         return None
     _dev("gemm", a, w, accumulate_into)
@@ -239,25 +273,31 @@ def gemm_fast(a: torch.Tensor, w: torch.Tensor, out_dtype=None,
             return None
         out = torch.empty((m, n), dtype=out_dtype, device=a.device)
         epi = EPI_STORE_BF16 if out_dtype == torch.bfloat16 else EPI_STORE_F32
-    name = "bc4g_gemm_skinny" if m <= SKINNY_MAX_ROWS else "bc4g_gemm_mfma"
-    library.call(name, _ptr(a), _ptr(w), _ptr(out), epi, m, n, k, _stream())
+    if m <= SKINNY_MAX_ROWS:
+        packed = packed if packed is not None else pack_weight(w)      # (packing per call: tests only)
+        library.call("bc4g_gemm_skinny", _ptr(a), _ptr(packed), _ptr(out), epi, m, n, k, _stream())
+    else:
+        library.call("bc4g_gemm_mfma", _ptr(a), _ptr(w), _ptr(out), epi, m, n, k, _stream())
     return out
 
 
 NORMED_MAX_ROWS = 16
 
 
-def gemm_normed_supported(x: torch.Tensor, n_rows: int, g: torch.Tensor, w: torch.Tensor) -> bool:
+def gemm_normed_supported(x: torch.Tensor, n_rows: int, g: torch.Tensor, w) -> bool:
     """Whether RMSNorm can be fused into the product: few rows, bfloat16 weights, k a multiple of 8."""
+    w, _ = _weight(w)
     staged = (-(-n_rows // 4) * 4) * (x.shape[1] + 8) * 2          # bytes of LDS the normed rows take
     return (x.is_cuda and x.dtype == torch.float32 and w.dtype == torch.bfloat16 and 0 < n_rows <= NORMED_MAX_ROWS
             and x.shape[1] == w.shape[1] and x.shape[1] % 8 == 0 and g.dtype in _CODE and staged <= 96 * 1024)
 
 
 def gemm_normed(x: torch.Tensor, rows: Optional[torch.Tensor], n_rows: int, g: torch.Tensor, eps: float,
-                w: torch.Tensor, epilogue: int) -> torch.Tensor:
+                w, epilogue: int) -> torch.Tensor:
     """rmsnorm(x[rows]) W^T with the norm fused into the product (see gemm_skinny.hip): epilogue
     EPI_STORE_BF16, EPI_STORE_F32 or EPI_SWIGLU (w = gate rows then up rows)."""
+    w, packed = _weight(w)
+    packed = packed if packed is not None else pack_weight(w)
     _dev("gemm_normed", x, rows, g, w)
     k, n = x.shape[1], w.shape[0]
     if tuple(g.shape) != (k,):
@@ -275,45 +315,52 @@ def gemm_normed(x: torch.Tensor, rows: Optional[torch.Tensor], n_rows: int, g: t
     else:
         raise KernelError(f"gemm_normed: epilogue {epilogue} is not supported")
     library.call("bc4g_gemm_skinny_normed", _ptr(x), _ptr(rows), _ptr(g), _code(g, "gemm_normed"), float(eps),
-                 _ptr(w), _ptr(out), epilogue, n_rows, n, k, _stream())
+                 _ptr(packed), _ptr(out), epilogue, n_rows, n, k, _stream())
     return out
 
 
-def gemm_swiglu(a: torch.Tensor, w_gate_up: torch.Tensor, interleaved: bool = False) -> torch.Tensor:
+def gemm_swiglu(a: torch.Tensor, w_gate_up, interleaved: bool = False) -> torch.Tensor:
     """silu(a Wg^T) * (a Wu^T), [M, I], for w_gate_up [2I, K].  interleaved: every 16 rows of the
     weight are eight gate rows and the eight up rows of the same outputs -- then the activation
     is applied to the float sums inside the product's kernel.  Otherwise the product is stored
     and the activation kernel follows."""
-    if interleaved and _fast_operands(a, w_gate_up) and w_gate_up.shape[0] % 16 == 0:
-        _dev("gemm_swiglu", a, w_gate_up)
+    rows, packed = _weight(w_gate_up)
+    if interleaved and _fast_operands(a, rows) and rows.shape[0] % 16 == 0:
+        _dev("gemm_swiglu", a, rows)
         m, k = a.shape
-        n = w_gate_up.shape[0]
+        n = rows.shape[0]
         out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=a.device)
-        name = "bc4g_gemm_skinny" if m <= SKINNY_MAX_ROWS else "bc4g_gemm_mfma"
-        library.call(name, _ptr(a), _ptr(w_gate_up), _ptr(out), EPI_SWIGLU, m, n, k, _stream())
+        if m <= SKINNY_MAX_ROWS:
+            packed = packed if packed is not None else pack_weight(rows)
+            library.call("bc4g_gemm_skinny", _ptr(a), _ptr(packed), _ptr(out), EPI_SWIGLU, m, n, k, _stream())
+        else:
+            library.call("bc4g_gemm_mfma", _ptr(a), _ptr(rows), _ptr(out), EPI_SWIGLU, m, n, k, _stream())
         return out
     gu = gemm_fast(a, w_gate_up, a.dtype)
     if gu is None:
-        gu = gemm_generic(a, w_gate_up, a.dtype)
+        gu = gemm_generic(a, rows, a.dtype)
     return swiglu(gu, interleaved)
 
 
-def gemm_qkv_rope_supported(x: torch.Tensor, n_rows: int, normed: bool, w: torch.Tensor, head_dim: int,
+def gemm_qkv_rope_supported(x: torch.Tensor, n_rows: int, normed: bool, w, head_dim: int,
                             rotary_dim: int) -> bool:
     """Whether the q|k|v product of these rows can rotate and write the cache in its epilogue."""
+    w, _ = _weight(w)
     rows_ok = n_rows <= (NORMED_MAX_ROWS if normed else SKINNY_MAX_ROWS)
     return (x.is_cuda and w.dtype == torch.bfloat16 and x.shape[1] % 8 == 0 and 0 < n_rows and rows_ok
             and head_dim % 16 == 0 and rotary_dim in (0, head_dim)
             and x.dtype == (torch.float32 if normed else torch.bfloat16))
 
 
-def gemm_qkv_rope(x: torch.Tensor, g: Optional[torch.Tensor], eps: float, w: torch.Tensor,
+def gemm_qkv_rope(x: torch.Tensor, g: Optional[torch.Tensor], eps: float, w,
                   positions: torch.Tensor, slot_map: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
                   v_cache: Optional[torch.Tensor], n_heads: int, n_kv_heads: int, head_dim: int, rotary_dim: int,
                   theta: float, write_kv: bool = True) -> torch.Tensor:
     """The q|k|v product of a decode step with rotary positions and the cache write in its
     epilogue (w in the reordered head layout).  With g the input is the float residual stream
     and RMSNorm is fused.  Returns the rotated queries [M, heads * head_dim]."""
+    w, packed = _weight(w)
+    packed = packed if packed is not None else pack_weight(w)
     _dev("gemm_qkv_rope", x, g, w, positions, slot_map, k_cache, v_cache)
     m, k = x.shape
     n = (n_heads + 2 * n_kv_heads) * head_dim
@@ -329,7 +376,7 @@ def gemm_qkv_rope(x: torch.Tensor, g: Optional[torch.Tensor], eps: float, w: tor
         raise KernelError("gemm_qkv_rope: the fused norm needs a float32 input and a scale of its width")
     q = torch.empty((m, n_heads * head_dim), dtype=torch.bfloat16, device=x.device)
     library.call("bc4g_gemm_skinny_qkv", _ptr(x), _ptr(g), _code(g, "gemm_qkv_rope") if g is not None else 0,
-                 float(eps), _ptr(w), _ptr(q), _ptr(positions), _ptr(slot_map), _ptr(k_cache), _ptr(v_cache),
+                 float(eps), _ptr(packed), _ptr(q), _ptr(positions), _ptr(slot_map), _ptr(k_cache), _ptr(v_cache),
                  m, k, n_heads, n_kv_heads, head_dim, int(rotary_dim), float(theta), page_tokens,
                  1 if write_kv else 0, _stream())
     return q

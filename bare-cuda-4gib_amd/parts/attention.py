@@ -82,8 +82,8 @@ class CausalAttention(Part):
             q, k, v = rows(q, self.num_heads), rows(k, self.num_kv_heads), rows(v, self.num_kv_heads)
             o = o.view(-1, self.num_heads, d)[:, :, order].reshape(-1, self.num_heads * d).contiguous()
         # one product for q, k and v: their rows one after the other
-        self.w_qkv = torch.cat([p.to(dt) for p in (q, k, v)], dim=0).contiguous()
-        self.w_o = o
+        self.w_qkv = ops.StreamedWeight(torch.cat([p.to(dt) for p in (q, k, v)], dim=0).contiguous())
+        self.w_o = ops.StreamedWeight(o)
         self.act_dtype = rt.act_dtype
 
     def forward(self, h, ctx, cache, residual, writes: bool = True) -> None:

@@ -44,7 +44,7 @@ class LMHead(Part):
         return {"weight": WeightSpec((self.vocab_size, self.hidden_size), optional=self.tied_to is not None)}
 
     def bind(self, tensors, rt) -> None:
-        self.weight = tensors["weight"]
+        self.weight = ops.StreamedWeight(tensors["weight"])
 
     accepts_lazy_norm = True
 

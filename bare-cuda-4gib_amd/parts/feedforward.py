@@ -40,7 +40,8 @@ class SwiGLU(Part):
             self.w_gu = torch.stack([g.view(i // 8, 8, h), u.view(i // 8, 8, h)], dim=1).reshape(2 * i, h).contiguous()
         else:
             self.w_gu = torch.cat([g.to(dt), u.to(dt)], dim=0).contiguous()
-        self.w_down = tensors["down_proj.weight"]
+        self.w_gu = ops.StreamedWeight(self.w_gu)
+        self.w_down = ops.StreamedWeight(tensors["down_proj.weight"])
         self.act_dtype = rt.act_dtype
 
     def forward(self, h, ctx, residual) -> None:

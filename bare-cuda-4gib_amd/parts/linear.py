@@ -14,7 +14,7 @@ from ..csrc import ops
 from .lazy import Normed
 
 
-def _fused_norm(x: Normed, w: torch.Tensor, epilogue: int) -> Optional[torch.Tensor]:
+def _fused_norm(x: Normed, w, epilogue: int) -> Optional[torch.Tensor]:
     if x._tensor is not None:
         return None
     scale = x.fusable_scale()
@@ -23,10 +23,10 @@ def _fused_norm(x: Normed, w: torch.Tensor, epilogue: int) -> Optional[torch.Ten
     return ops.gemm_normed(x.x, x.rows, x.n_rows, scale[0], scale[1], w, epilogue)
 
 
-def linear(x: Union[torch.Tensor, Normed], w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
+def linear(x: Union[torch.Tensor, Normed], w, out_dtype: Optional[torch.dtype] = None,
            accumulate_into: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """x [M, K] times w [N, K] transposed.  With ``accumulate_into`` (the
-    float32 residual stream) the product is added to it in place."""
+    """x [M, K] times w [N, K] transposed (w a tensor or an ops.StreamedWeight).  With
+    ``accumulate_into`` (the float32 residual stream) the product is added to it in place."""
     if isinstance(x, Normed):
         if accumulate_into is None and out_dtype in (torch.bfloat16, torch.float32):
             epi = ops.EPI_STORE_BF16 if out_dtype == torch.bfloat16 else ops.EPI_STORE_F32
@@ -40,7 +40,7 @@ def linear(x: Union[torch.Tensor, Normed], w: torch.Tensor, out_dtype: Optional[
     return ops.gemm_generic(x, w, out_dtype, accumulate_into)
 
 
-def linear_swiglu(x: Union[torch.Tensor, Normed], w_gate_up: torch.Tensor, interleaved: bool = False) -> torch.Tensor:
+def linear_swiglu(x: Union[torch.Tensor, Normed], w_gate_up, interleaved: bool = False) -> torch.Tensor:
     """silu(x Wg^T) * (x Wu^T) for w_gate_up = gate rows followed by up rows, or (interleaved)
     blocks of eight gate rows and the eight up rows of the same outputs."""
     if isinstance(x, Normed):

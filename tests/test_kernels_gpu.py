@@ -414,3 +414,25 @@ def test_qkv_product_with_rotation_and_cache_write(ops, nh, nkv, d, m, normed, r
         close(kc2, kc_c, 1e-2, 2e-2, "unfused keys")
         close(vc2, vc_c, 1e-2, 2e-2, "unfused values")
         close(buf.view(m, nh + 2 * nkv, d)[:, :nh], q.view(m, nh, d), 1e-2, 2e-2, "unfused queries")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("m,n,k", [(1, 48, 64), (7, 100, 200), (33, 272, 1000), (64, 16, 8)])
+def test_streamed_weight_packing(ops, m, n, k):
+    """The packed copy holds the same matrix: the weight-streaming kernel gives, bit for bit, what
+    it gives for a copy packed on the host by the layout's definition, and that is x w^T."""
+    torch.manual_seed(m + n + k)
+    w = (torch.randn(n, k) * 0.1).bfloat16()
+    x = torch.randn(m, k).bfloat16()
+    nb, ks = -(-n // 16), -(-k // 32)
+    host = torch.zeros(nb, ks, 64, 8, dtype=torch.bfloat16)
+    for row in range(n):
+        for kk in range(0, k, 8):
+            lane = ((kk % 32) // 8) * 16 + row % 16
+            host[row // 16, kk // 32, lane] = w[row, kk:kk + 8]
+    held = ops.StreamedWeight(w.cuda())
+    assert torch.equal(held.packed.cpu(), host.view(-1))
+    out = ops.gemm_fast(x.cuda(), held, torch.float32)
+    want = x.double() @ w.double().T
+    torch.testing.assert_close(out.cpu().double(), want, rtol=2e-3, atol=2e-3)
+    assert torch.equal(out, ops.gemm_fast(x.cuda(), w.cuda(), torch.float32))
