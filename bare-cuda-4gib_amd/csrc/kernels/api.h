@@ -73,7 +73,8 @@ int bc4g_sample(const float* logits, const float* temperature, const double* u, 
 extern "C" {
 // bfloat16 x [m, k] (m <= 64) times bfloat16 w [n, k] transposed, weights streamed once through
 // the matrix cores.  w comes packed in fragment order: [ceil(n/16)][ceil(k/32)][64][8], where lane l
-// of a k-step holds row l % 16 of the block and k 8 * (l / 16) .. + 7 of the step, zeros past n and k.  epilogue: 0 store bfloat16 [m, n]; 1 store float32; 2 add into float32;
+// of a k-step holds row l % 16 of the block and k 8 * (l / 16) .. + 7 of the step, zeros past n and k.
+// epilogue: 0 store bfloat16 [m, n]; 1 store float32; 2 add into float32;
 // 3 SwiGLU: every 16 rows of w are eight gate rows and the eight up rows of the same outputs
 // (n = 2 * inter), out bfloat16 [m, inter] = silu(gate) * up.
 int bc4g_gemm_skinny(const void* x, const void* w, void* out, int epilogue, int m, int n, int k, void* stream);
@@ -84,15 +85,17 @@ extern "C" {
 // 16 rows, each tokens_per_tile tokens times the query heads of one key/value head; tile_start[s]
 // is the first wave-sized piece of request s when every request's rows are cut into pieces of
 // q_tiles * tokens_per_tile tokens; n_tiles their total.  q_tiles is 1, or 4 for head sizes up to
-// 64 and 2 up to 128.  With n_splits > 1 the keys
-// are cut into that many parts whose float partials (part_o [n_splits, T, heads, d], part_ml
-// [n_splits, T, heads, 2]) are merged into out.
+// 64 and 2 up to 128.  With shared_tile (q_tiles 1 only) a workgroup is one tile whose waves cut
+// the tile's keys between them and combine in LDS: for few rows over long contexts.  With
+// n_splits > 1 the keys are, moreover, cut into that many parts over workgroups, whose float
+// partials (part_o [n_splits, T, heads, d], part_ml [n_splits, T, heads, 2]) a second kernel
+// merges into out.
 int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, float* part_o, float* part_ml, const void* k_cache,
                         const void* v_cache, const int32_t* block_table, int table_stride,
                         const int32_t* seq_start, const int32_t* seq_ctx, const int32_t* tile_start,
                         int n_seqs, int n_tiles, int n_tokens, int n_heads, int n_kv_heads, int head_dim,
                         int page_tokens, int window, float scale, int tokens_per_tile, int q_tiles,
-                        int n_splits, void* stream);
+                        int shared_tile, int n_splits, void* stream);
 }
 
 extern "C" {

@@ -10,8 +10,12 @@
 //   online softmax in float, base 2, masked by absolute position (and the window)
 //   O^T += V^T P^T   with P^T taken from the score registers as the B operand and V^T loaded
 //                 from the transposed value pages (8-byte loads of 4 consecutive tokens)
-// With n_splits > 1 the key range is cut into that many parts (grid z); each part writes
-// unnormalized float partials, and attention_merge_kernel combines them.
+// Prompt portions bring many tiles: there a workgroup is four independent waves (WS == 1).
+// Decoded tokens bring few tiles and long key walks: there a workgroup is one tile and its WS
+// waves cut the tile's keys between them, then combine their partial results in LDS (in wave
+// order).  On top of that, with n_splits > 1 the key range is cut into that many parts over
+// workgroups (grid z); each part writes unnormalized float partials, and
+// attention_merge_kernel combines them.
 //
 // A row reads keys max(0, p - window + 1) .. p only.  Keys beyond the tile's last position may
 // never have been written: their scores are replaced by -inf and their values by zero, so that
@@ -59,12 +63,19 @@ struct AttnArgs {
 // DJ: k-steps of 32 over head_dim for the scores; DB: blocks of 16 output dimensions; QT: 16-row
 // query tiles per wave (consecutive tokens), which share every key and value fragment the wave
 // loads -- prompt portions use 4 (or 2 for large heads), decoded tokens 1.
-template <int DJ, int DB, int QT>
-__global__ __launch_bounds__(kWavesPerBlock * kWave, 2) void attention_mfma_kernel(const AttnArgs a) {
-  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+// WS: 1, or the number of waves that share one tile's keys.
+constexpr int kMergePad = 4;   // floats between rows of the partial outputs in LDS
+
+template <int DJ, int DB, int QT, int WS>
+__global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, WS > 8 ? 4 : 2) void attention_mfma_kernel(
+    const AttnArgs a) {
+  static_assert(WS == 1 || QT == 1, "waves share a tile's keys for single query tiles only");
+  extern __shared__ __align__(16) float merge_raw[];   // WS > 1: [WS][16][d + pad] outputs, [WS][16][2] statistics
+  const int lane = threadIdx.x % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int col = lane % 16, grp = lane / 16;
-  const int tile = blockIdx.x * kWavesPerBlock + wave;
-  if (tile >= a.n_tiles) return;   // no block-wide barrier below: waves are independent
+  const int tile = WS > 1 ? blockIdx.x : blockIdx.x * kWavesPerBlock + wave;
+  if (WS == 1 && tile >= a.n_tiles) return;   // (waves are independent there: no barrier below)
 
   // which request this tile belongs to
   int lo_s = 0, hi_s = a.n_seqs - 1;
@@ -110,8 +121,9 @@ __global__ __launch_bounds__(kWavesPerBlock * kWave, 2) void attention_mfma_kern
   const int lo_min = (a.window > 0 && pos_min - a.window + 1 > 0) ? pos_min - a.window + 1 : 0;
   const int kt_first = lo_min / 32, kt_last = pos_max / 32;
   const int n_kt = kt_last - kt_first + 1;
-  const int per_split = (n_kt + a.n_splits - 1) / a.n_splits;
-  const int kt_begin = kt_first + blockIdx.z * per_split;
+  const int n_parts = a.n_splits * WS;
+  const int per_split = (n_kt + n_parts - 1) / n_parts;
+  const int kt_begin = kt_first + (blockIdx.z * WS + (WS > 1 ? wave : 0)) * per_split;
   const int kt_end = min(kt_last + 1, kt_begin + per_split);
 
   float m_run[QT], l_run[QT];
@@ -172,10 +184,17 @@ __global__ __launch_bounds__(kWavesPerBlock * kWave, 2) void attention_mfma_kern
     }
   };
 
+  // (sixteen waves a workgroup leave a wave 128 registers: no room for a second tile in flight,
+  // and with four waves on every SIMD the other waves cover a load's latency)
+  constexpr bool kAhead = WS <= 8;
   KeyTile cur, nxt;
-  if (kt_begin < kt_end) fetch(cur, kt_begin);
+  if (kAhead && kt_begin < kt_end) fetch(cur, kt_begin);
   for (int kt = kt_begin; kt < kt_end; ++kt) {
-    if (kt + 1 < kt_end) fetch(nxt, kt + 1);
+    if constexpr (kAhead) {
+      if (kt + 1 < kt_end) fetch(nxt, kt + 1);
+    } else {
+      fetch(cur, kt);
+    }
     const int key0 = kt * 32;
     // values of keys past the tile's last position are replaced by zero
     uint32_t vmask[4];
@@ -253,7 +272,58 @@ __global__ __launch_bounds__(kWavesPerBlock * kWave, 2) void attention_mfma_kern
         o[t][b] = mfma_16x16x32(vf, pf, o[t][b]);
       }
     }
-    if (kt + 1 < kt_end) cur = nxt;
+    if constexpr (kAhead) {
+      if (kt + 1 < kt_end) cur = nxt;
+    }
+  }
+
+  if constexpr (WS > 1) {
+    // The waves' partial results meet in LDS; then all threads share out the tile's 16 x d
+    // outputs and add the parts in wave order, weighted by 2^(m_part - m).
+    const int ostride = d + kMergePad;
+    float* part_o = merge_raw;
+    float* part_ml = merge_raw + WS * 16 * ostride;
+    float l_tot = l_run[0] + __shfl_xor(l_run[0], 16, kWave);
+    l_tot += __shfl_xor(l_tot, 32, kWave);
+#pragma unroll
+    for (int b = 0; b < DB; ++b) {
+      if (16 * b >= d) break;
+      *reinterpret_cast<floatx4*>(part_o + (wave * 16 + col) * ostride + 16 * b + 4 * grp) = o[0][b];
+    }
+    if (grp == 0) {
+      part_ml[(wave * 16 + col) * 2] = m_run[0];
+      part_ml[(wave * 16 + col) * 2 + 1] = l_tot;
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < 16 * d; idx += WS * kWave) {
+      const int r = idx / d, c = idx % d;
+      const int r_tok = r / a.hg, r_head_in_group = hsub * a.hg + r % a.hg;
+      if (r_tok >= a.tpt || r_tok >= ntok || r_head_in_group >= group) continue;
+      float m = -INFINITY;
+#pragma unroll
+      for (int w = 0; w < WS; ++w) m = fmaxf(m, part_ml[(w * 16 + r) * 2]);
+      float l = 0.f, acc = 0.f;
+#pragma unroll
+      for (int w = 0; w < WS; ++w) {
+        const float mw = part_ml[(w * 16 + r) * 2];
+        const float wt = (mw == -INFINITY) ? 0.f : fast_exp2(mw - m);
+        l += wt * part_ml[(w * 16 + r) * 2 + 1];
+        acc += wt * part_o[(w * 16 + r) * ostride + c];
+      }
+      const long row = row0 + tok0 + r_tok;
+      const int head = kvh * group + r_head_in_group;
+      if (a.n_splits == 1) {
+        a.out[(row * a.n_heads + head) * d + c] = from_float<bf16_t>(acc / l);
+      } else {
+        const long slot = (static_cast<long>(blockIdx.z) * a.n_tokens + row) * a.n_heads + head;
+        a.part_o[slot * d + c] = acc;
+        if (c == 0) {
+          a.part_ml[slot * 2] = m;
+          a.part_ml[slot * 2 + 1] = l;
+        }
+      }
+    }
+    return;
   }
 
 #pragma unroll
@@ -333,7 +403,7 @@ extern "C" int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, flo
                                    const int32_t* seq_start, const int32_t* seq_ctx, const int32_t* tile_start,
                                    int n_seqs, int n_tiles, int n_tokens, int n_heads, int n_kv_heads, int head_dim,
                                    int page_tokens, int window, float scale, int tokens_per_tile, int q_tiles,
-                                   int n_splits, void* stream) {
+                                   int shared_tile, int n_splits, void* stream) {
   BC4G_REQUIRE(n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0, "attention_mfma: bad heads %d/%d",
                n_heads, n_kv_heads);
   BC4G_REQUIRE(head_dim >= 16 && head_dim <= 256 && head_dim % 16 == 0,
@@ -380,17 +450,27 @@ extern "C" int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, flo
                "attention_mfma: %d query tiles per wave are not built for head_dim %d (1 or %d)", q_tiles, head_dim,
                max_qt);
   BC4G_REQUIRE(n_kv_heads * a.n_sub <= 65535, "attention_mfma: too many heads for the grid");
+  BC4G_REQUIRE(!shared_tile || q_tiles == 1, "attention_mfma: waves share the keys of single query tiles only");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  dim3 grid((n_tiles + kWavesPerBlock - 1) / kWavesPerBlock, n_kv_heads * a.n_sub, n_splits);
-  dim3 block(kWavesPerBlock * kWave);
-  if (dj <= 2 && db <= 4) {
-    if (q_tiles == 4) attention_mfma_kernel<2, 4, 4><<<grid, block, 0, s>>>(a);
-    else attention_mfma_kernel<2, 4, 1><<<grid, block, 0, s>>>(a);
-  } else if (dj <= 4 && db <= 8) {
-    if (q_tiles == 2) attention_mfma_kernel<4, 8, 2><<<grid, block, 0, s>>>(a);
-    else attention_mfma_kernel<4, 8, 1><<<grid, block, 0, s>>>(a);
+  if (shared_tile) {
+    // one workgroup per tile; its waves (16, 8 or 4 by head size) cut the keys between them
+    dim3 grid(n_tiles, n_kv_heads * a.n_sub, n_splits);
+    auto lds = [&](int ws) { return static_cast<size_t>(ws) * 16 * (head_dim + kMergePad + 2) * sizeof(float); };
+    if (dj <= 2 && db <= 4) attention_mfma_kernel<2, 4, 1, 16><<<grid, 16 * kWave, lds(16), s>>>(a);
+    else if (dj <= 4 && db <= 8) attention_mfma_kernel<4, 8, 1, 8><<<grid, 8 * kWave, lds(8), s>>>(a);
+    else attention_mfma_kernel<8, 16, 1, 4><<<grid, 4 * kWave, lds(4), s>>>(a);
   } else {
-    attention_mfma_kernel<8, 16, 1><<<grid, block, 0, s>>>(a);
+    dim3 grid((n_tiles + kWavesPerBlock - 1) / kWavesPerBlock, n_kv_heads * a.n_sub, n_splits);
+    dim3 block(kWavesPerBlock * kWave);
+    if (dj <= 2 && db <= 4) {
+      if (q_tiles == 4) attention_mfma_kernel<2, 4, 4, 1><<<grid, block, 0, s>>>(a);
+      else attention_mfma_kernel<2, 4, 1, 1><<<grid, block, 0, s>>>(a);
+    } else if (dj <= 4 && db <= 8) {
+      if (q_tiles == 2) attention_mfma_kernel<4, 8, 2, 1><<<grid, block, 0, s>>>(a);
+      else attention_mfma_kernel<4, 8, 1, 1><<<grid, block, 0, s>>>(a);
+    } else {
+      attention_mfma_kernel<8, 16, 1, 1><<<grid, block, 0, s>>>(a);
+    }
   }
   if (int e = check_launch("attention_mfma")) return e;
   if (n_splits > 1) {

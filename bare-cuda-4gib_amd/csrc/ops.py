@@ -402,14 +402,28 @@ ATTENTION_MAX_SPLITS = 64
 ATTENTION_ENOUGH_WAVES = 512      # from here on the rows alone occupy the GPU
 ATTENTION_TILES_PER_WALK = 16     # 32-key tiles one wave should walk at most, if parts are to be had
 ATTENTION_MAX_PROMPT_SPLITS = 8
+ATTENTION_SHARED_WALK = 4         # the same where a workgroup's waves share one tile's keys
+ATTENTION_ENOUGH_GROUPS = 512     # workgroups of that kind from which on the keys are not cut further
 
 
-def attention_splits(n_tiles: int, n_heads: int, n_kv_heads: int, max_kv_len: int) -> int:
-    """Into how many parts the keys are cut so that the GPU has enough waves: none if the rows
-    alone fill it, else towards ATTENTION_TARGET_WAVES waves with at least one 32-key tile each."""
+def attention_shared_waves(head_dim: int) -> int:
+    """Waves that share one tile's keys in the decode form of the matrix-core attention kernel."""
+    return 16 if head_dim <= 64 else (8 if head_dim <= 128 else 4)
+
+
+
+def attention_splits(n_tiles: int, n_heads: int, n_kv_heads: int, max_kv_len: int, shared_waves: int = 0) -> int:
+    """Into how many parts the keys are cut over workgroups so that the GPU has enough waves: none
+    if the rows alone fill it, else towards ATTENTION_TARGET_WAVES waves with at least one 32-key
+    tile each.  With ``shared_waves`` a workgroup's waves already cut a tile's keys between them;
+    the keys are cut further only while a wave would walk more than ATTENTION_SHARED_WALK tiles."""
     group = n_heads // n_kv_heads
     waves = n_tiles * n_kv_heads * (-(-group // 16))
     key_tiles = max(1, -(-max_kv_len // 32))
+    if shared_waves:
+        walk = -(-key_tiles // shared_waves)
+        return max(1, min(-(-walk // ATTENTION_SHARED_WALK), ATTENTION_ENOUGH_GROUPS // max(waves, 1),
+                          ATTENTION_MAX_SPLITS))
     if waves >= ATTENTION_ENOUGH_WAVES:
         # the rows alone occupy the GPU; what is left to shorten is the longest wave's walk over
         # its keys, which bounds the kernel's time
@@ -420,7 +434,7 @@ def attention_splits(n_tiles: int, n_heads: int, n_kv_heads: int, max_kv_len: in
 def attention_mfma(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                    seq_start: torch.Tensor, seq_ctx: torch.Tensor, tile_start: torch.Tensor, n_tiles: int,
                    n_heads: int, n_kv_heads: int, head_dim: int, window: int, scale: float,
-                   n_splits: int, q_tiles: int = 1) -> torch.Tensor:
+                   n_splits: int, q_tiles: int = 1, shared_tile: bool = False) -> torch.Tensor:
     _dev("attention_mfma", qkv, k_cache, v_cache, block_table, seq_start, seq_ctx, tile_start)
     t = qkv.shape[0]
     _check_queries("attention_mfma", qkv, n_heads, n_kv_heads, head_dim)
@@ -442,7 +456,7 @@ def attention_mfma(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
                  _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(seq_start), _ptr(seq_ctx),
                  _ptr(tile_start), n_seqs, n_tiles, t, n_heads, n_kv_heads, head_dim, k_cache.shape[2],
                  int(window), float(scale), attention_tile_tokens(n_heads, n_kv_heads), int(q_tiles),
-                 int(n_splits), _stream())
+                 int(bool(shared_tile)), int(n_splits), _stream())
     return out
 
 
@@ -453,11 +467,15 @@ def attention(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, b
     else the plain float kernel."""
     if attention_mfma_supported(qkv, k_cache, head_dim):
         tpt = attention_tile_tokens(n_heads, n_kv_heads)
-        # a wave takes several query tiles as soon as some request brings more than one tile of rows
-        q_tiles = attention_q_tiles(head_dim) if ctx.max_q_len > tpt else 1
+        # a wave takes several query tiles as soon as some request brings more than one tile of rows;
+        # while every request brings one tile at most, a workgroup's waves share the tile's keys
+        shared = ctx.max_q_len <= tpt
+        q_tiles = 1 if shared else attention_q_tiles(head_dim)
         tile_start, n_tiles = ctx.attention_tiles(tpt * q_tiles)
-        n_splits = ctx.fixed_attention_splits or attention_splits(n_tiles, n_heads, n_kv_heads, ctx.max_kv_len)
+        n_splits = ctx.fixed_attention_splits or attention_splits(
+            n_tiles, n_heads, n_kv_heads, ctx.max_kv_len, attention_shared_waves(head_dim) if shared else 0)
         return attention_mfma(qkv, k_cache, v_cache, block_table, ctx.seq_start_dev, ctx.seq_ctx_dev,
-                              tile_start, n_tiles, n_heads, n_kv_heads, head_dim, window, scale, n_splits, q_tiles)
+                              tile_start, n_tiles, n_heads, n_kv_heads, head_dim, window, scale, n_splits, q_tiles,
+                              shared)
     return attention_generic(qkv, k_cache, v_cache, block_table, ctx.row_seq, ctx.positions,
                              n_heads, n_kv_heads, head_dim, window, scale)

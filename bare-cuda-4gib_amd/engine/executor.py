@@ -217,7 +217,8 @@ class Executor:
         S = key[0]
         dev = torch.tensor(flat, dtype=torch.int32).to(self.rt.device)
         # the key split count is frozen into the graph: chosen for the bucket's longest context
-        splits = max((ops.attention_splits(S, m.num_heads, m.num_kv_heads, bucket)
+        splits = max((ops.attention_splits(S, m.num_heads, m.num_kv_heads, bucket,
+                                           ops.attention_shared_waves(m.head_dim))
                       for m in self._attention_parts), default=1)
         ctx = self._context_from(dev, layout, group_layout, dict(host, max_kv=bucket), fixed_splits=splits)
         self.model.forward(ctx)                      # once outside the graph: first-use work happens here

@@ -252,7 +252,7 @@ def test_attention_generic(ops, nh, nkv, d, page, window):
         close(got, plain_result(case, window), what=f"generic {dt}", **tol)
 
 
-def run_mfma(ops, case, window, n_splits, q_tiles=1):
+def run_mfma(ops, case, window, n_splits, q_tiles=1, shared=False):
     nh, nkv, d = case["nh"], case["nkv"], case["d"]
     tpt = ops.attention_tile_tokens(nh, nkv) * q_tiles
     starts = [0]
@@ -261,7 +261,7 @@ def run_mfma(ops, case, window, n_splits, q_tiles=1):
     dev = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
     return ops.attention_mfma(case["qkv"], case["kc"], case["vc"], case["table"], dev(case["seq_start"]),
                               dev(case["seq_ctx"]), dev(starts), starts[-1], nh, nkv, d, window,
-                              1.0 / math.sqrt(d), n_splits, q_tiles)
+                              1.0 / math.sqrt(d), n_splits, q_tiles, shared)
 
 
 @pytest.mark.parametrize("nh,nkv,d,page", SHAPES)
@@ -278,6 +278,9 @@ def test_attention_mfma(ops, nh, nkv, d, page, window, n_splits):
         close(again, plain_result(case, window), rtol=2e-2, atol=2e-2, what="mfma, several tiles a wave")
         if n_splits == 1:   # (with split keys the parts are cut elsewhere: equal up to rounding only)
             assert torch.equal(again, got), "a row's result must not depend on how rows are grouped into waves"
+    # a workgroup's waves sharing one tile's keys (the form decoded tokens use)
+    close(run_mfma(ops, case, window, n_splits, shared=True), plain_result(case, window), rtol=2e-2, atol=2e-2,
+          what="mfma, keys shared between a workgroup's waves")
 
 
 @pytest.mark.parametrize("n_splits", [1, 5])
@@ -290,6 +293,9 @@ def test_attention_far_key_among_hundreds(ops, n_splits):
         want = plain_result(case)
         if fn == "mfma":
             got = run_mfma(ops, case, 0, n_splits)
+            shared = run_mfma(ops, case, 0, n_splits, shared=True)
+            close(shared, want, rtol=2e-2, atol=2e-2, what="mfma, shared keys")
+            assert float((shared[419].double().cpu().view(4, 64)[1] - case["wants"][0][2][3, 0]).abs().max()) < 0.05
         else:
             got = ops.attention_generic(case["qkv"], case["kc"], case["vc"], case["table"], case["row_seq"],
                                         case["positions"], 4, 2, 64, 0)
@@ -304,6 +310,8 @@ def test_attention_window_edge(ops):
     case = paged_case([(0, 50)], 2, 1, 32, 16, torch.bfloat16, seed=6, poison=False)
     for window in (1, 16, 17, 31, 32, 33):
         close(run_mfma(ops, case, window, 1), plain_result(case, window), rtol=2e-2, atol=2e-2, what=f"window {window}")
+        close(run_mfma(ops, case, window, 1, shared=True), plain_result(case, window), rtol=2e-2, atol=2e-2,
+              what=f"window {window}, shared keys")
 
 
 def test_argmax_ties_and_sampling(ops):
