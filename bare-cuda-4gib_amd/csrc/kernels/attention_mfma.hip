@@ -77,17 +77,31 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, WS > 8 ? 4 
   const int tile = WS > 1 ? blockIdx.x : blockIdx.x * kWavesPerBlock + wave;
   if (WS == 1 && tile >= a.n_tiles) return;   // (waves are independent there: no barrier below)
 
-  // which request this tile belongs to
-  int lo_s = 0, hi_s = a.n_seqs - 1;
-  while (lo_s < hi_s) {
-    const int mid = (lo_s + hi_s + 1) >> 1;
-    if (a.tile_start[mid] <= tile) lo_s = mid; else hi_s = mid - 1;
+  // Which request this tile belongs to, and that request's rows and context.  Up to 63 requests
+  // are looked at by one lane each (three loads, all at once, and a vote); more by bisection.
+  int s, row0, q_len, ctx, tile0;
+  if (a.n_seqs < kWave) {
+    const int ts = lane <= a.n_seqs ? a.tile_start[lane] : 0;
+    const int ss = lane <= a.n_seqs ? a.seq_start[lane] : 0;
+    const int sc = lane < a.n_seqs ? a.seq_ctx[lane] : 0;
+    s = __popcll(__ballot(lane < a.n_seqs && ts <= tile)) - 1;
+    tile0 = __shfl(ts, s, kWave);
+    row0 = __shfl(ss, s, kWave);
+    q_len = __shfl(ss, s + 1, kWave) - row0;
+    ctx = __shfl(sc, s, kWave);
+  } else {
+    int lo_s = 0, hi_s = a.n_seqs - 1;
+    while (lo_s < hi_s) {
+      const int mid = (lo_s + hi_s + 1) >> 1;
+      if (a.tile_start[mid] <= tile) lo_s = mid; else hi_s = mid - 1;
+    }
+    s = lo_s;
+    tile0 = a.tile_start[s];
+    row0 = a.seq_start[s];
+    q_len = a.seq_start[s + 1] - row0;
+    ctx = a.seq_ctx[s];
   }
-  const int s = lo_s;
-  const int row0 = a.seq_start[s];
-  const int q_len = a.seq_start[s + 1] - row0;
-  const int ctx = a.seq_ctx[s];
-  const int tok0 = (tile - a.tile_start[s]) * a.tpt * QT;
+  const int tok0 = (tile - tile0) * a.tpt * QT;
   const int ntok = min(a.tpt * QT, q_len - tok0);
   const int kvh = blockIdx.y / a.n_sub, hsub = blockIdx.y % a.n_sub;
   const int group = a.n_heads / a.n_kv_heads;
@@ -184,8 +198,7 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, WS > 8 ? 4 
     }
   };
 
-  // (sixteen waves a workgroup leave a wave 128 registers: no room for a second tile in flight,
-  // and with four waves on every SIMD the other waves cover a load's latency)
+  // (more than eight waves a workgroup would leave a wave 128 registers: no room for a second tile)
   constexpr bool kAhead = WS <= 8;
   KeyTile cur, nxt;
   if (kAhead && kt_begin < kt_end) fetch(cur, kt_begin);
@@ -371,6 +384,11 @@ __global__ __launch_bounds__(kWave) void attention_merge_kernel(const float* __r
   __shared__ float weight[kMaxSplits];
   const long rh = blockIdx.x;
   const int lane = threadIdx.x;
+  // the first parts' outputs are asked for together with the statistics, not after them
+  constexpr int kEarly = 8;
+  float early[kEarly];
+#pragma unroll
+  for (int z = 0; z < kEarly; ++z) early[z] = (z < n_splits && lane < d) ? part_o[(z * n_rows_heads + rh) * d + lane] : 0.f;
   float mz = -INFINITY, lz = 0.f;
   if (lane < n_splits) {
     const float2 ml = *reinterpret_cast<const float2*>(part_ml + (lane * n_rows_heads + rh) * 2);
@@ -387,8 +405,13 @@ __global__ __launch_bounds__(kWave) void attention_merge_kernel(const float* __r
   const float inv = 1.0f / l;
   for (int c = lane; c < d; c += kWave) {
     float acc = 0.f;
+    int z = 0;
+    if (c == lane) {
+#pragma unroll
+      for (; z < kEarly; ++z) acc += weight[z] * early[z];      // (weights beyond n_splits are zero)
+    }
 #pragma unroll 8
-    for (int z = 0; z < n_splits; ++z) acc += weight[z] * part_o[(z * n_rows_heads + rh) * d + c];
+    for (; z < n_splits; ++z) acc += weight[z] * part_o[(z * n_rows_heads + rh) * d + c];
     out[rh * d + c] = from_float<bf16_t>(acc * inv);
   }
 }
@@ -453,10 +476,10 @@ extern "C" int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, flo
   BC4G_REQUIRE(!shared_tile || q_tiles == 1, "attention_mfma: waves share the keys of single query tiles only");
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (shared_tile) {
-    // one workgroup per tile; its waves (16, 8 or 4 by head size) cut the keys between them
+    // one workgroup per tile; its waves (8, or 4 for the largest heads) cut the keys between them
     dim3 grid(n_tiles, n_kv_heads * a.n_sub, n_splits);
     auto lds = [&](int ws) { return static_cast<size_t>(ws) * 16 * (head_dim + kMergePad + 2) * sizeof(float); };
-    if (dj <= 2 && db <= 4) attention_mfma_kernel<2, 4, 1, 16><<<grid, 16 * kWave, lds(16), s>>>(a);
+    if (dj <= 2 && db <= 4) attention_mfma_kernel<2, 4, 1, 8><<<grid, 8 * kWave, lds(8), s>>>(a);
     else if (dj <= 4 && db <= 8) attention_mfma_kernel<4, 8, 1, 8><<<grid, 8 * kWave, lds(8), s>>>(a);
     else attention_mfma_kernel<8, 16, 1, 4><<<grid, 4 * kWave, lds(4), s>>>(a);
   } else {

@@ -402,13 +402,14 @@ ATTENTION_MAX_SPLITS = 64
 ATTENTION_ENOUGH_WAVES = 512      # from here on the rows alone occupy the GPU
 ATTENTION_TILES_PER_WALK = 16     # 32-key tiles one wave should walk at most, if parts are to be had
 ATTENTION_MAX_PROMPT_SPLITS = 8
-ATTENTION_SHARED_WALK = 4         # the same where a workgroup's waves share one tile's keys
-ATTENTION_ENOUGH_GROUPS = 512     # workgroups of that kind from which on the keys are not cut further
+ATTENTION_SHARED_WALK = 1         # the same where a workgroup's waves share one tile's keys: a CU pulls
+                                  # only so much from memory, so few workgroups with long walks are slow
+ATTENTION_ENOUGH_GROUPS = 256     # workgroups of that kind from which on the keys are not cut further
 
 
 def attention_shared_waves(head_dim: int) -> int:
     """Waves that share one tile's keys in the decode form of the matrix-core attention kernel."""
-    return 16 if head_dim <= 64 else (8 if head_dim <= 128 else 4)
+    return 8 if head_dim <= 128 else 4
 
 
 
