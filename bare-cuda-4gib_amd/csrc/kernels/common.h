@@ -9,6 +9,13 @@ namespace bc4g {
 
 constexpr int kWave = 64;  // CDNA wavefront width
 
+// A workgroup barrier that waits for this wave's LDS traffic only.  __syncthreads() also waits for
+// every global load the wave has in flight, which undoes a prefetch; here those loads stay in flight
+// (the compiler still waits for a load's data where it is used).
+__device__ inline void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 // ---- storage types ---------------------------------------------------------
 // Activations, weights and cache are float or bfloat16; bfloat16 is handled as
 // its 16-bit pattern and widened/rounded by hand so that every kernel states

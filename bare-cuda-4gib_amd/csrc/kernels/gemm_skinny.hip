@@ -209,7 +209,7 @@ __global__ __launch_bounds__(kThreads, 4) void gemm_skinny_kernel(const SkinnyAr
       if (lane == 0 && row < 16) ssq_row[row] = ss;
     }
     if (first && k_begin < k_end) load(cur, k_begin);      // a wave without a row to stage
-    __syncthreads();
+    lds_barrier();                                         // (the weights stay in flight)
   } else {
     if (k_begin < k_end) load(cur, k_begin);
   }
