@@ -7,7 +7,8 @@
 //   S^T = K Q^T   16x16x32 MFMAs with the keys as rows, so that a lane holds one query row's
 //                 scores and the softmax statistics are reductions inside a lane plus two
 //                 shuffles;  K rows come straight from the cache pages as the A operand
-//   online softmax in float, base 2, masked by absolute position (and the window)
+//   online softmax in float, base 2, masked by absolute position (and the window); the running
+//                 maximum is kept over raw scores and the scale enters the exponent's argument
 //   O^T += V^T P^T   with P^T taken from the score registers as the B operand and V^T loaded
 //                 from the transposed value pages (8-byte loads of 4 consecutive tokens)
 // Prompt portions bring many tiles: there a workgroup is four independent waves (WS == 1).
@@ -40,6 +41,26 @@ __device__ inline uint32_t pack_bf16x2(float lo, float hi) {
   uint32_t r;
   asm volatile("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(r) : "v"(lo), "v"(hi));
   return r;
+}
+
+// max / sum of a value over the four lanes l, l ^ 16, l ^ 32, l ^ 48, in every lane: the swap
+// instructions of gfx950 exchange half-rows between two registers in the vector ALU, with no trip
+// through LDS.  swap16(x, x) leaves (x of rows 0,0,2,2 | x of rows 1,1,3,3), swap32 the halves alike.
+__device__ inline float max_16_32(float x) {
+  const uint32_t u = __float_as_uint(x);
+  const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  const float y = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  const uint32_t v = __float_as_uint(y);
+  const auto b = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ inline float sum_16_32(float x) {
+  const uint32_t u = __float_as_uint(x);
+  const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  const float y = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  const uint32_t v = __float_as_uint(y);
+  const auto b = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
 struct AttnArgs {
@@ -84,11 +105,12 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, WS > 8 ? 4 
     const int ts = lane <= a.n_seqs ? a.tile_start[lane] : 0;
     const int ss = lane <= a.n_seqs ? a.seq_start[lane] : 0;
     const int sc = lane < a.n_seqs ? a.seq_ctx[lane] : 0;
-    s = __popcll(__ballot(lane < a.n_seqs && ts <= tile)) - 1;
-    tile0 = __shfl(ts, s, kWave);
-    row0 = __shfl(ss, s, kWave);
-    q_len = __shfl(ss, s + 1, kWave) - row0;
-    ctx = __shfl(sc, s, kWave);
+    // (read as scalars: everything derived from them -- key ranges, pages, addresses -- stays scalar)
+    s = __builtin_amdgcn_readfirstlane(__popcll(__ballot(lane < a.n_seqs && ts <= tile)) - 1);
+    tile0 = __builtin_amdgcn_readlane(ts, s);
+    row0 = __builtin_amdgcn_readlane(ss, s);
+    q_len = __builtin_amdgcn_readlane(ss, s + 1) - row0;
+    ctx = __builtin_amdgcn_readlane(sc, s);
   } else {
     int lo_s = 0, hi_s = a.n_seqs - 1;
     while (lo_s < hi_s) {
@@ -160,13 +182,14 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, WS > 8 ? 4 
     const int idx = r * kWave + lane;
     tbl[r] = (idx < pages_needed && idx < a.table_stride) ? table[idx] : 0;
   }
-  auto page_of = [&](int page_index) -> long {
+  auto page_of = [&](int page_index) -> long {       // page_index is the same in every lane
     if (page_index >= kTableRegs * kWave) return table[page_index];
-    int32_t v = __shfl(tbl[0], page_index % kWave, kWave);
+    const int at = page_index % kWave, reg = page_index / kWave;
+    int32_t v = __builtin_amdgcn_readlane(tbl[0], at);
 #pragma unroll
     for (int r = 1; r < kTableRegs; ++r) {
-      const int32_t w = __shfl(tbl[r], page_index % kWave, kWave);
-      if (page_index / kWave == r) v = w;
+      const int32_t w = __builtin_amdgcn_readlane(tbl[r], at);
+      if (reg == r) v = w;
     }
     return v;
   };
@@ -199,7 +222,7 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, WS > 8 ? 4 
   };
 
   // (more than eight waves a workgroup would leave a wave 128 registers: no room for a second tile)
-  constexpr bool kAhead = WS <= 8;
+  constexpr bool kAhead = WS <= 8 && DB <= 8;   // (nor do the fragments of the largest heads leave room)
   KeyTile cur, nxt;
   if (kAhead && kt_begin < kt_end) fetch(cur, kt_begin);
   for (int kt = kt_begin; kt < kt_end; ++kt) {
@@ -209,81 +232,94 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, WS > 8 ? 4 
       fetch(cur, kt);
     }
     const int key0 = kt * 32;
-    // values of keys past the tile's last position are replaced by zero
-    uint32_t vmask[4];
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const int kb = key0 + 16 * h + 4 * grp;
-      vmask[2 * h] = (kb <= pos_max ? 0xffffu : 0u) | (kb + 1 <= pos_max ? 0xffff0000u : 0u);
-      vmask[2 * h + 1] = (kb + 2 <= pos_max ? 0xffffu : 0u) | (kb + 3 <= pos_max ? 0xffff0000u : 0u);
-    }
-#pragma unroll
-    for (int t = 0; t < QT; ++t) {
-      if (QT > 1 && t * a.tpt >= ntok) continue;          // a tile beyond the request's rows (uniform)
-      floatx4 sc[2];
+    // values of keys past the tile's last position are replaced by zero (the tile at the end only)
+    if (key0 + 31 > pos_max) {
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
-        sc[h] = floatx4{0.f, 0.f, 0.f, 0.f};
+        const int kb = key0 + 16 * h + 4 * grp;
+        const uint32_t m01 = (kb <= pos_max ? 0xffffu : 0u) | (kb + 1 <= pos_max ? 0xffff0000u : 0u);
+        const uint32_t m23 = (kb + 2 <= pos_max ? 0xffffu : 0u) | (kb + 3 <= pos_max ? 0xffff0000u : 0u);
 #pragma unroll
-        for (int j = 0; j < DJ; ++j) sc[h] = mfma_16x16x32(cur.k[h][j], qf[t][j], sc[h]);
+        for (int b = 0; b < DB; ++b) {
+          cur.v[h][b].x &= m01;
+          cur.v[h][b].y &= m23;
+        }
       }
-      // This lane holds, for its query row, the scores of keys key0 + 16h + 4*grp + r.  A tile
-      // that every row of the query tile sees whole needs no mask (the usual case away from the
-      // diagonal); otherwise scores are masked by position, window and row validity.
-      const int tile_first_pos = ctx + tok0 + t * a.tpt;
-      const int tile_last_pos = min(tile_first_pos + a.tpt - 1, pos_max);
-      const int tile_lo = (a.window > 0 && tile_last_pos - a.window + 1 > 0) ? tile_last_pos - a.window + 1 : 0;
-      const bool interior = key0 + 31 <= tile_first_pos && key0 >= tile_lo;
-      float sv[8];
-      float m_tile = -INFINITY;
-      if (interior) {
+    }
+    // The wave's query tiles go through each phase together -- all score MFMAs, then all the
+    // softmax arithmetic, then all output MFMAs -- with no branch between tiles, so that the
+    // independent chains of the tiles overlap.  (Tiles beyond the request's rows run masked.)
+    floatx4 sc[QT][2];
+#pragma unroll
+    for (int t = 0; t < QT; ++t)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        sc[t][h] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < DJ; ++j) sc[t][h] = mfma_16x16x32(cur.k[h][j], qf[t][j], sc[t][h]);
+      }
+    // A lane holds, for its query row, the raw scores of keys key0 + 16h + 4*grp + r.  A key tile
+    // that every row of the wave sees whole needs no mask (the usual case away from the diagonal);
+    // otherwise scores are masked by position, window and row validity.
+    const int last_lo = (a.window > 0 && pos_max - a.window + 1 > 0) ? pos_max - a.window + 1 : 0;
+    const bool interior = key0 + 31 <= pos_min && key0 >= last_lo && ntok == a.tpt * QT;
+    float sv[QT][8];
+    if (interior) {
+#pragma unroll
+      for (int t = 0; t < QT; ++t)
 #pragma unroll
         for (int h = 0; h < 2; ++h)
 #pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            sv[4 * h + r] = sc[h][r] * a.scale_log2;
-            m_tile = fmaxf(m_tile, sv[4 * h + r]);
-          }
-      } else {
+          for (int r = 0; r < 4; ++r) sv[t][4 * h + r] = sc[t][h][r];
+    } else {
+#pragma unroll
+      for (int t = 0; t < QT; ++t)
 #pragma unroll
         for (int h = 0; h < 2; ++h)
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             const int key = key0 + 16 * h + 4 * grp + r;
             const bool vis = cur.ok[h] && q_ok[t] && key <= q_pos[t] && key >= q_lo[t];
-            const float v = vis ? sc[h][r] * a.scale_log2 : -INFINITY;
-            sv[4 * h + r] = v;
-            m_tile = fmaxf(m_tile, v);
+            sv[t][4 * h + r] = vis ? sc[t][h][r] : -INFINITY;
           }
-      }
-      m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 16, kWave));
-      m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, kWave));
+    }
+    // the running maximum is kept over raw scores; the softmax scale (> 0) enters the exponent
+    float alpha[QT];
+    uint4 pf[QT];
+    bool moved = false;
+#pragma unroll
+    for (int t = 0; t < QT; ++t) {
+      float m_tile = fmaxf(fmaxf(fmaxf(sv[t][0], sv[t][1]), fmaxf(sv[t][2], sv[t][3])),
+                           fmaxf(fmaxf(sv[t][4], sv[t][5]), fmaxf(sv[t][6], sv[t][7])));
+      m_tile = max_16_32(m_tile);
       const float m_new = fmaxf(m_run[t], m_tile);
       const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-      const float alpha = fast_exp2(m_run[t] - m_safe);   // 0 while nothing has been seen
-      float psum = 0.f;
-      uint32_t pk[4];
+      alpha[t] = fast_exp2((m_run[t] - m_safe) * a.scale_log2);   // 0 while nothing has been seen
+      const float shift = -m_safe * a.scale_log2;
+      float p[8];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float p0 = fast_exp2(sv[2 * i] - m_safe), p1 = fast_exp2(sv[2 * i + 1] - m_safe);
-        psum += p0 + p1;
-        pk[i] = pack_bf16x2(p0, p1);
-      }
-      l_run[t] = l_run[t] * alpha + psum;
+      for (int i = 0; i < 8; ++i) p[i] = fast_exp2(fmaf(sv[t][i], a.scale_log2, shift));
+      const float psum = ((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]));
+      l_run[t] = l_run[t] * alpha[t] + psum;
       m_run[t] = m_new;
-      const uint4 pf = make_uint4(pk[0], pk[1], pk[2], pk[3]);
-      const bool rescale = __any(alpha != 1.0f);   // the running maximum moved for some row
+      pf[t] = make_uint4(pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3]), pack_bf16x2(p[4], p[5]),
+                         pack_bf16x2(p[6], p[7]));
+      moved = moved || alpha[t] != 1.0f;
+    }
+    if (__any(moved)) {                                    // the running maximum moved for some row
 #pragma unroll
-      for (int b = 0; b < DB; ++b) {
-        if (16 * b >= d) break;   // DB is the most blocks this instantiation holds
-        const uint4 vf = make_uint4(cur.v[0][b].x & vmask[0], cur.v[0][b].y & vmask[1],
-                                    cur.v[1][b].x & vmask[2], cur.v[1][b].y & vmask[3]);
-        if (rescale) {
+      for (int t = 0; t < QT; ++t)
 #pragma unroll
-          for (int r = 0; r < 4; ++r) o[t][b][r] *= alpha;
-        }
-        o[t][b] = mfma_16x16x32(vf, pf, o[t][b]);
-      }
+        for (int b = 0; b < DB; ++b)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) o[t][b][r] *= alpha[t];
+    }
+    // (blocks past the head size hold zeros and are never stored)
+#pragma unroll
+    for (int b = 0; b < DB; ++b) {
+      const uint4 vf = make_uint4(cur.v[0][b].x, cur.v[0][b].y, cur.v[1][b].x, cur.v[1][b].y);
+#pragma unroll
+      for (int t = 0; t < QT; ++t) o[t][b] = mfma_16x16x32(vf, pf[t], o[t][b]);
     }
     if constexpr (kAhead) {
       if (kt + 1 < kt_end) cur = nxt;
@@ -296,15 +332,14 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, WS > 8 ? 4 
     const int ostride = d + kMergePad;
     float* part_o = merge_raw;
     float* part_ml = merge_raw + WS * 16 * ostride;
-    float l_tot = l_run[0] + __shfl_xor(l_run[0], 16, kWave);
-    l_tot += __shfl_xor(l_tot, 32, kWave);
+    const float l_tot = sum_16_32(l_run[0]);
 #pragma unroll
     for (int b = 0; b < DB; ++b) {
       if (16 * b >= d) break;
       *reinterpret_cast<floatx4*>(part_o + (wave * 16 + col) * ostride + 16 * b + 4 * grp) = o[0][b];
     }
     if (grp == 0) {
-      part_ml[(wave * 16 + col) * 2] = m_run[0];
+      part_ml[(wave * 16 + col) * 2] = m_run[0] * a.scale_log2;      // (-inf stays -inf: the scale is > 0)
       part_ml[(wave * 16 + col) * 2 + 1] = l_tot;
     }
     __syncthreads();
@@ -341,8 +376,7 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, WS > 8 ? 4 
 
 #pragma unroll
   for (int t = 0; t < QT; ++t) {
-    float l_tot = l_run[t] + __shfl_xor(l_run[t], 16, kWave);
-    l_tot += __shfl_xor(l_tot, 32, kWave);
+    const float l_tot = sum_16_32(l_run[t]);
     if (!q_ok[t]) continue;
     const long row = row0 + tok0 + q_tok[t];
     if (a.n_splits == 1) {
@@ -365,7 +399,7 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, WS > 8 ? 4 
         *reinterpret_cast<floatx4*>(dst + 16 * b) = o[t][b];
       }
       if (grp == 0) {
-        a.part_ml[slot * 2] = m_run[t];
+        a.part_ml[slot * 2] = m_run[t] * a.scale_log2;
         a.part_ml[slot * 2 + 1] = l_tot;
       }
     }
@@ -436,6 +470,7 @@ extern "C" int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, flo
   BC4G_REQUIRE(n_splits >= 1 && n_splits <= kMaxSplits && (n_splits == 1 || (part_o && part_ml)),
                "attention_mfma: the split count %d must lie in 1..64", n_splits);
   BC4G_REQUIRE(window >= 0 && table_stride > 0 && n_seqs > 0, "attention_mfma: bad sizes");
+  BC4G_REQUIRE(scale > 0.f, "attention_mfma: the softmax scale must be positive, got %g", static_cast<double>(scale));
   BC4G_REQUIRE(q_stride >= n_heads * head_dim && q_stride % 8 == 0, "attention_mfma: bad query row stride %d", q_stride);
   if (n_tiles == 0 || n_tokens == 0) return 0;
   const int group = n_heads / n_kv_heads;
