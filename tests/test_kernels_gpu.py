@@ -132,6 +132,26 @@ def test_gemm_mfma(ops, m, n, k):
     assert ops.gemm_fast(a.float().to(DEV), w.to(DEV)) is None                      # float operands: not taken
 
 
+def test_gemm_mfma_both_forms_agree_bit_for_bit(ops):
+    """Few tiles go to the form with moving and multiplying waves, many to the plain one (two
+    workgroups a CU).  Both add over k in the same order: a row's result is the same bits
+    whichever form the number of rows selects, also for sizes that are no multiple of anything."""
+    n, k = 2060, 200                                    # 17 tiles across
+    a, w = bf(rnd(2500, k, seed=40)), bf(rnd(n, k, seed=41))
+    wd = w.to(DEV)
+    many = ops.gemm_fast(a.to(DEV), wd, torch.float32)                 # 20 x 17 = 340 tiles: plain form
+    few = ops.gemm_fast(a[:300].contiguous().to(DEV), wd, torch.float32)   # 3 x 17 tiles: split form
+    close(many, a.double() @ w.double().T, 1e-4, 2e-3, "many tiles")
+    assert torch.equal(few, many[:300])
+    gate_up = interleave8(w[:1024], w[1024:2048])
+    g = ops.gemm_swiglu(a.to(DEV), gate_up.to(DEV), interleaved=True)
+    assert torch.equal(ops.gemm_swiglu(a[:300].contiguous().to(DEV), gate_up.to(DEV), interleaved=True), g[:300])
+    acc_many, acc_few = torch.ones(2500, n, device=DEV), torch.ones(300, n, device=DEV)
+    ops.gemm_fast(a.to(DEV), wd, accumulate_into=acc_many)
+    ops.gemm_fast(a[:300].contiguous().to(DEV), wd, accumulate_into=acc_few)
+    assert torch.equal(acc_few, acc_many[:300])
+
+
 def test_gemm_mfma_xcd_numbering_covers_every_tile(ops):
     a, w = bf(rnd(1024, 64, seed=15)), bf(rnd(1024, 64, seed=16))                    # 8 x 8 tiles: remapped ids
     close(ops.gemm_fast(a.to(DEV), w.to(DEV), torch.float32), a.double() @ w.double().T, 1e-4, 1e-3, "xcd")
