@@ -64,7 +64,9 @@ __device__ inline uint32_t pack2(float a, float b) {
 }
 
 template <int MT, int EPI, int XMODE, int U>
-__global__ __launch_bounds__(kThreads, 4) void gemm_skinny_kernel(const SkinnyArgs a) {
+// (The normed form keeps to 80 registers, so that three workgroups share a CU and all the blocks of
+// a 5,632 x 2 wide gate-up matrix are in flight at once.)
+__global__ __launch_bounds__(kThreads, XMODE != kPlain ? 6 : 4) void gemm_skinny_kernel(const SkinnyArgs a) {
   constexpr int kSets = 1;
   constexpr bool kNormed = XMODE != kPlain;
   static_assert(!kNormed || MT == 1, "the fused norm handles one tile of rows");
@@ -151,7 +153,7 @@ __global__ __launch_bounds__(kThreads, 4) void gemm_skinny_kernel(const SkinnyAr
     // Stage bf16(x * g): wave w takes rows w, w + 8; a lane takes 8 elements of each 512.  The
     // loads of x and g are issued first and the first weights right after them: loads come back
     // in the order they were issued, so the (cached) x arrives while the weights are on their way.
-    constexpr int kStageIters = 4;                       // 2048 elements of a row per round
+    constexpr int kStageIters = 2;                       // 1024 elements of a row per round
     bf16_t* stage = reinterpret_cast<bf16_t*>(stage_raw);
     bool first = true;
     for (int row = wave; row < a.m_stage; row += kWaves) {
@@ -306,7 +308,7 @@ int launch(const SkinnyArgs& a, hipStream_t s) {
     if (mt != 1) return fail("gemm_skinny: the fused norm takes at most 16 rows, got %d", a.m);
     const size_t stage = static_cast<size_t>(a.m_stage) * (a.k + kStagePad) * 2;
     if (stage > kMaxStageBytes) return fail("gemm_skinny: %d rows of k=%d do not fit the staging buffer", a.m, a.k);
-    auto kernel = gemm_skinny_kernel<1, EPI, XMODE, 8>;
+    auto kernel = gemm_skinny_kernel<1, EPI, XMODE, 4>;
     static bool raised = false;   // per instantiation: allow more than the default dynamic LDS
     if (!raised) {
       if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
