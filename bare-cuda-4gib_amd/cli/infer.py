@@ -2,8 +2,9 @@
 print the generated ids.  Options as in the reference's program of the same
 name (bench/src/main.cc:18-95): ``--model --prompt id,id,... [--tokens N]
 [--max-seq N]``; ids in, ids out, no tokenizer.  Added here: ``--dtype``,
-the sampling options of the Python entry point, and ``--random-weights`` to
-write the model folder from a configuration and a seed first."""
+the sampling options of the Python entry point, ``--kv-pages`` /
+``--page-tokens`` for the cache pool, and ``--random-weights`` to write the
+model folder from a configuration and a seed first."""
 from __future__ import annotations
 
 import argparse
@@ -27,6 +28,8 @@ def main(argv=None) -> int:
     ap.add_argument("--top-p", type=float, default=1.0)
     ap.add_argument("--top-k", type=int, default=0)
     ap.add_argument("--seed", type=int, default=-1, help="sampling seed; -1 draws one")
+    ap.add_argument("--kv-pages", type=int, default=0, help="pages in the cache pool; 0 sizes it for --max-seq")
+    ap.add_argument("--page-tokens", type=int, default=64, help="tokens per cache page (a multiple of 16)")
     ap.add_argument("--random-weights", metavar="CONFIG_JSON", default=None,
                     help="first write --model from this config.json with random weights")
     ap.add_argument("--weights-seed", type=int, default=0)
@@ -45,7 +48,8 @@ def main(argv=None) -> int:
     from ..errors import EngineError
     max_seq = args.max_seq if args.max_seq > 0 else len(prompt) + args.tokens
     try:
-        engine = Engine(args.model, max_tokens=max_seq, max_seqs=1, dtype=args.dtype)
+        engine = Engine(args.model, max_tokens=max_seq, max_seqs=1, kv_pages=args.kv_pages, dtype=args.dtype,
+                        page_tokens=args.page_tokens)
         cache_mib = engine.executor.cache.storage_bytes() / 2**20
         print(f"[llm] {len(engine.model.layers)} layers, hidden {engine.model.hidden_size}, vocab "
               f"{engine.model.vocab_size} | weights {engine.model.weight_bytes / 2**20:.1f} MiB, cache "

@@ -145,11 +145,13 @@ def test_command_line(folders, tmp_path):
     folder = folders("A", "float32")
     prompt = helpers.random_ids(7, 256, 1)
     proc = subprocess.run([sys.executable, os.path.join(helpers.ROOT, "bin", "llm-infer"), "--model", folder,
-                           "--prompt", ",".join(map(str, prompt)), "--tokens", "5", "--dtype", "float32"],
+                           "--prompt", ",".join(map(str, prompt)), "--tokens", "5", "--dtype", "float32",
+                           "--page-tokens", "16", "--kv-pages", "3"],
                           capture_output=True, text=True, timeout=300)
     assert proc.returncode == 0, proc.stderr[-2000:]
     lines = proc.stdout.strip().splitlines()
     assert lines[0].startswith("[llm] 2 layers, hidden 64, vocab 256") and lines[1].split() == ["prompt:"] + [str(t) for t in prompt]
+    assert "(3 pages, max batch 1)" in lines[0]
     assert [int(t) for t in lines[2].split()[1:]] == PlainLlama(folder).greedy(prompt, 5)
     bad = subprocess.run([sys.executable, os.path.join(helpers.ROOT, "bin", "llm-infer"), "--model", str(tmp_path / "none"),
                           "--prompt", "1,2"], capture_output=True, text=True, timeout=300)
