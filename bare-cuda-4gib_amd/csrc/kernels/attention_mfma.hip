@@ -87,7 +87,8 @@ struct AttnArgs {
 // WS: 1, or the number of waves that share one tile's keys.
 constexpr int kMergePad = 4;   // floats between rows of the partial outputs in LDS
 
-template <int DJ, int DB, int QT, int WS>
+// EXACT: the head size is exactly 16 * DB (the usual sizes 64, 128, 256): no test against it is left.
+template <int DJ, int DB, int QT, int WS, bool EXACT>
 __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, WS > 8 ? 4 : 2) void attention_mfma_kernel(
     const AttnArgs a) {
   static_assert(WS == 1 || QT == 1, "waves share a tile's keys for single query tiles only");
@@ -127,7 +128,7 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, WS > 8 ? 4 
   const int ntok = min(a.tpt * QT, q_len - tok0);
   const int kvh = blockIdx.y / a.n_sub, hsub = blockIdx.y % a.n_sub;
   const int group = a.n_heads / a.n_kv_heads;
-  const int d = a.head_dim, P = a.page_tokens;
+  const int d = EXACT ? 16 * DB : a.head_dim, P = a.page_tokens;
   const int32_t* table = a.block_table + static_cast<long>(s) * a.table_stride;
 
   // this lane's query row in each tile (as B operand and as owner of one row's statistics)
@@ -147,7 +148,7 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, WS > 8 ? 4 
 #pragma unroll
     for (int j = 0; j < DJ; ++j) {
       const int c = 32 * j + 8 * grp;
-      qf[t][j] = (q_ok[t] && c < d)
+      qf[t][j] = (q_ok[t] && (EXACT || c < d))
                      ? load16(a.qkv + (row0 + tok0 + q_tok[t]) * qkv_stride + static_cast<long>(q_head) * d + c)
                      : zero16();
     }
@@ -201,23 +202,31 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, WS > 8 ? 4 
     uint2 v[2][DB];
     bool ok[2];
   };
-  auto fetch = [&](KeyTile& t, int kt) {
+  // Addresses are a scalar base (page, key/value head, offset in the page: the same in every lane)
+  // plus a 32-bit lane offset; where the next tile lies in its page is carried along from tile to
+  // tile (the wave walks its tiles in order), so a fetch costs no division.
+  const int k_lane = col * d + 8 * grp, v_lane = col * P + 4 * grp;
+  int next_page = (kt_begin * 32) / P, next_off = (kt_begin * 32) % P;
+  auto fetch = [&](KeyTile& t, int kt) {        // tiles are fetched in order, from kt_begin on
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       const int kb = kt * 32 + 16 * h;
       t.ok[h] = kb <= pos_max && kb + 15 >= lo_min;
-      long page = 0;
-      if (t.ok[h]) page = page_of(kb / P);
-      const int off = kb % P;
-      const bf16_t* kptr = a.k_cache + ((page * a.n_kv_heads + kvh) * P + off + col) * d + 8 * grp;
-      const bf16_t* vptr = a.v_cache + (page * a.n_kv_heads + kvh) * static_cast<long>(d) * P + off + 4 * grp +
-                           static_cast<long>(col) * P;
+      const long page = t.ok[h] ? page_of(next_page) : 0;
+      const bf16_t* kbase = a.k_cache + ((page * a.n_kv_heads + kvh) * P + next_off) * static_cast<long>(d);
+      const bf16_t* vbase = a.v_cache + (page * a.n_kv_heads + kvh) * static_cast<long>(d) * P + next_off;
 #pragma unroll
-      for (int j = 0; j < DJ; ++j) t.k[h][j] = (t.ok[h] && 32 * j + 8 * grp < d) ? load16(kptr + 32 * j) : zero16();
+      for (int j = 0; j < DJ; ++j)
+        t.k[h][j] = (t.ok[h] && (EXACT || 32 * j + 8 * grp < d)) ? load16(kbase + 32 * j + k_lane) : zero16();
 #pragma unroll
       for (int b = 0; b < DB; ++b)
-        t.v[h][b] = (t.ok[h] && 16 * b < d) ? *reinterpret_cast<const uint2*>(vptr + static_cast<long>(16 * b) * P)
+        t.v[h][b] = (t.ok[h] && (EXACT || 16 * b < d)) ? *reinterpret_cast<const uint2*>(vbase + 16 * b * P + v_lane)
                                             : make_uint2(0u, 0u);
+      next_off += 16;                           // pages hold a multiple of 16 tokens
+      if (next_off >= P) {
+        next_off = 0;
+        ++next_page;
+      }
     }
   };
 
@@ -335,7 +344,7 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, WS > 8 ? 4 
     const float l_tot = sum_16_32(l_run[0]);
 #pragma unroll
     for (int b = 0; b < DB; ++b) {
-      if (16 * b >= d) break;
+      if (!EXACT && 16 * b >= d) break;
       *reinterpret_cast<floatx4*>(part_o + (wave * 16 + col) * ostride + 16 * b + 4 * grp) = o[0][b];
     }
     if (grp == 0) {
@@ -384,7 +393,7 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, WS > 8 ? 4 
       bf16_t* dst = a.out + (row * a.n_heads + q_head) * d + 4 * grp;
 #pragma unroll
       for (int b = 0; b < DB; ++b) {
-        if (16 * b >= d) break;
+        if (!EXACT && 16 * b >= d) break;
         uint2 pack;
         pack.x = pack_bf16x2(o[t][b][0] * inv, o[t][b][1] * inv);
         pack.y = pack_bf16x2(o[t][b][2] * inv, o[t][b][3] * inv);
@@ -395,7 +404,7 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, WS > 8 ? 4 
       float* dst = a.part_o + slot * d + 4 * grp;
 #pragma unroll
       for (int b = 0; b < DB; ++b) {
-        if (16 * b >= d) break;
+        if (!EXACT && 16 * b >= d) break;
         *reinterpret_cast<floatx4*>(dst + 16 * b) = o[t][b];
       }
       if (grp == 0) {
@@ -454,6 +463,16 @@ __global__ __launch_bounds__(kWave) void attention_merge_kernel(const float* __r
 }  // namespace bc4g
 
 using namespace bc4g;
+
+namespace bc4g {
+namespace {
+template <int DJ, int DB, int QT, int WS>
+void launch_attention(const AttnArgs& a, dim3 grid, dim3 block, size_t lds, hipStream_t s) {
+  if (a.head_dim == 16 * DB) attention_mfma_kernel<DJ, DB, QT, WS, true><<<grid, block, lds, s>>>(a);
+  else attention_mfma_kernel<DJ, DB, QT, WS, false><<<grid, block, lds, s>>>(a);
+}
+}  // namespace
+}  // namespace bc4g
 
 extern "C" int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, float* part_o, float* part_ml, const void* k_cache,
                                    const void* v_cache, const int32_t* block_table, int table_stride,
@@ -514,20 +533,20 @@ extern "C" int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, flo
     // one workgroup per tile; its waves (8, or 4 for the largest heads) cut the keys between them
     dim3 grid(n_tiles, n_kv_heads * a.n_sub, n_splits);
     auto lds = [&](int ws) { return static_cast<size_t>(ws) * 16 * (head_dim + kMergePad + 2) * sizeof(float); };
-    if (dj <= 2 && db <= 4) attention_mfma_kernel<2, 4, 1, 8><<<grid, 8 * kWave, lds(8), s>>>(a);
-    else if (dj <= 4 && db <= 8) attention_mfma_kernel<4, 8, 1, 8><<<grid, 8 * kWave, lds(8), s>>>(a);
-    else attention_mfma_kernel<8, 16, 1, 4><<<grid, 4 * kWave, lds(4), s>>>(a);
+    if (dj <= 2 && db <= 4) launch_attention<2, 4, 1, 8>(a, grid, 8 * kWave, lds(8), s);
+    else if (dj <= 4 && db <= 8) launch_attention<4, 8, 1, 8>(a, grid, 8 * kWave, lds(8), s);
+    else launch_attention<8, 16, 1, 4>(a, grid, 4 * kWave, lds(4), s);
   } else {
     dim3 grid((n_tiles + kWavesPerBlock - 1) / kWavesPerBlock, n_kv_heads * a.n_sub, n_splits);
     dim3 block(kWavesPerBlock * kWave);
     if (dj <= 2 && db <= 4) {
-      if (q_tiles == 4) attention_mfma_kernel<2, 4, 4, 1><<<grid, block, 0, s>>>(a);
-      else attention_mfma_kernel<2, 4, 1, 1><<<grid, block, 0, s>>>(a);
+      if (q_tiles == 4) launch_attention<2, 4, 4, 1>(a, grid, block, 0, s);
+      else launch_attention<2, 4, 1, 1>(a, grid, block, 0, s);
     } else if (dj <= 4 && db <= 8) {
-      if (q_tiles == 2) attention_mfma_kernel<4, 8, 2, 1><<<grid, block, 0, s>>>(a);
-      else attention_mfma_kernel<4, 8, 1, 1><<<grid, block, 0, s>>>(a);
+      if (q_tiles == 2) launch_attention<4, 8, 2, 1>(a, grid, block, 0, s);
+      else launch_attention<4, 8, 1, 1>(a, grid, block, 0, s);
     } else {
-      attention_mfma_kernel<8, 16, 1, 1><<<grid, block, 0, s>>>(a);
+      launch_attention<8, 16, 1, 1>(a, grid, block, 0, s);
     }
   }
   if (int e = check_launch("attention_mfma")) return e;
