@@ -400,7 +400,7 @@ def attention_q_tiles(head_dim: int) -> int:
 ATTENTION_TARGET_WAVES = 2048
 ATTENTION_MAX_SPLITS = 64
 ATTENTION_ENOUGH_WAVES = 512      # from here on the rows alone occupy the GPU
-ATTENTION_TILES_PER_WALK = 16     # 32-key tiles one wave should walk at most, if parts are to be had
+ATTENTION_TILES_PER_WALK = 32     # 32-key tiles one wave should walk at most, if parts are to be had
 ATTENTION_MAX_PROMPT_SPLITS = 8
 ATTENTION_SHARED_WALK = 1         # the same where a workgroup's waves share one tile's keys: a CU pulls
                                   # only so much from memory, so few workgroups with long walks are slow
