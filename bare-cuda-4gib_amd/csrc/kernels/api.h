@@ -47,6 +47,16 @@ int bc4g_rope_kv_write(void* qkv, int dtype, const int32_t* positions, const int
                        int head_dim, int rotary_dim, float theta, int page_tokens, int num_pages,
                        int write_kv, int block_pairs, void* stream);
 
+// The angles of a step, for every layer to share: table [n_tokens, rotary_dim / 2, 2] = (cos, sin)
+// of position * theta^(-2i / rotary_dim).
+int bc4g_rope_table(const int32_t* positions, float* table, int n_tokens, int rotary_dim, float theta, void* stream);
+
+// bc4g_rope_kv_write for the block layout (block_pairs), rotating by a table from bc4g_rope_table
+// (rotate != 0: the whole head, rotary_dim == head_dim), in 16-byte pieces.
+int bc4g_rope_kv_write_blocks(void* qkv, int dtype, const float* table, const int32_t* slot_map, void* k_cache,
+                              void* v_cache, int n_tokens, int n_heads, int n_kv_heads, int head_dim, int rotate,
+                              int page_tokens, int write_kv, void* stream);
+
 // Causal softmax attention of every row over its request's cached keys
 // (attention_qk.cu:17-70, softmax.cu:22-43, attention_av.cu:18-46, fused).
 // Row t of request s = row_seq[t] at position p = positions[t] sees keys

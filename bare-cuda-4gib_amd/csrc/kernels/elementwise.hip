@@ -133,6 +133,104 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const int32_t* __restr
   }
 }
 
+// The angles of a step, once for all layers: table[token][i] = (cos, sin) of position * theta^(-2i/dim),
+// i < dim/2, with the precise powf / sincosf of the kernel above.
+__global__ void rope_table_kernel(const int32_t* __restrict__ positions, float2* __restrict__ table, long total,
+                                  int rhalf, float theta) {
+  const long stride = static_cast<long>(blockDim.x) * gridDim.x;
+  for (long idx = blockIdx.x * static_cast<long>(blockDim.x) + threadIdx.x; idx < total; idx += stride) {
+    const int i = static_cast<int>(idx % rhalf);
+    const long token = idx / rhalf;
+    const float inv_freq = 1.0f / powf(theta, (2.0f * static_cast<float>(i)) / static_cast<float>(2 * rhalf));
+    float s, c;
+    sincosf(static_cast<float>(positions[token]) * inv_freq, &s, &c);
+    table[idx] = make_float2(c, s);
+  }
+}
+
+// rope_kv_write for the block layout (block_pairs) with the step's table of angles: a thread takes
+// one block of 16 elements -- pairs 8b .. 8b+7 of one head of one token -- with 16-byte loads and
+// stores (values go to their transposed pages element by element).
+template <typename T>
+__global__ void rope_kv_write_blocks_kernel(T* __restrict__ qkv, const float2* __restrict__ table,
+                                            const int32_t* __restrict__ slot_map, T* __restrict__ k_cache,
+                                            T* __restrict__ v_cache, long total, int n_heads, int n_kv_heads,
+                                            int head_dim, int rotate, int page_tokens, int write_kv) {
+  const int blocks = head_dim / 16;
+  const int heads_total = n_heads + 2 * n_kv_heads;
+  const long stride = static_cast<long>(blockDim.x) * gridDim.x;
+  for (long idx = blockIdx.x * static_cast<long>(blockDim.x) + threadIdx.x; idx < total; idx += stride) {
+    const int b = static_cast<int>(idx % blocks);
+    const long rest = idx / blocks;
+    const int head = static_cast<int>(rest % heads_total);
+    const long token = rest / heads_total;
+    const bool is_q = head < n_heads, is_v = head >= n_heads + n_kv_heads;
+    if (!is_q && !write_kv) continue;
+    T* src = qkv + (token * heads_total + head) * head_dim + 16 * b;
+    float lo[8], hi[8];
+    if constexpr (sizeof(T) == 2) {
+      const uint4 l = *reinterpret_cast<const uint4*>(src), h = *reinterpret_cast<const uint4*>(src + 8);
+      const uint32_t lw[4] = {l.x, l.y, l.z, l.w}, hw[4] = {h.x, h.y, h.z, h.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        lo[2 * e] = __uint_as_float(lw[e] << 16);
+        lo[2 * e + 1] = __uint_as_float(lw[e] & 0xffff0000u);
+        hi[2 * e] = __uint_as_float(hw[e] << 16);
+        hi[2 * e + 1] = __uint_as_float(hw[e] & 0xffff0000u);
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        lo[e] = to_float(src[e]);
+        hi[e] = to_float(src[8 + e]);
+      }
+    }
+    if (rotate && !is_v) {
+      const float2* cs = table + token * (head_dim / 2) + 8 * b;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float2 a = cs[e];
+        const float l0 = lo[e], h0 = hi[e];
+        lo[e] = l0 * a.x - h0 * a.y;
+        hi[e] = h0 * a.x + l0 * a.y;
+      }
+    }
+    if (is_v) {   // values are kept transposed: [page][kv head][dim][token]
+      const int slot = slot_map[token];
+      const long page = slot / page_tokens, off = slot % page_tokens;
+      T* dst = v_cache + ((page * n_kv_heads + (head - n_heads - n_kv_heads)) * head_dim + 16 * b) * page_tokens + off;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        dst[static_cast<long>(e) * page_tokens] = from_float<T>(lo[e]);
+        dst[static_cast<long>(8 + e) * page_tokens] = from_float<T>(hi[e]);
+      }
+      continue;
+    }
+    T* dst = src;
+    if (!is_q) {   // keys: [page][kv head][token][dim]
+      const int slot = slot_map[token];
+      const long page = slot / page_tokens, off = slot % page_tokens;
+      dst = k_cache + ((page * n_kv_heads + (head - n_heads)) * page_tokens + off) * head_dim + 16 * b;
+    }
+    if constexpr (sizeof(T) == 2) {
+      uint32_t lw[4], hw[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        lw[e] = static_cast<uint32_t>(bf16_bits_from_float(lo[2 * e])) | (static_cast<uint32_t>(bf16_bits_from_float(lo[2 * e + 1])) << 16);
+        hw[e] = static_cast<uint32_t>(bf16_bits_from_float(hi[2 * e])) | (static_cast<uint32_t>(bf16_bits_from_float(hi[2 * e + 1])) << 16);
+      }
+      *reinterpret_cast<uint4*>(dst) = make_uint4(lw[0], lw[1], lw[2], lw[3]);
+      *reinterpret_cast<uint4*>(dst + 8) = make_uint4(hw[0], hw[1], hw[2], hw[3]);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        dst[e] = from_float<T>(lo[e]);
+        dst[8 + e] = from_float<T>(hi[e]);
+      }
+    }
+  }
+}
+
 // ---- argmax ----------------------------------------------------------------
 // Two stages so that a few rows still use many CUs: every block takes one slice of one row and
 // writes its best (value, index); one wave per row then picks among the slices.  Equal values
@@ -346,6 +444,44 @@ extern "C" int bc4g_rope_kv_write(void* qkv, int dtype, const int32_t* positions
     return fail("rope_kv_write: unknown dtype %d", dtype);
   }
   return check_launch("rope_kv_write");
+}
+
+extern "C" int bc4g_rope_table(const int32_t* positions, float* table, int n_tokens, int rotary_dim, float theta,
+                               void* stream) {
+  BC4G_REQUIRE(n_tokens >= 0 && rotary_dim > 0 && rotary_dim % 2 == 0 && theta > 0.f && positions && table,
+               "rope_table: bad arguments (T=%d, rotary_dim=%d)", n_tokens, rotary_dim);
+  if (n_tokens == 0) return 0;
+  const long total = static_cast<long>(n_tokens) * (rotary_dim / 2);
+  rope_table_kernel<<<grid_for(total), kBlock, 0, static_cast<hipStream_t>(stream)>>>(
+      positions, reinterpret_cast<float2*>(table), total, rotary_dim / 2, theta);
+  return check_launch("rope_table");
+}
+
+extern "C" int bc4g_rope_kv_write_blocks(void* qkv, int dtype, const float* table, const int32_t* slot_map,
+                                         void* k_cache, void* v_cache, int n_tokens, int n_heads, int n_kv_heads,
+                                         int head_dim, int rotate, int page_tokens, int write_kv, void* stream) {
+  BC4G_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads > 0, "rope_kv_write_blocks: bad sizes T=%d heads=%d/%d",
+               n_tokens, n_heads, n_kv_heads);
+  BC4G_REQUIRE(head_dim > 0 && head_dim % 16 == 0, "rope_kv_write_blocks: head_dim %d must be a multiple of 16", head_dim);
+  BC4G_REQUIRE(!write_kv || (page_tokens > 0 && k_cache && v_cache && slot_map),
+               "rope_kv_write_blocks: cache write asked for without a cache");
+  BC4G_REQUIRE(!rotate || table, "rope_kv_write_blocks: rotation needs the table of angles");
+  if (n_tokens == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const long total = static_cast<long>(n_tokens) * (n_heads + 2 * n_kv_heads) * (head_dim / 16);
+  const float2* tab = reinterpret_cast<const float2*>(table);
+  if (dtype == kF32) {
+    rope_kv_write_blocks_kernel<float><<<grid_for(total), kBlock, 0, s>>>(
+        static_cast<float*>(qkv), tab, slot_map, static_cast<float*>(k_cache), static_cast<float*>(v_cache), total,
+        n_heads, n_kv_heads, head_dim, rotate, page_tokens, write_kv);
+  } else if (dtype == kBF16) {
+    rope_kv_write_blocks_kernel<bf16_t><<<grid_for(total), kBlock, 0, s>>>(
+        static_cast<bf16_t*>(qkv), tab, slot_map, static_cast<bf16_t*>(k_cache), static_cast<bf16_t*>(v_cache), total,
+        n_heads, n_kv_heads, head_dim, rotate, page_tokens, write_kv);
+  } else {
+    return fail("rope_kv_write_blocks: unknown dtype %d", dtype);
+  }
+  return check_launch("rope_kv_write_blocks");
 }
 
 extern "C" int bc4g_argmax(const float* logits, int32_t* out, float* part_v, int32_t* part_i, int n_rows, int vocab,

@@ -19,6 +19,8 @@ _SIGNATURES = {
     "bc4g_rmsnorm": [_P, _P, _P, _I, _P, _I, _I, _I, _F, _P],
     "bc4g_gemm_generic": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _P],
     "bc4g_swiglu": [_P, _P, _I, _I, _I, _I, _P],
+    "bc4g_rope_table": [_P, _P, _I, _I, _F, _P],
+    "bc4g_rope_kv_write_blocks": [_P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
     "bc4g_rope_kv_write": [_P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _P],
     "bc4g_attention_generic": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _P],
     "bc4g_argmax": [_P, _P, _P, _P, _I, _I, _P],

@@ -154,6 +154,41 @@ def rope_kv_write(qkv: torch.Tensor, positions: Optional[torch.Tensor], slot_map
                  page_tokens, num_pages, 1 if write_kv else 0, 1 if block_pairs else 0, _stream())
 
 
+def rope_table(positions: torch.Tensor, rotary_dim: int, theta: float) -> torch.Tensor:
+    """(cos, sin) of every row's angles, float32 [T, rotary_dim / 2, 2]: computed once a step, read
+    by every layer's rope_kv_write_blocks."""
+    _dev("rope_table", positions)
+    t = positions.shape[0]
+    _i32("rope_table", "positions", positions, t)
+    table = torch.empty((t, rotary_dim // 2, 2), dtype=torch.float32, device=positions.device)
+    library.call("bc4g_rope_table", _ptr(positions), _ptr(table), t, int(rotary_dim), float(theta), _stream())
+    return table
+
+
+def rope_kv_write_blocks(qkv: torch.Tensor, table: Optional[torch.Tensor], slot_map: Optional[torch.Tensor],
+                         k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor], n_heads: int,
+                         n_kv_heads: int, head_dim: int, write_kv: bool = True) -> None:
+    """rope_kv_write for heads in block-pair order, rotating the whole head by a table of angles
+    (None: no rotation), 16 elements a thread."""
+    _dev("rope_kv_write_blocks", qkv, table, slot_map, k_cache, v_cache)
+    t = qkv.shape[0]
+    width = (n_heads + 2 * n_kv_heads) * head_dim
+    if qkv.dim() != 2 or qkv.shape[1] != width:
+        raise KernelError(f"rope_kv_write_blocks: qkv must be [T, {width}], got {tuple(qkv.shape)}")
+    if table is not None and (table.dtype != torch.float32 or tuple(table.shape) != (t, head_dim // 2, 2)
+                              or not table.is_contiguous()):
+        raise KernelError(f"rope_kv_write_blocks: the table must be float32 [{t}, {head_dim // 2}, 2], "
+                          f"got {table.dtype} {tuple(table.shape)}")
+    page_tokens = 0
+    if write_kv:
+        _check_cache("rope_kv_write_blocks", k_cache, v_cache, n_kv_heads, head_dim, qkv.dtype)
+        _i32("rope_kv_write_blocks", "slot_map", slot_map, t)
+        page_tokens = k_cache.shape[2]
+    library.call("bc4g_rope_kv_write_blocks", _ptr(qkv), _code(qkv, "rope_kv_write_blocks"), _ptr(table), _ptr(slot_map),
+                 _ptr(k_cache), _ptr(v_cache), t, n_heads, n_kv_heads, head_dim, 0 if table is None else 1,
+                 page_tokens, 1 if write_kv else 0, _stream())
+
+
 def _check_queries(what: str, q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int) -> None:
     """Queries come as the rows of the fused q|k|v product or as a buffer of queries alone."""
     widths = ((n_heads + 2 * n_kv_heads) * head_dim, n_heads * head_dim)

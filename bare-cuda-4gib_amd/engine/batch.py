@@ -37,10 +37,18 @@ class StepContext:
     cache_views: Dict[Hashable, Any] = dataclasses.field(default_factory=dict)
     # tokens per attention tile -> (device int32 [S+1] first tile of each request, number of tiles)
     tiles: Dict[int, Any] = dataclasses.field(default_factory=dict)
+    made: Dict[Any, Any] = dataclasses.field(default_factory=dict)      # see shared()
     fixed_attention_splits: int = 0      # non-zero: the key split count is fixed (a captured step)
 
     def cache(self, stream: Optional[Hashable]):
         return None if stream is None else self.cache_views.get(stream)
+
+    def shared(self, key, make):
+        """What several layers of one step share (a table of rotation angles, say): made by the
+        first that asks, kept until the step ends."""
+        if key not in self.made:
+            self.made[key] = make()
+        return self.made[key]
 
     def attention_tiles(self, tokens_per_tile: int):
         """Each request's rows cut into tiles of ``tokens_per_tile`` tokens: (first tile of each

@@ -223,6 +223,7 @@ class Executor:
         ctx = self._context_from(dev, layout, group_layout, dict(host, max_kv=bucket), fixed_splits=splits)
         self.model.forward(ctx)                      # once outside the graph: first-use work happens here
         torch.cuda.synchronize()
+        ctx.made.clear()                             # what layers share is made again inside the graph
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             logits = self.model.forward(ctx)

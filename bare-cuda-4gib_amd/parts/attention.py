@@ -98,8 +98,17 @@ class CausalAttention(Part):
             q = linear(h, self.w_qkv, out_dtype=self.act_dtype)
             if fused is None:
                 self.position.apply(q, ctx, self.num_heads, self.num_kv_heads, self.head_dim)
-            ops.rope_kv_write(q, ctx.positions, slot_map, k_cache, v_cache, self.num_heads, self.num_kv_heads,
-                              self.head_dim, rotary_dim, theta, write_kv=writes, block_pairs=self.block_pairs)
+            if self.block_pairs and fused is not None:
+                # the angles are the same in every layer: a table made once a step
+                table = None
+                if rotary_dim > 0:
+                    table = ctx.shared(("rope_table", rotary_dim, theta),
+                                       lambda: ops.rope_table(ctx.positions, rotary_dim, theta))
+                ops.rope_kv_write_blocks(q, table, slot_map, k_cache, v_cache, self.num_heads, self.num_kv_heads,
+                                         self.head_dim, write_kv=writes)
+            else:
+                ops.rope_kv_write(q, ctx.positions, slot_map, k_cache, v_cache, self.num_heads, self.num_kv_heads,
+                                  self.head_dim, rotary_dim, theta, write_kv=writes, block_pairs=self.block_pairs)
         o = ops.attention(q, cache.k, cache.v, ctx.block_tables[cache.group], ctx,
                           self.num_heads, self.num_kv_heads, self.head_dim, self.window, self.scale)
         linear(o, self.w_o, accumulate_into=residual)

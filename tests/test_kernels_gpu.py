@@ -164,6 +164,52 @@ def test_swiglu(ops, dt):
     close(ops.swiglu(gu.to(DEV)), want, 1e-5 if dt == torch.float32 else 8e-3, 1e-6 if dt == torch.float32 else 1e-3)
 
 
+def block_pair_order(d):
+    """Dimensions of a head in blocks of 16: eight dimensions, then their rotation partners."""
+    return [8 * b + t + (d // 2 if half else 0) for b in range(d // 16) for half in (0, 1) for t in range(8)]
+
+
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("d,rotate", [(16, True), (48, True), (64, True), (32, False)])
+def test_rope_kv_write_blocks_with_table(ops, dt, d, rotate):
+    """The block-order kernel with a table of angles: rows in block order in, rotated pairs out,
+    compared in the natural order with the plain rotation."""
+    nh, nkv, page, pages = 3, 2, 16, 5
+    positions = [0, 1, 2, 5, 8, 13, 21, 34, 3]
+    t = len(positions)
+    natural = rnd(t, nh + 2 * nkv, d, seed=60)
+    order = block_pair_order(d)
+    qkv = natural[:, :, order].reshape(t, -1).to(dt)
+    slots = [3 * page + i for i in range(4)] + [0, page + 15, 4 * page + 7, 2 * page + 1, 2 * page + 2]
+    kc = torch.full((pages, nkv, page, d), -7.5, dtype=dt, device=DEV)
+    vc = torch.full((pages, nkv, d, page), -7.5, dtype=dt, device=DEV)
+    pos_dev = torch.tensor(positions, dtype=torch.int32, device=DEV)
+    table = ops.rope_table(pos_dev, d, 10000.0) if rotate else None
+    if rotate:                                                           # the table itself: cos and sin of the angles
+        ang = torch.tensor(positions, dtype=torch.float64)[:, None] / 10000.0 ** (torch.arange(d // 2, dtype=torch.float64) * 2 / d)
+        close(table[..., 0], torch.cos(ang), 0, 5e-6, "cos")             # (float angles: 34 * 2^-24 off at most)
+        close(table[..., 1], torch.sin(ang), 0, 5e-6, "sin")
+    buf = qkv.clone().to(DEV)
+    ops.rope_kv_write_blocks(buf, table, torch.tensor(slots, dtype=torch.int32, device=DEV), kc, vc, nh, nkv, d)
+    x = qkv.double().view(t, nh + 2 * nkv, d)                            # (rounded as the kernel's input is)
+    inverse = torch.argsort(torch.tensor(order))
+    x_nat = x[:, :, inverse]
+    pos = torch.tensor(positions)
+    q_want = P.rope(x_nat[:, :nh], pos, 10000.0, d) if rotate else x_nat[:, :nh]
+    k_want = P.rope(x_nat[:, nh:nh + nkv], pos, 10000.0, d) if rotate else x_nat[:, nh:nh + nkv]
+    tol = dict(rtol=1e-5, atol=1e-5) if dt == torch.float32 else dict(rtol=8e-3, atol=8e-3)
+    out = buf.cpu().double().view(t, nh + 2 * nkv, d)
+    close(out[:, :nh][:, :, inverse], q_want, what="q", **tol)
+    kc_c, vc_c = kc.cpu().double(), vc.cpu().double()
+    touched = torch.zeros(pages, page, dtype=torch.bool)
+    for i, sl in enumerate(slots):
+        pg, off = divmod(sl, page)
+        close(kc_c[pg, :, off, :][:, inverse], k_want[i], what=f"k row {i}", **tol)
+        close(vc_c[pg, :, :, off][:, inverse], x_nat[i, nh + nkv:], what=f"v row {i}", **tol)
+        touched[pg, off] = True
+    assert bool((kc_c.permute(0, 2, 1, 3)[~touched] == -7.5).all()) and bool((vc_c.permute(0, 3, 1, 2)[~touched] == -7.5).all())
+
+
 @pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("rotary_dim", [16, 8, 0])
 def test_rope_kv_write(ops, dt, rotary_dim):
