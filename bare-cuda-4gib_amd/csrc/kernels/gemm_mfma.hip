@@ -222,16 +222,20 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_kernel(const bf16_t* __restr
   store_tile<EPI, 256>(tile_out, out, m, n, m0, n0, tid);
 }
 
-// The same product with the work split between waves: four waves only move operands (memory ->
-// registers -> LDS), four only multiply.  A wave issues its instructions in order, so a wave that
-// does both stands still at a full memory queue with its MFMAs behind it; here the multiplying
-// waves never wait for the memory pipeline, only for data.  LDS holds three k-steps: while step t
-// is multiplied, step t + 2 is written, and the three steps after that are in flight in the moving
-// waves' registers.
-constexpr int kStages = 3, kAhead = 3;
+// The same product with the work split between waves: four waves only multiply, eight only move
+// operands (memory -> registers -> LDS).  A wave issues its instructions in order, so a wave that
+// does everything stands still at a full memory queue with its MFMAs behind it; here the
+// multiplying waves wait for data only.  The moving waves form two groups that take the k-steps in
+// turn: in a round one group writes its step into LDS while the other asks memory for a later one
+// -- writing a step takes about as long as asking for one (measured: 900 and 1,300 clocks for a
+// 48 KB step), and one group doing both in a row was what a round waited for.  LDS holds three
+// k-steps: while step t is multiplied, step t + 2 is written; each group has two more in flight
+// in registers.
+constexpr int kStages = 3, kSets = 2;
+constexpr int kSplitThreads = 768;
 
 template <int EPI>
-__global__ __launch_bounds__(512) void gemm_mfma_split_kernel(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
+__global__ __launch_bounds__(kSplitThreads) void gemm_mfma_split_kernel(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
                                                               void* __restrict__ out, int m, int n, int k,
                                                               int m_blocks, int n_blocks) {
   __shared__ __align__(16) unsigned char lds_raw[sizeof(Tile) * kStages];
@@ -251,8 +255,9 @@ __global__ __launch_bounds__(512) void gemm_mfma_split_kernel(const bf16_t* __re
   const int wm = (wave % 4) / 2, wn = wave % 2;   // a multiplying wave's 64 x 64 quarter
 
   if (mover) {
-    // thread u of the 256 movers takes segment u % 8 of rows u / 8 + 32 i of both operands
-    const int u = tid - 256, seg = u % 8, lrow = u / 8;
+    // thread u of a group's 256 takes segment u % 8 of rows u / 8 + 32 i of both operands
+    const int group = (wave - 4) / 4;             // owns the k-steps s with s % 2 == group
+    const int u = tid - 256 - 256 * group, seg = u % 8, lrow = u / 8;
     struct Staged {
       uint4 a[4], w[4];
     };
@@ -283,25 +288,30 @@ __global__ __launch_bounds__(512) void gemm_mfma_split_kernel(const bf16_t* __re
         *reinterpret_cast<uint4*>(&tiles[buf].w[lrow + 32 * i][seg * 8]) = r.w[i];
       }
     };
-    // step s travels in register set s % kAhead and lands in LDS buffer s % kStages
-    Staged r[kAhead];
-    load_step(r[0], 0);
-    if (nk > 1) load_step(r[1], 1);
-    store_step(r[0], 0);
-    if (nk > 1) store_step(r[1], 1);
-    // (sets are numbered from step 2 on: step s >= 2 in set (s - 2) % kAhead)
+    // Step s lands in LDS buffer s % kStages; steps 0 and 1 before the first round, step t + 2 in
+    // round t.  A group's step s >= 2 travels in its register set (s / 2 - 1) % kSets.  In round t
+    // the group of step t + 2 (t % 2) stores it; the other group asks for step t + 1 + 2 kSets into
+    // the set its step t + 1 left the round before.
+    Staged r[kSets];
+    if (group < nk) {
+      load_step(r[0], group);
+      store_step(r[0], group);
+    }
 #pragma unroll
-    for (int s = 0; s < kAhead; ++s)
-      if (2 + s < nk) load_step(r[s], 2 + s);
+    for (int i = 0; i < kSets; ++i)
+      if (2 + group + 2 * i < nk) load_step(r[i], 2 + group + 2 * i);
     lds_barrier();
-    constexpr int kUnroll = 3;   // lcm(kStages, kAhead)
+    constexpr int kUnroll = 12;   // lcm(kStages, 2 groups x kSets)
     for (int kt = 0; kt < nk; kt += kUnroll) {
 #pragma unroll
       for (int j = 0; j < kUnroll; ++j) {
         const int t = kt + j;
         if (t >= nk) break;
-        if (t + 2 < nk) store_step(r[j % kAhead], (j + 2) % kStages);
-        if (t + 2 + kAhead < nk) load_step(r[j % kAhead], t + 2 + kAhead);
+        if (group == j % 2) {
+          if (t + 2 < nk) store_step(r[(j / 2) % kSets], (j + 2) % kStages);
+        } else if (t >= 1) {
+          if (t + 1 + 2 * kSets < nk) load_step(r[((j + 1) / 2 + kSets - 1) % kSets], t + 1 + 2 * kSets);
+        }
         lds_barrier();
       }
     }
@@ -339,7 +349,7 @@ __global__ __launch_bounds__(512) void gemm_mfma_split_kernel(const bf16_t* __re
     }
   }
 
-  // The tile goes out through LDS (as float [128][128 + 4]): all 512 threads store it, four
+  // The tile goes out through LDS (as float [128][128 + 4]): all threads store it, four
   // neighbouring columns of a row at once.
   constexpr int kOutStride = kBN + 4;
   float* tile_out = reinterpret_cast<float*>(lds_raw);
@@ -354,7 +364,7 @@ __global__ __launch_bounds__(512) void gemm_mfma_split_kernel(const bf16_t* __re
               acc[i][j][r];
   }
   lds_barrier();
-  store_tile<EPI, 512>(tile_out, out, m, n, m0, n0, tid);
+  store_tile<EPI, kSplitThreads>(tile_out, out, m, n, m0, n0, tid);
 }
 
 int compute_units() {
@@ -374,10 +384,10 @@ void launch_tiled(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, i
                   hipStream_t s) {
   dim3 grid(static_cast<unsigned>(m_blocks * n_blocks)), block(256);
   // With at most one tile a CU nothing else runs beside a workgroup: then the split form, whose
-  // moving and multiplying waves overlap, is the faster one (measured: 31 against 35 us for
+  // moving and multiplying waves overlap, is the faster one (measured: 29 against 35 us for
   // 2048 x 2048 x 2048); with more tiles two workgroups of the plain form share a CU and do better.
   if (m_blocks * n_blocks <= compute_units()) {
-    gemm_mfma_split_kernel<EPI><<<grid, dim3(512), 0, s>>>(ap, wp, out, m, n, k, m_blocks, n_blocks);
+    gemm_mfma_split_kernel<EPI><<<grid, dim3(kSplitThreads), 0, s>>>(ap, wp, out, m, n, k, m_blocks, n_blocks);
     return;
   }
   gemm_mfma_kernel<EPI, 2><<<grid, block, 0, s>>>(ap, wp, out, m, n, k, m_blocks, n_blocks);
