@@ -4,6 +4,7 @@ here without a change to the framework's files, with
   - attention with a window (its cache group gives pages back as the window moves on),
   - a layer that runs twice (own cache each time) and a layer that reads another layer's cache,
   - attention without any position encoding,
+  - (a second toy) a feed-forward with routing and a position encoding of another pairing,
 is built, loaded from a random model folder, and stepped whole, in portions, and mixed with few
 pages -- against a plain implementation of the same toy model written with the plain functions.
 Each part of a layer is also run alone against its plain function."""
@@ -263,3 +264,163 @@ def test_parts_alone(dtype):
     got = head.forward(hrows.to(DEV).contiguous())
     assert got.dtype == torch.float32
     assert torch.allclose(got.cpu().double(), hrows.double() @ table.double().T, **tol)
+
+
+# --- a second toy: a feed-forward with routing, and another position encoding ---------------
+# Both are defined here and never leave the tests.  The feed-forward picks, per token, the
+# likeliest of three small experts (router logits in float32) and scales the expert's output by
+# the router's softmax weight; the position encoding rotates neighbouring pairs (2i, 2i + 1) --
+# a pairing the framework's fused kernels do not have, so it goes through the ``apply`` interface.
+# Routing is a discontinuous choice, so this model is stepped in float32 only, and the plain
+# implementation asserts that no router decision was a near-tie.
+
+E_EXPERTS, E_INTER = 3, 40
+
+
+def register_routed_toy():
+    from bare_cuda_4gib_amd.config import Architecture, ModelConfig, field_from_json, register_architecture
+    from bare_cuda_4gib_amd.config.registry import unregister_architecture
+    from bare_cuda_4gib_amd.engine.spec import LayerSpec, ModelSpec, PartSpec, ScheduleEntry
+    from bare_cuda_4gib_amd.parts import Part, register_part
+    from bare_cuda_4gib_amd.weights import WeightSpec
+
+    class TopOneExperts(Part):
+        category = "feedforward"
+
+        def __init__(self, hidden_size, intermediate_size, experts):
+            self.h, self.i, self.e = hidden_size, intermediate_size, experts
+
+        def weight_specs(self):
+            specs = {"router.weight": WeightSpec((self.e, self.h))}
+            for e in range(self.e):
+                specs[f"experts.{e}.w1.weight"] = WeightSpec((self.i, self.h))
+                specs[f"experts.{e}.w2.weight"] = WeightSpec((self.h, self.i))
+            return specs
+
+        def bind(self, tensors, rt):
+            self.router = tensors["router.weight"].float()
+            self.w1 = [tensors[f"experts.{e}.w1.weight"].float() for e in range(self.e)]
+            self.w2 = [tensors[f"experts.{e}.w2.weight"].float() for e in range(self.e)]
+
+        def forward(self, h, ctx, residual):
+            h = h.float()
+            logits = h @ self.router.T
+            weight, choice = torch.softmax(logits, dim=-1).max(dim=-1)
+            for e in range(self.e):
+                rows = (choice == e).nonzero().flatten()
+                if rows.numel():
+                    out = torch.relu(h[rows] @ self.w1[e].T) @ self.w2[e].T
+                    residual[rows] += out * weight[rows, None]
+
+    class NeighbourRotary(Part):
+        category = "position"
+
+        def __init__(self, theta):
+            self.theta = float(theta)
+
+        def fused(self):
+            return None                                   # no kernel of the framework's rotates this pairing
+
+        def apply(self, qkv, ctx, n_heads, n_kv_heads, head_dim):
+            t = qkv.shape[0]
+            x = qkv.view(t, n_heads + 2 * n_kv_heads, head_dim)[:, :n_heads + n_kv_heads].float()
+            inv = self.theta ** (-torch.arange(0, head_dim, 2, device=qkv.device, dtype=torch.float32) / head_dim)
+            ang = ctx.positions.float()[:, None] * inv
+            cos, sin = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+            even, odd = x[..., 0::2], x[..., 1::2]
+            rot = torch.stack([even * cos - odd * sin, odd * cos + even * sin], dim=-1).flatten(-2)
+            qkv.view(t, n_heads + 2 * n_kv_heads, head_dim)[:, :n_heads + n_kv_heads] = rot.to(qkv.dtype)
+
+    @dataclasses.dataclass
+    class RoutedConfig(ModelConfig):
+        vocab_size: int = field_from_json("vocab_size")
+        hidden_size: int = field_from_json("hidden_size")
+        experts: int = field_from_json("experts")
+
+    def describe(cfg):
+        norm = dict(size=cfg.hidden_size, eps=1e-5)
+        def layer(i, position):
+            p = f"blocks.{i}."
+            attn = PartSpec("attention", dict(hidden_size=cfg.hidden_size, num_heads=NH, num_kv_heads=NKV, head_dim=D,
+                                              window=0, position=position), prefix=p + "attn.")
+            ffn = PartSpec("toy_top_one_experts", dict(hidden_size=cfg.hidden_size, intermediate_size=E_INTER,
+                                                       experts=cfg.experts), prefix=p + "moe.")
+            return LayerSpec("prenorm", attn, ffn, PartSpec("rmsnorm", dict(norm), prefix=p + "norm1."),
+                             PartSpec("rmsnorm", dict(norm), prefix=p + "norm2."))
+        layers = [layer(0, PartSpec("toy_neighbour_rotary", dict(theta=50.0))),
+                  layer(1, PartSpec("rotary", dict(theta=10000.0, dim=D)))]
+        return ModelSpec(vocab_size=cfg.vocab_size, hidden_size=cfg.hidden_size, max_seq_len=4096,
+                         embedding=PartSpec("embedding", dict(vocab_size=cfg.vocab_size, hidden_size=cfg.hidden_size), prefix="embed."),
+                         layers=layers, schedule=[ScheduleEntry(0, "kv0"), ScheduleEntry(1, "kv1")],
+                         final_norm=PartSpec("rmsnorm", dict(norm), prefix="final_norm."),
+                         head=PartSpec("lm_head", dict(vocab_size=cfg.vocab_size, hidden_size=cfg.hidden_size), prefix="head."))
+
+    for category, kind, cls in (("feedforward", "toy_top_one_experts", TopOneExperts),
+                                ("position", "toy_neighbour_rotary", NeighbourRotary)):
+        try:
+            register_part(category, kind, cls)
+        except Exception:
+            pass
+    unregister_architecture("ToyRoutedForTests")
+    register_architecture(Architecture("ToyRoutedForTests", "toy_routed_for_tests", RoutedConfig, describe))
+
+
+ROUTED_CONFIG = dict(architectures=["ToyRoutedForTests"], vocab_size=VOCAB, hidden_size=H, experts=E_EXPERTS)
+
+
+def plain_routed_logits(folder, ids):
+    from safetensors import safe_open
+    with safe_open(os.path.join(folder, "model.safetensors"), "pt") as f:
+        w = {n: f.get_tensor(n).double() for n in f.keys()}
+    t = len(ids)
+    pos = torch.arange(t)
+    x = w["embed.weight"][torch.tensor(ids)]
+    smallest_margin = float("inf")
+    for i in range(2):
+        p = f"blocks.{i}."
+        h = P.rmsnorm(x, w[p + "norm1.weight"], 1e-5)
+        q = (h @ w[p + "attn.q_proj.weight"].T).view(t, NH, D)
+        k = (h @ w[p + "attn.k_proj.weight"].T).view(t, NKV, D)
+        v = (h @ w[p + "attn.v_proj.weight"].T).view(t, NKV, D)
+        if i == 0:      # neighbouring pairs: the rotate-half rotation of the de-interleaved head, interleaved again
+            def rot(z):
+                split = torch.cat([z[..., 0::2], z[..., 1::2]], dim=-1)
+                r = P.rope(split, pos, 50.0)
+                return torch.stack([r[..., :D // 2], r[..., D // 2:]], dim=-1).flatten(-2)
+            q, k = rot(q), rot(k)
+        else:
+            q, k = P.rope(q, pos, 10000.0), P.rope(k, pos, 10000.0)
+        x = x + P.attention(q, k, v).reshape(t, -1) @ w[p + "attn.o_proj.weight"].T
+        h = P.rmsnorm(x, w[p + "norm2.weight"], 1e-5)
+        logits = h @ w[p + "moe.router.weight"].T
+        top2 = torch.topk(logits, 2, dim=-1).values
+        smallest_margin = min(smallest_margin, float((top2[:, 0] - top2[:, 1]).min()))
+        prob = torch.softmax(logits, dim=-1)
+        choice = logits.argmax(dim=-1)
+        out = torch.zeros_like(x)
+        for r in range(t):
+            e = int(choice[r])
+            out[r] = torch.relu(h[r] @ w[p + f"moe.experts.{e}.w1.weight"].T) @ w[p + f"moe.experts.{e}.w2.weight"].T * prob[r, e]
+        x = x + out
+    assert smallest_margin > 1e-4, "a router decision is a near-tie: pick other seeds"
+    return P.rmsnorm(x, w["final_norm.weight"], 1e-5) @ w["head.weight"].T
+
+
+def test_routed_feed_forward_and_another_position_encoding(tmp_path):
+    register_routed_toy()
+    from bare_cuda_4gib_amd.engine import Executor, load_model
+    from bare_cuda_4gib_amd.weights import write_random_model
+    folder = write_random_model(ROUTED_CONFIG, 21, str(tmp_path / "routed"), "float32", std=0.1)
+    requests = {f"r{i}": helpers.random_ids(n, VOCAB, 500 + i) for i, n in enumerate([4, 37, 90, 65])}
+    plain = {r: plain_routed_logits(folder, ids).numpy() for r, ids in requests.items()}
+    model, _ = load_model(folder, "float32")
+    page = 16
+    steps, where, peak = helpers.trace_mixed(requests, seed=4, max_live=3, page_tokens=page)
+    for label, (st, wh), pages in (("whole", helpers.trace_whole(requests), 16),
+                                   ("portions", helpers.trace_portions(requests, seed=3), 16),
+                                   ("mixed", (steps, where), peak // page)):
+        ex = Executor(model, num_pages=pages, max_requests=4, max_tokens=96, page_tokens=page, poison=True)
+        assert not ex.use_graphs                                      # the toy parts are not graph-safe
+        got = helpers.replay_in_process(ex, st)
+        helpers.compare_with_plain(got, wh, plain, label=f"routed toy {label}", rtol=2e-4, atol=2e-5)
+        assert ex.cache.pages_in_use() == 0
