@@ -42,6 +42,55 @@ __global__ void rmsnorm_kernel(const float* __restrict__ x, const int32_t* __res
   }
 }
 
+// The same for widths that are a multiple of 8 and at most 256 * 8 * CHUNKS: a thread keeps its
+// elements (CHUNKS pieces of 8) in registers between the sum and the scaling -- the row is read
+// once, in 16-byte pieces, and written in 16-byte (bfloat16) or 32-byte pieces.
+template <typename TW, typename TO, int CHUNKS>
+__global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const float* __restrict__ x, const int32_t* __restrict__ rows,
+                                                           const TW* __restrict__ w, TO* __restrict__ out, int hidden,
+                                                           float eps) {
+  __shared__ float scratch[16];
+  const size_t src_row = rows ? static_cast<size_t>(rows[blockIdx.x]) : blockIdx.x;
+  const float* xr = x + src_row * hidden;
+  TO* orow = out + static_cast<size_t>(blockIdx.x) * hidden;
+  float v[CHUNKS][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c) {
+    const int i = (c * 256 + threadIdx.x) * 8;
+    if (i < hidden) {
+      const float4 a = *reinterpret_cast<const float4*>(xr + i), b = *reinterpret_cast<const float4*>(xr + i + 4);
+      v[c][0] = a.x; v[c][1] = a.y; v[c][2] = a.z; v[c][3] = a.w;
+      v[c][4] = b.x; v[c][5] = b.y; v[c][6] = b.z; v[c][7] = b.w;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[c][e] = 0.f;
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss += v[c][e] * v[c][e];
+  }
+  const float mean_sq = block_sum(ss, scratch) / static_cast<float>(hidden);
+  const float scale = 1.0f / sqrtf(mean_sq + eps);
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c) {
+    const int i = (c * 256 + threadIdx.x) * 8;
+    if (i >= hidden) continue;
+    float y[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) y[e] = v[c][e] * scale * to_float(w[i + e]);
+    if constexpr (sizeof(TO) == 2) {
+      uint32_t pk[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        pk[e] = static_cast<uint32_t>(bf16_bits_from_float(y[2 * e])) | (static_cast<uint32_t>(bf16_bits_from_float(y[2 * e + 1])) << 16);
+      *reinterpret_cast<uint4*>(orow + i) = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) orow[i + e] = from_float<TO>(y[e]);
+    }
+  }
+}
+
 // ---- SwiGLU ----------------------------------------------------------------
 // interleaved 0: a row of gu holds the gate values, then the up values.  1: blocks of 16 -- eight
 // gate values followed by the eight up values of the same outputs (the layout the fused
@@ -382,9 +431,18 @@ extern "C" int bc4g_rmsnorm(const float* x, const int32_t* rows, const void* w, 
   BC4G_REQUIRE(n_rows >= 0 && hidden > 0, "rmsnorm: bad sizes rows=%d H=%d", n_rows, hidden);
   if (n_rows == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
-#define BC4G_RMS(TW, TO)                                                                         \
-  rmsnorm_kernel<TW, TO><<<n_rows, kBlock, 0, s>>>(x, rows, static_cast<const TW*>(w),           \
-                                                   static_cast<TO*>(out), hidden, eps)
+  // widths that are a multiple of 8, up to 8,192: the row stays in registers
+  const int chunks = hidden % 8 == 0 ? (hidden + 2047) / 2048 : 0;
+#define BC4G_RMS(TW, TO)                                                                                    \
+  do {                                                                                                      \
+    const TW* wp = static_cast<const TW*>(w);                                                               \
+    TO* op = static_cast<TO*>(out);                                                                         \
+    if (chunks == 1) rmsnorm_rows_kernel<TW, TO, 1><<<n_rows, 256, 0, s>>>(x, rows, wp, op, hidden, eps);      \
+    else if (chunks == 2) rmsnorm_rows_kernel<TW, TO, 2><<<n_rows, 256, 0, s>>>(x, rows, wp, op, hidden, eps); \
+    else if (chunks == 3 || chunks == 4)                                                                    \
+      rmsnorm_rows_kernel<TW, TO, 4><<<n_rows, 256, 0, s>>>(x, rows, wp, op, hidden, eps);                   \
+    else rmsnorm_kernel<TW, TO><<<n_rows, kBlock, 0, s>>>(x, rows, wp, op, hidden, eps);                     \
+  } while (0)
   if (w_dtype == kF32 && out_dtype == kF32) BC4G_RMS(float, float);
   else if (w_dtype == kF32 && out_dtype == kBF16) BC4G_RMS(float, bf16_t);
   else if (w_dtype == kBF16 && out_dtype == kF32) BC4G_RMS(bf16_t, float);
