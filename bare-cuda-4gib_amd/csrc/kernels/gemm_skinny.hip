@@ -110,6 +110,19 @@ __global__ __launch_bounds__(kThreads, XMODE != kPlain ? 6 : 4) void gemm_skinny
     }
   }
 
+  // The float sums that the product is added to (the residual stream) are asked for now, not
+  // after the weights: item j of a thread is output (threadIdx.x + j * kThreads) of the block.
+  constexpr int kAccItems = (MT * 256 + kThreads - 1) / kThreads;
+  float prev[kAccItems];
+  if constexpr (EPI == kAccumF32) {
+#pragma unroll
+    for (int j = 0; j < kAccItems; ++j) {
+      const int idx = threadIdx.x + j * kThreads;
+      const int row = idx / 16, gn = n0 + idx % 16;
+      prev[j] = (idx < MT * 256 && row < m && gn < a.n) ? static_cast<const float*>(a.out)[static_cast<long>(row) * a.n + gn] : 0.f;
+    }
+  }
+
   struct Batch {
     uint4 w[kSets][U];
     uint4 x[kNormed ? 1 : MT][kNormed ? 1 : U];
@@ -234,7 +247,11 @@ __global__ __launch_bounds__(kThreads, XMODE != kPlain ? 6 : 4) void gemm_skinny
 
   constexpr bool kPaired = EPI == kSwigluBf16 || EPI == kRopeKvBf16;   // columns nl and nl + 8 belong together
   constexpr int kCols = kPaired ? 8 : 16;
-  for (int idx = threadIdx.x; idx < MT * 16 * kCols; idx += kThreads) {
+  constexpr int kItems = (MT * 16 * kCols + kThreads - 1) / kThreads;
+#pragma unroll
+  for (int j = 0; j < kItems; ++j) {
+    const int idx = threadIdx.x + j * kThreads;
+    if (idx >= MT * 16 * kCols) continue;
     const int nl = idx % kCols, row = idx / kCols;
     const int gn = n0 + nl;
     if (row >= m || gn >= a.n) continue;
@@ -255,7 +272,7 @@ __global__ __launch_bounds__(kThreads, XMODE != kPlain ? 6 : 4) void gemm_skinny
     } else if constexpr (EPI == kStoreF32) {
       static_cast<float*>(a.out)[static_cast<long>(row) * a.n + gn] = sum;
     } else if constexpr (EPI == kAccumF32) {
-      static_cast<float*>(a.out)[static_cast<long>(row) * a.n + gn] += sum;
+      static_cast<float*>(a.out)[static_cast<long>(row) * a.n + gn] = prev[j] + sum;
     } else if constexpr (EPI == kSwigluBf16) {
       // block b = n0 / 16 holds gates and ups of outputs 8b .. 8b + 7
       const long o = static_cast<long>(row) * (a.n / 2) + (n0 / 2 + nl);
