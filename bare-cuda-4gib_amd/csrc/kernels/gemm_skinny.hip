@@ -123,6 +123,32 @@ __global__ __launch_bounds__(kThreads, XMODE != kPlain ? 6 : 4) void gemm_skinny
     }
   }
 
+  // The rotation a thread will apply in the epilogue (its output's angle: position and pair are
+  // known now) and the place in the cache it will write to are worked out while the weights are
+  // on their way: item j of a thread is pair (threadIdx.x + j * kThreads) % 8 of row ... / 8.
+  constexpr int kRopeItems = (MT * 128 + kThreads - 1) / kThreads;
+  float rope_cs[kRopeItems], rope_sn[kRopeItems];
+  int rope_slot[kRopeItems];
+  if constexpr (EPI == kRopeKvBf16) {
+    const RopeKvArgs& r = a.rope;
+    const int head = n0 / r.head_dim;
+    const bool is_v = head >= r.n_heads + r.n_kv_heads;
+#pragma unroll
+    for (int j = 0; j < kRopeItems; ++j) {
+      const int idx = threadIdx.x + j * kThreads;
+      const int row = idx / 8, nl = idx % 8;
+      const bool live = idx < MT * 128 && row < m;
+      rope_cs[j] = 1.f;
+      rope_sn[j] = 0.f;
+      if (live && r.rotary_dim > 0 && !is_v) {
+        const int pair = (n0 % r.head_dim) / 2 + nl;            // 8 * block + nl
+        const float inv_freq = 1.0f / powf(r.theta, (2.0f * static_cast<float>(pair)) / static_cast<float>(r.head_dim));
+        sincosf(static_cast<float>(r.positions[row]) * inv_freq, &rope_sn[j], &rope_cs[j]);
+      }
+      rope_slot[j] = (live && head >= r.n_heads && r.write_kv) ? r.slot_map[row] : 0;
+    }
+  }
+
   struct Batch {
     uint4 w[kSets][U];
     uint4 x[kNormed ? 1 : MT][kNormed ? 1 : U];
@@ -281,15 +307,10 @@ __global__ __launch_bounds__(kThreads, XMODE != kPlain ? 6 : 4) void gemm_skinny
       const RopeKvArgs& r = a.rope;
       const int d = r.head_dim;
       const int head = n0 / d, in_head = n0 % d + nl;         // the pair lies at in_head and in_head + 8
-      const int pair = (n0 % d) / 2 + nl;                     // 8 * block + nl
       float lo = sum, hi = partner;
       const bool is_v = head >= r.n_heads + r.n_kv_heads;
       if (r.rotary_dim > 0 && !is_v) {
-        const float inv_freq = 1.0f / powf(r.theta, (2.0f * static_cast<float>(pair)) / static_cast<float>(d));
-        const float angle = static_cast<float>(r.positions[row]) * inv_freq;
-        float sn, cs;
-        sincosf(angle, &sn, &cs);
-        const float l0 = lo, h0 = hi;
+        const float cs = rope_cs[j], sn = rope_sn[j], l0 = lo, h0 = hi;
         lo = l0 * cs - h0 * sn;
         hi = h0 * cs + l0 * sn;
       }
@@ -299,7 +320,7 @@ __global__ __launch_bounds__(kThreads, XMODE != kPlain ? 6 : 4) void gemm_skinny
         q[8] = from_float<bf16_t>(hi);
       } else if (r.write_kv) {
         const int kvh = is_v ? head - r.n_heads - r.n_kv_heads : head - r.n_heads;
-        const int slot = r.slot_map[row];
+        const int slot = rope_slot[j];
         const long page = slot / r.page_tokens, off = slot % r.page_tokens;
         if (is_v) {
           bf16_t* dst = r.v_cache + ((page * r.n_kv_heads + kvh) * d + in_head) * r.page_tokens + off;
