@@ -11,7 +11,12 @@
 // and are added in wave order, so a result does not depend on the number of rows or on timing.
 //
 // What comes in (XMODE):
-//   plain    x is bfloat16 [m, k], read from cache as the B operand
+//   plain    x is bfloat16 [m, k].  The B operand's own pattern (a lane group reads 16 bytes of
+//            each of 16 rows) keeps the texture path busy four times as long as a load of whole
+//            cache lines, and with 64 rows x is four times the weights' traffic: so x comes in row
+//            by row (eight or sixteen lanes read a row's part of the batch) and is turned into
+//            operand order through a buffer in LDS that belongs to the wave -- no barrier, and the
+//            next batch's loads are in flight meanwhile.
 //   normed   x is the float residual stream (rows taken through `rows` if given) and RMSNorm is
 //            fused (up to 16 rows): while the first weights are already on their way, the
 //            workgroup writes bf16(x * g) into LDS and sums x^2 per row; the MFMAs read their B
@@ -69,8 +74,16 @@ template <int MT, int EPI, int XMODE, int U>
 __global__ __launch_bounds__(kThreads, XMODE != kPlain ? 6 : 4) void gemm_skinny_kernel(const SkinnyArgs a) {
   constexpr int kSets = 1;
   constexpr bool kNormed = XMODE != kPlain;
+  constexpr bool kTurned = !kNormed;                      // x reaches operand order through LDS
+  constexpr int kPieces = 4 * U;                       // 16-byte pieces of a row in one batch of k-steps
   static_assert(!kNormed || MT == 1, "the fused norm handles one tile of rows");
-  __shared__ float red[kWaves][kSets][MT][16][kRedPad];
+  static_assert(!kTurned || 64 % kPieces == 0, "a load instruction covers whole rows of a batch");
+  // The waves' partial sums, and before them (kTurned) every wave's buffer for x: the same memory.
+  typedef float Red[kSets][MT][16][kRedPad];
+  constexpr int kRedBytes = kWaves * static_cast<int>(sizeof(Red));
+  constexpr int kTurnBytes = kTurned ? kWaves * MT * 16 * kPieces * 16 : 0;
+  __shared__ __align__(16) unsigned char pool[kRedBytes > kTurnBytes ? kRedBytes : kTurnBytes];
+  Red* red = reinterpret_cast<Red*>(pool);
   __shared__ float ssq_row[16];
   extern __shared__ __align__(16) unsigned char stage_raw[];   // normed: bf16 [m_stage][k + kStagePad]
   const int lane = threadIdx.x % kWave;
@@ -79,7 +92,9 @@ __global__ __launch_bounds__(kThreads, XMODE != kPlain ? 6 : 4) void gemm_skinny
   const int n0 = blockIdx.x * 16;
   const int k = a.k, m = a.m;
 
-  const int chunk = ((k + kWaves * 32 - 1) / (kWaves * 32)) * 32;
+  // every wave's part of k starts on a cache line of x (64 elements), whatever the number of rows:
+  // the order of the additions, and so the rounding, is the same in every form of the kernel
+  const int chunk = ((k + kWaves * 64 - 1) / (kWaves * 64)) * 64;
   const int k_begin = wave * chunk;
   const int k_end = min(k, k_begin + chunk);
 
@@ -149,6 +164,14 @@ __global__ __launch_bounds__(kThreads, XMODE != kPlain ? 6 : 4) void gemm_skinny
     }
   }
 
+  // kTurned: load i of a batch brings piece (i * 64 + lane) % kPieces of row (i * 64 + lane) / kPieces;
+  // in the wave's buffer piece p of row r lies at r * kPieces + (p ^ (r % 8)), which keeps both the
+  // row-wise writes and the operand-wise reads (16 rows at one piece) off each other's banks.
+  constexpr int kRowsPerLoad = kTurned ? 64 / kPieces : 1;
+  const int turn_row = lane / kPieces, turn_piece = lane % kPieces;
+  const bf16_t* turn_src = static_cast<const bf16_t*>(a.x) + static_cast<long>(turn_row) * k + turn_piece * 8;
+  uint4* turn = reinterpret_cast<uint4*>(pool) + wave * (MT * 16 * kPieces);
+
   struct Batch {
     uint4 w[kSets][U];
     uint4 x[kNormed ? 1 : MT][kNormed ? 1 : U];
@@ -161,13 +184,32 @@ __global__ __launch_bounds__(kThreads, XMODE != kPlain ? 6 : 4) void gemm_skinny
 #pragma unroll
       for (int s = 0; s < kSets; ++s)
         b.w[s][u] = k0 + 32 * u < k_end ? load16(wblock + static_cast<long>(k0 / 32 + u) * (kWave * 8) + wlane) : zero16();
-      if constexpr (!kNormed) {
+      if constexpr (!kNormed && !kTurned) {
 #pragma unroll
         for (int t = 0; t < MT; ++t) b.x[t][u] = (ok && xrow_ok[t]) ? load16(xptr[t] + kk) : zero16();
       }
     }
+    if constexpr (kTurned) {
+      const bool k_ok = k0 + turn_piece * 8 < k_end;
+#pragma unroll
+      for (int i = 0; i < MT * U; ++i) {
+        const bool ok = k_ok && turn_row + i * kRowsPerLoad < m;
+        b.x[i / U][i % U] = ok ? load16(turn_src + static_cast<long>(i * kRowsPerLoad) * k + k0) : zero16();
+      }
+    }
   };
   auto compute = [&](const Batch& b, int k0) {
+    if constexpr (kTurned) {
+#pragma unroll
+      for (int i = 0; i < MT * U; ++i) {
+        const int row = turn_row + i * kRowsPerLoad;
+        turn[row * kPieces + (turn_piece ^ (row % 8))] = b.x[i / U][i % U];
+      }
+      // the wave's own lanes wrote what its lanes now read: LDS serves a wave's accesses in order
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
 #pragma unroll
@@ -176,12 +218,19 @@ __global__ __launch_bounds__(kThreads, XMODE != kPlain ? 6 : 4) void gemm_skinny
         if constexpr (kNormed) {
           const int kk = k0 + 32 * u + 8 * grp;
           xb = kk < k_end ? *reinterpret_cast<const uint4*>(xptr[t] + kk) : zero16();
+        } else if constexpr (kTurned) {
+          xb = turn[(t * 16 + col) * kPieces + ((4 * u + grp) ^ (col % 8))];
         } else {
           xb = b.x[t][u];
         }
 #pragma unroll
         for (int s = 0; s < kSets; ++s) acc[s][t] = mfma_16x16x32(b.w[s][u], xb, acc[s][t]);
       }
+    }
+    if constexpr (kTurned) {                             // read before the next batch is written
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     }
   };
 
@@ -262,6 +311,7 @@ __global__ __launch_bounds__(kThreads, XMODE != kPlain ? 6 : 4) void gemm_skinny
     if (more) cur = nxt;
   }
 
+  if constexpr (kTurned) __syncthreads();               // the partial sums take the buffers' place
   // acc[s][t][r] is the partial sum for output column n0 + 4*grp + r and row t*16 + col
 #pragma unroll
   for (int s = 0; s < kSets; ++s)
@@ -359,7 +409,7 @@ int launch(const SkinnyArgs& a, hipStream_t s) {
     switch (mt) {
       // k-steps per batch chosen so that two batches of operands fit 128 registers (two workgroups a CU)
       case 1: gemm_skinny_kernel<1, EPI, XMODE, 4><<<grid, block, 0, s>>>(a); break;
-      case 2: gemm_skinny_kernel<2, EPI, XMODE, 4><<<grid, block, 0, s>>>(a); break;
+      case 2: gemm_skinny_kernel<2, EPI, XMODE, 2><<<grid, block, 0, s>>>(a); break;
       case 3: gemm_skinny_kernel<3, EPI, XMODE, 2><<<grid, block, 0, s>>>(a); break;
       case 4: gemm_skinny_kernel<4, EPI, XMODE, 2><<<grid, block, 0, s>>>(a); break;
       default: return fail("gemm_skinny: M=%d is beyond 64 rows", a.m);

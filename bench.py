@@ -25,16 +25,24 @@ TINYLLAMA = dict(architectures=["LlamaForCausalLM"], model_type="llama", vocab_s
                  num_hidden_layers=22, num_attention_heads=32, num_key_value_heads=4, head_dim=64,
                  intermediate_size=5632, rope_theta=10000.0, rms_norm_eps=1e-5,
                  max_position_embeddings=2048, tie_word_embeddings=False)
-FULL_LAYERS = 22
+# Other shapes of the same architecture, for measurements beside the headline (--shape).
+SHAPES = {
+    "tinyllama-1.1b": TINYLLAMA,
+    "llama-2-7b": dict(TINYLLAMA, hidden_size=4096, num_hidden_layers=32, num_attention_heads=32,
+                       num_key_value_heads=32, head_dim=128, intermediate_size=11008, max_position_embeddings=4096),
+    "llama-3-8b": dict(TINYLLAMA, vocab_size=128256, hidden_size=4096, num_hidden_layers=32, num_attention_heads=32,
+                       num_key_value_heads=8, head_dim=128, intermediate_size=14336, rope_theta=500000.0,
+                       max_position_embeddings=8192),
+}
 BASELINE_DECODE_B1 = 77.3                   # the reference's only FP16 decode number (batch 1, RTX 3050)
 
 
-def build_model(layers, dtype, seed=0):
+def build_model(layers, dtype, seed=0, shape=TINYLLAMA):
     import torch
     from bare_cuda_4gib_amd.config import architecture_for
     from bare_cuda_4gib_amd.engine import Model, Runtime, parse_dtype
     from bare_cuda_4gib_amd.weights.random_device import random_tensors_on_device
-    raw = dict(TINYLLAMA, num_hidden_layers=layers)
+    raw = dict(shape, num_hidden_layers=layers)
     arch = architecture_for(raw)
     cfg = arch.config_class.from_dict(raw)
     model = Model(arch.describe(cfg))
@@ -137,7 +145,9 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--prompt-len", type=int, default=512)
     ap.add_argument("--prefill-tokens", type=int, default=2048)
-    ap.add_argument("--layers", type=int, default=FULL_LAYERS, help="fewer than 22 only where time needs it")
+    ap.add_argument("--shape", choices=sorted(SHAPES), default="tinyllama-1.1b",
+                    help="layer sizes; the headline is measured on the default")
+    ap.add_argument("--layers", type=int, default=None, help="fewer than the shape has only where time needs it")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--no-points", action="store_true", help="skip decoding at batch 1 and 64")
     ap.add_argument("--only", choices=["decode", "prefill"], default=None,
@@ -153,16 +163,24 @@ def main() -> int:
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dtype = "bfloat16" if args.dtype == "bf16" else "float32"
     elem = 2 if args.dtype == "bf16" else 4
-    model, cfg = build_model(args.layers, dtype)
+    shape = SHAPES[args.shape]
+    full_layers = shape["num_hidden_layers"]
+    if args.layers is None:
+        args.layers = full_layers
+    model, cfg = build_model(args.layers, dtype, shape=shape)
 
     if args.only == "decode":
         dt, contexts = run_decode(model, cfg, args.batch, args.prompt_len, args.steps, args.warmup)
-        print(json.dumps({"only": "decode", "batch": args.batch, "ms_per_step": round(dt / args.steps * 1e3, 4),
+        gbs = decode_bytes(cfg, elem, contexts) / (dt / args.steps) / 1e9
+        print(json.dumps({"only": "decode", "shape": args.shape, "batch": args.batch, "context": contexts[0],
+                          "hbm_frac": round(gbs / HBM_PEAK_GBS, 4), "ms_per_step": round(dt / args.steps * 1e3, 4),
                           "tokens_per_s": round(args.batch * args.steps / dt, 1)}), flush=True)
         return 0
     if args.only == "prefill":
         pre_s = run_prefill(model, cfg, args.prefill_tokens)
-        print(json.dumps({"only": "prefill", "tokens": args.prefill_tokens, "ms": round(pre_s * 1e3, 3),
+        frac = prefill_flops(cfg, args.prefill_tokens) / pre_s / (PEAK_TFLOPS[args.dtype] * 1e12)
+        print(json.dumps({"only": "prefill", "shape": args.shape, "tokens": args.prefill_tokens,
+                          "ms": round(pre_s * 1e3, 3), "frac": round(frac, 4),
                           "tokens_per_s": round(args.prefill_tokens / pre_s, 1)}), flush=True)
         return 0
 
@@ -187,7 +205,8 @@ def main() -> int:
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": round(points.get("decode_b1", 0.0) / BASELINE_DECODE_B1, 2) if points else None,
         "dtype": args.dtype, "data": "synthetic: random weights N(0, 0.02), uniform random token ids",
-        "config": {"model": "TinyLlama-1.1B shape", "layers": args.layers, "layers_full": FULL_LAYERS,
+        "config": {"model": "TinyLlama-1.1B shape" if args.shape == "tinyllama-1.1b" else args.shape + " shape",
+                   "layers": args.layers, "layers_full": full_layers,
                    "hidden": cfg.hidden_size, "heads": cfg.num_heads, "kv_heads": cfg.num_kv_heads,
                    "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
                    "global_batch": args.batch, "seq_len": cfg.max_seq_len, "prompt_len": args.prompt_len,
