@@ -36,8 +36,14 @@ int bc4g_swiglu(const void* gu, void* out, int dtype, int n_tokens, int inter, i
 // their cache pages (rope.cu:18-55, kv_cache_write.cu:10-20).
 // qkv: [n_tokens, (n_heads + 2 n_kv_heads) * head_dim]; slot_map[t] = page * page_tokens +
 // offset of the row's token; k_cache: [pages, n_kv_heads, page_tokens, head_dim]; v_cache is kept
-// transposed, [pages, n_kv_heads, head_dim, page_tokens], so that the matrix-core kernels can load
-// consecutive tokens of one dimension.
+// transposed, [pages, n_kv_heads, head_dim, page_tokens].  That is the plain layout, of float caches
+// and of sizes the matrix-core attention kernel does not take.  A bfloat16 cache with head_dim
+// (16 .. 256) and page_tokens multiples of 16 is in *fragment order*: the same tensors, but inside
+// every [page_tokens, head_dim] region the elements lie as that kernel's lanes read them,
+//   keys    [token / 16][dim / 8][token % 16][dim % 8]
+//   values  [token / 16][dim / 16][(token % 16) / 4][dim % 16][token % 4]
+// (cache_fragment_order and the two offset functions in common.h).  Every writer below and the
+// matrix-core kernel apply this rule by themselves; bc4g_attention_generic reads the plain layout only.
 // rotary_dim 0 switches the rotation off; write_kv 0 leaves the cache alone.  block_pairs 1: every
 // head's dimensions come reordered in blocks of 16 (dimensions 8b..8b+7, then their rotation
 // partners head_dim/2 + 8b..), the order the fused weight-streaming kernel works in; queries, keys and

@@ -6,11 +6,13 @@
 // tiles of 32 and never writes scores to memory:
 //   S^T = K Q^T   16x16x32 MFMAs with the keys as rows, so that a lane holds one query row's
 //                 scores and the softmax statistics are reductions inside a lane plus two
-//                 shuffles;  K rows come straight from the cache pages as the A operand
+//                 shuffles;  K comes straight from the cache pages as the A operand (the pages
+//                 are stored in the operand's order: a fragment is one contiguous kilobyte)
 //   online softmax in float, base 2, masked by absolute position (and the window); the running
 //                 maximum is kept over raw scores and the scale enters the exponent's argument
 //   O^T += V^T P^T   with P^T taken from the score registers as the B operand and V^T loaded
-//                 from the transposed value pages (8-byte loads of 4 consecutive tokens)
+//                 from the value pages, stored in that operand's order too (8-byte loads of 4
+//                 consecutive tokens, the 64 lanes' loads contiguous)
 // Prompt portions bring many tiles: there a workgroup is four independent waves (WS == 1).
 // Decoded tokens bring few tiles and long key walks: there a workgroup is one tile and its WS
 // waves cut the tile's keys between them, then combine their partial results in LDS (in wave
@@ -68,8 +70,8 @@ struct AttnArgs {
   bf16_t* out;                 // [T, n_heads * d]               (n_splits == 1)
   float* part_o;               // [n_splits, T, n_heads, d]      (n_splits > 1), unnormalized
   float* part_ml;              // [n_splits, T, n_heads, 2]      running max (base 2) and sum
-  const bf16_t* k_cache;       // [pages, n_kv, P, d]
-  const bf16_t* v_cache;       // [pages, n_kv, d, P]
+  const bf16_t* k_cache;       // [pages, n_kv, P * d], every page and head in fragment order (common.h)
+  const bf16_t* v_cache;       // likewise
   const int32_t* block_table;  // [S, table_stride]
   const int32_t* seq_start;    // [S + 1] first row of each request in the batch
   const int32_t* seq_ctx;      // [S] tokens cached before this step
@@ -202,10 +204,11 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, WS > 8 ? 4 
     uint2 v[2][DB];
     bool ok[2];
   };
-  // Addresses are a scalar base (page, key/value head, offset in the page: the same in every lane)
-  // plus a 32-bit lane offset; where the next tile lies in its page is carried along from tile to
-  // tile (the wave walks its tiles in order), so a fetch costs no division.
-  const int k_lane = col * d + 8 * grp, v_lane = col * P + 4 * grp;
+  // The cache is in fragment order: the 16 keys at next_off of a page are one block of 16 * d
+  // elements in which a key fragment is 1 KB and a value fragment 512 bytes, both in lane order --
+  // a scalar base (page, key/value head, block) plus the lane's place.  Where the next tile lies in
+  // its page is carried along from tile to tile (the wave walks its tiles in order): no division.
+  const int k_lane = lane * 8, v_lane = lane * 4;
   int next_page = (kt_begin * 32) / P, next_off = (kt_begin * 32) % P;
   auto fetch = [&](KeyTile& t, int kt) {        // tiles are fetched in order, from kt_begin on
 #pragma unroll
@@ -213,14 +216,15 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, WS > 8 ? 4 
       const int kb = kt * 32 + 16 * h;
       t.ok[h] = kb <= pos_max && kb + 15 >= lo_min;
       const long page = t.ok[h] ? page_of(next_page) : 0;
-      const bf16_t* kbase = a.k_cache + ((page * a.n_kv_heads + kvh) * P + next_off) * static_cast<long>(d);
-      const bf16_t* vbase = a.v_cache + (page * a.n_kv_heads + kvh) * static_cast<long>(d) * P + next_off;
+      const long block = ((page * a.n_kv_heads + kvh) * P + next_off) * static_cast<long>(d);
+      const bf16_t* kbase = a.k_cache + block;
+      const bf16_t* vbase = a.v_cache + block;
 #pragma unroll
       for (int j = 0; j < DJ; ++j)
-        t.k[h][j] = (t.ok[h] && (EXACT || 32 * j + 8 * grp < d)) ? load16(kbase + 32 * j + k_lane) : zero16();
+        t.k[h][j] = (t.ok[h] && (EXACT || 32 * j + 8 * grp < d)) ? load16(kbase + 512 * j + k_lane) : zero16();
 #pragma unroll
       for (int b = 0; b < DB; ++b)
-        t.v[h][b] = (t.ok[h] && (EXACT || 16 * b < d)) ? *reinterpret_cast<const uint2*>(vbase + 16 * b * P + v_lane)
+        t.v[h][b] = (t.ok[h] && (EXACT || 16 * b < d)) ? *reinterpret_cast<const uint2*>(vbase + 256 * b + v_lane)
                                             : make_uint2(0u, 0u);
       next_off += 16;                           // pages hold a multiple of 16 tokens
       if (next_off >= P) {

@@ -49,6 +49,29 @@ template <> __host__ __device__ inline bf16_t from_float<bf16_t>(float f) {
   return r;
 }
 
+// ---- the key/value cache in fragment order -----------------------------------
+// A bfloat16 cache whose head size (16 .. 256) and page size are multiples of 16 -- the caches the
+// matrix-core attention kernel reads -- keeps the elements of every (page, key/value head) region of
+// page_tokens * head_dim elements in the order in which that kernel's lanes take them, one block of
+// 16 tokens after the other:
+//   keys    [token / 16][dim / 8][token % 16][dim % 8]
+//           the A operand of the scores for 16 keys x 32 dims (lane l: key l % 16, dims 8 * (l / 16) ..)
+//           is 1 KB that the 64 lanes read in lane order
+//   values  [token / 16][dim / 16][(token % 16) / 4][dim % 16][token % 4]
+//           the A operand of the output for 16 dims x 16 keys (lane l: dim l % 16, keys 4 * (l / 16) ..)
+//           is 512 bytes in lane order
+// Every other cache (float, other sizes) is plain: keys [token][dim], values [dim][token].
+__host__ __device__ inline bool cache_fragment_order(bool is_bf16, int head_dim, int page_tokens) {
+  return is_bf16 && head_dim % 16 == 0 && head_dim >= 16 && head_dim <= 256 && page_tokens % 16 == 0;
+}
+__host__ __device__ inline long frag_k_offset(int token, int dim, int head_dim) {
+  return static_cast<long>(token / 16) * (16 * head_dim) + ((dim / 8) * 16 + token % 16) * 8 + dim % 8;
+}
+__host__ __device__ inline long frag_v_offset(int token, int dim, int head_dim) {
+  return static_cast<long>(token / 16) * (16 * head_dim) + (((dim / 16) * 4 + (token % 16) / 4) * 16 + dim % 16) * 4 +
+         token % 4;
+}
+
 // ---- wave64 / block reductions --------------------------------------------
 __device__ inline float wave_sum(float v) {
 #pragma unroll

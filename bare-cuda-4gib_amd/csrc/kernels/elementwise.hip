@@ -122,7 +122,7 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const int32_t* __restr
                                      const int32_t* __restrict__ slot_map, T* __restrict__ k_cache,
                                      T* __restrict__ v_cache, long total, int n_heads, int n_kv_heads,
                                      int head_dim, int rotary_dim, float theta, int page_tokens,
-                                     int write_kv, int block_pairs) {
+                                     int write_kv, int block_pairs, int frag) {
   const int half = head_dim / 2;          // threads per head: each moves two elements
   const int rhalf = rotary_dim / 2;
   const int heads_total = n_heads + 2 * n_kv_heads;
@@ -169,12 +169,18 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const int32_t* __restr
       const int kvh = is_v ? head - n_heads - n_kv_heads : head - n_heads;
       const int slot = slot_map[token];
       const long page = slot / page_tokens, off = slot % page_tokens;
-      if (is_v) {  // values are kept transposed: [page][kv head][dim][token]
-        T* dst = v_cache + (page * n_kv_heads + kvh) * head_dim * page_tokens + off;
+      const long region = (page * n_kv_heads + kvh) * head_dim * page_tokens;
+      if (frag) {  // the cache in fragment order
+        T* dst = (is_v ? v_cache : k_cache) + region;
+        const int o = static_cast<int>(off);
+        dst[is_v ? frag_v_offset(o, i0, head_dim) : frag_k_offset(o, i0, head_dim)] = from_float<T>(a);
+        dst[is_v ? frag_v_offset(o, i1, head_dim) : frag_k_offset(o, i1, head_dim)] = from_float<T>(b);
+      } else if (is_v) {  // values are kept transposed: [page][kv head][dim][token]
+        T* dst = v_cache + region + off;
         dst[static_cast<long>(i0) * page_tokens] = from_float<T>(a);
         dst[static_cast<long>(i1) * page_tokens] = from_float<T>(b);
       } else {     // keys: [page][kv head][token][dim]
-        T* dst = k_cache + ((page * n_kv_heads + kvh) * page_tokens + off) * head_dim;
+        T* dst = k_cache + region + off * head_dim;
         dst[i0] = from_float<T>(a);
         dst[i1] = from_float<T>(b);
       }
@@ -199,12 +205,12 @@ __global__ void rope_table_kernel(const int32_t* __restrict__ positions, float2*
 
 // rope_kv_write for the block layout (block_pairs) with the step's table of angles: a thread takes
 // one block of 16 elements -- pairs 8b .. 8b+7 of one head of one token -- with 16-byte loads and
-// stores (values go to their transposed pages element by element).
+// stores (values go to their pages element by element).  frag: the cache is in fragment order.
 template <typename T>
 __global__ void rope_kv_write_blocks_kernel(T* __restrict__ qkv, const float2* __restrict__ table,
                                             const int32_t* __restrict__ slot_map, T* __restrict__ k_cache,
                                             T* __restrict__ v_cache, long total, int n_heads, int n_kv_heads,
-                                            int head_dim, int rotate, int page_tokens, int write_kv) {
+                                            int head_dim, int rotate, int page_tokens, int write_kv, int frag) {
   const int blocks = head_dim / 16;
   const int heads_total = n_heads + 2 * n_kv_heads;
   const long stride = static_cast<long>(blockDim.x) * gridDim.x;
@@ -247,19 +253,25 @@ __global__ void rope_kv_write_blocks_kernel(T* __restrict__ qkv, const float2* _
     if (is_v) {   // values are kept transposed: [page][kv head][dim][token]
       const int slot = slot_map[token];
       const long page = slot / page_tokens, off = slot % page_tokens;
-      T* dst = v_cache + ((page * n_kv_heads + (head - n_heads - n_kv_heads)) * head_dim + 16 * b) * page_tokens + off;
+      T* region = v_cache + (page * n_kv_heads + (head - n_heads - n_kv_heads)) * head_dim * page_tokens;
+      // dimension 16b + c of the token: 4 elements further for every c in fragment order, a page row otherwise
+      T* dst = frag ? region + frag_v_offset(static_cast<int>(off), 16 * b, head_dim) : region + 16L * b * page_tokens + off;
+      const long step = frag ? 4 : page_tokens;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        dst[static_cast<long>(e) * page_tokens] = from_float<T>(lo[e]);
-        dst[static_cast<long>(8 + e) * page_tokens] = from_float<T>(hi[e]);
+        dst[e * step] = from_float<T>(lo[e]);
+        dst[(8 + e) * step] = from_float<T>(hi[e]);
       }
       continue;
     }
     T* dst = src;
-    if (!is_q) {   // keys: [page][kv head][token][dim]
+    long second = 8;   // where the block's second eight elements go, from dst
+    if (!is_q) {   // keys: [page][kv head][token][dim], or in fragment order: eight dimensions of 16 tokens together
       const int slot = slot_map[token];
       const long page = slot / page_tokens, off = slot % page_tokens;
-      dst = k_cache + ((page * n_kv_heads + (head - n_heads)) * page_tokens + off) * head_dim + 16 * b;
+      T* region = k_cache + (page * n_kv_heads + (head - n_heads)) * page_tokens * head_dim;
+      dst = frag ? region + frag_k_offset(static_cast<int>(off), 16 * b, head_dim) : region + off * head_dim + 16 * b;
+      if (frag) second = 16 * 8;
     }
     if constexpr (sizeof(T) == 2) {
       uint32_t lw[4], hw[4];
@@ -269,12 +281,12 @@ __global__ void rope_kv_write_blocks_kernel(T* __restrict__ qkv, const float2* _
         hw[e] = static_cast<uint32_t>(bf16_bits_from_float(hi[2 * e])) | (static_cast<uint32_t>(bf16_bits_from_float(hi[2 * e + 1])) << 16);
       }
       *reinterpret_cast<uint4*>(dst) = make_uint4(lw[0], lw[1], lw[2], lw[3]);
-      *reinterpret_cast<uint4*>(dst + 8) = make_uint4(hw[0], hw[1], hw[2], hw[3]);
+      *reinterpret_cast<uint4*>(dst + second) = make_uint4(hw[0], hw[1], hw[2], hw[3]);
     } else {
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         dst[e] = from_float<T>(lo[e]);
-        dst[8 + e] = from_float<T>(hi[e]);
+        dst[second + e] = from_float<T>(hi[e]);
       }
     }
   }
@@ -492,12 +504,12 @@ extern "C" int bc4g_rope_kv_write(void* qkv, int dtype, const int32_t* positions
     rope_kv_write_kernel<float><<<grid_for(total), kBlock, 0, s>>>(
         static_cast<float*>(qkv), positions, slot_map, static_cast<float*>(k_cache),
         static_cast<float*>(v_cache), total, n_heads, n_kv_heads, head_dim, rotary_dim, theta, page_tokens, write_kv,
-        block_pairs);
+        block_pairs, 0);
   } else if (dtype == kBF16) {
     rope_kv_write_kernel<bf16_t><<<grid_for(total), kBlock, 0, s>>>(
         static_cast<bf16_t*>(qkv), positions, slot_map, static_cast<bf16_t*>(k_cache),
         static_cast<bf16_t*>(v_cache), total, n_heads, n_kv_heads, head_dim, rotary_dim, theta, page_tokens, write_kv,
-        block_pairs);
+        block_pairs, cache_fragment_order(true, head_dim, page_tokens) ? 1 : 0);
   } else {
     return fail("rope_kv_write: unknown dtype %d", dtype);
   }
@@ -531,11 +543,12 @@ extern "C" int bc4g_rope_kv_write_blocks(void* qkv, int dtype, const float* tabl
   if (dtype == kF32) {
     rope_kv_write_blocks_kernel<float><<<grid_for(total), kBlock, 0, s>>>(
         static_cast<float*>(qkv), tab, slot_map, static_cast<float*>(k_cache), static_cast<float*>(v_cache), total,
-        n_heads, n_kv_heads, head_dim, rotate, page_tokens, write_kv);
+        n_heads, n_kv_heads, head_dim, rotate, page_tokens, write_kv, 0);
   } else if (dtype == kBF16) {
     rope_kv_write_blocks_kernel<bf16_t><<<grid_for(total), kBlock, 0, s>>>(
         static_cast<bf16_t*>(qkv), tab, slot_map, static_cast<bf16_t*>(k_cache), static_cast<bf16_t*>(v_cache), total,
-        n_heads, n_kv_heads, head_dim, rotate, page_tokens, write_kv);
+        n_heads, n_kv_heads, head_dim, rotate, page_tokens, write_kv,
+        cache_fragment_order(true, head_dim, page_tokens) ? 1 : 0);
   } else {
     return fail("rope_kv_write_blocks: unknown dtype %d", dtype);
   }

@@ -45,9 +45,10 @@ enum Epilogue : int { kStoreBf16 = 0, kStoreF32 = 1, kAccumF32 = 2, kSwigluBf16 
 struct RopeKvArgs {
   const int32_t* positions;   // [m]
   const int32_t* slot_map;    // [m] page * page_tokens + offset
-  bf16_t* k_cache;            // [pages, n_kv, page_tokens, d]
-  bf16_t* v_cache;            // [pages, n_kv, d, page_tokens]
+  bf16_t* k_cache;            // [pages, n_kv, page_tokens, d], or every [page_tokens, d] in fragment order
+  bf16_t* v_cache;            // [pages, n_kv, d, page_tokens], or likewise
   int n_heads, n_kv_heads, head_dim, rotary_dim, page_tokens, write_kv;
+  int fragment_order;         // how the cache's pages are laid out (cache_fragment_order)
   float theta;
 };
 enum XMode : int { kPlain = 0, kNormedG16 = 1, kNormedG32 = 2 };   // norm scale g in bfloat16 / float
@@ -372,12 +373,18 @@ __global__ __launch_bounds__(kThreads, XMODE != kPlain ? 6 : 4) void gemm_skinny
         const int kvh = is_v ? head - r.n_heads - r.n_kv_heads : head - r.n_heads;
         const int slot = rope_slot[j];
         const long page = slot / r.page_tokens, off = slot % r.page_tokens;
-        if (is_v) {
-          bf16_t* dst = r.v_cache + ((page * r.n_kv_heads + kvh) * d + in_head) * r.page_tokens + off;
+        const long region = (page * r.n_kv_heads + kvh) * d * r.page_tokens;
+        if (r.fragment_order) {
+          bf16_t* dst = (is_v ? r.v_cache : r.k_cache) + region;
+          const int o = static_cast<int>(off);
+          dst[is_v ? frag_v_offset(o, in_head, d) : frag_k_offset(o, in_head, d)] = from_float<bf16_t>(lo);
+          dst[is_v ? frag_v_offset(o, in_head + 8, d) : frag_k_offset(o, in_head + 8, d)] = from_float<bf16_t>(hi);
+        } else if (is_v) {
+          bf16_t* dst = r.v_cache + region + in_head * r.page_tokens + off;
           dst[0] = from_float<bf16_t>(lo);
           dst[8L * r.page_tokens] = from_float<bf16_t>(hi);
         } else {
-          bf16_t* dst = r.k_cache + ((page * r.n_kv_heads + kvh) * r.page_tokens + off) * d + in_head;
+          bf16_t* dst = r.k_cache + region + off * d + in_head;
           dst[0] = from_float<bf16_t>(lo);
           dst[8] = from_float<bf16_t>(hi);
         }
@@ -489,7 +496,8 @@ extern "C" int bc4g_gemm_skinny_qkv(const void* x, const void* g, int g_dtype, f
                                     int m, int k, int n_heads, int n_kv_heads, int head_dim, int rotary_dim,
                                     float theta, int page_tokens, int write_kv, void* stream) {
   RopeKvArgs r{positions, slot_map, static_cast<bf16_t*>(k_cache), static_cast<bf16_t*>(v_cache), n_heads, n_kv_heads,
-               head_dim, rotary_dim, page_tokens, write_kv, theta};
+               head_dim, rotary_dim, page_tokens, write_kv,
+               cache_fragment_order(true, head_dim, page_tokens) ? 1 : 0, theta};
   const int n = (n_heads + 2 * n_kv_heads) * head_dim;
   if (int e = check_common("gemm_skinny_qkv", m, g ? 16 : 64, n, k, kRopeKvBf16)) return e;
   if (int e = check_rope("gemm_skinny_qkv", r, n)) return e;

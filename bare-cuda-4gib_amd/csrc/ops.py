@@ -120,8 +120,37 @@ def swiglu(gu: torch.Tensor, interleaved: bool = False) -> torch.Tensor:
     return out
 
 
+def cache_fragment_order(dtype: torch.dtype, head_dim: int, page_tokens: int) -> bool:
+    """Whether a cache of these sizes is kept in fragment order -- inside every page and head the
+    elements lie as the matrix-core attention kernel's lanes read them -- rather than plain (keys
+    [token][dim], values [dim][token]).  The kernels that write and read the cache apply the same rule."""
+    return dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= 256 and page_tokens % 16 == 0
+
+
+def cache_from_plain(k: torch.Tensor, v: torch.Tensor):
+    """Caches in the layout the kernels expect for their sizes, from plain ones (keys [pages, heads,
+    page_tokens, d], values [pages, heads, d, page_tokens]); the shapes stay."""
+    n, h, p, d = k.shape
+    if not cache_fragment_order(k.dtype, d, p):
+        return k, v
+    kf = k.view(n, h, p // 16, 16, d // 8, 8).permute(0, 1, 2, 4, 3, 5).contiguous().view(n, h, p, d)
+    vf = v.view(n, h, d // 16, 16, p // 16, 4, 4).permute(0, 1, 4, 2, 5, 3, 6).contiguous().view(n, h, d, p)
+    return kf, vf
+
+
+def cache_to_plain(k: torch.Tensor, v: torch.Tensor):
+    """The inverse of cache_from_plain: what the kernels wrote, as keys [.., token, dim] and values [.., dim, token]."""
+    n, h, p, d = k.shape
+    if not cache_fragment_order(k.dtype, d, p):
+        return k, v
+    kp = k.view(n, h, p // 16, d // 8, 16, 8).permute(0, 1, 2, 4, 3, 5).reshape(n, h, p, d)
+    vp = v.view(n, h, p // 16, d // 16, 4, 16, 4).permute(0, 1, 3, 5, 2, 4, 6).reshape(n, h, d, p)
+    return kp, vp
+
+
 def _check_cache(what: str, k: torch.Tensor, v: torch.Tensor, n_kv_heads: int, head_dim: int, dtype: torch.dtype):
-    """k: [pages, kv_heads, page_tokens, head_dim]; v transposed: [pages, kv_heads, head_dim, page_tokens]."""
+    """k: [pages, kv_heads, page_tokens, head_dim]; v transposed: [pages, kv_heads, head_dim, page_tokens]
+    (the order inside a page and head: see cache_fragment_order)."""
     ok = (k.dim() == 4 and v.dim() == 4 and k.shape[1] == n_kv_heads and k.shape[3] == head_dim
           and k.dtype == dtype and v.dtype == dtype
           and tuple(v.shape) == (k.shape[0], n_kv_heads, head_dim, k.shape[2]))

@@ -200,7 +200,7 @@ def test_rope_kv_write_blocks_with_table(ops, dt, d, rotate):
     tol = dict(rtol=1e-5, atol=1e-5) if dt == torch.float32 else dict(rtol=8e-3, atol=8e-3)
     out = buf.cpu().double().view(t, nh + 2 * nkv, d)
     close(out[:, :nh][:, :, inverse], q_want, what="q", **tol)
-    kc_c, vc_c = kc.cpu().double(), vc.cpu().double()
+    kc_c, vc_c = (c.cpu().double() for c in ops.cache_to_plain(kc, vc))   # by token and dimension
     touched = torch.zeros(pages, page, dtype=torch.bool)
     for i, sl in enumerate(slots):
         pg, off = divmod(sl, page)
@@ -233,7 +233,7 @@ def test_rope_kv_write(ops, dt, rotary_dim):
     out = buf.cpu().double().view(t, nh + 2 * nkv, d)
     close(out[:, :nh], q_want, what="q", **tol)
     assert torch.equal(out[:, nh:], x[:, nh:]) or rotary_dim       # k, v in the buffer are not the product
-    kc_c, vc_c = kc.cpu().double(), vc.cpu().double()
+    kc_c, vc_c = (c.cpu().double() for c in ops.cache_to_plain(kc, vc))   # by token and dimension
     touched_k = torch.zeros_like(kc_c, dtype=torch.bool)
     touched_v = torch.zeros_like(vc_c, dtype=torch.bool)
     for i, s in enumerate(slots):
@@ -325,7 +325,8 @@ def run_mfma(ops, case, window, n_splits, q_tiles=1, shared=False):
     for s in range(len(case["seq_ctx"])):
         starts.append(starts[-1] + -(-(case["seq_start"][s + 1] - case["seq_start"][s]) // tpt))
     dev = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
-    return ops.attention_mfma(case["qkv"], case["kc"], case["vc"], case["table"], dev(case["seq_start"]),
+    kc, vc = ops.cache_from_plain(case["kc"], case["vc"])      # the layout the writers leave for these sizes
+    return ops.attention_mfma(case["qkv"], kc, vc, case["table"], dev(case["seq_start"]),
                               dev(case["seq_ctx"]), dev(starts), starts[-1], nh, nkv, d, window,
                               1.0 / math.sqrt(d), n_splits, q_tiles, shared)
 
@@ -470,7 +471,7 @@ def test_qkv_product_with_rotation_and_cache_write(ops, nh, nkv, d, m, normed, r
                           torch.tensor(slots, dtype=torch.int32, device=DEV), kc, vc, nh, nkv, d, rd, theta)
     tol = dict(rtol=2e-2, atol=3e-2)
     close(q.view(m, nh, d), q_want[:, :, order], what="q", **tol)
-    kc_c, vc_c = kc.cpu().double(), vc.cpu().double()
+    kc_c, vc_c = (c.cpu().double() for c in ops.cache_to_plain(kc, vc))   # by token and dimension
     seen_k, seen_v = torch.zeros_like(kc_c, dtype=torch.bool), torch.zeros_like(vc_c, dtype=torch.bool)
     for i, s in enumerate(slots):
         pg, off = divmod(s, page)
@@ -485,6 +486,7 @@ def test_qkv_product_with_rotation_and_cache_write(ops, nh, nkv, d, m, normed, r
         ops.rope_kv_write(buf, torch.tensor(positions, dtype=torch.int32, device=DEV),
                           torch.tensor(slots, dtype=torch.int32, device=DEV), kc2, vc2, nh, nkv, d, rd, theta,
                           block_pairs=True)
+        kc2, vc2 = ops.cache_to_plain(kc2, vc2)
         close(kc2, kc_c, 1e-2, 2e-2, "unfused keys")
         close(vc2, vc_c, 1e-2, 2e-2, "unfused values")
         close(buf.view(m, nh + 2 * nkv, d)[:, :nh], q.view(m, nh, d), 1e-2, 2e-2, "unfused queries")
