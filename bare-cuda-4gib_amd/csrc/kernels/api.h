@@ -97,13 +97,17 @@ int bc4g_gemm_skinny(const void* x, const void* w, void* out, int epilogue, int 
 }
 
 extern "C" {
-// Attention on the matrix cores (bfloat16): see attention_mfma.hip.  A wave takes q_tiles tiles of
-// 16 rows, each tokens_per_tile tokens times the query heads of one key/value head; tile_start[s]
-// is the first wave-sized piece of request s when every request's rows are cut into pieces of
-// q_tiles * tokens_per_tile tokens; n_tiles their total.  q_tiles is 1, or 4 for head sizes up to
-// 64 and 2 up to 128.  With shared_tile (q_tiles 1 only) a workgroup is one tile whose waves cut
-// the tile's keys between them and combine in LDS: for few rows over long contexts.  With
-// n_splits > 1 the keys are, moreover, cut into that many parts over workgroups, whose float
+// Attention on the matrix cores (bfloat16, the cache in fragment order): see attention_mfma.hip.
+// A wave takes q_tiles tiles of 16 rows, each tokens_per_tile tokens times the query heads of one
+// key/value head.  q_tiles is 1, or 4 for head sizes up to 64 and 2 up to 128.  `form` says what a
+// workgroup is, and with it what tile_start counts (tile_start[s]: the first piece of request s when
+// every request's rows are cut into pieces; n_tiles their total):
+//   0  four independent waves; pieces of q_tiles * tokens_per_tile tokens (a wave's)
+//   1  one tile (q_tiles 1) whose waves cut the tile's keys between them and combine in LDS, for
+//      few rows over long contexts; pieces of tokens_per_tile tokens
+//   2  four waves with consecutive tiles of one request that walk their keys together, every key
+//      tile staged in LDS once for all of them; pieces of 4 * q_tiles * tokens_per_tile tokens
+// With n_splits > 1 the keys are, moreover, cut into that many parts over workgroups, whose float
 // partials (part_o [n_splits, T, heads, d], part_ml [n_splits, T, heads, 2]) a second kernel
 // merges into out.
 int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, float* part_o, float* part_ml, const void* k_cache,
@@ -111,7 +115,7 @@ int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, float* part_o,
                         const int32_t* seq_start, const int32_t* seq_ctx, const int32_t* tile_start,
                         int n_seqs, int n_tiles, int n_tokens, int n_heads, int n_kv_heads, int head_dim,
                         int page_tokens, int window, float scale, int tokens_per_tile, int q_tiles,
-                        int shared_tile, int n_splits, void* stream);
+                        int form, int n_splits, void* stream);
 }
 
 extern "C" {

@@ -13,7 +13,13 @@
 //   O^T += V^T P^T   with P^T taken from the score registers as the B operand and V^T loaded
 //                 from the value pages, stored in that operand's order too (8-byte loads of 4
 //                 consecutive tokens, the 64 lanes' loads contiguous)
-// Prompt portions bring many tiles: there a workgroup is four independent waves (WS == 1).
+// Prompt portions bring many tiles of one request: there a workgroup is four waves with
+// consecutive tiles that walk their keys together (WS == 0) -- all threads copy a key tile from the
+// cache into LDS once (a straight copy: the pages are in operand order already) and every wave
+// takes its operands from there, so a key is fetched once for 4 * QT * 16 query rows; the next
+// tile's loads are in flight during the arithmetic, and there is one barrier a tile.  (WS == 1 is
+// the same without LDS, four independent waves: kept for comparison and for tiles of different
+// requests in one workgroup.)
 // Decoded tokens bring few tiles and long key walks: there a workgroup is one tile and its WS
 // waves cut the tile's keys between them, then combine their partial results in LDS (in wave
 // order).  On top of that, with n_splits > 1 the key range is cut into that many parts over
@@ -93,12 +99,18 @@ constexpr int kMergePad = 4;   // floats between rows of the partial outputs in 
 template <int DJ, int DB, int QT, int WS, bool EXACT>
 __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, WS > 8 ? 4 : 2) void attention_mfma_kernel(
     const AttnArgs a) {
-  static_assert(WS == 1 || QT == 1, "waves share a tile's keys for single query tiles only");
-  extern __shared__ __align__(16) float merge_raw[];   // WS > 1: [WS][16][d + pad] outputs, [WS][16][2] statistics
+  static_assert(WS <= 1 || QT == 1, "waves share a tile's keys for single query tiles only");
+  constexpr bool kStaged = WS == 0;
+  // WS > 1: [WS][16][d + pad] outputs, [WS][16][2] statistics; WS == 0: two key tiles of 128 * d bytes
+  extern __shared__ __align__(16) float merge_raw[];
   const int lane = threadIdx.x % kWave;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int col = lane % 16, grp = lane / 16;
-  const int tile = WS > 1 ? blockIdx.x : blockIdx.x * kWavesPerBlock + wave;
+  // what tile_start counts: a wave's tiles (WS == 1), or a workgroup's (one tile, or four waves' tiles)
+  // (prompt forms: the last workgroups first -- under the causal mask a request's last rows walk
+  // the most keys, and the longest walks should not be the ones that start last)
+  const int block_x = WS > 1 ? blockIdx.x : gridDim.x - 1 - blockIdx.x;
+  const int tile = WS == 1 ? block_x * kWavesPerBlock + wave : block_x;
   if (WS == 1 && tile >= a.n_tiles) return;   // (waves are independent there: no barrier below)
 
   // Which request this tile belongs to, and that request's rows and context.  Up to 63 requests
@@ -126,8 +138,10 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, WS > 8 ? 4 
     q_len = a.seq_start[s + 1] - row0;
     ctx = a.seq_ctx[s];
   }
-  const int tok0 = (tile - tile0) * a.tpt * QT;
-  const int ntok = min(a.tpt * QT, q_len - tok0);
+  // the workgroup's rows (kStaged: four waves' worth) and this wave's among them
+  const int tok0_wg = (tile - tile0) * a.tpt * QT * (kStaged ? kWavesPerBlock : 1);
+  const int tok0 = tok0_wg + (kStaged ? wave * a.tpt * QT : 0);
+  const int ntok = max(0, min(a.tpt * QT, q_len - tok0));     // (0: a wave past the request's rows)
   const int kvh = blockIdx.y / a.n_sub, hsub = blockIdx.y % a.n_sub;
   const int group = a.n_heads / a.n_kv_heads;
   const int d = EXACT ? 16 * DB : a.head_dim, P = a.page_tokens;
@@ -156,14 +170,21 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, WS > 8 ? 4 
     }
   }
 
+  // the wave's own positions (masks), and those of the rows whose keys the walk covers: the
+  // wave's, or (kStaged) the four waves' together
   const int pos_min = ctx + tok0, pos_max = ctx + tok0 + ntok - 1;
-  const int lo_min = (a.window > 0 && pos_min - a.window + 1 > 0) ? pos_min - a.window + 1 : 0;
-  const int kt_first = lo_min / 32, kt_last = pos_max / 32;
+  const int walk_min = ctx + tok0_wg;
+  const int walk_max = kStaged ? ctx + min(q_len, tok0_wg + kWavesPerBlock * a.tpt * QT) - 1 : pos_max;
+  const int lo_min = (a.window > 0 && walk_min - a.window + 1 > 0) ? walk_min - a.window + 1 : 0;
+  const int kt_first = lo_min / 32, kt_last = walk_max / 32;
   const int n_kt = kt_last - kt_first + 1;
-  const int n_parts = a.n_splits * WS;
+  const int n_parts = a.n_splits * (WS > 1 ? WS : 1);
   const int per_split = (n_kt + n_parts - 1) / n_parts;
-  const int kt_begin = kt_first + (blockIdx.z * WS + (WS > 1 ? wave : 0)) * per_split;
+  const int kt_begin = kt_first + (blockIdx.z * (WS > 1 ? WS : 1) + (WS > 1 ? wave : 0)) * per_split;
   const int kt_end = min(kt_last + 1, kt_begin + per_split);
+  // kStaged: the tiles of the walk that hold keys of this wave's rows
+  const int own_lo = (a.window > 0 && pos_min - a.window + 1 > 0) ? pos_min - a.window + 1 : 0;
+  const int own_first = own_lo / 32, own_last = ntok > 0 ? pos_max / 32 : -1;
 
   float m_run[QT], l_run[QT];
   floatx4 o[QT][DB];
@@ -179,7 +200,7 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, WS > 8 ? 4 
   // i / 64), so that finding a tile's page is a lane read and not a trip to memory.
   constexpr int kTableRegs = 4;
   int32_t tbl[kTableRegs];
-  const int pages_needed = pos_max / P + 1;
+  const int pages_needed = walk_max / P + 1;
 #pragma unroll
   for (int r = 0; r < kTableRegs; ++r) {
     const int idx = r * kWave + lane;
@@ -200,8 +221,8 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, WS > 8 ? 4 
   // one tile of 32 keys: key fragments (A operand of the scores) and value fragments (A operand
   // of the output), fetched one tile ahead of their use
   struct KeyTile {
-    uint4 k[2][DJ];
-    uint2 v[2][DB];
+    uint4 k[2][kStaged ? 1 : DJ];
+    uint2 v[2][kStaged ? 1 : DB];
     bool ok[2];
   };
   // The cache is in fragment order: the 16 keys at next_off of a page are one block of 16 * d
@@ -210,22 +231,14 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, WS > 8 ? 4 
   // its page is carried along from tile to tile (the wave walks its tiles in order): no division.
   const int k_lane = lane * 8, v_lane = lane * 4;
   int next_page = (kt_begin * 32) / P, next_off = (kt_begin * 32) % P;
-  auto fetch = [&](KeyTile& t, int kt) {        // tiles are fetched in order, from kt_begin on
+  long block_at[2];                              // where the tile's two blocks of 16 keys lie in the cache
+  auto locate = [&](bool (&ok)[2], int kt) {    // tiles are located in order, from kt_begin on
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       const int kb = kt * 32 + 16 * h;
-      t.ok[h] = kb <= pos_max && kb + 15 >= lo_min;
-      const long page = t.ok[h] ? page_of(next_page) : 0;
-      const long block = ((page * a.n_kv_heads + kvh) * P + next_off) * static_cast<long>(d);
-      const bf16_t* kbase = a.k_cache + block;
-      const bf16_t* vbase = a.v_cache + block;
-#pragma unroll
-      for (int j = 0; j < DJ; ++j)
-        t.k[h][j] = (t.ok[h] && (EXACT || 32 * j + 8 * grp < d)) ? load16(kbase + 512 * j + k_lane) : zero16();
-#pragma unroll
-      for (int b = 0; b < DB; ++b)
-        t.v[h][b] = (t.ok[h] && (EXACT || 16 * b < d)) ? *reinterpret_cast<const uint2*>(vbase + 256 * b + v_lane)
-                                            : make_uint2(0u, 0u);
+      ok[h] = kb <= walk_max && kb + 15 >= lo_min;
+      const long page = ok[h] ? page_of(next_page) : 0;
+      block_at[h] = ((page * a.n_kv_heads + kvh) * P + next_off) * static_cast<long>(d);
       next_off += 16;                           // pages hold a multiple of 16 tokens
       if (next_off >= P) {
         next_off = 0;
@@ -233,32 +246,111 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, WS > 8 ? 4 
       }
     }
   };
+  auto fetch = [&](KeyTile& t, int kt) {
+    locate(t.ok, kt);
+    if constexpr (!kStaged) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const bf16_t* kbase = a.k_cache + block_at[h];
+        const bf16_t* vbase = a.v_cache + block_at[h];
+#pragma unroll
+        for (int j = 0; j < DJ; ++j)
+          t.k[h][j] = (t.ok[h] && (EXACT || 32 * j + 8 * grp < d)) ? load16(kbase + 512 * j + k_lane) : zero16();
+#pragma unroll
+        for (int b = 0; b < DB; ++b)
+          t.v[h][b] = (t.ok[h] && (EXACT || 16 * b < d)) ? *reinterpret_cast<const uint2*>(vbase + 256 * b + v_lane)
+                                              : make_uint2(0u, 0u);
+      }
+    }
+  };
+
+  // kStaged: a tile in LDS is four segments of 16 * d elements -- keys of its first and second 16
+  // tokens, then their values -- each a copy of the block in the cache.  A thread copies the same
+  // 16-byte pieces of every tile: piece c = threadIdx.x + 256 * r lies in segment c / (2 * d).
+  constexpr int kPieces = kStaged ? (4 * 2 * 16 * DB + 255) / 256 : 1;    // per thread, for the largest d of this form
+  int piece_seg[kPieces], piece_off[kPieces];
+  if constexpr (kStaged) {
+#pragma unroll
+    for (int r = 0; r < kPieces; ++r) {
+      const int c = threadIdx.x + 256 * r;
+      piece_seg[r] = c < 8 * d ? c / (2 * d) : -1;
+      piece_off[r] = (c % (2 * d)) * 8;
+    }
+  }
+  uint4 staged[kPieces];
+  bool staged_ok[2];
+  auto stage_load = [&](int kt) {               // cache -> registers
+    locate(staged_ok, kt);
+#pragma unroll
+    for (int r = 0; r < kPieces; ++r) {
+      const int seg = piece_seg[r];
+      const bool live = seg >= 0 && staged_ok[seg & 1];
+      const bf16_t* base = (seg >= 2 ? a.v_cache : a.k_cache) + block_at[seg & 1];
+      staged[r] = live ? load16(base + piece_off[r]) : zero16();
+    }
+  };
+  bf16_t* tiles = reinterpret_cast<bf16_t*>(merge_raw);
+  auto stage_store = [&](int buf) {             // registers -> LDS
+#pragma unroll
+    for (int r = 0; r < kPieces; ++r)
+      if (piece_seg[r] >= 0)
+        *reinterpret_cast<uint4*>(tiles + buf * (64 * d) + piece_seg[r] * (16 * d) + piece_off[r]) = staged[r];
+  };
 
   // (more than eight waves a workgroup would leave a wave 128 registers: no room for a second tile)
   constexpr bool kAhead = WS <= 8 && DB <= 8;   // (nor do the fragments of the largest heads leave room)
   KeyTile cur, nxt;
-  if (kAhead && kt_begin < kt_end) fetch(cur, kt_begin);
+  if constexpr (kStaged) {
+    if (kt_begin < kt_end) stage_load(kt_begin);
+  } else {
+    if (kAhead && kt_begin < kt_end) fetch(cur, kt_begin);
+  }
   for (int kt = kt_begin; kt < kt_end; ++kt) {
-    if constexpr (kAhead) {
+    const bf16_t* tile_lds = tiles + ((kt - kt_begin) & 1) * (64 * d);
+    if constexpr (kStaged) {
+      // This tile goes into the buffer that the tile before the last was read from: every wave has
+      // passed the last barrier, so it has finished with that one.  The next tile's loads start now.
+      stage_store((kt - kt_begin) & 1);
+      cur.ok[0] = staged_ok[0];
+      cur.ok[1] = staged_ok[1];
+      if (kt + 1 < kt_end) stage_load(kt + 1);
+      lds_barrier();
+      if (kt < own_first || kt > own_last) continue;      // no key of this wave's rows in the tile
+    } else if constexpr (kAhead) {
       if (kt + 1 < kt_end) fetch(nxt, kt + 1);
     } else {
       fetch(cur, kt);
     }
     const int key0 = kt * 32;
-    // values of keys past the tile's last position are replaced by zero (the tile at the end only)
-    if (key0 + 31 > pos_max) {
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        const int kb = key0 + 16 * h + 4 * grp;
-        const uint32_t m01 = (kb <= pos_max ? 0xffffu : 0u) | (kb + 1 <= pos_max ? 0xffff0000u : 0u);
-        const uint32_t m23 = (kb + 2 <= pos_max ? 0xffffu : 0u) | (kb + 3 <= pos_max ? 0xffff0000u : 0u);
-#pragma unroll
-        for (int b = 0; b < DB; ++b) {
-          cur.v[h][b].x &= m01;
-          cur.v[h][b].y &= m23;
-        }
+    // values of keys past the walk's last position may never have been written: they are replaced
+    // by zero (in the tile at the end only)
+    const bool edge = key0 + 31 > walk_max;
+    auto value_fragment = [&](int b) -> uint4 {
+      uint2 v0, v1;
+      if constexpr (kStaged) {
+        v0 = *reinterpret_cast<const uint2*>(tile_lds + 32 * d + 256 * b + v_lane);
+        v1 = *reinterpret_cast<const uint2*>(tile_lds + 48 * d + 256 * b + v_lane);
+      } else {
+        v0 = cur.v[0][b];
+        v1 = cur.v[1][b];
       }
-    }
+      if (edge) {
+        const int kb = key0 + 4 * grp;
+        v0.x &= (kb <= walk_max ? 0xffffu : 0u) | (kb + 1 <= walk_max ? 0xffff0000u : 0u);
+        v0.y &= (kb + 2 <= walk_max ? 0xffffu : 0u) | (kb + 3 <= walk_max ? 0xffff0000u : 0u);
+        v1.x &= (kb + 16 <= walk_max ? 0xffffu : 0u) | (kb + 17 <= walk_max ? 0xffff0000u : 0u);
+        v1.y &= (kb + 18 <= walk_max ? 0xffffu : 0u) | (kb + 19 <= walk_max ? 0xffff0000u : 0u);
+      }
+      return make_uint4(v0.x, v0.y, v1.x, v1.y);
+    };
+    auto key_fragment = [&](int h, int j) -> uint4 {
+      if constexpr (kStaged) {
+        return (EXACT || 32 * j + 8 * grp < d) ? *reinterpret_cast<const uint4*>(tile_lds + 16 * d * h + 512 * j + k_lane)
+                                               : zero16();
+      } else {
+        return cur.k[h][j];
+      }
+    };
     // The wave's query tiles go through each phase together -- all score MFMAs, then all the
     // softmax arithmetic, then all output MFMAs -- with no branch between tiles, so that the
     // independent chains of the tiles overlap.  (Tiles beyond the request's rows run masked.)
@@ -266,10 +358,14 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, WS > 8 ? 4 
 #pragma unroll
     for (int t = 0; t < QT; ++t)
 #pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        sc[t][h] = floatx4{0.f, 0.f, 0.f, 0.f};
+      for (int h = 0; h < 2; ++h) sc[t][h] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int j = 0; j < DJ; ++j) sc[t][h] = mfma_16x16x32(cur.k[h][j], qf[t][j], sc[t][h]);
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int j = 0; j < DJ; ++j) {
+        const uint4 kf = key_fragment(h, j);
+#pragma unroll
+        for (int t = 0; t < QT; ++t) sc[t][h] = mfma_16x16x32(kf, qf[t][j], sc[t][h]);
       }
     // A lane holds, for its query row, the raw scores of keys key0 + 16h + 4*grp + r.  A key tile
     // that every row of the wave sees whole needs no mask (the usual case away from the diagonal);
@@ -330,11 +426,11 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, WS > 8 ? 4 
     // (blocks past the head size hold zeros and are never stored)
 #pragma unroll
     for (int b = 0; b < DB; ++b) {
-      const uint4 vf = make_uint4(cur.v[0][b].x, cur.v[0][b].y, cur.v[1][b].x, cur.v[1][b].y);
+      const uint4 vf = value_fragment(b);
 #pragma unroll
       for (int t = 0; t < QT; ++t) o[t][b] = mfma_16x16x32(vf, pf[t], o[t][b]);
     }
-    if constexpr (kAhead) {
+    if constexpr (kAhead && !kStaged) {
       if (kt + 1 < kt_end) cur = nxt;
     }
   }
@@ -483,7 +579,7 @@ extern "C" int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, flo
                                    const int32_t* seq_start, const int32_t* seq_ctx, const int32_t* tile_start,
                                    int n_seqs, int n_tiles, int n_tokens, int n_heads, int n_kv_heads, int head_dim,
                                    int page_tokens, int window, float scale, int tokens_per_tile, int q_tiles,
-                                   int shared_tile, int n_splits, void* stream) {
+                                   int form, int n_splits, void* stream) {
   BC4G_REQUIRE(n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0, "attention_mfma: bad heads %d/%d",
                n_heads, n_kv_heads);
   BC4G_REQUIRE(head_dim >= 16 && head_dim <= 256 && head_dim % 16 == 0,
@@ -531,9 +627,24 @@ extern "C" int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, flo
                "attention_mfma: %d query tiles per wave are not built for head_dim %d (1 or %d)", q_tiles, head_dim,
                max_qt);
   BC4G_REQUIRE(n_kv_heads * a.n_sub <= 65535, "attention_mfma: too many heads for the grid");
-  BC4G_REQUIRE(!shared_tile || q_tiles == 1, "attention_mfma: waves share the keys of single query tiles only");
+  BC4G_REQUIRE(form >= 0 && form <= 2, "attention_mfma: unknown form %d", form);
+  BC4G_REQUIRE(form != 1 || q_tiles == 1, "attention_mfma: waves share the keys of single query tiles only");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (shared_tile) {
+  if (form == 2) {
+    // four waves' tiles per workgroup (n_tiles counts workgroups), key tiles staged in LDS twice over
+    dim3 grid(n_tiles, n_kv_heads * a.n_sub, n_splits);
+    dim3 block(kWavesPerBlock * kWave);
+    const size_t lds = static_cast<size_t>(2) * 128 * head_dim;
+    if (dj <= 2 && db <= 4) {
+      if (q_tiles == 4) launch_attention<2, 4, 4, 0>(a, grid, block, lds, s);
+      else launch_attention<2, 4, 1, 0>(a, grid, block, lds, s);
+    } else if (dj <= 4 && db <= 8) {
+      if (q_tiles == 2) launch_attention<4, 8, 2, 0>(a, grid, block, lds, s);
+      else launch_attention<4, 8, 1, 0>(a, grid, block, lds, s);
+    } else {
+      launch_attention<8, 16, 1, 0>(a, grid, block, lds, s);
+    }
+  } else if (form == 1) {
     // one workgroup per tile; its waves (8, or 4 for the largest heads) cut the keys between them
     dim3 grid(n_tiles, n_kv_heads * a.n_sub, n_splits);
     auto lds = [&](int ws) { return static_cast<size_t>(ws) * 16 * (head_dim + kMergePad + 2) * sizeof(float); };

@@ -70,8 +70,12 @@ def load(build_if_missing: bool = True) -> ctypes.CDLL:
     return lib
 
 
+_entry: dict = {}
+
+
 def call(name: str, *args) -> None:
-    lib = load()
-    status = getattr(lib, name)(*args)
-    if status != 0:
-        raise KernelError(lib.bc4g_last_error().decode("utf-8", "replace"))
+    fn = _entry.get(name)
+    if fn is None:
+        fn = _entry[name] = getattr(load(), name)
+    if fn(*args) != 0:
+        raise KernelError(load().bc4g_last_error().decode("utf-8", "replace"))

@@ -42,7 +42,9 @@ def _i32(what: str, name: str, t: torch.Tensor, n: int) -> None:
 
 
 def _stream() -> int:
-    return torch.cuda.current_stream().cuda_stream
+    """The current stream's handle (asked for at every launch: a step runs a few hundred of them, so
+    by the short way, without a Stream object)."""
+    return torch._C._cuda_getCurrentRawStream(torch._C._cuda_getDevice())
 
 
 def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
@@ -451,6 +453,9 @@ def attention_mfma_supported(qkv: torch.Tensor, k_cache: torch.Tensor, head_dim:
             and k_cache.shape[2] % 16 == 0)
 
 
+ATTENTION_STAGED_WAVES = 4      # waves of a workgroup whose tiles share every key tile through LDS
+
+
 def attention_tile_tokens(n_heads: int, n_kv_heads: int) -> int:
     """Tokens of one request per 16-row tile of the matrix-core attention kernel."""
     return 16 // min(n_heads // n_kv_heads, 16)
@@ -461,13 +466,13 @@ def attention_q_tiles(head_dim: int) -> int:
     return 4 if head_dim <= 64 else (2 if head_dim <= 128 else 1)
 
 
-ATTENTION_TARGET_WAVES = 2048
 ATTENTION_MAX_SPLITS = 64
-ATTENTION_ENOUGH_WAVES = 512      # from here on the rows alone occupy the GPU
-ATTENTION_TILES_PER_WALK = 32     # 32-key tiles one wave should walk at most, if parts are to be had
+ATTENTION_PROMPT_GROUPS = 512     # workgroups a prompt step should bring: the longest walks run first, and
+                                  # with two rounds of workgroups the short ones fill in behind them
 ATTENTION_MAX_PROMPT_SPLITS = 8
-ATTENTION_SHARED_WALK = 1         # the same where a workgroup's waves share one tile's keys: a CU pulls
-                                  # only so much from memory, so few workgroups with long walks are slow
+ATTENTION_MIN_WALK = 4            # 32-key tiles a part of a prompt's keys should hold at least
+ATTENTION_SHARED_WALK = 1         # 32-key tiles a wave walks where a workgroup's waves share one tile's keys:
+                                  # a CU pulls only so much from memory, so few workgroups with long walks are slow
 ATTENTION_ENOUGH_GROUPS = 256     # workgroups of that kind from which on the keys are not cut further
 
 
@@ -478,9 +483,10 @@ def attention_shared_waves(head_dim: int) -> int:
 
 
 def attention_splits(n_tiles: int, n_heads: int, n_kv_heads: int, max_kv_len: int, shared_waves: int = 0) -> int:
-    """Into how many parts the keys are cut over workgroups so that the GPU has enough waves: none
-    if the rows alone fill it, else towards ATTENTION_TARGET_WAVES waves with at least one 32-key
-    tile each.  With ``shared_waves`` a workgroup's waves already cut a tile's keys between them;
+    """Into how many parts the keys are cut over workgroups so that the GPU has enough of them.
+    n_tiles counts waves' tiles.  Prompt forms (four waves a workgroup): towards
+    ATTENTION_PROMPT_GROUPS workgroups, while a part keeps ATTENTION_MIN_WALK tiles of 32 keys.
+    With ``shared_waves`` a workgroup is one tile whose waves already cut the keys between them;
     the keys are cut further only while a wave would walk more than ATTENTION_SHARED_WALK tiles."""
     group = n_heads // n_kv_heads
     waves = n_tiles * n_kv_heads * (-(-group // 16))
@@ -489,17 +495,18 @@ def attention_splits(n_tiles: int, n_heads: int, n_kv_heads: int, max_kv_len: in
         walk = -(-key_tiles // shared_waves)
         return max(1, min(-(-walk // ATTENTION_SHARED_WALK), ATTENTION_ENOUGH_GROUPS // max(waves, 1),
                           ATTENTION_MAX_SPLITS))
-    if waves >= ATTENTION_ENOUGH_WAVES:
-        # the rows alone occupy the GPU; what is left to shorten is the longest wave's walk over
-        # its keys, which bounds the kernel's time
-        return max(1, min(ATTENTION_MAX_PROMPT_SPLITS, -(-key_tiles // ATTENTION_TILES_PER_WALK)))
-    return max(1, min(ATTENTION_TARGET_WAVES // max(waves, 1), key_tiles, ATTENTION_MAX_SPLITS))
+    groups = max(1, -(-waves // ATTENTION_STAGED_WAVES))
+    return max(1, min(-(-ATTENTION_PROMPT_GROUPS // groups), ATTENTION_MAX_PROMPT_SPLITS,
+                      key_tiles // ATTENTION_MIN_WALK))
 
 
 def attention_mfma(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                    seq_start: torch.Tensor, seq_ctx: torch.Tensor, tile_start: torch.Tensor, n_tiles: int,
                    n_heads: int, n_kv_heads: int, head_dim: int, window: int, scale: float,
-                   n_splits: int, q_tiles: int = 1, shared_tile: bool = False) -> torch.Tensor:
+                   n_splits: int, q_tiles: int = 1, form: int = 0) -> torch.Tensor:
+    """form 0: four independent waves a workgroup, tile_start counts pieces of q_tiles tiles; 1: one
+    tile a workgroup, its waves share the keys (q_tiles 1); 2: four waves a workgroup that walk their
+    keys together through LDS, tile_start counts pieces of 4 * q_tiles tiles (ATTENTION_STAGED_WAVES)."""
     _dev("attention_mfma", qkv, k_cache, v_cache, block_table, seq_start, seq_ctx, tile_start)
     t = qkv.shape[0]
     _check_queries("attention_mfma", qkv, n_heads, n_kv_heads, head_dim)
@@ -521,7 +528,7 @@ def attention_mfma(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
                  _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(seq_start), _ptr(seq_ctx),
                  _ptr(tile_start), n_seqs, n_tiles, t, n_heads, n_kv_heads, head_dim, k_cache.shape[2],
                  int(window), float(scale), attention_tile_tokens(n_heads, n_kv_heads), int(q_tiles),
-                 int(bool(shared_tile)), int(n_splits), _stream())
+                 int(form), int(n_splits), _stream())
     return out
 
 
@@ -534,13 +541,15 @@ def attention(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, b
         tpt = attention_tile_tokens(n_heads, n_kv_heads)
         # a wave takes several query tiles as soon as some request brings more than one tile of rows;
         # while every request brings one tile at most, a workgroup's waves share the tile's keys
+        # (else four waves with consecutive tiles of a request walk their keys together)
         shared = ctx.max_q_len <= tpt
         q_tiles = 1 if shared else attention_q_tiles(head_dim)
-        tile_start, n_tiles = ctx.attention_tiles(tpt * q_tiles)
+        waves = 1 if shared else ATTENTION_STAGED_WAVES
+        tile_start, n_tiles = ctx.attention_tiles(tpt * q_tiles * waves)
         n_splits = ctx.fixed_attention_splits or attention_splits(
-            n_tiles, n_heads, n_kv_heads, ctx.max_kv_len, attention_shared_waves(head_dim) if shared else 0)
+            n_tiles * waves, n_heads, n_kv_heads, ctx.max_kv_len, attention_shared_waves(head_dim) if shared else 0)
         return attention_mfma(qkv, k_cache, v_cache, block_table, ctx.seq_start_dev, ctx.seq_ctx_dev,
                               tile_start, n_tiles, n_heads, n_kv_heads, head_dim, window, scale, n_splits, q_tiles,
-                              shared)
+                              1 if shared else 2)
     return attention_generic(qkv, k_cache, v_cache, block_table, ctx.row_seq, ctx.positions,
                              n_heads, n_kv_heads, head_dim, window, scale)

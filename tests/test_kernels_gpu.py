@@ -318,9 +318,9 @@ def test_attention_generic(ops, nh, nkv, d, page, window):
         close(got, plain_result(case, window), what=f"generic {dt}", **tol)
 
 
-def run_mfma(ops, case, window, n_splits, q_tiles=1, shared=False):
+def run_mfma(ops, case, window, n_splits, q_tiles=1, shared=False, staged=False):
     nh, nkv, d = case["nh"], case["nkv"], case["d"]
-    tpt = ops.attention_tile_tokens(nh, nkv) * q_tiles
+    tpt = ops.attention_tile_tokens(nh, nkv) * q_tiles * (ops.ATTENTION_STAGED_WAVES if staged else 1)
     starts = [0]
     for s in range(len(case["seq_ctx"])):
         starts.append(starts[-1] + -(-(case["seq_start"][s + 1] - case["seq_start"][s]) // tpt))
@@ -328,7 +328,7 @@ def run_mfma(ops, case, window, n_splits, q_tiles=1, shared=False):
     kc, vc = ops.cache_from_plain(case["kc"], case["vc"])      # the layout the writers leave for these sizes
     return ops.attention_mfma(case["qkv"], kc, vc, case["table"], dev(case["seq_start"]),
                               dev(case["seq_ctx"]), dev(starts), starts[-1], nh, nkv, d, window,
-                              1.0 / math.sqrt(d), n_splits, q_tiles, shared)
+                              1.0 / math.sqrt(d), n_splits, q_tiles, 2 if staged else int(shared))
 
 
 @pytest.mark.parametrize("nh,nkv,d,page", SHAPES)
@@ -345,6 +345,12 @@ def test_attention_mfma(ops, nh, nkv, d, page, window, n_splits):
         close(again, plain_result(case, window), rtol=2e-2, atol=2e-2, what="mfma, several tiles a wave")
         if n_splits == 1:   # (with split keys the parts are cut elsewhere: equal up to rounding only)
             assert torch.equal(again, got), "a row's result must not depend on how rows are grouped into waves"
+    # four waves of a workgroup walking their keys together through LDS (the form prompts use)
+    for qt in sorted({1, many}):
+        staged = run_mfma(ops, case, window, n_splits, qt, staged=True)
+        close(staged, plain_result(case, window), rtol=2e-2, atol=2e-2, what=f"mfma, key tiles staged in LDS, {qt} tiles a wave")
+        if n_splits == 1:   # the same keys in the same order for every row: the same bits
+            assert torch.equal(staged, got), "a row's result must not depend on which waves share its keys"
     # a workgroup's waves sharing one tile's keys (the form decoded tokens use)
     close(run_mfma(ops, case, window, n_splits, shared=True), plain_result(case, window), rtol=2e-2, atol=2e-2,
           what="mfma, keys shared between a workgroup's waves")
@@ -360,6 +366,7 @@ def test_attention_far_key_among_hundreds(ops, n_splits):
         want = plain_result(case)
         if fn == "mfma":
             got = run_mfma(ops, case, 0, n_splits)
+            close(run_mfma(ops, case, 0, n_splits, 4, staged=True), want, rtol=2e-2, atol=2e-2, what="mfma, staged keys")
             shared = run_mfma(ops, case, 0, n_splits, shared=True)
             close(shared, want, rtol=2e-2, atol=2e-2, what="mfma, shared keys")
             assert float((shared[419].double().cpu().view(4, 64)[1] - case["wants"][0][2][3, 0]).abs().max()) < 0.05
@@ -379,6 +386,8 @@ def test_attention_window_edge(ops):
         close(run_mfma(ops, case, window, 1), plain_result(case, window), rtol=2e-2, atol=2e-2, what=f"window {window}")
         close(run_mfma(ops, case, window, 1, shared=True), plain_result(case, window), rtol=2e-2, atol=2e-2,
               what=f"window {window}, shared keys")
+        close(run_mfma(ops, case, window, 1, ops.attention_q_tiles(32), staged=True), plain_result(case, window), rtol=2e-2, atol=2e-2,
+              what=f"window {window}, staged keys")
 
 
 def test_argmax_ties_and_sampling(ops):
