@@ -209,16 +209,30 @@ __global__ void rope_table_kernel(const int32_t* __restrict__ positions, float2*
 template <typename T>
 __global__ void rope_kv_write_blocks_kernel(T* __restrict__ qkv, const float2* __restrict__ table,
                                             const int32_t* __restrict__ slot_map, T* __restrict__ k_cache,
-                                            T* __restrict__ v_cache, long total, int n_heads, int n_kv_heads,
-                                            int head_dim, int rotate, int page_tokens, int write_kv, int frag) {
+                                            T* __restrict__ v_cache, long total, long n_tokens, int n_heads,
+                                            int n_kv_heads, int head_dim, int rotate, int page_tokens, int write_kv,
+                                            int frag) {
   const int blocks = head_dim / 16;
   const int heads_total = n_heads + 2 * n_kv_heads;
   const long stride = static_cast<long>(blockDim.x) * gridDim.x;
+  // Items of the query heads first, a row's blocks next to each other (they are rotated in place);
+  // then those of the key and value heads with 16 consecutive rows next to each other: in a cache in
+  // fragment order the same 8 dimensions of 16 consecutive tokens lie together.
+  const long q_items = n_tokens * n_heads * blocks;
   for (long idx = blockIdx.x * static_cast<long>(blockDim.x) + threadIdx.x; idx < total; idx += stride) {
-    const int b = static_cast<int>(idx % blocks);
-    const long rest = idx / blocks;
-    const int head = static_cast<int>(rest % heads_total);
-    const long token = rest / heads_total;
+    int b, head;
+    long token;
+    if (idx < q_items) {
+      b = static_cast<int>(idx % blocks);
+      head = static_cast<int>((idx / blocks) % n_heads);
+      token = idx / (static_cast<long>(blocks) * n_heads);
+    } else {
+      const long j = idx - q_items;
+      b = static_cast<int>((j / 16) % blocks);
+      head = n_heads + static_cast<int>((j / (16 * blocks)) % (2 * n_kv_heads));
+      token = (j / (16L * blocks * 2 * n_kv_heads)) * 16 + j % 16;
+      if (token >= n_tokens) continue;
+    }
     const bool is_q = head < n_heads, is_v = head >= n_heads + n_kv_heads;
     if (!is_q && !write_kv) continue;
     T* src = qkv + (token * heads_total + head) * head_dim + 16 * b;
@@ -538,16 +552,17 @@ extern "C" int bc4g_rope_kv_write_blocks(void* qkv, int dtype, const float* tabl
   BC4G_REQUIRE(!rotate || table, "rope_kv_write_blocks: rotation needs the table of angles");
   if (n_tokens == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const long total = static_cast<long>(n_tokens) * (n_heads + 2 * n_kv_heads) * (head_dim / 16);
+  // (the key and value heads' items are counted for whole groups of 16 rows)
+  const long total = (static_cast<long>(n_tokens) * n_heads + ((n_tokens + 15) / 16) * 16L * 2 * n_kv_heads) * (head_dim / 16);
   const float2* tab = reinterpret_cast<const float2*>(table);
   if (dtype == kF32) {
     rope_kv_write_blocks_kernel<float><<<grid_for(total), kBlock, 0, s>>>(
         static_cast<float*>(qkv), tab, slot_map, static_cast<float*>(k_cache), static_cast<float*>(v_cache), total,
-        n_heads, n_kv_heads, head_dim, rotate, page_tokens, write_kv, 0);
+        n_tokens, n_heads, n_kv_heads, head_dim, rotate, page_tokens, write_kv, 0);
   } else if (dtype == kBF16) {
     rope_kv_write_blocks_kernel<bf16_t><<<grid_for(total), kBlock, 0, s>>>(
         static_cast<bf16_t*>(qkv), tab, slot_map, static_cast<bf16_t*>(k_cache), static_cast<bf16_t*>(v_cache), total,
-        n_heads, n_kv_heads, head_dim, rotate, page_tokens, write_kv,
+        n_tokens, n_heads, n_kv_heads, head_dim, rotate, page_tokens, write_kv,
         cache_fragment_order(true, head_dim, page_tokens) ? 1 : 0);
   } else {
     return fail("rope_kv_write_blocks: unknown dtype %d", dtype);
