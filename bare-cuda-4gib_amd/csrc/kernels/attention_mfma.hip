@@ -18,8 +18,8 @@
 // cache into LDS once (a straight copy: the pages are in operand order already) and every wave
 // takes its operands from there, so a key is fetched once for 4 * QT * 16 query rows; the next
 // tile's loads are in flight during the arithmetic, and there is one barrier a tile.  (WS == 1 is
-// the same without LDS, four independent waves: kept for comparison and for tiles of different
-// requests in one workgroup.)
+// the same without LDS, four independent waves each fetching its own keys: the simpler form, kept as
+// a cross-check -- both give the same bits.)
 // Decoded tokens bring few tiles and long key walks: there a workgroup is one tile and its WS
 // waves cut the tile's keys between them, then combine their partial results in LDS (in wave
 // order).  On top of that, with n_splits > 1 the key range is cut into that many parts over

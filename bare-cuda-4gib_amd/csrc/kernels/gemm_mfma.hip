@@ -10,6 +10,11 @@
 // Rows and columns beyond the matrix are read as zero and not stored; k must be a multiple of 8.
 // Every output element is accumulated over k in ascending order, whatever the number of rows.
 //
+// What bounds this kernel is not the matrix cores but what a CU can pull through its cache: at
+// 128 x 128 a k-step of 64 brings 32 KB for 2 MFLOP, and 256 CUs doing so reach ~10 TB/s together
+// (measured: ~650 TFLOP/s).  Where the output has tiles enough, a workgroup of 8 waves therefore
+// takes a 256 x 128 tile (the same waves a CU, the same per-wave work, a quarter less traffic).
+//
 // Workgroups are numbered so that those sharing a tile of w run on the same XCD (workgroups are
 // dealt to the 8 XCDs in turn, each with an L2 of its own).
 #include <math.h>
@@ -95,14 +100,25 @@ __device__ inline void store_tile(const float* tile_out, void* __restrict__ out,
 }
 
 // SETS: register sets; SETS - 1 k-steps are in flight from memory while one is written to LDS.
-template <int EPI, int SETS>
-__global__ __launch_bounds__(256, 2) void gemm_mfma_kernel(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
-                                                           void* __restrict__ out, int m, int n, int k,
-                                                           int m_blocks, int n_blocks) {
+// WMS: rows of waves (64 output rows each) -- 2 for the 128 x 128 tile, 4 for the 256 x 128 one.
+template <int WMS>
+struct TileOf {
+  bf16_t a[64 * WMS][kLdsStride];
+  bf16_t w[kBN][kLdsStride];
+};
+
+template <int EPI, int SETS, int WMS>
+__global__ __launch_bounds__(128 * WMS, WMS == 2 ? 2 : 1) void gemm_mfma_kernel(
+    const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, void* __restrict__ out, int m, int n, int k,
+    int m_blocks, int n_blocks) {
+  constexpr int kRows = 64 * WMS, kThreads = 128 * WMS;
+  constexpr int kChunkRows = kThreads / 8;           // rows one chunk of a thread's loads covers
+  constexpr int kChunksA = kRows / kChunkRows, kChunksW = kBN / kChunkRows;
+  typedef TileOf<WMS> Tile;
   __shared__ __align__(16) unsigned char lds_raw[sizeof(Tile) * 2];
   Tile* tiles = reinterpret_cast<Tile*>(lds_raw);
   const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
-  const int wm = wave / 2, wn = wave % 2;   // this wave's 64 x 64 quarter
+  const int wm = wave / 2, wn = wave % 2;   // this wave's 64 x 64 part
 
   // XCD-aware numbering: consecutive logical ids stay on one XCD; m runs fastest so that
   // neighbours share a tile of w.
@@ -110,34 +126,39 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_kernel(const bf16_t* __restr
   int logical = blockIdx.x;
   if (total % kXcds == 0) logical = (blockIdx.x % kXcds) * (total / kXcds) + blockIdx.x / kXcds;
   const int bm = logical % m_blocks, bn = logical / m_blocks;
-  const long m0 = static_cast<long>(bm) * kBM, n0 = static_cast<long>(bn) * kBN;
+  const long m0 = static_cast<long>(bm) * kRows, n0 = static_cast<long>(bn) * kBN;
 
-  // global -> LDS: a tile is 128 rows x 8 segments of 16 bytes; thread t moves segment t%8 of rows
-  // t/8 + 32 i (chunk i = 0..3 of each operand).
+  // global -> LDS: a tile's rows are 8 segments of 16 bytes; thread t moves segment t%8 of rows
+  // t/8 + kChunkRows * i (chunk i of each operand; chunks 0..3 carry both where both have as many).
   const int seg = tid % 8, lrow = tid / 8;
   struct Staged {
-    uint4 a[4], w[4];
+    uint4 a[kChunksA], w[kChunksW];
   };
-  const bf16_t* arow[4];
-  const bf16_t* wrow[4];
-  bool a_ok[4], w_ok[4];
+  const bf16_t* arow[kChunksA];
+  const bf16_t* wrow[kChunksW];
+  bool a_ok[kChunksA], w_ok[kChunksW];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const long gm = m0 + lrow + 32 * i, gn = n0 + lrow + 32 * i;
+  for (int i = 0; i < kChunksA; ++i) {
+    const long gm = m0 + lrow + kChunkRows * i;
     a_ok[i] = gm < m;
-    w_ok[i] = gn < n;
     arow[i] = a + (a_ok[i] ? gm : 0) * k + seg * 8;
+  }
+#pragma unroll
+  for (int i = 0; i < kChunksW; ++i) {
+    const long gn = n0 + lrow + kChunkRows * i;
+    w_ok[i] = gn < n;
     wrow[i] = w + (w_ok[i] ? gn : 0) * k + seg * 8;
   }
+  static_assert(kChunksA == 4, "the loop below moves four chunks a k-step");
   auto load_chunk = [&](Staged& r, int kt, int i) {
     const int kk = kt * kBK;
     const bool k_ok = kk + seg * 8 < k;
     r.a[i] = (k_ok && a_ok[i]) ? load16(arow[i] + kk) : zero16();
-    r.w[i] = (k_ok && w_ok[i]) ? load16(wrow[i] + kk) : zero16();
+    if (i < kChunksW) r.w[i] = (k_ok && w_ok[i]) ? load16(wrow[i] + kk) : zero16();
   };
   auto store_chunk = [&](const Staged& r, int buf, int i) {
-    *reinterpret_cast<uint4*>(&tiles[buf].a[lrow + 32 * i][seg * 8]) = r.a[i];
-    *reinterpret_cast<uint4*>(&tiles[buf].w[lrow + 32 * i][seg * 8]) = r.w[i];
+    *reinterpret_cast<uint4*>(&tiles[buf].a[lrow + kChunkRows * i][seg * 8]) = r.a[i];
+    if (i < kChunksW) *reinterpret_cast<uint4*>(&tiles[buf].w[lrow + kChunkRows * i][seg * 8]) = r.w[i];
   };
 
   floatx16 acc[2][2];
@@ -179,19 +200,24 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_kernel(const bf16_t* __restr
       if (t >= nk) break;
       const int cur = j % 2;
       const bool st = t + 1 < nk;
+      // all the k-step's fragments are asked for at once: LDS answers in order, so the MFMAs of the
+      // first slice start when its four reads are back while the other twelve are on their way
+      uint4 fa[kBK / 16][2], fw[kBK / 16][2];
 #pragma unroll
-      for (int ks = 0; ks < kBK / 16; ++ks) {
-        uint4 fa[2], fw[2];
+      for (int ks = 0; ks < kBK / 16; ++ks)
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
-          fa[i] = *reinterpret_cast<const uint4*>(&tiles[cur].a[wm * 64 + i * 32 + frow][ks * 16 + fk]);
-          fw[i] = *reinterpret_cast<const uint4*>(&tiles[cur].w[wn * 64 + i * 32 + frow][ks * 16 + fk]);
+          fa[ks][i] = *reinterpret_cast<const uint4*>(&tiles[cur].a[wm * 64 + i * 32 + frow][ks * 16 + fk]);
+          fw[ks][i] = *reinterpret_cast<const uint4*>(&tiles[cur].w[wn * 64 + i * 32 + frow][ks * 16 + fk]);
         }
+      __builtin_amdgcn_sched_group_barrier(0x100, 16, 0);   // the 16 LDS reads first
+#pragma unroll
+      for (int ks = 0; ks < kBK / 16; ++ks)
 #pragma unroll
         for (int i = 0; i < 2; ++i)
 #pragma unroll
-          for (int jj = 0; jj < 2; ++jj) acc[i][jj] = mfma_32x32x16(fa[i], fw[jj], acc[i][jj]);
-      }
+          for (int jj = 0; jj < 2; ++jj) acc[i][jj] = mfma_32x32x16(fa[ks][i], fw[ks][jj], acc[i][jj]);
+      __builtin_amdgcn_sched_group_barrier(0x008, 16, 0);   // then the 16 MFMAs
       if (st) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) store_chunk(r[(j + 1) % SETS], 1 - cur, i);
@@ -204,22 +230,28 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_kernel(const bf16_t* __restr
     }
   }
 
-  // The tile goes out through LDS (as float [128][128 + 4]), so that a thread stores four
-  // neighbouring columns of a row at once.  acc[i][j][r] is row wm*64 + i*32 + 8*(r/4) +
+  // The tile goes out through LDS (as float [128][128 + 4], 128 rows at a time), so that a thread
+  // stores four neighbouring columns of a row at once.  acc[i][j][r] is row wm*64 + i*32 + 8*(r/4) +
   // 4*(lane/32) + r%4 and column wn*64 + j*32 + lane%32 of the tile.
   constexpr int kOutStride = kBN + 4;
   static_assert(sizeof(float) * kBM * kOutStride <= sizeof(Tile) * 2, "the output tile must fit the operand buffers");
   float* tile_out = reinterpret_cast<float*>(lds_raw);
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int half = 0; half < WMS / 2; ++half) {
+    if (half > 0) lds_barrier();                      // the half before has been read
+    if (wm / 2 == half) {
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+      for (int i = 0; i < 2; ++i)
 #pragma unroll
-      for (int r = 0; r < 16; ++r)
-        tile_out[(wm * 64 + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + r % 4) * kOutStride + wn * 64 + j * 32 + lane % 32] =
-            acc[i][j][r];
-  lds_barrier();
-  store_tile<EPI, 256>(tile_out, out, m, n, m0, n0, tid);
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            tile_out[((wm % 2) * 64 + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + r % 4) * kOutStride + wn * 64 + j * 32 +
+                     lane % 32] = acc[i][j][r];
+    }
+    lds_barrier();
+    store_tile<EPI, kThreads>(tile_out, out, m, n, m0 + 128 * half, n0, tid);
+  }
 }
 
 // The same product with the work split between waves: four waves only multiply, eight only move
@@ -382,6 +414,14 @@ int compute_units() {
 template <int EPI>
 void launch_tiled(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, int k, long m_blocks, long n_blocks,
                   hipStream_t s) {
+  // With tiles enough for every CU to have two of them and more, the 256 x 128 tile: a quarter less
+  // traffic per FLOP, which is what bounds this kernel.
+  const long tall_blocks = (m + 255) / 256;
+  if (tall_blocks * n_blocks >= 2L * compute_units()) {
+    gemm_mfma_kernel<EPI, 2, 4><<<dim3(static_cast<unsigned>(tall_blocks * n_blocks)), dim3(512), 0, s>>>(
+        ap, wp, out, m, n, k, static_cast<int>(tall_blocks), static_cast<int>(n_blocks));
+    return;
+  }
   dim3 grid(static_cast<unsigned>(m_blocks * n_blocks)), block(256);
   // With at most one tile a CU nothing else runs beside a workgroup: then the split form, whose
   // moving and multiplying waves overlap, is the faster one (measured: 29 against 35 us for
@@ -390,7 +430,7 @@ void launch_tiled(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, i
     gemm_mfma_split_kernel<EPI><<<grid, dim3(kSplitThreads), 0, s>>>(ap, wp, out, m, n, k, m_blocks, n_blocks);
     return;
   }
-  gemm_mfma_kernel<EPI, 2><<<grid, block, 0, s>>>(ap, wp, out, m, n, k, m_blocks, n_blocks);
+  gemm_mfma_kernel<EPI, 2, 2><<<grid, block, 0, s>>>(ap, wp, out, m, n, k, m_blocks, n_blocks);
 }
 
 }  // namespace

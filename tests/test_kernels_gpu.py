@@ -134,8 +134,9 @@ def test_gemm_mfma(ops, m, n, k):
 
 def test_gemm_mfma_both_forms_agree_bit_for_bit(ops):
     """Few tiles go to the form with moving and multiplying waves, many to the plain one (two
-    workgroups a CU).  Both add over k in the same order: a row's result is the same bits
-    whichever form the number of rows selects, also for sizes that are no multiple of anything."""
+    workgroups a CU), very many to the one with 256 x 128 tiles.  All add over k in the same order:
+    a row's result is the same bits whichever form the number of rows selects, also for sizes that
+    are no multiple of anything."""
     n, k = 2060, 200                                    # 17 tiles across
     a, w = bf(rnd(2500, k, seed=40)), bf(rnd(n, k, seed=41))
     wd = w.to(DEV)
@@ -150,6 +151,16 @@ def test_gemm_mfma_both_forms_agree_bit_for_bit(ops):
     ops.gemm_fast(a.to(DEV), wd, accumulate_into=acc_many)
     ops.gemm_fast(a[:300].contiguous().to(DEV), wd, accumulate_into=acc_few)
     assert torch.equal(acc_few, acc_many[:300])
+    # 7,700 rows: 31 x 17 tiles of 256 x 128, the last of them with 20 rows and 12 columns
+    big = torch.cat([a, bf(rnd(5200, k, seed=42))]).to(DEV)
+    most = ops.gemm_fast(big, wd, torch.float32)
+    assert torch.equal(most[:2500], many)
+    close(most[2500:], big[2500:].double().cpu() @ w.double().T, 1e-4, 2e-3, "very many tiles")
+    assert torch.equal(ops.gemm_swiglu(big, gate_up.to(DEV), interleaved=True)[:2500], g)
+    acc_most = torch.ones(7700, n, device=DEV)
+    ops.gemm_fast(big, wd, accumulate_into=acc_most)
+    assert torch.equal(acc_most[:2500], acc_many)
+    assert torch.equal(ops.gemm_fast(big, wd, torch.bfloat16)[:2500], ops.gemm_fast(a.to(DEV), wd, torch.bfloat16))
 
 
 def test_gemm_mfma_xcd_numbering_covers_every_tile(ops):
