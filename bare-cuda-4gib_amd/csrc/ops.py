@@ -348,14 +348,20 @@ def gemm_fast(a: torch.Tensor, w, out_dtype=None,
 
 
 NORMED_MAX_ROWS = 16
+NORMED_STAGE_BYTES = 96 * 1024      # LDS the fused norm may fill with its rows of bf16(x * g)
+
+
+def _normed_rows_fit(n_rows: int, k: int) -> bool:
+    """Whether the rows a fused RMSNorm stages in LDS (rounded up to 4, each k + 8 bfloat16) fit there:
+    16 rows do up to k = 3,064, 8 rows up to 6,136."""
+    return 0 < n_rows <= NORMED_MAX_ROWS and (-(-n_rows // 4) * 4) * (k + 8) * 2 <= NORMED_STAGE_BYTES
 
 
 def gemm_normed_supported(x: torch.Tensor, n_rows: int, g: torch.Tensor, w) -> bool:
     """Whether RMSNorm can be fused into the product: few rows, bfloat16 weights, k a multiple of 8."""
     w, _ = _weight(w)
-    staged = (-(-n_rows // 4) * 4) * (x.shape[1] + 8) * 2          # bytes of LDS the normed rows take
-    return (x.is_cuda and x.dtype == torch.float32 and w.dtype == torch.bfloat16 and 0 < n_rows <= NORMED_MAX_ROWS
-            and x.shape[1] == w.shape[1] and x.shape[1] % 8 == 0 and g.dtype in _CODE and staged <= 96 * 1024)
+    return (x.is_cuda and x.dtype == torch.float32 and w.dtype == torch.bfloat16 and _normed_rows_fit(n_rows, x.shape[1])
+            and x.shape[1] == w.shape[1] and x.shape[1] % 8 == 0 and g.dtype in _CODE)
 
 
 def gemm_normed(x: torch.Tensor, rows: Optional[torch.Tensor], n_rows: int, g: torch.Tensor, eps: float,
@@ -412,7 +418,7 @@ def gemm_qkv_rope_supported(x: torch.Tensor, n_rows: int, normed: bool, w, head_
                             rotary_dim: int) -> bool:
     """Whether the q|k|v product of these rows can rotate and write the cache in its epilogue."""
     w, _ = _weight(w)
-    rows_ok = n_rows <= (NORMED_MAX_ROWS if normed else SKINNY_MAX_ROWS)
+    rows_ok = _normed_rows_fit(n_rows, x.shape[1]) if normed else n_rows <= SKINNY_MAX_ROWS
     return (x.is_cuda and w.dtype == torch.bfloat16 and x.shape[1] % 8 == 0 and 0 < n_rows and rows_ok
             and head_dim % 16 == 0 and rotary_dim in (0, head_dim)
             and x.dtype == (torch.float32 if normed else torch.bfloat16))

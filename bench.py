@@ -8,6 +8,11 @@ weights, a batch of 8 requests with 512-token prompts, and times K decode steps 
 token for every request through the engine's step function, greedy choice on the device, the
 chosen ids read back).  It prints ONE JSON line: decoded tokens a second, the prefill of one
 2,048-token prompt, the decode step against the HBM roofline, and decoding at batch 1 and 64.
+
+Beside the headline: `--shape` runs the same measurements at the sizes of Llama-2-7B or Llama-3-8B;
+`--only decode|prefill` runs one part and prints a short line of its own (what the profiles use);
+`--only serve` submits `--requests` requests of mixed lengths to the scheduler and times the whole
+run, prompts in portions of `--chunk` tokens beside the others' decoded tokens.
 """
 import argparse
 import json
@@ -137,6 +142,50 @@ def run_prefill(model, cfg, tokens, runs=3, seed=2):
     return best
 
 
+def run_serve(model, cfg, n_requests, new_tokens, chunk, seed=3):
+    """A mixed batch through the scheduler: n_requests submitted at once, prompt lengths uniform in
+    [128, max context - new_tokens], prompts cut into portions of `chunk` tokens beside the decoded
+    tokens of the others, temperature 1.0.  Returns (seconds, scheduler statistics)."""
+    import torch
+    from bare_cuda_4gib_amd.engine import Executor
+    from bare_cuda_4gib_amd.engine.scheduler import Request, Scheduler
+    from bare_cuda_4gib_amd.sampling.device import DevicePicker
+    from bare_cuda_4gib_amd.sampling.params import SamplingParams
+    page = 64
+    longest = min(cfg.max_seq_len - new_tokens, 4096)
+    gen = torch.Generator().manual_seed(seed)
+    lengths = torch.randint(128, longest + 1, (n_requests,), generator=gen).tolist()
+    pages = sum(-(-(n + new_tokens) // page) for n in lengths)
+    ex = Executor(model, num_pages=pages, max_requests=n_requests, max_tokens=cfg.max_seq_len, page_tokens=page,
+                  max_batch_tokens=2048)
+    sched = Scheduler(ex, DevicePicker(), max_batch_tokens=2048, prefill_chunk=chunk)
+
+    def submit_all(tag):
+        for i, n in enumerate(lengths):
+            prompt = torch.randint(0, cfg.vocab_size, (n,), generator=gen).tolist()
+            sched.submit(Request(id=tag * n_requests + i, prompt=prompt, max_new_tokens=new_tokens,
+                                 sampling=SamplingParams(temperature=1.0, seed=i)))
+
+    def drain():
+        made = 0
+        while not sched.idle():
+            made += sum(1 for e in sched.step() if e.token >= 0)
+        return made
+
+    submit_all(0)                     # once untimed: graphs are captured, buffers made
+    drain()
+    before = sched.stats()
+    submit_all(1)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    made = drain()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    after = sched.stats()
+    return dt, dict(requests=n_requests, generated=made, prompt_tokens=sum(lengths),
+                    steps=after.steps - before.steps, preemptions=after.preemptions - before.preemptions)
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -150,7 +199,10 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="fewer than the shape has only where time needs it")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--no-points", action="store_true", help="skip decoding at batch 1 and 64")
-    ap.add_argument("--only", choices=["decode", "prefill"], default=None,
+    ap.add_argument("--requests", type=int, default=64, help="--only serve: requests submitted at once")
+    ap.add_argument("--new-tokens", type=int, default=256, help="--only serve: tokens generated per request")
+    ap.add_argument("--chunk", type=int, default=512, help="--only serve: prompt portion size")
+    ap.add_argument("--only", choices=["decode", "prefill", "serve"], default=None,
                     help="run one part only and print its own short line (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -182,6 +234,13 @@ def main() -> int:
         print(json.dumps({"only": "prefill", "shape": args.shape, "tokens": args.prefill_tokens,
                           "ms": round(pre_s * 1e3, 3), "frac": round(frac, 4),
                           "tokens_per_s": round(args.prefill_tokens / pre_s, 1)}), flush=True)
+        return 0
+
+    if args.only == "serve":
+        dt, st = run_serve(model, cfg, args.requests, args.new_tokens, args.chunk)
+        print(json.dumps(dict(only="serve", shape=args.shape, **st, seconds=round(dt, 3),
+                              generated_per_s=round(st["generated"] / dt, 1),
+                              all_tokens_per_s=round((st["generated"] + st["prompt_tokens"]) / dt, 1))), flush=True)
         return 0
 
     dt, contexts = run_decode(model, cfg, args.batch, args.prompt_len, args.steps, args.warmup)

@@ -76,3 +76,33 @@ def test_sizes_through_the_engine(made, name, dtype):
         got = helpers.replay_in_process(ex, steps)
         helpers.compare_with_plain(got, where, plain, label=f"{label} {name} {dtype}", **TOL[dtype])
         assert ex.cache.pages_in_use() == 0
+
+
+def test_sixteen_decoded_rows_at_a_width_whose_fused_norm_does_not_fit(tmp_path):
+    """Hidden size 4,096: sixteen rows of it do not fit the LDS buffer of the product with the norm
+    fused (eight do), so a step of sixteen decoded tokens takes the norm and the product apart --
+    and gives the plain implementation's logits, like a step of eight."""
+    import torch
+    from bare_cuda_4gib_amd.csrc import ops
+    from bare_cuda_4gib_amd.engine import Executor, StepEntry, load_model
+    from bare_cuda_4gib_amd.weights import write_random_model
+    cfg = _cfg(vocab_size=72, hidden_size=4096, num_attention_heads=2, num_key_value_heads=1, head_dim=64,
+               intermediate_size=48, num_hidden_layers=1)
+    folder = os.path.join(str(tmp_path), "wide")
+    write_random_model(cfg, 5, folder, "bfloat16", std=0.01)
+    x = torch.zeros(16, 4096, device="cuda")
+    w = torch.zeros(256, 4096, dtype=torch.bfloat16, device="cuda")
+    assert ops.gemm_qkv_rope_supported(x[:8], 8, True, w, 64, 64) and not ops.gemm_qkv_rope_supported(x, 16, True, w, 64, 64)
+    assert ops.gemm_normed_supported(x[:8], 8, w[0], w) and not ops.gemm_normed_supported(x, 16, w[0], w)
+    plain = PlainLlama(folder)
+    model, _ = load_model(folder, "bfloat16", "cuda:0")
+    for n in (8, 16):
+        ex = Executor(model, num_pages=n, max_requests=n, max_tokens=64, page_tokens=64)
+        prompts = [helpers.random_ids(3 + i % 5, 72, 500 + i) for i in range(n)]
+        for i, ids in enumerate(prompts):
+            ex.admit(i)
+            ex.step([StepEntry(i, ids[:-1], [])])
+        got = ex.step([StepEntry(i, ids[-1:], [0]) for i, ids in enumerate(prompts)]).float().cpu().numpy()
+        for i, ids in enumerate(prompts):
+            want = plain.logits(ids).numpy()[-1]
+            assert abs(got[i] - want).max() <= 6e-3 + 2e-2 * abs(want).max(), f"{n} rows, request {i}"
