@@ -390,6 +390,30 @@ def test_attention_far_key_among_hundreds(ops, n_splits):
         assert float((last - v_far).abs().max()) < 0.05, "the far key's value must dominate"
 
 
+@pytest.mark.parametrize("nh,nkv,d,page", [(8, 2, 128, 64), (16, 2, 64, 16)])
+def test_attention_long_context(ops, nh, nkv, d, page):
+    """A whole prompt of 2,200 tokens, a portion of 40 after 2,100 cached ones, single tokens after
+    2,177 and 1,030: hundreds of key tiles a row, the block table beyond one register a lane for the
+    small pages, a window that ends inside the cached part; every form and several ways to cut the keys."""
+    seqs = [(0, 2200), (2100, 40), (2177, 1), (1030, 1)]
+    case = paged_case(seqs, nh, nkv, d, page, torch.bfloat16, seed=12, poison=False)
+    qt = ops.attention_q_tiles(d)
+    for window in (0, 700):
+        want = plain_result(case, window)
+        for n_splits in (1, 8):
+            close(run_mfma(ops, case, window, n_splits, qt, staged=True), want, rtol=2e-2, atol=2e-2,
+                  what=f"staged, window {window}, {n_splits} parts")
+            close(run_mfma(ops, case, window, n_splits, qt), want, rtol=2e-2, atol=2e-2,
+                  what=f"independent waves, window {window}, {n_splits} parts")
+    # (4,300 tokens in pages of 16 are 269 pages: more than the 256 table entries a wave keeps in its lanes)
+    more = [(2199, 1)] + ([(4300, 2)] if page == 16 else [])
+    decode = paged_case(seqs[2:] + more, nh, nkv, d, page, torch.bfloat16, seed=13, poison=False)
+    for window in (0, 700):
+        for n_splits in (1, 5, 64):
+            close(run_mfma(ops, decode, window, n_splits, shared=True), plain_result(decode, window), rtol=2e-2, atol=2e-2,
+                  what=f"shared keys, window {window}, {n_splits} parts")
+
+
 def test_attention_window_edge(ops):
     """Keys exactly at the window's edge: position p sees p - window + 1 but not p - window."""
     case = paged_case([(0, 50)], 2, 1, 32, 16, torch.bfloat16, seed=6, poison=False)

@@ -106,3 +106,38 @@ def test_sixteen_decoded_rows_at_a_width_whose_fused_norm_does_not_fit(tmp_path)
         for i, ids in enumerate(prompts):
             want = plain.logits(ids).numpy()[-1]
             assert abs(got[i] - want).max() <= 6e-3 + 2e-2 * abs(want).max(), f"{n} rows, request {i}"
+
+
+def test_one_layer_at_the_widths_of_an_8b_model(tmp_path):
+    """One layer with the widths of a large model -- hidden 4,096, 32 query / 8 key-value heads of
+    128, a feed-forward of 11,000 (no multiple of 16 x 16) -- so that every kernel meets its long
+    k and its many blocks: prompts of 64 requests in batches of sixteen, then all 64 decoded together,
+    then groups of 1, 8, 16, 17 and 22."""
+    from bare_cuda_4gib_amd.engine import Executor, StepEntry, load_model
+    from bare_cuda_4gib_amd.weights import write_random_model
+    cfg = _cfg(vocab_size=1000, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+               intermediate_size=11000, num_hidden_layers=1)
+    folder = os.path.join(str(tmp_path), "wide8b")
+    write_random_model(cfg, 9, folder, "bfloat16", std=0.008)
+    plain = PlainLlama(folder)
+    model, _ = load_model(folder, "bfloat16", "cuda:0")
+    n = 64
+    prompts = [helpers.random_ids(4 + (7 * i) % 37, 1000, 700 + i) for i in range(n)]
+    want = [plain.logits(ids).numpy() for ids in prompts]
+    ex = Executor(model, num_pages=n, max_requests=n, max_tokens=64, page_tokens=64, max_batch_tokens=1024)
+    for lo in range(0, n, 16):                        # prompts but for their last two tokens, sixteen requests a step
+        for i in range(lo, lo + 16):
+            ex.admit(i)
+        ex.step([StepEntry(i, prompts[i][:-2], []) for i in range(lo, lo + 16)])
+
+    def check(got, ids, at):
+        got = got.float().cpu().numpy()
+        for row, i in enumerate(ids):
+            w = want[i][at]
+            assert abs(got[row] - w).max() <= 6e-3 + 2e-2 * abs(w).max(), f"request {i}, token {at}, {len(ids)} rows"
+
+    everyone = list(range(n))
+    check(ex.step([StepEntry(i, prompts[i][-2:-1], [0]) for i in everyone]), everyone, -2)
+    for lo, hi in ((0, 1), (1, 9), (9, 25), (25, 42), (42, 64)):
+        ids = list(range(lo, hi))
+        check(ex.step([StepEntry(i, prompts[i][-1:], [0]) for i in ids]), ids, -1)
