@@ -26,6 +26,7 @@ from __future__ import annotations
 import dataclasses
 from typing import Any, Dict, Hashable, Iterable, List, Optional, Sequence, Tuple
 
+import numpy as np
 import torch
 
 from ..errors import EngineError, OutOfPages
@@ -110,6 +111,12 @@ class CacheManager:
                 raise EngineError(f"cache: stream {sid!r} has an unknown spec {spec!r}")
         self._requests: Dict[Hashable, _Request] = {}
         self._free_slots: List[int] = list(range(max_requests - 1, -1, -1))
+        # The same bookkeeping as arrays by request slot, for whoever describes a batch of many
+        # requests to the device without a Python loop over them: lengths, and every group's block
+        # tables as rows of a matrix (-1 where there is no page), kept in step with the lists above.
+        self.lengths_by_slot = np.zeros(max_requests, dtype=np.int32)
+        self.tables_by_slot: Dict[Hashable, np.ndarray] = {
+            g: np.full((max_requests, self.max_pages_per_request), -1, dtype=np.int32) for g in self.groups}
 
     # ---- requests ---------------------------------------------------------
     def has(self, request: Hashable) -> bool:
@@ -130,6 +137,7 @@ class CacheManager:
             raise EngineError(f"cache: all {self.max_requests} request slots are taken")
         slot = self._free_slots.pop()
         self._requests[request] = _Request(slot, self.groups)
+        self.lengths_by_slot[slot] = 0
         for view in self._views.values():
             if isinstance(view, StateView):
                 view.state[slot].zero_()
@@ -146,6 +154,13 @@ class CacheManager:
 
     def length(self, request: Hashable) -> int:
         return self._req(request).length
+
+    def slots(self, requests: Sequence[Hashable]) -> np.ndarray:
+        """The requests' slots as an array: the index into lengths_by_slot and tables_by_slot."""
+        try:
+            return np.fromiter((self._requests[r].slot for r in requests), dtype=np.int32, count=len(requests))
+        except KeyError as e:
+            raise EngineError(f"cache: unknown request {e.args[0]!r}") from None
 
     def table(self, group: Hashable, request: Hashable) -> List[int]:
         """The request's pages in token order (-1 where the window has passed)."""
@@ -175,6 +190,7 @@ class CacheManager:
         """
         seen = set()
         need: Dict[Hashable, int] = {g: 0 for g in self.groups}
+        short = False
         for request, n_new in asks:
             if request in seen:
                 raise EngineError(f"cache: request {request!r} appears twice in one reservation")
@@ -185,8 +201,13 @@ class CacheManager:
             if r.length + n_new > self.max_tokens:
                 raise EngineError(f"cache: request {request!r} would hold {r.length + n_new} tokens, "
                                   f"the cache is sized for {self.max_tokens} per request")
-            for g, n in self.new_pages_needed(request, n_new).items():
-                need[g] += n
+            want = -(-(r.length + n_new) // self.page_tokens)
+            for g, t in r.tables.items():
+                if len(t) < want:
+                    need[g] += want - len(t)
+                    short = True
+        if not short:
+            return
         for g, n in need.items():
             free = self.groups[g].pool.free_count
             if n > free:
@@ -199,6 +220,7 @@ class CacheManager:
                 while len(t) < want:
                     page = self.groups[g].pool.acquire()
                     assert page >= 0
+                    self.tables_by_slot[g][r.slot, len(t)] = page
                     t.append(page)
 
     def advance(self, request: Hashable, n_new: int) -> None:
@@ -209,6 +231,7 @@ class CacheManager:
                          r.length + n_new > min(len(t) for t in r.tables.values()) * self.page_tokens):
             raise EngineError(f"cache: request {request!r} advanced past its reserved pages")
         r.length += n_new
+        self.lengths_by_slot[r.slot] = r.length
         for g, t in r.tables.items():
             window = self.groups[g].window
             if window <= 0:
@@ -218,6 +241,7 @@ class CacheManager:
             for idx in range(r.released[g], min(first_needed, len(t))):
                 self._give_back(g, t[idx])
                 t[idx] = -1
+                self.tables_by_slot[g][r.slot, idx] = -1
             r.released[g] = max(r.released[g], min(first_needed, len(t)))
 
     def _give_back(self, group: Hashable, page: int) -> None:
@@ -237,6 +261,8 @@ class CacheManager:
             for page in t:
                 if page >= 0:
                     self._give_back(g, page)
+            self.tables_by_slot[g][r.slot, :len(t)] = -1
+        self.lengths_by_slot[r.slot] = 0
         self._free_slots.append(r.slot)
         del self._requests[request]
 

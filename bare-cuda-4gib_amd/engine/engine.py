@@ -63,7 +63,7 @@ class Engine:
                                  max_tokens=max_tokens, page_tokens=page_tokens,
                                  max_batch_tokens=max_batch_tokens)
         self.scheduler = Scheduler(self.executor, DevicePicker(), max_batch_tokens=max_batch_tokens,
-                                   prefill_chunk=prefill_chunk)
+                                   prefill_chunk=prefill_chunk, run_ahead=True)
         self._max_waiting = max_waiting
         self._outbox: Deque[Event] = collections.deque()
         self._live = set()

@@ -12,6 +12,7 @@ from __future__ import annotations
 import dataclasses
 from typing import Hashable, List, Optional, Sequence
 
+import numpy as np
 import torch
 
 from ..cache.manager import CacheManager
@@ -186,29 +187,46 @@ class Executor:
         return (self.use_graphs and len(entries) <= self.graph_max_batch
                 and all(len(e.tokens) == 1 for e in entries))
 
-    def _graph_step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def _graph_step(self, entries: Sequence[StepEntry], device_tokens: Optional[torch.Tensor] = None) -> torch.Tensor:
         """A step in which every request brings one token, replayed from a HIP graph captured
         for this batch size and context bucket.  Only the int32 batch description changes
         between replays; it is copied into the graph's own buffer first.  Logits of every row
         come back ([S, vocab]); the buffer is the graph's and is overwritten by its next replay."""
+        cache, P = self.cache, self.cache.page_tokens
         S = len(entries)
-        width = self.cache.max_pages_per_request
-        flat, layout, group_layout, host = self._host_arrays(entries, table_width=width, all_logits=True)
+        width = cache.max_pages_per_request
+        slots = cache.slots([e.request for e in entries])
+        ctx = cache.lengths_by_slot[slots]
         bucket = 256
-        while bucket < host["max_kv"]:
+        while bucket < int(ctx.max()) + 1:
             bucket *= 2
         key = (S, bucket)
         slot = self._graphs.get(key)
         if slot is None:
+            flat, layout, group_layout, host = self._host_arrays(entries, table_width=width, all_logits=True)
             slot = self._capture(key, flat, layout, group_layout, host, bucket)
         # a ring of pinned staging buffers, each with an event that says its copy has been done
         ring = slot["ring"]
         buf, view, event = ring[slot["next"] % len(ring)]
         slot["next"] += 1
         event.synchronize()
-        view[:] = flat
+        # What changes from step to step is written from the cache manager's arrays by slot, with no
+        # loop over the requests; what does not (rows 0..S-1 one per request) is in the buffers since
+        # the capture.  The layout is that of _host_arrays.
+        at = slot["at"]
+        view[0:S] = [e.tokens[0] for e in entries]
+        view[at["positions"]:at["positions"] + S] = ctx
+        view[at["seq_ctx"]:at["seq_ctx"] + S] = ctx
+        view[at["seq_slots"]:at["seq_slots"] + S] = slots
+        rows = slot["rows"]
+        for g, tables_at, slots_at in at["groups"]:
+            tables = cache.tables_by_slot[g][slots]
+            view[tables_at:tables_at + S * width] = tables.reshape(-1)
+            view[slots_at:slots_at + S] = tables[rows, ctx // P] * P + ctx % P
         slot["dev"].copy_(buf, non_blocking=True)
         event.record()
+        if device_tokens is not None:
+            slot["dev"][:S].copy_(device_tokens)
         slot["graph"].replay()
         return slot["logits"]
 
@@ -230,24 +248,45 @@ class Executor:
         ring = []
         for _ in range(4):
             buf = torch.empty(len(flat), dtype=torch.int32).pin_memory()
+            buf.numpy()[:] = flat
             event = torch.cuda.Event()
             event.record()
             ring.append((buf, buf.numpy(), event))
-        slot = dict(graph=graph, dev=dev, logits=logits, ring=ring, next=0)
+        # where the parts that change between steps lie in the flat array
+        at, off = {}, 0
+        for name, n in layout:
+            at[name] = off
+            off += n
+        at["groups"] = []
+        for g, width in group_layout:
+            at["groups"].append((g, off, off + S * width))
+            off += S * width + host["T"]
+        slot = dict(graph=graph, dev=dev, logits=logits, ring=ring, next=0, at=at, rows=np.arange(S))
         self._graphs[key] = slot
         return slot
 
-    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+    def step(self, entries: Sequence[StepEntry], device_tokens: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         """Run the entries as one batch.  Returns float32 logits
         [number of wanted places, vocab] on the device, in the order of the
         entries and of their ``want`` lists; None if nothing is wanted.
 
+        ``device_tokens`` (int32 on the device, one per entry): every entry brings one token, and it
+        is this tensor's -- what a sampling kernel has just chosen -- not the placeholder in the
+        entry.  The host can then describe the next step before it has seen the ids of this one,
+        and read them while the next step runs.  The ids must lie in the vocabulary: they are not
+        looked at on the host.
+
         Raises OutOfPages, with nothing changed, if the cache cannot hold the
         batch's tokens."""
         self._validate(entries)
+        if device_tokens is not None:
+            if (not device_tokens.is_cuda or device_tokens.dtype != torch.int32 or device_tokens.dim() != 1
+                    or device_tokens.numel() != len(entries) or any(len(e.tokens) != 1 for e in entries)):
+                raise EngineError("step: device_tokens must be int32 on the device, one for each entry, "
+                                  "and every entry must bring one (placeholder) token")
         self.cache.reserve([(e.request, len(e.tokens)) for e in entries])
         if self._graph_eligible(entries):
-            every = self._graph_step(entries)
+            every = self._graph_step(entries, device_tokens)
             wanted = [i for i, e in enumerate(entries) if len(e.want)]
             if not wanted:
                 logits = None
@@ -256,7 +295,10 @@ class Executor:
             else:
                 logits = every[torch.tensor(wanted, device=every.device)]
         else:
-            logits = self.model.forward(self.build_context(entries))
+            ctx = self.build_context(entries)
+            if device_tokens is not None:
+                ctx.token_ids.copy_(device_tokens)
+            logits = self.model.forward(ctx)
         for e in entries:
             self.cache.advance(e.request, len(e.tokens))
         return logits

@@ -126,11 +126,19 @@ class Scheduler:
     """
 
     def __init__(self, executor, picker, *, max_batch_tokens: int = 2048, prefill_chunk: int = 512,
-                 clock=time.monotonic):
+                 clock=time.monotonic, run_ahead: bool = False):
+        """``run_ahead``: while every running request is decoding and none can be admitted, the next
+        step is launched with its tokens taken from what the sampling kernel has just chosen, on
+        the device, before the host has read them; the host reads a step's tokens (and emits its
+        events) while the next step runs.  The tokens are the same; the events of a step come out
+        of the following call to step().  Needs a picker with ``pick_later`` and an executor whose
+        step takes ``device_tokens``."""
         if max_batch_tokens <= 0 or prefill_chunk <= 0:
             raise EngineError("scheduler: max_batch_tokens and prefill_chunk must be positive")
         self.executor = executor
         self.picker = picker
+        self.run_ahead = run_ahead
+        self._ahead = None                # (requests, picked): a step whose tokens have not been read yet
         self.max_batch_tokens = max_batch_tokens
         self.prefill_chunk = prefill_chunk
         self._clock = clock
@@ -180,7 +188,7 @@ class Scheduler:
         return False
 
     def idle(self) -> bool:
-        return not self.waiting and not self.running
+        return not self.waiting and not self.running and self._ahead is None
 
     def stats(self) -> SchedulerStats:
         s = dataclasses.replace(self._totals)
@@ -271,6 +279,15 @@ class Scheduler:
     def _run_step(self) -> List[TokenEvent]:
         events: List[TokenEvent] = []
         self._expire(events)
+        if self._ahead is not None:
+            # the step launched last has not been read: launch the one after it if nothing but
+            # decoding goes on, then read the first while the second runs
+            ahead, self._ahead = self._ahead, None
+            following = self._launch_following(ahead)
+            self._read(ahead, events)
+            if following is not None:
+                self._ahead = following
+                return events
         batch = self.plan()
         if not batch:
             return events
@@ -289,10 +306,49 @@ class Scheduler:
         for r, n in batch:
             r.computed += n
         if wanted:
+            if self.run_ahead:
+                picked = self.picker.pick_later(logits, [r.sampling for r in wanted], [r.rng for r in wanted])
+                if picked is not None:
+                    self._ahead = (wanted, picked)
+                    return events
             tokens = self.picker.pick(logits, [r.sampling for r in wanted], [r.rng for r in wanted])
             for r, token in zip(wanted, tokens):
                 self._emit(r, int(token), events)
         return events
+
+    def _launch_following(self, ahead):
+        """The step after one whose tokens are still on the device, if it can be decided without
+        them: every running request took part in that step and goes on decoding (those that reach
+        their length with it leave; one that turns out to have met a stop id has run a token too
+        far, into pages that its end gives back), nothing waits that could be admitted, the pages
+        are there, and the tokens can be chosen on the device again.  None otherwise."""
+        requests, picked = ahead
+        running = {id(r) for r in self.running}
+        live = sum(1 for r in requests if id(r) in running)
+        if live != len(self.running) or (self.waiting and self.executor.cache.free_slots > 0):
+            return None
+        rows = [i for i, r in enumerate(requests) if id(r) in running and r.generated + 1 < r.target]
+        if not rows or len(rows) > self.max_batch_tokens:
+            return None
+        going = [requests[i] for i in rows]
+        if not self.executor.cache.can_reserve([(r.id, 1) for r in going]):
+            return None
+        tokens = picked.tokens_for(rows)
+        logits = self.executor.step([StepEntry(r.id, [0], [0]) for r in going], device_tokens=tokens)
+        self._totals.steps += 1
+        self._totals.decode_tokens += len(going)
+        for r in going:
+            r.computed += 1
+        following = self.picker.pick_later(logits, [r.sampling for r in going], [r.rng for r in going])
+        assert following is not None, "the same requests' tokens were chosen on the device a step ago"
+        return (going, following)
+
+    def _read(self, ahead, events: List[TokenEvent]) -> None:
+        requests, picked = ahead
+        running = {id(r) for r in self.running}
+        for r, token in zip(requests, picked.result()):
+            if id(r) in running:           # (not cancelled, expired or ended by a stop id meanwhile)
+                self._emit(r, int(token), events)
 
     def _emit(self, r: _Live, token: int, events: List[TokenEvent]) -> None:
         e = TokenEvent(r.id, token, r.generated)

@@ -6,7 +6,7 @@ The default run has the layer sizes of TinyLlama-1.1B (22 layers, hidden 2048, 3
 4 key-value heads, head size 64, feed-forward 5632, vocabulary 32000, context 2048) with random
 weights, a batch of 8 requests with 512-token prompts, and times K decode steps (each step: one
 token for every request through the engine's step function, greedy choice on the device, the
-chosen ids read back).  It prints ONE JSON line: decoded tokens a second, the prefill of one
+chosen ids read back while the next step runs).  It prints ONE JSON line: decoded tokens a second, the prefill of one
 2,048-token prompt, the decode step against the HBM roofline, and decoding at batch 1 and 64.
 
 Beside the headline: `--shape` runs the same measurements at the sizes of Llama-2-7B or Llama-3-8B;
@@ -98,18 +98,37 @@ def run_decode(model, cfg, batch, prompt_len, steps, warmup, seed=1):
         logits = ex.step([StepEntry(b, prompt, [prompt_len - 1])])
         last.append(int(ops.argmax(logits)[0]))
 
-    def one_step(tokens):
-        logits = ex.step([StepEntry(b, [tokens[b]], [0]) for b in range(batch)])
-        return ops.argmax(logits).tolist()
+    # Every step's tokens are the ids the step before chose, taken on the device; the host reads a
+    # step's ids (through pinned memory) while the next step runs, so describing a step to the
+    # device costs the GPU no time.
+    entries = [StepEntry(b, [0], [0]) for b in range(batch)]
+    stage = [torch.empty(batch, dtype=torch.int32).pin_memory() for _ in range(2)]
+    copied = [torch.cuda.Event() for _ in range(2)]
+    read = []
 
-    for _ in range(warmup):
-        last = one_step(last)
+    def launch(ids, i):
+        chosen = ops.argmax(ex.step(entries, device_tokens=ids))
+        stage[i % 2].copy_(chosen, non_blocking=True)
+        copied[i % 2].record()
+        return chosen
+
+    def run(n, ids):
+        for i in range(n):
+            ids = launch(ids, i)
+            if i > 0:                                    # the ids of the step before, now that this one is under way
+                copied[(i - 1) % 2].synchronize()
+                read.append(stage[(i - 1) % 2].tolist())
+        copied[(n - 1) % 2].synchronize()
+        read.append(stage[(n - 1) % 2].tolist())
+        return ids
+
+    ids = run(warmup, torch.tensor(last, dtype=torch.int32, device="cuda:0"))
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(steps):
-        last = one_step(last)
+    ids = run(steps, ids)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
+    assert len(read) == warmup + steps and all(len(r) == batch for r in read)
     mid = prompt_len + warmup + steps // 2
     for b in range(batch):
         ex.release(b)
@@ -158,7 +177,7 @@ def run_serve(model, cfg, n_requests, new_tokens, chunk, seed=3):
     pages = sum(-(-(n + new_tokens) // page) for n in lengths)
     ex = Executor(model, num_pages=pages, max_requests=n_requests, max_tokens=cfg.max_seq_len, page_tokens=page,
                   max_batch_tokens=2048)
-    sched = Scheduler(ex, DevicePicker(), max_batch_tokens=2048, prefill_chunk=chunk)
+    sched = Scheduler(ex, DevicePicker(), max_batch_tokens=2048, prefill_chunk=chunk, run_ahead=True)   # as Engine does
 
     def submit_all(tag):
         for i, n in enumerate(lengths):

@@ -58,6 +58,17 @@ def _check_invariants(cm, lengths):
         assert all(group.pool.in_use(p) for p in held)
         assert group.pool.pages_in_use == len(held), "a page is lost"
         assert group.pool.pages_in_use + group.pool.free_count == group.pool.num_pages
+        # the arrays by slot say what the lists say, and nothing in the rows of free slots
+        mirror = cm.tables_by_slot[gkey]
+        live_slots = set()
+        for rid in cm.live_requests():
+            slot, table = cm.slot(rid), cm.table(gkey, rid)
+            live_slots.add(slot)
+            assert mirror[slot, :len(table)].tolist() == table and (mirror[slot, len(table):] == -1).all()
+            assert cm.lengths_by_slot[slot] == cm.length(rid)
+        for slot in range(cm.max_requests):
+            if slot not in live_slots:
+                assert (mirror[slot] == -1).all() and cm.lengths_by_slot[slot] == 0
 
 
 def test_reserve_is_all_or_nothing_and_pages_are_lazy():

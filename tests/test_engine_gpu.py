@@ -53,6 +53,72 @@ def test_long_decoding(folders, dtype):
     helpers.compare_with_plain({(0, p): got[p] for p in range(400)}, where, {"r": plain}, label=f"long {dtype}", **TOL[dtype])
 
 
+@pytest.mark.parametrize("graphs", [True, False])
+def test_tokens_taken_on_the_device_give_the_same_sequence(folders, graphs):
+    """Decoding with every step's tokens taken from the ids the step before chose, on the device
+    (the host sees them a step late), gives the ids of decoding with the host in between."""
+    from bare_cuda_4gib_amd.csrc import ops
+    from bare_cuda_4gib_amd.engine import Executor, StepEntry, load_model
+    folder = folders("B", "bfloat16")
+    model, _ = load_model(folder, "bfloat16")
+    vocab = helpers.TINY_B["vocab_size"]
+    prompts = [helpers.random_ids(n, vocab, 60 + n) for n in (5, 17, 2)]
+
+    def start():
+        ex = Executor(model, num_pages=12, max_requests=3, max_tokens=64, page_tokens=16)
+        ex.use_graphs = ex.use_graphs and graphs
+        first = []
+        for i, ids in enumerate(prompts):
+            ex.admit(i)
+            first.append(int(ops.argmax(ex.step([StepEntry(i, ids, [len(ids) - 1])]))[0]))
+        return ex, first
+
+    ex, last = start()
+    by_host = []
+    for _ in range(30):
+        last = ops.argmax(ex.step([StepEntry(i, [last[i]], [0]) for i in range(3)])).tolist()
+        by_host.append(last)
+    ex, first = start()
+    ids = torch.tensor(first, dtype=torch.int32, device="cuda:0")
+    entries = [StepEntry(i, [0], [0]) for i in range(3)]
+    on_device = []
+    for _ in range(30):
+        ids = ops.argmax(ex.step(entries, device_tokens=ids))
+        on_device.append(ids)                       # read only after everything has been launched
+    assert [t.tolist() for t in on_device] == by_host
+    with pytest.raises(Exception, match="device_tokens"):
+        ex.step(entries[:2], device_tokens=ids)
+
+
+def test_decode_step_description_from_the_arrays_by_slot(folders):
+    """A step of decoded tokens is described to the device from the cache manager's arrays by slot;
+    the description is, number for number, the one the general builder makes -- for requests of
+    different lengths, in another order than their slots, across page edges, with one left out."""
+    from bare_cuda_4gib_amd.engine import Executor, StepEntry, load_model
+    folder = folders("A", "bfloat16")
+    model, _ = load_model(folder, "bfloat16")
+    ex = Executor(model, num_pages=40, max_requests=6, max_tokens=96, page_tokens=16)
+    assert ex.use_graphs
+    vocab = helpers.TINY_A["vocab_size"]
+    names = ["a", "b", "c", "d", "e"]
+    for i, r in enumerate(names):
+        ex.admit(r)
+        ex.step([StepEntry(r, helpers.random_ids(3 + 6 * i, vocab, 40 + i), [])])
+    ex.release("b")
+    ex.admit("f")
+    ex.step([StepEntry("f", helpers.random_ids(15, vocab, 50), [])])
+    width = ex.cache.max_pages_per_request
+    for step in range(40):
+        order = [r for r in ("e", "a", "f", "d", "c") if not (r == "d" and step % 3 == 0)]
+        entries = [StepEntry(r, [(7 * step + j) % vocab], [0]) for j, r in enumerate(order)]
+        ex.cache.reserve([(e.request, 1) for e in entries])
+        want = ex._host_arrays(entries, table_width=width, all_logits=True)[0]
+        ex.step(entries)
+        used = [slot for slot in ex._graphs.values() if slot["next"] and len(slot["rows"]) == len(entries)]
+        latest = [s["ring"][(s["next"] - 1) % len(s["ring"])][1].tolist() for s in used]
+        assert want in latest, f"step {step}"
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_first_tokens_one_by_one(folders, dtype):
     """Positions 0, 1, 2, ... each as a step of its own: one key, then two, then three."""

@@ -8,6 +8,7 @@ import pytest
 import torch
 
 from bare_cuda_4gib_amd.cache import CacheManager, PagedKV
+from bare_cuda_4gib_amd.engine.executor import StepEntry
 from bare_cuda_4gib_amd.engine.scheduler import Request, Scheduler, check_request, EngineLimits
 from bare_cuda_4gib_amd.errors import EngineError
 from bare_cuda_4gib_amd.sampling import SamplingParams, sample_token
@@ -29,6 +30,7 @@ class FakeExecutor:
                                   max_requests=max_requests, max_tokens=max_tokens, dtype=torch.float32, device="cpu")
         self.history = {}
         self.batches = []
+        self.ahead_steps = 0
 
     def admit(self, rid):
         self.history[rid] = []
@@ -41,7 +43,11 @@ class FakeExecutor:
     def has(self, rid):
         return self.cache.has(rid)
 
-    def step(self, entries):
+    def step(self, entries, device_tokens=None):
+        if device_tokens is not None:      # (here: a list that stands for the ids on the device)
+            assert len(device_tokens) == len(entries) and all(e.tokens == [0] for e in entries)
+            entries = [StepEntry(e.request, [t], e.want) for e, t in zip(entries, device_tokens)]
+            self.ahead_steps += 1
         self.cache.reserve([(e.request, len(e.tokens)) for e in entries])
         self.batches.append([(e.request, len(e.tokens)) for e in entries])
         rows = []
@@ -57,6 +63,21 @@ class FakeExecutor:
 class HostPicker:
     def pick(self, logits, params, rngs):
         return [sample_token(logits[i].numpy(), p, r) for i, (p, r) in enumerate(zip(params, rngs))]
+
+    def pick_later(self, logits, params, rngs):
+        """What DevicePicker.pick_later gives, with a list in the place of the device tensor; rows
+        with top-k or top-p cannot be chosen "on the device" here either."""
+        if any(p.filtered() and not p.greedy() for p in params):
+            return None
+        tokens = self.pick(logits, params, rngs)
+
+        class Later:
+            def tokens_for(self, rows):
+                return [tokens[i] for i in rows]
+
+            def result(self):
+                return tokens
+        return Later()
 
 
 def expected_greedy(prompt, n, stop=()):
@@ -86,7 +107,7 @@ def run(sched, max_steps=500):
 
 
 def make(**kw):
-    sched_kw = {k: kw.pop(k) for k in ("max_batch_tokens", "prefill_chunk", "clock") if k in kw}
+    sched_kw = {k: kw.pop(k) for k in ("max_batch_tokens", "prefill_chunk", "clock", "run_ahead") if k in kw}
     ex = FakeExecutor(**kw)
     return Scheduler(ex, HostPicker(), **{"max_batch_tokens": 16, "prefill_chunk": 6, **sched_kw}), ex
 
@@ -226,3 +247,54 @@ def test_when_pages_run_out_the_latest_request_is_recomputed():
     assert ex.cache.pages_in_use() == 0 and ex.cache.free_slots == 3
     assert max(g.pool.high_water_mark for g in ex.cache.groups.values()) <= 9
     assert sched.stats().prefill_tokens > 18                              # recomputed tokens are counted
+
+
+@pytest.mark.parametrize("temperature", [0.0, 0.9])
+def test_running_ahead_changes_nothing_but_when_events_come(temperature):
+    """With run_ahead the step after a decode step is launched before the host has read the first
+    one's tokens: same tokens, same finishes, same pages given back -- with requests that end by a
+    stop id (one step too far on the device), by length, one cancelled while a step is unread,
+    others admitted when a slot frees, and under preemption."""
+    def scenario(run_ahead):
+        sched, ex = make(num_pages=8, max_requests=3, max_tokens=32, run_ahead=run_ahead)   # pages for 32 tokens
+        prompts = {i: prompt(n, 10 + i) for i, n in enumerate([5, 9, 3, 7, 2])}
+        free_run = expected_greedy(prompts[1], 12)
+        for i, p in prompts.items():
+            sched.submit(Request(id=i, prompt=p, max_new_tokens=[12, 12, 20, 9, 15][i],
+                                 stop_ids=[free_run[5]] if i == 1 and temperature == 0.0 else [],
+                                 sampling=SamplingParams(temperature=temperature, seed=i)))
+        out, finish, steps = {}, {}, 0
+        while not sched.idle():
+            steps += 1
+            assert steps < 400
+            for e in sched.step():
+                if e.token >= 0:
+                    assert e.index == len(out.setdefault(e.id, []))
+                    out[e.id].append(e.token)
+                if e.finish:
+                    finish[e.id] = e.finish
+            if len(out.get(2, [])) == 6 and 2 not in finish and sched.cancel(2):
+                finish[2] = "cancelled here"
+        assert ex.cache.pages_in_use() == 0 and ex.cache.free_slots == 3
+        return out, finish, ex, sched.stats()
+
+    plain_out, plain_finish, _, plain_stats = scenario(False)
+    out, finish, ex, stats = scenario(True)
+    assert ex.ahead_steps > 10, "steps were expected to be launched from tokens the host had not read"
+    cancelled = out.pop(2), plain_out.pop(2)
+    assert cancelled[0][:6] == cancelled[1][:6]            # (how many more it got before the cancel may differ)
+    assert out == plain_out and finish == plain_finish
+    # (a request that runs one token too far, or is cancelled a step later, may tip a page decision:
+    # the number of preemptions may differ, the tokens may not)
+    assert stats.preemptions > 0 and plain_stats.preemptions > 0
+    if temperature == 0.0:
+        assert finish[1] == "stop" and len(out[1]) == 6
+
+
+def test_running_ahead_leaves_rows_for_the_host_alone():
+    """A request with top-k cannot have its tokens chosen on the device: no step runs ahead."""
+    sched, ex = make(num_pages=12, run_ahead=True)
+    sched.submit(Request(id=0, prompt=prompt(4, 1), max_new_tokens=8, sampling=SamplingParams(temperature=0.7, top_k=5, seed=3)))
+    sched.submit(Request(id=1, prompt=prompt(6, 2), max_new_tokens=8))
+    out, finish = run(sched)
+    assert ex.ahead_steps == 0 and len(out[0]) == 8 and out[1] == expected_greedy(prompt(6, 2), 8)
