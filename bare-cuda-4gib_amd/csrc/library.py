@@ -8,6 +8,7 @@ from typing import Optional
 
 from ..errors import KernelError
 from . import build as _build
+from .profile import profiler
 
 _P = c_void_p
 _I = c_int
@@ -71,11 +72,20 @@ def load(build_if_missing: bool = True) -> ctypes.CDLL:
 
 
 _entry: dict = {}
+_profiler = profiler()
 
 
-def call(name: str, *args) -> None:
+def call(name: str, *args, cost=None) -> None:
+    """Calls an entry point of the library.  ``cost``: a function that gives (floating-point
+    operations, bytes to move at least) of this call, asked only while the profiler is on."""
     fn = _entry.get(name)
     if fn is None:
         fn = _entry[name] = getattr(load(), name)
-    if fn(*args) != 0:
+    if _profiler.enabled:
+        mark = _profiler.begin(name[5:] if name.startswith("bc4g_") else name, cost)
+        status = fn(*args)
+        _profiler.end(mark)
+    else:
+        status = fn(*args)
+    if status != 0:
         raise KernelError(load().bc4g_last_error().decode("utf-8", "replace"))

@@ -51,6 +51,11 @@ def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
     return None if t is None else t.data_ptr()
 
 
+def _gemm_cost(m: int, n: int, k: int, in_bytes: int, w_bytes: int, out_bytes: float):
+    """(operations, bytes moved at least) of an [m, k] x [n, k]^T product; out_bytes per output element."""
+    return lambda: (2.0 * m * n * k, m * k * in_bytes + n * k * w_bytes + m * n * out_bytes)
+
+
 def embed_gather(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out[t, :] = float(table[ids[t], :]); ids must already be known to lie in [0, vocab)."""
     _dev("embed_gather", table, ids, out)
@@ -62,7 +67,7 @@ def embed_gather(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Ten
     elif out.dtype != torch.float32 or tuple(out.shape) != (n, hidden):
         raise KernelError(f"embed_gather: out must be float32 [{n}, {hidden}]")
     library.call("bc4g_embed_gather", _ptr(table), _code(table, "embed_gather"), _ptr(ids), _ptr(out),
-                 n, hidden, vocab, _stream())
+                 n, hidden, vocab, _stream(), cost=lambda: (0.0, n * hidden * (table.element_size() + 4)))
     return out
 
 
@@ -83,7 +88,8 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.
         _i32("rmsnorm", "rows", rows, n)
     out = torch.empty((n, hidden), dtype=out_dtype, device=x.device)
     library.call("bc4g_rmsnorm", _ptr(x), _ptr(rows), _ptr(weight), _code(weight, "rmsnorm"), _ptr(out),
-                 _code(out, "rmsnorm"), n, hidden, float(eps), _stream())
+                 _code(out, "rmsnorm"), n, hidden, float(eps), _stream(),
+                 cost=lambda: (3.0 * n * hidden, n * hidden * (4 + out.element_size()) + hidden * weight.element_size()))
     return out
 
 
@@ -104,7 +110,9 @@ def gemm_generic(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = None
     else:
         out = torch.empty((m, n), dtype=out_dtype or a.dtype, device=a.device)
     library.call("bc4g_gemm_generic", _ptr(a), _code(a, "gemm"), _ptr(w), _code(w, "gemm"), _ptr(out),
-                 _code(out, "gemm"), 1 if accumulate_into is not None else 0, m, n, k, _stream())
+                 _code(out, "gemm"), 1 if accumulate_into is not None else 0, m, n, k, _stream(),
+                 cost=_gemm_cost(m, n, k, a.element_size(), w.element_size(),
+                                 8 if accumulate_into is not None else out.element_size()))
     return out
 
 
@@ -118,7 +126,8 @@ def swiglu(gu: torch.Tensor, interleaved: bool = False) -> torch.Tensor:
     out = torch.empty((t, inter), dtype=gu.dtype, device=gu.device)
     if interleaved and inter % 8:
         raise KernelError(f"swiglu: the interleaved layout needs I={inter} to be a multiple of 8")
-    library.call("bc4g_swiglu", _ptr(gu), _ptr(out), _code(gu, "swiglu"), t, inter, 1 if interleaved else 0, _stream())
+    library.call("bc4g_swiglu", _ptr(gu), _ptr(out), _code(gu, "swiglu"), t, inter, 1 if interleaved else 0, _stream(),
+                 cost=lambda: (4.0 * t * inter, 3 * t * inter * gu.element_size()))
     return out
 
 
@@ -182,7 +191,8 @@ def rope_kv_write(qkv: torch.Tensor, positions: Optional[torch.Tensor], slot_map
         num_pages, page_tokens = k_cache.shape[0], k_cache.shape[2]
     library.call("bc4g_rope_kv_write", _ptr(qkv), _code(qkv, "rope_kv_write"), _ptr(positions), _ptr(slot_map),
                  _ptr(k_cache), _ptr(v_cache), t, n_heads, n_kv_heads, head_dim, rotary_dim, float(theta),
-                 page_tokens, num_pages, 1 if write_kv else 0, 1 if block_pairs else 0, _stream())
+                 page_tokens, num_pages, 1 if write_kv else 0, 1 if block_pairs else 0, _stream(),
+                 cost=lambda: (3.0 * t * (n_heads + n_kv_heads) * head_dim, 2 * t * width * qkv.element_size()))
 
 
 def rope_table(positions: torch.Tensor, rotary_dim: int, theta: float) -> torch.Tensor:
@@ -192,7 +202,8 @@ def rope_table(positions: torch.Tensor, rotary_dim: int, theta: float) -> torch.
     t = positions.shape[0]
     _i32("rope_table", "positions", positions, t)
     table = torch.empty((t, rotary_dim // 2, 2), dtype=torch.float32, device=positions.device)
-    library.call("bc4g_rope_table", _ptr(positions), _ptr(table), t, int(rotary_dim), float(theta), _stream())
+    library.call("bc4g_rope_table", _ptr(positions), _ptr(table), t, int(rotary_dim), float(theta), _stream(),
+                 cost=lambda: (0.0, t * rotary_dim * 4))
     return table
 
 
@@ -217,7 +228,8 @@ def rope_kv_write_blocks(qkv: torch.Tensor, table: Optional[torch.Tensor], slot_
         page_tokens = k_cache.shape[2]
     library.call("bc4g_rope_kv_write_blocks", _ptr(qkv), _code(qkv, "rope_kv_write_blocks"), _ptr(table), _ptr(slot_map),
                  _ptr(k_cache), _ptr(v_cache), t, n_heads, n_kv_heads, head_dim, 0 if table is None else 1,
-                 page_tokens, 1 if write_kv else 0, _stream())
+                 page_tokens, 1 if write_kv else 0, _stream(),
+                 cost=lambda: (3.0 * t * (n_heads + n_kv_heads) * head_dim, 2 * t * qkv.shape[1] * qkv.element_size()))
 
 
 def _check_queries(what: str, q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int) -> None:
@@ -230,8 +242,9 @@ def _check_queries(what: str, q: torch.Tensor, n_heads: int, n_kv_heads: int, he
 def attention_generic(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                       block_table: torch.Tensor, row_seq: torch.Tensor, positions: torch.Tensor,
                       n_heads: int, n_kv_heads: int, head_dim: int, window: int = 0,
-                      scale: Optional[float] = None) -> torch.Tensor:
-    """Causal attention of every row over its request's cache; returns [T, n_heads*head_dim]."""
+                      scale: Optional[float] = None, work=None) -> torch.Tensor:
+    """Causal attention of every row over its request's cache; returns [T, n_heads*head_dim].
+    (``work``: what the profiler is told about the call, see attention_work.)"""
     _dev("attention", qkv, k_cache, v_cache, block_table, row_seq, positions)
     t = qkv.shape[0]
     _check_queries("attention", qkv, n_heads, n_kv_heads, head_dim)
@@ -244,7 +257,7 @@ def attention_generic(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.T
     library.call("bc4g_attention_generic", _ptr(qkv), qkv.shape[1], _ptr(out), _code(qkv, "attention"), _ptr(k_cache),
                  _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(row_seq), _ptr(positions), t,
                  n_heads, n_kv_heads, head_dim, k_cache.shape[2], k_cache.shape[0], int(window),
-                 float(scale if scale is not None else 1.0 / math.sqrt(head_dim)), _stream())
+                 float(scale if scale is not None else 1.0 / math.sqrt(head_dim)), _stream(), cost=work)
     return out
 
 
@@ -257,7 +270,8 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
     out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
     part_v = torch.empty((rows, 64), dtype=torch.float32, device=logits.device)
     part_i = torch.empty((rows, 64), dtype=torch.int32, device=logits.device)
-    library.call("bc4g_argmax", _ptr(logits), _ptr(out), _ptr(part_v), _ptr(part_i), rows, logits.shape[1], _stream())
+    library.call("bc4g_argmax", _ptr(logits), _ptr(out), _ptr(part_v), _ptr(part_i), rows, logits.shape[1], _stream(),
+                 cost=lambda: (0.0, rows * logits.shape[1] * 4))
     return out
 
 
@@ -273,7 +287,8 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, u: torch.Tensor) -> 
     if u.dtype != torch.float64 or u.numel() != rows:
         raise KernelError("sample: u must be float64 [rows]")
     out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
-    library.call("bc4g_sample", _ptr(logits), _ptr(temperature), _ptr(u), _ptr(out), rows, logits.shape[1], _stream())
+    library.call("bc4g_sample", _ptr(logits), _ptr(temperature), _ptr(u), _ptr(out), rows, logits.shape[1], _stream(),
+                 cost=lambda: (3.0 * rows * logits.shape[1], rows * logits.shape[1] * 4))
     return out
 
 
@@ -339,11 +354,12 @@ def gemm_fast(a: torch.Tensor, w, out_dtype=None,
             return None
         out = torch.empty((m, n), dtype=out_dtype, device=a.device)
         epi = EPI_STORE_BF16 if out_dtype == torch.bfloat16 else EPI_STORE_F32
+    cost = _gemm_cost(m, n, k, 2, 2, 8 if accumulate_into is not None else out.element_size())
     if m <= SKINNY_MAX_ROWS:
         packed = packed if packed is not None else pack_weight(w)      # (packing per call: tests only)
-        library.call("bc4g_gemm_skinny", _ptr(a), _ptr(packed), _ptr(out), epi, m, n, k, _stream())
+        library.call("bc4g_gemm_skinny", _ptr(a), _ptr(packed), _ptr(out), epi, m, n, k, _stream(), cost=cost)
     else:
-        library.call("bc4g_gemm_mfma", _ptr(a), _ptr(w), _ptr(out), epi, m, n, k, _stream())
+        library.call("bc4g_gemm_mfma", _ptr(a), _ptr(w), _ptr(out), epi, m, n, k, _stream(), cost=cost)
     return out
 
 
@@ -388,7 +404,8 @@ def gemm_normed(x: torch.Tensor, rows: Optional[torch.Tensor], n_rows: int, g: t
     else:
         raise KernelError(f"gemm_normed: epilogue {epilogue} is not supported")
     library.call("bc4g_gemm_skinny_normed", _ptr(x), _ptr(rows), _ptr(g), _code(g, "gemm_normed"), float(eps),
-                 _ptr(packed), _ptr(out), epilogue, n_rows, n, k, _stream())
+                 _ptr(packed), _ptr(out), epilogue, n_rows, n, k, _stream(),
+                 cost=_gemm_cost(n_rows, n, k, 4, 2, out.element_size() * out.shape[1] / n))
     return out
 
 
@@ -405,9 +422,11 @@ def gemm_swiglu(a: torch.Tensor, w_gate_up, interleaved: bool = False) -> torch.
         out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=a.device)
         if m <= SKINNY_MAX_ROWS:
             packed = packed if packed is not None else pack_weight(rows)
-            library.call("bc4g_gemm_skinny", _ptr(a), _ptr(packed), _ptr(out), EPI_SWIGLU, m, n, k, _stream())
+            library.call("bc4g_gemm_skinny", _ptr(a), _ptr(packed), _ptr(out), EPI_SWIGLU, m, n, k, _stream(),
+                         cost=_gemm_cost(m, n, k, 2, 2, 1))
         else:
-            library.call("bc4g_gemm_mfma", _ptr(a), _ptr(rows), _ptr(out), EPI_SWIGLU, m, n, k, _stream())
+            library.call("bc4g_gemm_mfma", _ptr(a), _ptr(rows), _ptr(out), EPI_SWIGLU, m, n, k, _stream(),
+                         cost=_gemm_cost(m, n, k, 2, 2, 1))
         return out
     gu = gemm_fast(a, w_gate_up, a.dtype)
     if gu is None:
@@ -451,7 +470,7 @@ def gemm_qkv_rope(x: torch.Tensor, g: Optional[torch.Tensor], eps: float, w,
     library.call("bc4g_gemm_skinny_qkv", _ptr(x), _ptr(g), _code(g, "gemm_qkv_rope") if g is not None else 0,
                  float(eps), _ptr(packed), _ptr(q), _ptr(positions), _ptr(slot_map), _ptr(k_cache), _ptr(v_cache),
                  m, k, n_heads, n_kv_heads, head_dim, int(rotary_dim), float(theta), page_tokens,
-                 1 if write_kv else 0, _stream())
+                 1 if write_kv else 0, _stream(), cost=_gemm_cost(m, n, k, x.element_size(), 2, 2))
     return q
 
 
@@ -510,7 +529,7 @@ def attention_splits(n_tiles: int, n_heads: int, n_kv_heads: int, max_kv_len: in
 def attention_mfma(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                    seq_start: torch.Tensor, seq_ctx: torch.Tensor, tile_start: torch.Tensor, n_tiles: int,
                    n_heads: int, n_kv_heads: int, head_dim: int, window: int, scale: float,
-                   n_splits: int, q_tiles: int = 1, form: int = 0) -> torch.Tensor:
+                   n_splits: int, q_tiles: int = 1, form: int = 0, work=None) -> torch.Tensor:
     """form 0: four independent waves a workgroup, tile_start counts pieces of q_tiles tiles; 1: one
     tile a workgroup, its waves share the keys (q_tiles 1); 2: four waves a workgroup that walk their
     keys together through LDS, tile_start counts pieces of 4 * q_tiles tiles (ATTENTION_STAGED_WAVES)."""
@@ -535,7 +554,7 @@ def attention_mfma(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
                  _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(seq_start), _ptr(seq_ctx),
                  _ptr(tile_start), n_seqs, n_tiles, t, n_heads, n_kv_heads, head_dim, k_cache.shape[2],
                  int(window), float(scale), attention_tile_tokens(n_heads, n_kv_heads), int(q_tiles),
-                 int(form), int(n_splits), _stream())
+                 int(form), int(n_splits), _stream(), cost=work)
     return out
 
 
@@ -544,6 +563,7 @@ def attention(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, b
     """Attention of a step's rows over the cache: the matrix-core kernel where it takes the
     sizes (bfloat16, head size a multiple of 16 up to 256, pages of a multiple of 16 tokens),
     else the plain float kernel."""
+    work = lambda: attention_work(ctx, n_heads, n_kv_heads, head_dim, window, qkv.element_size())
     if attention_mfma_supported(qkv, k_cache, head_dim):
         tpt = attention_tile_tokens(n_heads, n_kv_heads)
         # a wave takes several query tiles as soon as some request brings more than one tile of rows;
@@ -557,6 +577,23 @@ def attention(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, b
             n_tiles * waves, n_heads, n_kv_heads, ctx.max_kv_len, attention_shared_waves(head_dim) if shared else 0)
         return attention_mfma(qkv, k_cache, v_cache, block_table, ctx.seq_start_dev, ctx.seq_ctx_dev,
                               tile_start, n_tiles, n_heads, n_kv_heads, head_dim, window, scale, n_splits, q_tiles,
-                              1 if shared else 2)
+                              1 if shared else 2, work=work)
     return attention_generic(qkv, k_cache, v_cache, block_table, ctx.row_seq, ctx.positions,
-                             n_heads, n_kv_heads, head_dim, window, scale)
+                             n_heads, n_kv_heads, head_dim, window, scale, work=work)
+
+
+def attention_work(ctx, n_heads: int, n_kv_heads: int, head_dim: int, window: int, elem: int):
+    """(operations, bytes moved at least) of a step's attention, for the profiler: two products
+    of head_dim per query head and visible key; every visible key and value read once per
+    request, queries read and outputs written once."""
+    pairs = keys = 0
+    for s in range(ctx.n_seqs):
+        cached, new = ctx.seq_ctx[s], ctx.seq_start[s + 1] - ctx.seq_start[s]
+        if window > 0:
+            pairs += sum(min(window, cached + i + 1) for i in range(new))
+            keys += min(cached + new, window + new - 1)
+        else:
+            pairs += new * cached + new * (new + 1) // 2
+            keys += cached + new
+    return (4.0 * pairs * n_heads * head_dim,
+            (2 * keys * n_kv_heads * head_dim + 2 * ctx.n_tokens * n_heads * head_dim) * elem)
