@@ -71,6 +71,23 @@ class Engine:
         self._stopped = False
         self._injected = ""
 
+    @classmethod
+    def from_config(cls, config: dict, seed: int = 0, dtype: str = "bfloat16", folder: Optional[str] = None,
+                    **engine_args) -> "Engine":
+        """An engine over random weights: the model folder (config.json, model.safetensors) is written
+        from the configuration and the seed by the random-weights mode -- into ``folder``, or into a
+        temporary one that lives as long as the engine -- and loaded like any other."""
+        import tempfile
+        from ..weights import write_random_model
+        keep = None
+        if folder is None:
+            keep = tempfile.TemporaryDirectory(prefix="bc4g_model_")
+            folder = keep.name
+        write_random_model(config, seed, folder, dtype)
+        engine = cls(folder, dtype=dtype, **engine_args)
+        engine._model_folder = keep
+        return engine
+
     # ---- properties ---------------------------------------------------------
     @property
     def healthy(self) -> bool:

@@ -156,6 +156,17 @@ def test_greedy_generation_through_the_entry_point(folders, name, dtype):
     assert stats["kv_pages_used"] == 0 and stats["running"] == 0 and stats["prefill_tokens"] == 2 * sum(map(len, prompts))
 
 
+def test_engine_from_a_configuration_and_a_seed(folders):
+    """Engine.from_config writes the model folder by the random-weights mode and loads it: the
+    same tokens as the engine over the folder the tests wrote with the same seed."""
+    from bare_cuda_4gib_amd.engine.engine import Engine, generate_batch
+    cfg, seed = helpers.TINY["A"]
+    prompts = [helpers.random_ids(n, cfg["vocab_size"], 90 + n) for n in (3, 11)]
+    over_folder = generate_batch(Engine(folders("A", "bfloat16"), max_tokens=32, max_seqs=2), prompts, 8)
+    fresh = Engine.from_config(cfg, seed, "bfloat16", max_tokens=32, max_seqs=2)
+    assert generate_batch(fresh, prompts, 8) == over_folder
+
+
 def test_entry_point_statuses_and_failure_path(folders):
     from bare_cuda_4gib_amd.engine import Engine
     engine = Engine(folders("A", "bfloat16"), max_tokens=32, max_seqs=1, max_waiting=1, page_tokens=16)
