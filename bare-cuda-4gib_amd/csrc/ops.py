@@ -325,6 +325,9 @@ def _weight(w):
 
 
 SKINNY_MAX_ROWS = 64
+SKINNY_PASSES_ROWS = 128            # up to here the weights are streamed once per 64 rows rather than tiled: the
+                                    # tiled kernel has one row of tiles to give to 256 CUs (measured at 65 rows:
+                                    # 3.8 ms a step tiled)
 EPI_STORE_BF16, EPI_STORE_F32, EPI_ACCUM_F32, EPI_SWIGLU = 0, 1, 2, 3
 
 
@@ -354,12 +357,16 @@ def gemm_fast(a: torch.Tensor, w, out_dtype=None,
             return None
         out = torch.empty((m, n), dtype=out_dtype, device=a.device)
         epi = EPI_STORE_BF16 if out_dtype == torch.bfloat16 else EPI_STORE_F32
-    cost = _gemm_cost(m, n, k, 2, 2, 8 if accumulate_into is not None else out.element_size())
-    if m <= SKINNY_MAX_ROWS:
+    out_bytes = 8 if accumulate_into is not None else out.element_size()
+    if m <= SKINNY_PASSES_ROWS:
         packed = packed if packed is not None else pack_weight(w)      # (packing per call: tests only)
-        library.call("bc4g_gemm_skinny", _ptr(a), _ptr(packed), _ptr(out), epi, m, n, k, _stream(), cost=cost)
+        for r0 in range(0, m, SKINNY_MAX_ROWS):                        # the weights once for every 64 rows
+            rows = min(SKINNY_MAX_ROWS, m - r0)
+            library.call("bc4g_gemm_skinny", _ptr(a[r0:]), _ptr(packed), _ptr(out[r0:]), epi, rows, n, k, _stream(),
+                         cost=_gemm_cost(rows, n, k, 2, 2, out_bytes))
     else:
-        library.call("bc4g_gemm_mfma", _ptr(a), _ptr(w), _ptr(out), epi, m, n, k, _stream(), cost=cost)
+        library.call("bc4g_gemm_mfma", _ptr(a), _ptr(w), _ptr(out), epi, m, n, k, _stream(),
+                     cost=_gemm_cost(m, n, k, 2, 2, out_bytes))
     return out
 
 
@@ -420,10 +427,12 @@ def gemm_swiglu(a: torch.Tensor, w_gate_up, interleaved: bool = False) -> torch.
         m, k = a.shape
         n = rows.shape[0]
         out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=a.device)
-        if m <= SKINNY_MAX_ROWS:
+        if m <= SKINNY_PASSES_ROWS:
             packed = packed if packed is not None else pack_weight(rows)
-            library.call("bc4g_gemm_skinny", _ptr(a), _ptr(packed), _ptr(out), EPI_SWIGLU, m, n, k, _stream(),
-                         cost=_gemm_cost(m, n, k, 2, 2, 1))
+            for r0 in range(0, m, SKINNY_MAX_ROWS):
+                part = min(SKINNY_MAX_ROWS, m - r0)
+                library.call("bc4g_gemm_skinny", _ptr(a[r0:]), _ptr(packed), _ptr(out[r0:]), EPI_SWIGLU, part, n, k,
+                             _stream(), cost=_gemm_cost(part, n, k, 2, 2, 1))
         else:
             library.call("bc4g_gemm_mfma", _ptr(a), _ptr(rows), _ptr(out), EPI_SWIGLU, m, n, k, _stream(),
                          cost=_gemm_cost(m, n, k, 2, 2, 1))

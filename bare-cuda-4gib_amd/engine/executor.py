@@ -47,7 +47,7 @@ class Executor:
 
     def __init__(self, model: Model, *, num_pages: int, max_requests: int, max_tokens: int,
                  page_tokens: int = 64, max_batch_tokens: int = 0, poison: bool = False,
-                 use_graphs: bool = True, graph_max_batch: int = 64):
+                 use_graphs: bool = True, graph_max_batch: int = 256):
         if model.rt is None:
             raise EngineError("executor: the model has no weights bound")
         self.model = model

@@ -115,7 +115,8 @@ def test_gemm_swiglu(ops, m, inter, k):
           "interleaved: the activation sees the float sums")
 
 
-@pytest.mark.parametrize("m,n,k", [(65, 130, 304), (150, 257, 64), (300, 128, 2048), (128, 384, 96), (129, 61, 8)])
+@pytest.mark.parametrize("m,n,k", [(65, 130, 304), (150, 257, 64), (300, 128, 2048), (128, 384, 96), (129, 61, 8),
+                                   (200, 384, 96)])
 def test_gemm_mfma(ops, m, n, k):
     a, w = bf(rnd(m, k, seed=12)), bf(rnd(n, k, seed=13))
     want = a.double() @ w.double().T
@@ -127,8 +128,11 @@ def test_gemm_mfma(ops, m, n, k):
     acc = base.clone().to(DEV)
     ops.gemm_fast(a.to(DEV), w.to(DEV), accumulate_into=acc)
     close(acc, want + base.double(), 1e-4, 1e-4 * scale, "mfma accumulate")
-    fewer = ops.gemm_fast(a[:70].contiguous().to(DEV), w.to(DEV), torch.float32)   # rows do not depend on M
-    assert torch.equal(fewer, got[:70])
+    # rows do not depend on M (while the same kind of kernel serves them: up to SKINNY_PASSES_ROWS rows the
+    # weights are streamed in passes of 64 rows, beyond that the output is tiled)
+    part = m - 3 if m - 3 > ops.SKINNY_PASSES_ROWS else min(m, 40)
+    fewer = ops.gemm_fast(a[:part].contiguous().to(DEV), w.to(DEV), torch.float32)
+    assert torch.equal(fewer, got[:part])
     assert ops.gemm_fast(a.float().to(DEV), w.to(DEV)) is None                      # float operands: not taken
 
 
