@@ -51,16 +51,29 @@ __device__ inline uint32_t pack_bf16x2(float lo, float hi) {
   return r;
 }
 
+// Maxima in one instruction each.  (fmaxf would first quiet a possible signalling NaN in every operand
+// with an instruction of its own; the operands here are MFMA results, -inf or earlier maxima.)
+__device__ inline float max2(float a, float b) {
+  float r;
+  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+__device__ inline float max3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+
 // max / sum of a value over the four lanes l, l ^ 16, l ^ 32, l ^ 48, in every lane: the swap
 // instructions of gfx950 exchange half-rows between two registers in the vector ALU, with no trip
 // through LDS.  swap16(x, x) leaves (x of rows 0,0,2,2 | x of rows 1,1,3,3), swap32 the halves alike.
 __device__ inline float max_16_32(float x) {
   const uint32_t u = __float_as_uint(x);
   const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
-  const float y = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  const float y = max2(__uint_as_float(a[0]), __uint_as_float(a[1]));
   const uint32_t v = __float_as_uint(y);
   const auto b = __builtin_amdgcn_permlane32_swap(v, v, false, false);
-  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+  return max2(__uint_as_float(b[0]), __uint_as_float(b[1]));
 }
 __device__ inline float sum_16_32(float x) {
   const uint32_t u = __float_as_uint(x);
@@ -393,36 +406,45 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, WS > 8 ? 4 
           }
     }
     // the running maximum is kept over raw scores; the softmax scale (> 0) enters the exponent
-    float alpha[QT];
+    float m_new[QT], psum[QT];
     uint4 pf[QT];
     bool moved = false;
 #pragma unroll
     for (int t = 0; t < QT; ++t) {
-      float m_tile = fmaxf(fmaxf(fmaxf(sv[t][0], sv[t][1]), fmaxf(sv[t][2], sv[t][3])),
-                           fmaxf(fmaxf(sv[t][4], sv[t][5]), fmaxf(sv[t][6], sv[t][7])));
-      m_tile = max_16_32(m_tile);
-      const float m_new = fmaxf(m_run[t], m_tile);
-      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-      alpha[t] = fast_exp2((m_run[t] - m_safe) * a.scale_log2);   // 0 while nothing has been seen
+      float m_tile = max3(sv[t][0], sv[t][1], sv[t][2]);
+      m_tile = max3(m_tile, sv[t][3], sv[t][4]);
+      m_tile = max3(m_tile, sv[t][5], sv[t][6]);
+      m_tile = max_16_32(max2(m_tile, sv[t][7]));
+      m_new[t] = max2(m_run[t], m_tile);
+      const float m_safe = (m_new[t] == -INFINITY) ? 0.f : m_new[t];
       const float shift = -m_safe * a.scale_log2;
       float p[8];
 #pragma unroll
       for (int i = 0; i < 8; ++i) p[i] = fast_exp2(fmaf(sv[t][i], a.scale_log2, shift));
-      const float psum = ((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]));
-      l_run[t] = l_run[t] * alpha[t] + psum;
-      m_run[t] = m_new;
+      psum[t] = ((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]));
       pf[t] = make_uint4(pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3]), pack_bf16x2(p[4], p[5]),
                          pack_bf16x2(p[6], p[7]));
-      moved = moved || alpha[t] != 1.0f;
+      moved = moved || m_new[t] != m_run[t];
     }
-    if (__any(moved)) {                                    // the running maximum moved for some row
+    if (__any(moved)) {
+      // the running maximum moved for some row of the wave (early in a walk, rarely later): what has
+      // been summed so far is scaled down by 2^(old maximum - new maximum), 0 while nothing had been seen
 #pragma unroll
-      for (int t = 0; t < QT; ++t)
+      for (int t = 0; t < QT; ++t) {
+        const float m_safe = (m_new[t] == -INFINITY) ? 0.f : m_new[t];
+        const float alpha = fast_exp2((m_run[t] - m_safe) * a.scale_log2);
+        l_run[t] = l_run[t] * alpha + psum[t];
 #pragma unroll
         for (int b = 0; b < DB; ++b)
 #pragma unroll
-          for (int r = 0; r < 4; ++r) o[t][b][r] *= alpha[t];
+          for (int r = 0; r < 4; ++r) o[t][b][r] *= alpha;
+      }
+    } else {
+#pragma unroll
+      for (int t = 0; t < QT; ++t) l_run[t] += psum[t];
     }
+#pragma unroll
+    for (int t = 0; t < QT; ++t) m_run[t] = m_new[t];
     // (blocks past the head size hold zeros and are never stored)
 #pragma unroll
     for (int b = 0; b < DB; ++b) {
