@@ -110,7 +110,7 @@ constexpr int kMergePad = 4;   // floats between rows of the partial outputs in 
 
 // EXACT: the head size is exactly 16 * DB (the usual sizes 64, 128, 256): no test against it is left.
 template <int DJ, int DB, int QT, int WS, bool EXACT>
-__global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, WS > 8 ? 4 : 2) void attention_mfma_kernel(
+__global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, 2) void attention_mfma_kernel(
     const AttnArgs a) {
   static_assert(WS <= 1 || QT == 1, "waves share a tile's keys for single query tiles only");
   constexpr bool kStaged = WS == 0;
@@ -310,8 +310,8 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, WS > 8 ? 4 
         *reinterpret_cast<uint4*>(tiles + buf * (64 * d) + piece_seg[r] * (16 * d) + piece_off[r]) = staged[r];
   };
 
-  // (more than eight waves a workgroup would leave a wave 128 registers: no room for a second tile)
-  constexpr bool kAhead = WS <= 8 && DB <= 8;   // (nor do the fragments of the largest heads leave room)
+  // (the fragments of the largest heads leave no room for a second tile)
+  constexpr bool kAhead = DB <= 8;
   KeyTile cur, nxt;
   if constexpr (kStaged) {
     if (kt_begin < kt_end) stage_load(kt_begin);

@@ -73,14 +73,13 @@ template <int MT, int EPI, int XMODE, int U>
 // (The normed form keeps to 80 registers, so that three workgroups share a CU and all the blocks of
 // a 5,632 x 2 wide gate-up matrix are in flight at once.)
 __global__ __launch_bounds__(kThreads, XMODE != kPlain ? 6 : 4) void gemm_skinny_kernel(const SkinnyArgs a) {
-  constexpr int kSets = 1;
   constexpr bool kNormed = XMODE != kPlain;
   constexpr bool kTurned = !kNormed;                      // x reaches operand order through LDS
   constexpr int kPieces = 4 * U;                       // 16-byte pieces of a row in one batch of k-steps
   static_assert(!kNormed || MT == 1, "the fused norm handles one tile of rows");
   static_assert(!kTurned || 64 % kPieces == 0, "a load instruction covers whole rows of a batch");
   // The waves' partial sums, and before them (kTurned) every wave's buffer for x: the same memory.
-  typedef float Red[kSets][MT][16][kRedPad];
+  typedef float Red[MT][16][kRedPad];
   constexpr int kRedBytes = kWaves * static_cast<int>(sizeof(Red));
   constexpr int kTurnBytes = kTurned ? kWaves * MT * 16 * kPieces * 16 : 0;
   __shared__ __align__(16) unsigned char pool[kRedBytes > kTurnBytes ? kRedBytes : kTurnBytes];
@@ -99,11 +98,9 @@ __global__ __launch_bounds__(kThreads, XMODE != kPlain ? 6 : 4) void gemm_skinny
   const int k_begin = wave * chunk;
   const int k_end = min(k, k_begin + chunk);
 
-  floatx4 acc[kSets][MT];
+  floatx4 acc[MT];
 #pragma unroll
-  for (int s = 0; s < kSets; ++s)
-#pragma unroll
-    for (int t = 0; t < MT; ++t) acc[s][t] = floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int t = 0; t < MT; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
   // this workgroup's block of 16 rows in the packed weights: k-step ks at wblock + ks * 512 elements
   // (a scalar base and a 32-bit lane offset, so the loads of a batch differ in their scalar part only)
@@ -174,7 +171,7 @@ __global__ __launch_bounds__(kThreads, XMODE != kPlain ? 6 : 4) void gemm_skinny
   uint4* turn = reinterpret_cast<uint4*>(pool) + wave * (MT * 16 * kPieces);
 
   struct Batch {
-    uint4 w[kSets][U];
+    uint4 w[U];
     uint4 x[kNormed ? 1 : MT][kNormed ? 1 : U];
   };
   auto load = [&](Batch& b, int k0) {
@@ -182,9 +179,7 @@ __global__ __launch_bounds__(kThreads, XMODE != kPlain ? 6 : 4) void gemm_skinny
     for (int u = 0; u < U; ++u) {
       const int kk = k0 + 32 * u + 8 * grp;
       const bool ok = kk < k_end;
-#pragma unroll
-      for (int s = 0; s < kSets; ++s)
-        b.w[s][u] = k0 + 32 * u < k_end ? load16(wblock + static_cast<long>(k0 / 32 + u) * (kWave * 8) + wlane) : zero16();
+      b.w[u] = k0 + 32 * u < k_end ? load16(wblock + static_cast<long>(k0 / 32 + u) * (kWave * 8) + wlane) : zero16();
       if constexpr (!kNormed && !kTurned) {
 #pragma unroll
         for (int t = 0; t < MT; ++t) b.x[t][u] = (ok && xrow_ok[t]) ? load16(xptr[t] + kk) : zero16();
@@ -224,8 +219,7 @@ __global__ __launch_bounds__(kThreads, XMODE != kPlain ? 6 : 4) void gemm_skinny
         } else {
           xb = b.x[t][u];
         }
-#pragma unroll
-        for (int s = 0; s < kSets; ++s) acc[s][t] = mfma_16x16x32(b.w[s][u], xb, acc[s][t]);
+        acc[t] = mfma_16x16x32(b.w[u], xb, acc[t]);
       }
     }
     if constexpr (kTurned) {                             // read before the next batch is written
@@ -313,13 +307,11 @@ __global__ __launch_bounds__(kThreads, XMODE != kPlain ? 6 : 4) void gemm_skinny
   }
 
   if constexpr (kTurned) __syncthreads();               // the partial sums take the buffers' place
-  // acc[s][t][r] is the partial sum for output column n0 + 4*grp + r and row t*16 + col
+  // acc[t][r] is the partial sum for output column n0 + 4*grp + r and row t*16 + col
 #pragma unroll
-  for (int s = 0; s < kSets; ++s)
+  for (int t = 0; t < MT; ++t)
 #pragma unroll
-    for (int t = 0; t < MT; ++t)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) red[wave][s][t][4 * grp + r][col] = acc[s][t][r];
+    for (int r = 0; r < 4; ++r) red[wave][t][4 * grp + r][col] = acc[t][r];
   __syncthreads();
 
   constexpr bool kPaired = EPI == kSwigluBf16 || EPI == kRopeKvBf16;   // columns nl and nl + 8 belong together
@@ -334,10 +326,10 @@ __global__ __launch_bounds__(kThreads, XMODE != kPlain ? 6 : 4) void gemm_skinny
     if (row >= m || gn >= a.n) continue;
     float sum = 0.f, partner = 0.f;
 #pragma unroll
-    for (int wv = 0; wv < kWaves; ++wv) sum += red[wv][0][row / 16][nl][row % 16];
+    for (int wv = 0; wv < kWaves; ++wv) sum += red[wv][row / 16][nl][row % 16];
     if constexpr (kPaired) {
 #pragma unroll
-      for (int wv = 0; wv < kWaves; ++wv) partner += red[wv][0][row / 16][nl + 8][row % 16];
+      for (int wv = 0; wv < kWaves; ++wv) partner += red[wv][row / 16][nl + 8][row % 16];
     }
     if constexpr (kNormed) {
       const float scale = 1.0f / sqrtf(ssq_row[row] / static_cast<float>(k) + a.eps);
