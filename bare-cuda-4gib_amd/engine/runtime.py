@@ -41,8 +41,12 @@ class Runtime:
     def place_weight(self, t: torch.Tensor) -> torch.Tensor:
         """A loaded tensor on the device: kept as stored (bfloat16 stays
         bfloat16, 32-bit stays 32-bit, integers int32), except that the 32-bit
-        path widens everything to float."""
+        path widens everything to float and that a tensor stored in float16 is
+        kept in bfloat16 otherwise (rounded to nearest, ties to even: a
+        float16 checkpoint then runs on the same kernels as a bfloat16 one)."""
         t = t.to(self.device)
         if t.is_floating_point() and self.full_precision and t.dtype != torch.float32:
             t = t.to(torch.float32)
+        elif t.dtype == torch.float16:
+            t = t.to(torch.float32).to(torch.bfloat16)
         return t.contiguous()

@@ -37,14 +37,15 @@ class WeightSpec:
 def _kept_dtype_ok(spec: WeightSpec, t: torch.Tensor) -> bool:
     if spec.kind == "int_table":
         return t.dtype == torch.int32
-    return t.dtype in (torch.bfloat16, torch.float32)
+    return t.dtype in (torch.bfloat16, torch.float32, torch.float16)
 
 
 def load_weights(model_dir: str, expected: Dict[str, WeightSpec],
                  ignore: Iterable[str] = ()) -> Dict[str, torch.Tensor]:
     """Read every expected tensor from ``model_dir``.
 
-    Returns name -> CPU tensor (bfloat16 stays bfloat16, 32-bit stays 32-bit,
+    Returns name -> CPU tensor (bfloat16 stays bfloat16, 32-bit stays 32-bit, float16 stays
+    float16 until it is placed on the device, where the 16-bit path keeps it in bfloat16,
     integers are int32).  ``ignore`` holds glob patterns of tensor names a file
     may carry that the engine does not need.  Raises one WeightError that lists
     every missing tensor, unexpected tensor and wrong shape.

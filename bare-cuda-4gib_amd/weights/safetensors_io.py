@@ -78,9 +78,9 @@ class SafetensorsFile:
         return self.entries[name]["dtype"]
 
     def tensor(self, name: str) -> torch.Tensor:
-        """The tensor in the dtype the engine keeps it in: BF16 stays bfloat16;
-        F32 stays float32; F16 and F64 become float32 (F16 widens exactly);
-        integers become int32."""
+        """The tensor as the host hands it on: BF16 stays bfloat16, F32 stays float32, F16 stays
+        float16 (the device then keeps it in bfloat16, or widens it for the 32-bit path), F64 becomes
+        float32; integers become int32."""
         e = self.entries[name]
         npdt, _ = _NP_VIEW[e["dtype"]]
         arr = np.frombuffer(self._mm, dtype=npdt, count=int(np.prod(e["shape"], dtype=np.int64)) if e["shape"] else 1,
@@ -90,7 +90,9 @@ class SafetensorsFile:
             return torch.from_numpy(arr.copy()).view(torch.bfloat16)
         if dt in ("F32",):
             return torch.from_numpy(arr.copy())
-        if dt in ("F16", "F64"):
+        if dt == "F16":
+            return torch.from_numpy(arr.copy())
+        if dt == "F64":
             return torch.from_numpy(arr.astype(np.float32))
         if dt == "BOOL":
             return torch.from_numpy(arr.astype(np.int32))

@@ -51,8 +51,15 @@ def test_kept_dtypes(tmp_path):
     assert torch.equal(w["model.norm.weight"], tensors["model.norm.weight"])
     assert w["lm_head.weight"].dtype == torch.bfloat16                                   # stays bfloat16
     assert torch.equal(w["lm_head.weight"], tensors["lm_head.weight"])
-    assert w["model.layers.0.mlp.up_proj.weight"].dtype == torch.float32                 # float16 widens exactly
-    assert torch.equal(w["model.layers.0.mlp.up_proj.weight"], tensors["model.layers.0.mlp.up_proj.weight"].float())
+    half = w["model.layers.0.mlp.up_proj.weight"]
+    assert half.dtype == torch.float16 and torch.equal(half, tensors["model.layers.0.mlp.up_proj.weight"])
+    # on the device: a float16 tensor is kept in bfloat16 by the 16-bit path, widened by the 32-bit one
+    from bare_cuda_4gib_amd.engine.runtime import Runtime
+    cpu = torch.device("cpu")
+    placed = Runtime(cpu, torch.bfloat16).place_weight(half)
+    assert placed.dtype == torch.bfloat16 and torch.equal(placed, half.float().to(torch.bfloat16))
+    assert torch.equal(Runtime(cpu, torch.float32).place_weight(half), half.float())
+    assert Runtime(cpu, torch.bfloat16).place_weight(w["model.norm.weight"]).dtype == torch.float32
 
 
 def test_integer_tables_become_int32(tmp_path):
