@@ -109,13 +109,15 @@ extern "C" {
 //      tile staged in LDS once for all of them; pieces of 4 * q_tiles * tokens_per_tile tokens
 // With n_splits > 1 the keys are, moreover, cut into that many parts over workgroups, whose float
 // partials (part_o [n_splits, T, heads, d], part_ml [n_splits, T, heads, 2]) a second kernel
-// merges into out.
+// merges into out.  A request without pieces (tile_start[s + 1] == tile_start[s]) is left out: its
+// rows of out are not written, provided row_seq ([T]: each row's request) is given for the merge
+// to see which rows those are -- so two launches of different forms can share one out.
 int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, float* part_o, float* part_ml, const void* k_cache,
                         const void* v_cache, const int32_t* block_table, int table_stride,
                         const int32_t* seq_start, const int32_t* seq_ctx, const int32_t* tile_start,
                         int n_seqs, int n_tiles, int n_tokens, int n_heads, int n_kv_heads, int head_dim,
                         int page_tokens, int window, float scale, int tokens_per_tile, int q_tiles,
-                        int form, int n_splits, void* stream);
+                        int form, int n_splits, const int32_t* row_seq, void* stream);
 }
 
 extern "C" {

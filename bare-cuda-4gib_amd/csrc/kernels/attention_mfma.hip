@@ -539,16 +539,24 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, 2) void att
 
 // out[row, head, :] = sum_z 2^(m_z - M) O_z / sum_z 2^(m_z - M) l_z, parts added in order of z.
 // One wave per (row, head), up to 64 parts: lane z reads part z's statistics, the weights go
-// through LDS, and every lane then sums its output dimensions over the parts.
+// through LDS, and every lane then sums its output dimensions over the parts.  With row_seq given,
+// rows of requests that had no tile in this launch (tile_start[s + 1] == tile_start[s]) are left
+// alone: another launch writes them.
 constexpr int kMaxSplits = 64;
 
 __global__ __launch_bounds__(kWave) void attention_merge_kernel(const float* __restrict__ part_o,
                                                                 const float* __restrict__ part_ml,
                                                                 bf16_t* __restrict__ out, int n_splits,
-                                                                long n_rows_heads, int d) {
+                                                                long n_rows_heads, int d, int n_heads,
+                                                                const int32_t* __restrict__ row_seq,
+                                                                const int32_t* __restrict__ tile_start) {
   __shared__ float weight[kMaxSplits];
   const long rh = blockIdx.x;
   const int lane = threadIdx.x;
+  if (row_seq != nullptr) {
+    const int s = row_seq[rh / n_heads];
+    if (tile_start[s + 1] == tile_start[s]) return;
+  }
   // the first parts' outputs are asked for together with the statistics, not after them
   constexpr int kEarly = 8;
   float early[kEarly];
@@ -601,7 +609,7 @@ extern "C" int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, flo
                                    const int32_t* seq_start, const int32_t* seq_ctx, const int32_t* tile_start,
                                    int n_seqs, int n_tiles, int n_tokens, int n_heads, int n_kv_heads, int head_dim,
                                    int page_tokens, int window, float scale, int tokens_per_tile, int q_tiles,
-                                   int form, int n_splits, void* stream) {
+                                   int form, int n_splits, const int32_t* row_seq, void* stream) {
   BC4G_REQUIRE(n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0, "attention_mfma: bad heads %d/%d",
                n_heads, n_kv_heads);
   BC4G_REQUIRE(head_dim >= 16 && head_dim <= 256 && head_dim % 16 == 0,
@@ -691,7 +699,8 @@ extern "C" int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, flo
     const long rows_heads = static_cast<long>(n_tokens) * n_heads;
     BC4G_REQUIRE(rows_heads <= 2147483647L, "attention_mfma: too many rows to merge");
     attention_merge_kernel<<<static_cast<unsigned>(rows_heads), 64, 0, s>>>(part_o, part_ml, a.out, n_splits,
-                                                                             rows_heads, head_dim);
+                                                                             rows_heads, head_dim, n_heads, row_seq,
+                                                                             tile_start);
     return check_launch("attention_merge");
   }
   return 0;

@@ -506,6 +506,8 @@ ATTENTION_PROMPT_GROUPS = 512     # workgroups a prompt step should bring: the l
                                   # with two rounds of workgroups the short ones fill in behind them
 ATTENTION_MAX_PROMPT_SPLITS = 8
 ATTENTION_MIN_WALK = 4            # 32-key tiles a part of a prompt's keys should hold at least
+ATTENTION_APART_CONTEXT = 256     # cached tokens from which on a single-tile request beside prompt portions gets a
+                                  # launch of the decode form for itself
 ATTENTION_SHARED_WALK = 1         # 32-key tiles a wave walks where a workgroup's waves share one tile's keys:
                                   # a CU pulls only so much from memory, so few workgroups with long walks are slow
 ATTENTION_ENOUGH_GROUPS = 256     # workgroups of that kind from which on the keys are not cut further
@@ -538,10 +540,13 @@ def attention_splits(n_tiles: int, n_heads: int, n_kv_heads: int, max_kv_len: in
 def attention_mfma(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                    seq_start: torch.Tensor, seq_ctx: torch.Tensor, tile_start: torch.Tensor, n_tiles: int,
                    n_heads: int, n_kv_heads: int, head_dim: int, window: int, scale: float,
-                   n_splits: int, q_tiles: int = 1, form: int = 0, work=None) -> torch.Tensor:
+                   n_splits: int, q_tiles: int = 1, form: int = 0, work=None,
+                   out: Optional[torch.Tensor] = None, row_seq: Optional[torch.Tensor] = None) -> torch.Tensor:
     """form 0: four independent waves a workgroup, tile_start counts pieces of q_tiles tiles; 1: one
     tile a workgroup, its waves share the keys (q_tiles 1); 2: four waves a workgroup that walk their
-    keys together through LDS, tile_start counts pieces of 4 * q_tiles tiles (ATTENTION_STAGED_WAVES)."""
+    keys together through LDS, tile_start counts pieces of 4 * q_tiles tiles (ATTENTION_STAGED_WAVES).
+    Requests without pieces are left out; with ``out`` (the result of another launch over the other
+    requests) and ``row_seq`` (each row's request) their rows of it stay as they are."""
     _dev("attention_mfma", qkv, k_cache, v_cache, block_table, seq_start, seq_ctx, tile_start)
     t = qkv.shape[0]
     _check_queries("attention_mfma", qkv, n_heads, n_kv_heads, head_dim)
@@ -554,7 +559,13 @@ def attention_mfma(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     _i32("attention_mfma", "seq_start", seq_start, n_seqs + 1)
     _i32("attention_mfma", "seq_ctx", seq_ctx, n_seqs)
     _i32("attention_mfma", "tile_start", tile_start, n_seqs + 1)
-    out = torch.empty((t, n_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
+    if out is None:
+        out = torch.empty((t, n_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
+    elif out.dtype != qkv.dtype or tuple(out.shape) != (t, n_heads * head_dim) or not out.is_contiguous():
+        raise KernelError(f"attention_mfma: out must be {qkv.dtype} [{t}, {n_heads * head_dim}]")
+    if row_seq is not None:
+        _dev("attention_mfma", row_seq)
+        _i32("attention_mfma", "row_seq", row_seq, t)
     part_o = part_ml = None
     if n_splits > 1:
         part_o = torch.empty((n_splits, t, n_heads, head_dim), dtype=torch.float32, device=qkv.device)
@@ -563,7 +574,7 @@ def attention_mfma(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
                  _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(seq_start), _ptr(seq_ctx),
                  _ptr(tile_start), n_seqs, n_tiles, t, n_heads, n_kv_heads, head_dim, k_cache.shape[2],
                  int(window), float(scale), attention_tile_tokens(n_heads, n_kv_heads), int(q_tiles),
-                 int(form), int(n_splits), _stream(), cost=work)
+                 int(form), int(n_splits), _ptr(row_seq), _stream(), cost=work)
     return out
 
 
@@ -575,18 +586,32 @@ def attention(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, b
     work = lambda: attention_work(ctx, n_heads, n_kv_heads, head_dim, window, qkv.element_size())
     if attention_mfma_supported(qkv, k_cache, head_dim):
         tpt = attention_tile_tokens(n_heads, n_kv_heads)
-        # a wave takes several query tiles as soon as some request brings more than one tile of rows;
-        # while every request brings one tile at most, a workgroup's waves share the tile's keys
-        # (else four waves with consecutive tiles of a request walk their keys together)
-        shared = ctx.max_q_len <= tpt
-        q_tiles = 1 if shared else attention_q_tiles(head_dim)
-        waves = 1 if shared else ATTENTION_STAGED_WAVES
-        tile_start, n_tiles = ctx.attention_tiles(tpt * q_tiles * waves)
-        n_splits = ctx.fixed_attention_splits or attention_splits(
-            n_tiles * waves, n_heads, n_kv_heads, ctx.max_kv_len, attention_shared_waves(head_dim) if shared else 0)
-        return attention_mfma(qkv, k_cache, v_cache, block_table, ctx.seq_start_dev, ctx.seq_ctx_dev,
-                              tile_start, n_tiles, n_heads, n_kv_heads, head_dim, window, scale, n_splits, q_tiles,
-                              1 if shared else 2, work=work)
+        args = (qkv, k_cache, v_cache, block_table, ctx.seq_start_dev, ctx.seq_ctx_dev)
+        sizes = (n_heads, n_kv_heads, head_dim, window, scale)
+        # While every request brings one tile of rows at most (decoded tokens), a workgroup is one
+        # tile and its waves share the tile's keys.
+        if ctx.max_q_len <= tpt:
+            tile_start, n_tiles = ctx.attention_tiles(tpt)
+            n_splits = ctx.fixed_attention_splits or attention_splits(
+                n_tiles, n_heads, n_kv_heads, ctx.max_kv_len, attention_shared_waves(head_dim))
+            return attention_mfma(*args, tile_start, n_tiles, *sizes, n_splits, 1, 1, work=work)
+        # Else four waves with consecutive tiles of a request walk their keys together -- but a
+        # request that brings a single tile beside them (a decoded token in a step with prompt
+        # portions) would walk its whole context with one wave: those requests get a launch of their
+        # own in the other form, into the same output.
+        q_tiles = attention_q_tiles(head_dim)
+        short = [s for s in range(ctx.n_seqs) if ctx.seq_start[s + 1] - ctx.seq_start[s] <= tpt]
+        apart = bool(short) and max(ctx.seq_ctx[s] for s in short) >= ATTENTION_APART_CONTEXT
+        long_tiles = ctx.attention_tiles(tpt * q_tiles * ATTENTION_STAGED_WAVES, *((False, tpt) if apart else ()))
+        n_splits = attention_splits(long_tiles[1] * ATTENTION_STAGED_WAVES, n_heads, n_kv_heads, ctx.max_kv_len)
+        out = attention_mfma(*args, long_tiles[0], long_tiles[1], *sizes, n_splits, q_tiles, 2, work=work,
+                             row_seq=ctx.row_seq if apart else None)
+        if apart:
+            short_tiles = ctx.attention_tiles(tpt, True, tpt)
+            longest = max(ctx.seq_ctx[s] for s in short) + tpt
+            n_splits = attention_splits(short_tiles[1], n_heads, n_kv_heads, longest, attention_shared_waves(head_dim))
+            attention_mfma(*args, short_tiles[0], short_tiles[1], *sizes, n_splits, 1, 1, out=out, row_seq=ctx.row_seq)
+        return out
     return attention_generic(qkv, k_cache, v_cache, block_table, ctx.row_seq, ctx.positions,
                              n_heads, n_kv_heads, head_dim, window, scale, work=work)
 

@@ -50,14 +50,19 @@ class StepContext:
             self.made[key] = make()
         return self.made[key]
 
-    def attention_tiles(self, tokens_per_tile: int):
+    def attention_tiles(self, tokens_per_tile: int, short: Optional[bool] = None, short_max: int = 0):
         """Each request's rows cut into tiles of ``tokens_per_tile`` tokens: (first tile of each
-        request as a device tensor, total).  Made once per step and tile size."""
-        if tokens_per_tile not in self.tiles:
+        request as a device tensor, total).  With ``short`` given, only the requests that bring at
+        most ``short_max`` rows (True) or more than that (False) get tiles; the others get none.
+        Made once per step, tile size and choice."""
+        key = tokens_per_tile if short is None else (tokens_per_tile, short, short_max)
+        if key not in self.tiles:
             starts = [0]
             for s in range(self.n_seqs):
                 n = self.seq_start[s + 1] - self.seq_start[s]
+                if short is not None and (n <= short_max) != short:
+                    n = 0
                 starts.append(starts[-1] + -(-n // tokens_per_tile))
             dev = torch.tensor(starts, dtype=torch.int32).to(self.token_ids.device, non_blocking=True)
-            self.tiles[tokens_per_tile] = (dev, starts[-1])
-        return self.tiles[tokens_per_tile]
+            self.tiles[key] = (dev, starts[-1])
+        return self.tiles[key]

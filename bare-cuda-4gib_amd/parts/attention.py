@@ -51,9 +51,9 @@ class CausalAttention(Part):
 
     def attention_tile_tokens(self):
         """The piece sizes (in tokens) the matrix-core kernel wants each request's rows cut into:
-        one 16-row tile for decoded tokens, several for prompt portions."""
+        one 16-row tile for decoded tokens, four waves' tiles for prompt portions."""
         tpt = ops.attention_tile_tokens(self.num_heads, self.num_kv_heads)
-        return (tpt, tpt * ops.attention_q_tiles(self.head_dim))
+        return (tpt, tpt * ops.attention_q_tiles(self.head_dim) * ops.ATTENTION_STAGED_WAVES)
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
         q, kv, h = self.num_heads * self.head_dim, self.num_kv_heads * self.head_dim, self.hidden_size

@@ -53,6 +53,46 @@ def test_long_decoding(folders, dtype):
     helpers.compare_with_plain({(0, p): got[p] for p in range(400)}, where, {"r": plain}, label=f"long {dtype}", **TOL[dtype])
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decoded_tokens_at_long_contexts_beside_prompt_portions(folders, dtype):
+    """Requests with hundreds of cached tokens decode one token each in the same step in which others
+    bring portions of their prompts: in bfloat16 the decoded rows then get an attention launch of their
+    own (keys cut between a workgroup's waves and over workgroups) into the same output as the
+    portions' launch.  Every row's logits against the plain implementation; one decoding request
+    stays below the context at which that happens and goes with the portions."""
+    from bare_cuda_4gib_amd.engine import Executor, StepEntry, load_model
+    folder = folders("C", dtype)
+    vocab = helpers.TINY_C["vocab_size"]
+    plain = PlainLlama(folder)
+    model, _ = load_model(folder, dtype)
+    ex = Executor(model, num_pages=80, max_requests=6, max_tokens=512, page_tokens=16, poison=True)
+    ex.cache.shuffle_free_pages(9)
+    ids = {"far": helpers.random_ids(460, vocab, 1), "mid": helpers.random_ids(300, vocab, 2),
+           "near": helpers.random_ids(40, vocab, 3), "p1": helpers.random_ids(90, vocab, 4),
+           "p2": helpers.random_ids(37, vocab, 5)}
+    want = {r: plain.logits(t).numpy() for r, t in ids.items()}
+    done = {"far": 450, "mid": 290, "near": 30, "p1": 0, "p2": 0}
+    for r in ("far", "mid", "near"):
+        ex.admit(r)
+        ex.step([StepEntry(r, ids[r][:done[r]], [])])
+    ex.admit("p1"), ex.admit("p2")
+    portions = {"p1": [33, 2, 40, 15], "p2": [5, 20, 12]}
+    tol = TOL[dtype]
+    for step in range(4):
+        entries, rows = [], []
+        for r in ("p1", "far", "near", "p2", "mid"):
+            n = 1 if r in ("far", "mid", "near") else (portions[r][step] if step < len(portions[r]) else 0)
+            if n == 0:
+                continue
+            entries.append(StepEntry(r, ids[r][done[r]:done[r] + n], list(range(n))))
+            rows += [(r, done[r] + i) for i in range(n)]
+            done[r] += n
+        got = ex.step(entries).float().cpu().numpy()
+        for row, (r, pos) in enumerate(rows):
+            w = want[r][pos]
+            assert abs(got[row] - w).max() <= tol["atol"] + tol["rtol"] * abs(w).max(), f"step {step}: {r} at {pos}"
+
+
 @pytest.mark.parametrize("graphs", [True, False])
 def test_tokens_taken_on_the_device_give_the_same_sequence(folders, graphs):
     """Decoding with every step's tokens taken from the ids the step before chose, on the device
