@@ -560,3 +560,44 @@ def test_streamed_weight_packing(ops, m, n, k):
     want = x.double() @ w.double().T
     torch.testing.assert_close(out.cpu().double(), want, rtol=2e-3, atol=2e-3)
     assert torch.equal(out, ops.gemm_fast(x.cuda(), w.cuda(), torch.float32))
+
+
+def test_products_at_random_sizes(ops):
+    """Forty seeded draws of (rows, outputs, k): every row count from 1 to 140 crosses the kernels'
+    borders (16 rows a tile, 64 a pass, 128 rows to the tiled kernel), outputs are multiples of
+    nothing, k any multiple of 8 -- each against the product in double precision, stored as bfloat16,
+    as float, and added into a float matrix."""
+    rng = random.Random(2024)
+    for case in range(40):
+        m = rng.choice([1, 2, 7, 15, 16, 17, 31, 33, 63, 64, 65, 100, 127, 128, 129, 140])
+        n = rng.choice([1, 5, 16, 17, 40, 129, 250, 511])
+        k = 8 * rng.choice([1, 2, 3, 5, 8, 13, 32, 33, 64, 100, 129])
+        a, w = bf(rnd(m, k, seed=100 + case)), bf(rnd(n, k, seed=200 + case))
+        want = a.double() @ w.double().T
+        scale = math.sqrt(k)
+        ad, wd = a.to(DEV), ops.StreamedWeight(w.to(DEV))
+        close(ops.gemm_fast(ad, wd, torch.float32), want, 1e-4, 1e-4 * scale, f"case {case}: {m}x{n}x{k} -> f32")
+        close(ops.gemm_fast(ad, wd, torch.bfloat16), want, 8e-3, 1e-3 * scale, f"case {case}: {m}x{n}x{k} -> bf16")
+        base = rnd(m, n, seed=300 + case).float()
+        acc = base.clone().to(DEV)
+        ops.gemm_fast(ad, wd, accumulate_into=acc)
+        close(acc, want + base.double(), 1e-4, 1e-4 * scale, f"case {case}: {m}x{n}x{k} accumulate")
+
+
+def test_attention_at_random_batches(ops):
+    """Twelve seeded batches of up to five requests -- cached lengths and new tokens at random, pages
+    of 16 or 32 tokens, with and without a window -- through the three forms of the matrix-core
+    kernel with random cuts of the keys, each against the plain result."""
+    rng = random.Random(77)
+    for case in range(12):
+        nh, nkv, d, page = rng.choice([(4, 2, 16, 16), (6, 2, 48, 32), (8, 2, 64, 16), (4, 4, 128, 32), (16, 1, 32, 16)])
+        seqs = [(rng.choice([0, 1, 15, 16, 17, 63, 64, 200]), rng.choice([1, 1, 2, 3, 16, 33, 70])) for _ in range(rng.randint(1, 5))]
+        window = rng.choice([0, 0, 24, 65])
+        data = paged_case(seqs, nh, nkv, d, page, torch.bfloat16, seed=500 + case)
+        want = plain_result(data, window)
+        what = f"case {case}: heads {nh}/{nkv} d={d} page={page} window={window} {seqs}"
+        qt = ops.attention_q_tiles(d)
+        for n_splits in (1, rng.choice([2, 3, 7])):
+            close(run_mfma(ops, data, window, n_splits, qt, staged=True), want, rtol=2e-2, atol=2e-2, what=what + " staged")
+            close(run_mfma(ops, data, window, n_splits, qt), want, rtol=2e-2, atol=2e-2, what=what + " independent")
+            close(run_mfma(ops, data, window, n_splits, shared=True), want, rtol=2e-2, atol=2e-2, what=what + " shared")
