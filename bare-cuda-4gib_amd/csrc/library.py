@@ -3,7 +3,7 @@ from __future__ import annotations
 
 import ctypes
 import sys
-from ctypes import c_char_p, c_double, c_float, c_int, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_void_p
 from typing import Optional
 
 from ..errors import KernelError

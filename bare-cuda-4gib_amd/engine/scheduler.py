@@ -25,7 +25,7 @@ from __future__ import annotations
 import collections
 import dataclasses
 import time
-from typing import Deque, Dict, Hashable, List, Optional, Sequence
+from typing import Deque, List, Sequence
 
 from ..errors import EngineError, OutOfPages
 from ..sampling.mt19937_64 import MT19937_64

@@ -21,7 +21,7 @@ head         forward(h) -> float32 logits [rows, vocab]
 """
 from __future__ import annotations
 
-from typing import Any, Callable, Dict, List
+from typing import Callable, Dict, List
 
 import torch
 

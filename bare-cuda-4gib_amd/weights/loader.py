@@ -10,7 +10,7 @@ from __future__ import annotations
 
 import dataclasses
 import fnmatch
-from typing import Dict, Iterable, Optional, Tuple
+from typing import Dict, Iterable, Tuple
 
 import torch
 

@@ -9,7 +9,6 @@ import sys
 from typing import Dict, List, Sequence, Tuple
 
 import numpy as np
-import torch
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 

@@ -3,7 +3,6 @@ that reduce to a library routine, invariants, and the constants the reference's 
 Each check is chosen so that a plausible mistake fails it."""
 import math
 
-import numpy as np
 import pytest
 import torch
 import torch.nn.functional as F

@@ -2,9 +2,7 @@
 in one step and the last 32 tokens one by one; in portions of changing size down to two tokens;
 and mixed, up to four live requests with so few pages that they are used again -- in 32-bit and
 in bfloat16, for every tiny configuration."""
-import numpy as np
 import pytest
-import torch
 
 import helpers
 from plain_llama import PlainLlama
