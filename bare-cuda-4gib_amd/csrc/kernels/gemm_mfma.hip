@@ -15,8 +15,8 @@
 // (measured: ~650 TFLOP/s).  Where the output has tiles enough, a workgroup of 8 waves therefore
 // takes a 256 x 128 tile (the same waves a CU, the same per-wave work, a quarter less traffic).
 //
-// Workgroups are numbered so that those sharing a tile of w run on the same XCD (workgroups are
-// dealt to the 8 XCDs in turn, each with an L2 of its own).
+// Workgroups are numbered so that those sharing tiles of a and w run on the same XCD at the same
+// time (tile_of).  Where 256 x 256 tiles fill the CUs, a third form takes those (gemm_mfma_wide_kernel).
 #include <math.h>
 
 #include "api.h"
@@ -32,6 +32,25 @@ constexpr int kXcds = 8;
 // kSwigluBf16: every 16 rows of w are eight gate rows and the eight up rows of the same outputs;
 // out [m, n / 2] = silu(gate) * up.  A gate and its up lie eight lanes apart in the MFMA result.
 enum Epilogue : int { kStoreBf16 = 0, kStoreF32 = 1, kAccumF32 = 2, kSwigluBf16 = 3 };
+
+
+// Which tile a workgroup takes.  Workgroups are dealt to the 8 XCDs in turn, each with an L2 of its
+// own: consecutive logical ids stay on one XCD and walk the output in bands of kBand rows of tiles,
+// m fastest inside a band -- so the 32 tiles an XCD works on at one time are 8 x 4 of them, which
+// share their rows of a and of w in that L2 (with all of m fastest, 8,192 rows were 32 tiles of one
+// column, each with rows of a of its own: measured 807 -> 896 TFLOP/s for 8192 x 28672 x 4096).
+constexpr int kBand = 8;
+__device__ inline void tile_of(int block, int m_blocks, int n_blocks, int& bm, int& bn) {
+  const int total = m_blocks * n_blocks;
+  int logical = block;
+  if (total % kXcds == 0) logical = (block % kXcds) * (total / kXcds) + block / kXcds;
+  const int per_band = kBand * n_blocks;
+  const int first = (logical / per_band) * kBand;
+  const int rows = min(kBand, m_blocks - first);
+  const int in_band = logical % per_band;
+  bm = first + in_band % rows;
+  bn = in_band / rows;
+}
 
 struct Tile {
   bf16_t a[kBM][kLdsStride];
@@ -120,12 +139,8 @@ __global__ __launch_bounds__(128 * WMS, WMS == 2 ? 2 : 1) void gemm_mfma_kernel(
   const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
   const int wm = wave / 2, wn = wave % 2;   // this wave's 64 x 64 part
 
-  // XCD-aware numbering: consecutive logical ids stay on one XCD; m runs fastest so that
-  // neighbours share a tile of w.
-  const int total = m_blocks * n_blocks;
-  int logical = blockIdx.x;
-  if (total % kXcds == 0) logical = (blockIdx.x % kXcds) * (total / kXcds) + blockIdx.x / kXcds;
-  const int bm = logical % m_blocks, bn = logical / m_blocks;
+  int bm, bn;
+  tile_of(blockIdx.x, m_blocks, n_blocks, bm, bn);
   const long m0 = static_cast<long>(bm) * kRows, n0 = static_cast<long>(bn) * kBN;
 
   // global -> LDS: a tile's rows are 8 segments of 16 bytes; thread t moves segment t%8 of rows
@@ -276,10 +291,8 @@ __global__ __launch_bounds__(kSplitThreads) void gemm_mfma_split_kernel(const bf
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const bool mover = wave >= 4;
 
-  const int total = m_blocks * n_blocks;
-  int logical = blockIdx.x;
-  if (total % kXcds == 0) logical = (blockIdx.x % kXcds) * (total / kXcds) + blockIdx.x / kXcds;
-  const int bm = logical % m_blocks, bn = logical / m_blocks;
+  int bm, bn;
+  tile_of(blockIdx.x, m_blocks, n_blocks, bm, bn);
   const long m0 = static_cast<long>(bm) * kBM, n0 = static_cast<long>(bn) * kBN;
   const int nk = (k + kBK - 1) / kBK;
 
@@ -399,6 +412,163 @@ __global__ __launch_bounds__(kSplitThreads) void gemm_mfma_split_kernel(const bf
   store_tile<EPI, kSplitThreads>(tile_out, out, m, n, m0, n0, tid);
 }
 
+// The same product for outputs with very many tiles: a workgroup of 8 waves takes a 256 x 256 tile
+// and a wave a 128 x 64 part of it (4 x 2 MFMA blocks).  Per FLOP the tile brings two thirds of the
+// bytes of a 256 x 128 one through the CU's cache, which is what bounds these kernels, and a wave
+// reads three quarters of the fragments from LDS (measured, with the banded tile order:
+// 4096 x 4096 x 4096 833 -> 1,015 TFLOP/s, 8192 x 6144 x 4096 917 -> 1,044; no gain where k is long
+// and the output wide, 8192 x 28672 x 4096).  A k-step of 64 is 72 KB in LDS, in two buffers; the
+// step after the next is in flight in registers: between the MFMAs of each slice of 16 a quarter of it
+// is written to LDS and asked for again, two steps ahead, and the next slice's fragments are read
+// while this slice's MFMAs run.  The order of the additions over k is that of the other forms.
+constexpr int kWide = 256;
+struct WideTile {
+  bf16_t a[kWide][kLdsStride];
+  bf16_t w[kWide][kLdsStride];
+};
+constexpr size_t kWideLdsBytes = sizeof(WideTile) * 2;
+
+template <int EPI>
+__global__ __launch_bounds__(512, 1) void gemm_mfma_wide_kernel(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
+                                                                     void* __restrict__ out, int m, int n, int k,
+                                                                     int m_blocks, int n_blocks) {
+  constexpr int WN = 4;                         // waves along n (two rows of them along m)
+  constexpr int kThreads = 128 * WN;
+  constexpr int kWaveN = kWide / WN;            // columns of a wave's part
+  constexpr int kJ = kWaveN / 32;               // MFMA blocks along n
+  extern __shared__ __align__(16) unsigned char wide_raw[];
+  WideTile* tiles = reinterpret_cast<WideTile*>(wide_raw);
+  const int tid = threadIdx.x, lane = tid % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int wm = wave / WN, wn = wave % WN;
+
+  int bm, bn;
+  tile_of(blockIdx.x, m_blocks, n_blocks, bm, bn);
+  const long m0 = static_cast<long>(bm) * kWide, n0 = static_cast<long>(bn) * kWide;
+
+  // global -> LDS: thread t moves segment t % 8 (16 bytes) of rows t / 8 + kChunkRows i of both operands
+  constexpr int kChunkRows = kThreads / 8;
+  constexpr int kChunks = kWide / kChunkRows;
+  constexpr int kPerSlice = kChunks / (kBK / 16);   // chunks written and asked for again per slice of k
+  static_assert(kPerSlice >= 1, "a slice moves at least one chunk");
+  const int seg = tid % 8, lrow = tid / 8;
+  uint4 ra[kChunks], rw[kChunks];
+  const bf16_t* arow[kChunks];
+  const bf16_t* wrow[kChunks];
+  bool a_ok[kChunks], w_ok[kChunks];
+#pragma unroll
+  for (int i = 0; i < kChunks; ++i) {
+    const long gm = m0 + lrow + kChunkRows * i, gn = n0 + lrow + kChunkRows * i;
+    a_ok[i] = gm < m;
+    w_ok[i] = gn < n;
+    arow[i] = a + (a_ok[i] ? gm : 0) * k + seg * 8;
+    wrow[i] = w + (w_ok[i] ? gn : 0) * k + seg * 8;
+  }
+  auto load_chunk = [&](int kt, int i) {
+    const int kk = kt * kBK;
+    const bool k_ok = kk + seg * 8 < k;
+    ra[i] = (k_ok && a_ok[i]) ? load16(arow[i] + kk) : zero16();
+    rw[i] = (k_ok && w_ok[i]) ? load16(wrow[i] + kk) : zero16();
+  };
+  auto store_chunk = [&](int buf, int i) {
+    *reinterpret_cast<uint4*>(&tiles[buf].a[lrow + kChunkRows * i][seg * 8]) = ra[i];
+    *reinterpret_cast<uint4*>(&tiles[buf].w[lrow + kChunkRows * i][seg * 8]) = rw[i];
+  };
+
+  floatx16 acc[4][kJ];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < kJ; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  const int frow = lane % 32, fk = (lane / 32) * 8;
+  const int nk = (k + kBK - 1) / kBK;
+#pragma unroll
+  for (int i = 0; i < kChunks; ++i) load_chunk(0, i);
+#pragma unroll
+  for (int i = 0; i < kChunks; ++i) store_chunk(0, i);
+  if (nk > 1) {
+#pragma unroll
+    for (int i = 0; i < kChunks; ++i) load_chunk(1, i);
+  }
+  lds_barrier();
+  uint4 fa[2][4], fw[2][kJ];
+  auto read_fragments = [&](int set, int buf, int ks) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      fa[set][i] = *reinterpret_cast<const uint4*>(&tiles[buf].a[wm * 128 + i * 32 + frow][ks * 16 + fk]);
+#pragma unroll
+    for (int j = 0; j < kJ; ++j)
+      fw[set][j] = *reinterpret_cast<const uint4*>(&tiles[buf].w[wn * kWaveN + j * 32 + frow][ks * 16 + fk]);
+  };
+  for (int t = 0; t < nk; ++t) {
+    const int cur = t & 1;
+    const bool st = t + 1 < nk, ld = t + 2 < nk;
+    read_fragments(0, cur, 0);
+#pragma unroll
+    for (int ks = 0; ks < kBK / 16; ++ks) {
+      // the next slice's fragments are asked for before this slice's MFMAs, which hide the wait
+      if (ks + 1 < kBK / 16) read_fragments((ks + 1) % 2, cur, ks + 1);
+      // a part of the next step goes to the other buffer and is asked for again, two steps ahead
+#pragma unroll
+      for (int c = 0; c < kPerSlice; ++c) {
+        if (st) store_chunk(1 - cur, kPerSlice * ks + c);
+        if (ld) load_chunk(t + 2, kPerSlice * ks + c);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < kJ; ++j) acc[i][j] = mfma_32x32x16(fa[ks % 2][i], fw[ks % 2][j], acc[i][j]);
+    }
+    lds_barrier();
+  }
+
+  // The tile goes out through LDS, its upper and its lower half in turn, each as two float
+  // [128][128 + 4] quarters.  acc[i][j][r] is row wm*128 + i*32 + 8*(r/4) + 4*(lane/32) + r%4 and
+  // column wn*kWaveN + j*32 + lane%32 of the tile.
+  constexpr int kOutStride = kBN + 4;
+  static_assert(2 * sizeof(float) * kBM * kOutStride <= kWideLdsBytes, "two output quarters must fit the operand buffers");
+  float* tile_out = reinterpret_cast<float*>(wide_raw);
+#pragma unroll
+  for (int half = 0; half < 2; ++half) {
+    if (half > 0) lds_barrier();
+    if (wm == half) {
+      const int col0 = wn * kWaveN;
+      float* mine = tile_out + (col0 / kBN) * (kBM * kOutStride) + col0 % kBN;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < kJ; ++j)
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            mine[(i * 32 + 8 * (r / 4) + 4 * (lane / 32) + r % 4) * kOutStride + j * 32 + lane % 32] = acc[i][j][r];
+    }
+    lds_barrier();
+#pragma unroll
+    for (int q = 0; q < 2; ++q)
+      store_tile<EPI, kThreads>(tile_out + q * (kBM * kOutStride), out, m, n, m0 + 128 * half, n0 + 128 * q, tid);
+  }
+}
+
+template <int EPI>
+int launch_wide(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, int k, long m_blocks, long n_blocks,
+                hipStream_t s) {
+  auto kernel = gemm_mfma_wide_kernel<EPI>;
+  static bool raised = false;   // per instantiation: allow more than the default dynamic LDS
+  if (!raised) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            static_cast<int>(kWideLdsBytes)) != hipSuccess)
+      return fail("gemm_mfma: cannot raise the dynamic LDS limit");
+    raised = true;
+  }
+  kernel<<<dim3(static_cast<unsigned>(m_blocks * n_blocks)), dim3(512), kWideLdsBytes, s>>>(
+      ap, wp, out, m, n, k, static_cast<int>(m_blocks), static_cast<int>(n_blocks));
+  return 0;
+}
+
+
 int compute_units() {
   static int cus[64] = {0};
   int dev = 0;
@@ -412,15 +582,22 @@ int compute_units() {
 }
 
 template <int EPI>
-void launch_tiled(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, int k, long m_blocks, long n_blocks,
-                  hipStream_t s) {
+int launch_tiled(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, int k, long m_blocks, long n_blocks,
+                 hipStream_t s) {
+  // Where 256 x 256 tiles fill the CUs round after round (nine tenths of the rounds' places taken),
+  // the form with those tiles; with fewer, the idle places of its last round cost more than it gains
+  // (measured: 2048 x 28672 x 4096, 3.5 rounds, 633 against 576 us).
+  const long wide_blocks = ((m + kWide - 1) / kWide) * ((n + kWide - 1) / kWide);
+  const long rounds = (wide_blocks + compute_units() - 1) / compute_units();
+  if (wide_blocks * 10 >= rounds * compute_units() * 9)
+    return launch_wide<EPI>(ap, wp, out, m, n, k, (m + kWide - 1) / kWide, (n + kWide - 1) / kWide, s);
   // With tiles enough for every CU to have two of them and more, the 256 x 128 tile: a quarter less
   // traffic per FLOP, which is what bounds this kernel.
   const long tall_blocks = (m + 255) / 256;
   if (tall_blocks * n_blocks >= 2L * compute_units()) {
     gemm_mfma_kernel<EPI, 2, 4><<<dim3(static_cast<unsigned>(tall_blocks * n_blocks)), dim3(512), 0, s>>>(
         ap, wp, out, m, n, k, static_cast<int>(tall_blocks), static_cast<int>(n_blocks));
-    return;
+    return 0;
   }
   dim3 grid(static_cast<unsigned>(m_blocks * n_blocks)), block(256);
   // With at most one tile a CU nothing else runs beside a workgroup: then the split form, whose
@@ -428,9 +605,10 @@ void launch_tiled(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, i
   // 2048 x 2048 x 2048); with more tiles two workgroups of the plain form share a CU and do better.
   if (m_blocks * n_blocks <= compute_units()) {
     gemm_mfma_split_kernel<EPI><<<grid, dim3(kSplitThreads), 0, s>>>(ap, wp, out, m, n, k, m_blocks, n_blocks);
-    return;
+    return 0;
   }
   gemm_mfma_kernel<EPI, 2, 2><<<grid, block, 0, s>>>(ap, wp, out, m, n, k, m_blocks, n_blocks);
+  return 0;
 }
 
 }  // namespace
@@ -448,15 +626,17 @@ extern "C" int bc4g_gemm_mfma(const void* a, const void* w, void* out, int epilo
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bf16_t* ap = static_cast<const bf16_t*>(a);
   const bf16_t* wp = static_cast<const bf16_t*>(w);
+  int e = 0;
   switch (epilogue) {
-    case kStoreBf16: launch_tiled<kStoreBf16>(ap, wp, out, m, n, k, m_blocks, n_blocks, s); break;
-    case kStoreF32: launch_tiled<kStoreF32>(ap, wp, out, m, n, k, m_blocks, n_blocks, s); break;
-    case kAccumF32: launch_tiled<kAccumF32>(ap, wp, out, m, n, k, m_blocks, n_blocks, s); break;
+    case kStoreBf16: e = launch_tiled<kStoreBf16>(ap, wp, out, m, n, k, m_blocks, n_blocks, s); break;
+    case kStoreF32: e = launch_tiled<kStoreF32>(ap, wp, out, m, n, k, m_blocks, n_blocks, s); break;
+    case kAccumF32: e = launch_tiled<kAccumF32>(ap, wp, out, m, n, k, m_blocks, n_blocks, s); break;
     case kSwigluBf16:
       BC4G_REQUIRE(n % 16 == 0, "gemm_mfma: SwiGLU needs blocks of eight gate and eight up rows, N=%d is no multiple of 16", n);
-      launch_tiled<kSwigluBf16>(ap, wp, out, m, n, k, m_blocks, n_blocks, s);
+      e = launch_tiled<kSwigluBf16>(ap, wp, out, m, n, k, m_blocks, n_blocks, s);
       break;
     default: return fail("gemm_mfma: unknown epilogue %d", epilogue);
   }
+  if (e) return e;
   return check_launch("gemm_mfma");
 }

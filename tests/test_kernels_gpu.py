@@ -167,6 +167,39 @@ def test_gemm_mfma_both_forms_agree_bit_for_bit(ops):
     assert torch.equal(ops.gemm_fast(big, wd, torch.bfloat16)[:2500], ops.gemm_fast(a.to(DEV), wd, torch.bfloat16))
 
 
+def test_gemm_mfma_wide_tiles_agree_bit_for_bit(ops):
+    """Outputs that fill every CU with 256 x 256 tiles go to the form with those tiles (eight waves,
+    128 x 64 each): same order over k, same bits as the other forms, whose results for the first rows
+    are taken from a product with fewer rows; edges in both directions (20 rows, 12 columns) and a k
+    that is no multiple of the k-step."""
+    n, k = 16 * 256 - 244, 200                          # 16 tiles across, the last with 12 columns
+    a, w = bf(rnd(16 * 256 - 236, k, seed=43)), bf(rnd(n, k, seed=44))     # 16 tiles down, the last with 20 rows
+    ad, wd = a.to(DEV), w.to(DEV)
+    wide = ops.gemm_fast(ad, wd, torch.float32)                        # 256 tiles of 256 x 256
+    close(wide, a.double() @ w.double().T, 1e-4, 2e-3, "wide tiles")
+    few = ops.gemm_fast(ad[:700].contiguous(), wd, torch.float32)      # 3 x 16 wide tiles: the other forms
+    assert torch.equal(few, wide[:700])
+    assert torch.equal(ops.gemm_fast(ad[:700].contiguous(), wd, torch.bfloat16), ops.gemm_fast(ad, wd, torch.bfloat16)[:700])
+    acc_wide, acc_few = torch.ones(a.shape[0], n, device=DEV), torch.ones(700, n, device=DEV)
+    ops.gemm_fast(ad, wd, accumulate_into=acc_wide)
+    ops.gemm_fast(ad[:700].contiguous(), wd, accumulate_into=acc_few)
+    assert torch.equal(acc_few, acc_wide[:700])
+    gate_up = interleave8(w[:1920], w[1920:3840]).to(DEV)               # 15 tiles across: 240 of 256 places
+    g = ops.gemm_swiglu(ad, gate_up, interleaved=True)
+    assert torch.equal(ops.gemm_swiglu(ad[:700].contiguous(), gate_up, interleaved=True), g[:700])
+    gu = a.double() @ w[:3840].double().T
+    close(g, P.swiglu(gu[:, :1920], gu[:, 1920:]), 8e-3, 3e-2, "wide tiles, SwiGLU")
+
+
+@pytest.mark.parametrize("m,n", [(1024, 1024), (2304, 640), (1280 + 5, 384), (4352, 256)])
+def test_gemm_mfma_tile_numbering_covers_every_tile(ops, m, n):
+    """Tiles are dealt to the XCDs and walked in bands of eight rows of tiles: every tile is computed
+    once, whether the rows of tiles are a multiple of the band or not (9, 11 and 17 or 34 rows of
+    tiles here) and whether the tile count is a multiple of the XCDs or not."""
+    a, w = bf(rnd(m, 64, seed=15)), bf(rnd(n, 64, seed=16))
+    close(ops.gemm_fast(a.to(DEV), w.to(DEV), torch.float32), a.double() @ w.double().T, 1e-4, 1e-3, "numbering")
+
+
 def test_gemm_mfma_xcd_numbering_covers_every_tile(ops):
     a, w = bf(rnd(1024, 64, seed=15)), bf(rnd(1024, 64, seed=16))                    # 8 x 8 tiles: remapped ids
     close(ops.gemm_fast(a.to(DEV), w.to(DEV), torch.float32), a.double() @ w.double().T, 1e-4, 1e-3, "xcd")
