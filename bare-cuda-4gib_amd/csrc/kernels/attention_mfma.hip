@@ -589,6 +589,53 @@ __global__ __launch_bounds__(kWave) void attention_merge_kernel(const float* __r
   }
 }
 
+// The same for up to MAXS parts (the usual case: prompts are cut into at most 8, decode steps of
+// short contexts into few): a thread takes four neighbouring output dimensions of one (row, head),
+// asks for every part's statistics and outputs at once -- one trip to memory, no LDS, no barrier --
+// and adds the parts in order of z.
+template <int MAXS>
+__global__ __launch_bounds__(256) void attention_merge_few_kernel(const float* __restrict__ part_o,
+                                                                  const float* __restrict__ part_ml,
+                                                                  bf16_t* __restrict__ out, int n_splits,
+                                                                  long n_rows_heads, int d, int n_heads,
+                                                                  const int32_t* __restrict__ row_seq,
+                                                                  const int32_t* __restrict__ tile_start) {
+  const long item = blockIdx.x * 256L + threadIdx.x;
+  const int per = d / 4;
+  const long rh = item / per;
+  const int c = static_cast<int>(item % per) * 4;
+  if (rh >= n_rows_heads) return;
+  if (row_seq != nullptr) {
+    const int s = row_seq[rh / n_heads];
+    if (tile_start[s + 1] == tile_start[s]) return;
+  }
+  float2 ml[MAXS];
+  floatx4 o[MAXS];
+#pragma unroll
+  for (int z = 0; z < MAXS; ++z) {
+    const bool live = z < n_splits;
+    ml[z] = live ? *reinterpret_cast<const float2*>(part_ml + (z * n_rows_heads + rh) * 2) : make_float2(-INFINITY, 0.f);
+    o[z] = live ? *reinterpret_cast<const floatx4*>(part_o + (z * n_rows_heads + rh) * d + c) : floatx4{0.f, 0.f, 0.f, 0.f};
+  }
+  float m = -INFINITY;
+#pragma unroll
+  for (int z = 0; z < MAXS; ++z) m = fmaxf(m, ml[z].x);
+  float l = 0.f;
+  floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int z = 0; z < MAXS; ++z) {
+    const float wz = (ml[z].x == -INFINITY) ? 0.f : exp2f(ml[z].x - m);
+    l += wz * ml[z].y;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) acc[e] += wz * o[z][e];
+  }
+  const float inv = 1.0f / l;
+  uint2 pack;
+  pack.x = pack_bf16x2(acc[0] * inv, acc[1] * inv);
+  pack.y = pack_bf16x2(acc[2] * inv, acc[3] * inv);
+  *reinterpret_cast<uint2*>(out + rh * d + c) = pack;
+}
+
 }  // namespace
 }  // namespace bc4g
 
@@ -698,9 +745,16 @@ extern "C" int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, flo
   if (n_splits > 1) {
     const long rows_heads = static_cast<long>(n_tokens) * n_heads;
     BC4G_REQUIRE(rows_heads <= 2147483647L, "attention_mfma: too many rows to merge");
-    attention_merge_kernel<<<static_cast<unsigned>(rows_heads), 64, 0, s>>>(part_o, part_ml, a.out, n_splits,
-                                                                             rows_heads, head_dim, n_heads, row_seq,
-                                                                             tile_start);
+    constexpr int kFew = 8;
+    if (n_splits <= kFew) {
+      const long items = rows_heads * (head_dim / 4);
+      attention_merge_few_kernel<kFew><<<static_cast<unsigned>((items + 255) / 256), 256, 0, s>>>(
+          part_o, part_ml, a.out, n_splits, rows_heads, head_dim, n_heads, row_seq, tile_start);
+    } else {
+      attention_merge_kernel<<<static_cast<unsigned>(rows_heads), 64, 0, s>>>(part_o, part_ml, a.out, n_splits,
+                                                                               rows_heads, head_dim, n_heads, row_seq,
+                                                                               tile_start);
+    }
     return check_launch("attention_merge");
   }
   return 0;
