@@ -60,6 +60,7 @@ struct SkinnyArgs {
   const bf16_t* w;          // packed: [ceil(n / 16)][ceil(k / 32)][64 lanes][8]
   void* out;
   int m, n, k, n_out;
+  int rows_per_block;       // plain mode: blockIdx.y takes rows y * rows_per_block .. of x and out (0: all rows)
   int m_stage;              // normed modes: rows of x staged in LDS (m rounded up to 4)
   float eps;
   RopeKvArgs rope;          // kRopeKvBf16 only
@@ -72,8 +73,23 @@ __device__ inline uint32_t pack2(float a, float b) {
 template <int MT, int EPI, int XMODE, int U>
 // (The normed form keeps to 80 registers, so that three workgroups share a CU and all the blocks of
 // a 5,632 x 2 wide gate-up matrix are in flight at once.)
-__global__ __launch_bounds__(kThreads, XMODE != kPlain ? 6 : 4) void gemm_skinny_kernel(const SkinnyArgs a) {
+__global__ __launch_bounds__(kThreads, XMODE != kPlain ? 6 : 4) void gemm_skinny_kernel(const SkinnyArgs args) {
   constexpr bool kNormed = XMODE != kPlain;
+  // Where the weight blocks are too few to occupy the CUs, the rows are shared out over blockIdx.y:
+  // such a workgroup sees its own rows only, as if they were the whole batch.
+  SkinnyArgs a = args;
+  if (!kNormed && args.rows_per_block > 0) {
+    const long row0 = static_cast<long>(blockIdx.y) * args.rows_per_block;
+    a.m = min(args.rows_per_block, args.m - static_cast<int>(row0));
+    a.x = static_cast<const bf16_t*>(args.x) + row0 * args.k;
+    if constexpr (EPI == kStoreBf16) a.out = static_cast<bf16_t*>(args.out) + row0 * args.n;
+    else if constexpr (EPI == kSwigluBf16) a.out = static_cast<bf16_t*>(args.out) + row0 * (args.n / 2);
+    else if constexpr (EPI == kRopeKvBf16) {
+      a.out = static_cast<bf16_t*>(args.out) + row0 * args.rope.n_heads * args.rope.head_dim;
+      a.rope.positions = args.rope.positions ? args.rope.positions + row0 : nullptr;
+      a.rope.slot_map = args.rope.slot_map ? args.rope.slot_map + row0 : nullptr;
+    } else a.out = static_cast<float*>(args.out) + row0 * args.n;
+  }
   constexpr bool kTurned = !kNormed;                      // x reaches operand order through LDS
   constexpr int kPieces = 4 * U;                       // 16-byte pieces of a row in one batch of k-steps
   static_assert(!kNormed || MT == 1, "the fused norm handles one tile of rows");
@@ -386,6 +402,7 @@ __global__ __launch_bounds__(kThreads, XMODE != kPlain ? 6 : 4) void gemm_skinny
 }
 
 constexpr int kMaxStageBytes = 96 * 1024;
+constexpr int kSplitMaxBlocks = 256, kSplitMinRows = 8;
 
 template <int EPI, int XMODE>
 int launch(const SkinnyArgs& a, hipStream_t s) {
@@ -405,12 +422,25 @@ int launch(const SkinnyArgs& a, hipStream_t s) {
     }
     kernel<<<grid, block, stage, s>>>(a);
   } else {
-    switch (mt) {
+    // Every workgroup reads all its rows of x, and what a CU can pull through its cache is what bounds
+    // the kernel once x is as large as the block's weights (16 rows).  Where the weight blocks are
+    // few (up to kSplitMaxBlocks: n = 4,096), two workgroups share a block's rows: each pulls half of
+    // x, and the block's weights are read twice, once of it from L2 (measured at TinyLlama's sizes:
+    // 1.80 -> 1.51 ms a step at 64 rows, 1.36 -> 1.26 at 32, 1.15 -> 1.12 at 16; four workgroups a
+    // block, or splitting the wide gate-up product too, are no faster).
+    SkinnyArgs b = a;
+    int tiles = mt;
+    if (a.m > kSplitMinRows && static_cast<int>(grid.x) <= kSplitMaxBlocks) {
+      b.rows_per_block = (a.m + 1) / 2;
+      tiles = (b.rows_per_block + 15) / 16;
+      grid.y = 2;
+    }
+    switch (tiles) {
       // k-steps per batch chosen so that two batches of operands fit 128 registers (two workgroups a CU)
-      case 1: gemm_skinny_kernel<1, EPI, XMODE, 4><<<grid, block, 0, s>>>(a); break;
-      case 2: gemm_skinny_kernel<2, EPI, XMODE, 2><<<grid, block, 0, s>>>(a); break;
-      case 3: gemm_skinny_kernel<3, EPI, XMODE, 2><<<grid, block, 0, s>>>(a); break;
-      case 4: gemm_skinny_kernel<4, EPI, XMODE, 2><<<grid, block, 0, s>>>(a); break;
+      case 1: gemm_skinny_kernel<1, EPI, XMODE, 4><<<grid, block, 0, s>>>(b); break;
+      case 2: gemm_skinny_kernel<2, EPI, XMODE, 2><<<grid, block, 0, s>>>(b); break;
+      case 3: gemm_skinny_kernel<3, EPI, XMODE, 2><<<grid, block, 0, s>>>(b); break;
+      case 4: gemm_skinny_kernel<4, EPI, XMODE, 2><<<grid, block, 0, s>>>(b); break;
       default: return fail("gemm_skinny: M=%d is beyond 64 rows", a.m);
     }
   }
@@ -462,7 +492,7 @@ extern "C" int bc4g_gemm_skinny(const void* x, const void* w, void* out, int epi
   if (int e = check_common("gemm_skinny", m, 64, n, k, epilogue)) return e;
   BC4G_REQUIRE(epilogue != kRopeKvBf16, "gemm_skinny: use bc4g_gemm_skinny_qkv for the rotary epilogue");
   if (m == 0) return 0;
-  SkinnyArgs a{x, nullptr, nullptr, static_cast<const bf16_t*>(w), out, m, n, k, n, 0, 0.f, {}};
+  SkinnyArgs a{x, nullptr, nullptr, static_cast<const bf16_t*>(w), out, m, n, k, n, 0, 0, 0.f, {}};
   return launch_epilogue<kPlain>(a, epilogue, static_cast<hipStream_t>(stream));
 }
 
@@ -473,7 +503,7 @@ extern "C" int bc4g_gemm_skinny_normed(const float* x, const int32_t* rows, cons
   BC4G_REQUIRE(epilogue != kAccumF32 && epilogue != kRopeKvBf16, "gemm_skinny_normed: epilogue %d is not supported here",
                epilogue);
   if (m == 0) return 0;
-  SkinnyArgs a{x, rows, g, static_cast<const bf16_t*>(w), out, m, n, k, n, ((m + 3) / 4) * 4, eps, {}};
+  SkinnyArgs a{x, rows, g, static_cast<const bf16_t*>(w), out, m, n, k, n, 0, ((m + 3) / 4) * 4, eps, {}};
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (g_dtype == kBF16) return launch_epilogue<kNormedG16>(a, epilogue, s);
   if (g_dtype == kF32) return launch_epilogue<kNormedG32>(a, epilogue, s);
@@ -495,7 +525,7 @@ extern "C" int bc4g_gemm_skinny_qkv(const void* x, const void* g, int g_dtype, f
   if (int e = check_rope("gemm_skinny_qkv", r, n)) return e;
   if (m == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  SkinnyArgs a{x, nullptr, g, static_cast<const bf16_t*>(w), q_out, m, n, k, n, g ? ((m + 3) / 4) * 4 : 0, eps, r};
+  SkinnyArgs a{x, nullptr, g, static_cast<const bf16_t*>(w), q_out, m, n, k, n, 0, g ? ((m + 3) / 4) * 4 : 0, eps, r};
   if (!g) return launch<kRopeKvBf16, kPlain>(a, s);
   if (g_dtype == kBF16) return launch<kRopeKvBf16, kNormedG16>(a, s);
   if (g_dtype == kF32) return launch<kRopeKvBf16, kNormedG32>(a, s);

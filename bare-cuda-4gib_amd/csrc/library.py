@@ -52,6 +52,10 @@ def load(build_if_missing: bool = True) -> ctypes.CDLL:
     elif _build.is_stale():
         print(f"[bc4g] warning: {_build.LIB_PATH} is older than its sources; "
               "run __graft_entry__.build() to rebuild", file=sys.stderr, flush=True)
+    # PyTorch first: it brings a HIP runtime of its own, and the library must bind to that one.  Loaded
+    # before torch, the library pulls in the system's runtime instead, the process then holds two, and
+    # the library's launches fail ("no ROCm-capable device is detected").
+    import torch  # noqa: F401
     try:
         lib = ctypes.CDLL(_build.LIB_PATH)
     except OSError as e:
