@@ -116,6 +116,7 @@ enum DType : int { kF32 = 0, kBF16 = 1 };
 // Records a message for bc4g_last_error() and returns a non-zero status.
 int fail(const char* fmt, ...);
 int check_launch(const char* what);
+int compute_units();   // of the current device (256 if it cannot be asked)
 
 inline int ceil_div(long a, long b) { return static_cast<int>((a + b - 1) / b); }
 

@@ -23,6 +23,18 @@ int check_launch(const char* what) {
   return 0;
 }
 
+int compute_units() {
+  static int cus[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cus[dev] == 0) {
+    int v = 0;
+    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) v = 256;
+    cus[dev] = v;
+  }
+  return cus[dev];
+}
+
 }  // namespace bc4g
 
 extern "C" const char* bc4g_last_error() { return bc4g::g_error; }

@@ -569,18 +569,6 @@ int launch_wide(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, int
 }
 
 
-int compute_units() {
-  static int cus[64] = {0};
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-  if (cus[dev] == 0) {
-    int v = 0;
-    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) v = 256;
-    cus[dev] = v;
-  }
-  return cus[dev];
-}
-
 template <int EPI>
 int launch_tiled(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, int k, long m_blocks, long n_blocks,
                  hipStream_t s) {

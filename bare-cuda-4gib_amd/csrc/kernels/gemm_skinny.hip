@@ -9,6 +9,9 @@
 // straight through memory (rows past n and k past the matrix are stored as zeros).  Loads run
 // one batch of k-steps ahead of the MFMAs that use them.  The waves' partial sums meet in LDS
 // and are added in wave order, so a result does not depend on the number of rows or on timing.
+// Where the weight blocks are few and the rows of x more than eight, two workgroups share a block,
+// each with half of the rows of x (what a CU can pull through its cache bounds the kernel, so the
+// pulling is spread).
 //
 // What comes in (XMODE):
 //   plain    x is bfloat16 [m, k].  The B operand's own pattern (a lane group reads 16 bytes of
@@ -402,7 +405,7 @@ __global__ __launch_bounds__(kThreads, XMODE != kPlain ? 6 : 4) void gemm_skinny
 }
 
 constexpr int kMaxStageBytes = 96 * 1024;
-constexpr int kSplitMaxBlocks = 256, kSplitMinRows = 8;
+constexpr int kSplitMinRows = 8;
 
 template <int EPI, int XMODE>
 int launch(const SkinnyArgs& a, hipStream_t s) {
@@ -424,13 +427,13 @@ int launch(const SkinnyArgs& a, hipStream_t s) {
   } else {
     // Every workgroup reads all its rows of x, and what a CU can pull through its cache is what bounds
     // the kernel once x is as large as the block's weights (16 rows).  Where the weight blocks are
-    // few (up to kSplitMaxBlocks: n = 4,096), two workgroups share a block's rows: each pulls half of
+    // few (up to one a CU: n = 4,096), two workgroups share a block's rows: each pulls half of
     // x, and the block's weights are read twice, once of it from L2 (measured at TinyLlama's sizes:
     // 1.80 -> 1.51 ms a step at 64 rows, 1.36 -> 1.26 at 32, 1.15 -> 1.12 at 16; four workgroups a
     // block, or splitting the wide gate-up product too, are no faster).
     SkinnyArgs b = a;
     int tiles = mt;
-    if (a.m > kSplitMinRows && static_cast<int>(grid.x) <= kSplitMaxBlocks) {
+    if (a.m > kSplitMinRows && static_cast<int>(grid.x) <= compute_units()) {
       b.rows_per_block = (a.m + 1) / 2;
       tiles = (b.rows_per_block + 15) / 16;
       grid.y = 2;
