@@ -59,11 +59,12 @@ struct Tile {
 
 // Stores a finished tile (float [128][kBN + 4] in LDS) with the epilogue, THREADS threads together.
 template <int EPI, int THREADS>
-__device__ inline void store_tile(const float* tile_out, void* __restrict__ out, int m, int n, long ldo, long m0, long n0, int tid) {
+__device__ inline void store_tile(const float* tile_out, void* __restrict__ out, int m, int n, long m0, long n0, int tid) {
   constexpr int kOutStride = kBN + 4;
-  const bool vec = ldo % 4 == 0;    // rows of the output start on 16-byte (bfloat16: 8-byte) boundaries
+  const bool vec = n % 4 == 0;      // rows of the output start on 16-byte (bfloat16: 8-byte) boundaries
   if constexpr (EPI == kSwigluBf16) {
     // every 16 columns: eight gates, then the eight ups of the same outputs; a thread takes four gates
+    const long n_out = n / 2;
     for (int c = tid; c < kBM * (kBN / 8); c += THREADS) {
       const int row = c / (kBN / 8), q = c % (kBN / 8);           // q: group of four outputs
       const int col = (q / 2) * 16 + (q % 2) * 4;                 // first gate column in the tile
@@ -73,8 +74,8 @@ __device__ inline void store_tile(const float* tile_out, void* __restrict__ out,
       float v[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) v[e] = (src[e] / (1.0f + expf(-src[e]))) * src[e + 8];
-      bf16_t* dst = static_cast<bf16_t*>(out) + gm * ldo + (gn / 16) * 8 + gn % 16;
-      if (vec) {
+      bf16_t* dst = static_cast<bf16_t*>(out) + gm * n_out + (gn / 16) * 8 + gn % 16;
+      if (n_out % 4 == 0) {
         uint2 pk;
         pk.x = static_cast<uint32_t>(bf16_bits_from_float(v[0])) | (static_cast<uint32_t>(bf16_bits_from_float(v[1])) << 16);
         pk.y = static_cast<uint32_t>(bf16_bits_from_float(v[2])) | (static_cast<uint32_t>(bf16_bits_from_float(v[3])) << 16);
@@ -90,7 +91,7 @@ __device__ inline void store_tile(const float* tile_out, void* __restrict__ out,
       const long gm = m0 + row, gn = n0 + col;
       if (gm >= m || gn >= n) continue;
       const floatx4 v = *reinterpret_cast<const floatx4*>(tile_out + row * kOutStride + col);
-      const long o = gm * ldo + gn;
+      const long o = gm * n + gn;
       if (vec) {
         if constexpr (EPI == kStoreBf16) {
           uint2 pk;
@@ -127,7 +128,7 @@ struct TileOf {
 
 template <int EPI, int SETS, int WMS>
 __global__ __launch_bounds__(128 * WMS, WMS == 2 ? 2 : 1) void gemm_mfma_kernel(
-    const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, void* __restrict__ out, int m, int n, int k, long ldo,
+    const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, void* __restrict__ out, int m, int n, int k,
     int m_blocks, int n_blocks) {
   constexpr int kRows = 64 * WMS, kThreads = 128 * WMS;
   constexpr int kChunkRows = kThreads / 8;           // rows one chunk of a thread's loads covers
@@ -264,7 +265,7 @@ __global__ __launch_bounds__(128 * WMS, WMS == 2 ? 2 : 1) void gemm_mfma_kernel(
                      lane % 32] = acc[i][j][r];
     }
     lds_barrier();
-    store_tile<EPI, kThreads>(tile_out, out, m, n, ldo, m0 + 128 * half, n0, tid);
+    store_tile<EPI, kThreads>(tile_out, out, m, n, m0 + 128 * half, n0, tid);
   }
 }
 
@@ -282,7 +283,7 @@ constexpr int kSplitThreads = 768;
 
 template <int EPI>
 __global__ __launch_bounds__(kSplitThreads) void gemm_mfma_split_kernel(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
-                                                              void* __restrict__ out, int m, int n, int k, long ldo,
+                                                              void* __restrict__ out, int m, int n, int k,
                                                               int m_blocks, int n_blocks) {
   __shared__ __align__(16) unsigned char lds_raw[sizeof(Tile) * kStages];
   Tile* tiles = reinterpret_cast<Tile*>(lds_raw);
@@ -408,7 +409,7 @@ __global__ __launch_bounds__(kSplitThreads) void gemm_mfma_split_kernel(const bf
               acc[i][j][r];
   }
   lds_barrier();
-  store_tile<EPI, kSplitThreads>(tile_out, out, m, n, ldo, m0, n0, tid);
+  store_tile<EPI, kSplitThreads>(tile_out, out, m, n, m0, n0, tid);
 }
 
 // The same product for outputs with very many tiles: a workgroup of 8 waves takes a 256 x 256 tile
@@ -429,7 +430,7 @@ constexpr size_t kWideLdsBytes = sizeof(WideTile) * 2;
 
 template <int EPI>
 __global__ __launch_bounds__(512, 1) void gemm_mfma_wide_kernel(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
-                                                                     void* __restrict__ out, int m, int n, int k, long ldo,
+                                                                     void* __restrict__ out, int m, int n, int k,
                                                                      int m_blocks, int n_blocks) {
   constexpr int WN = 4;                         // waves along n (two rows of them along m)
   constexpr int kThreads = 128 * WN;
@@ -547,12 +548,13 @@ __global__ __launch_bounds__(512, 1) void gemm_mfma_wide_kernel(const bf16_t* __
     lds_barrier();
 #pragma unroll
     for (int q = 0; q < 2; ++q)
-      store_tile<EPI, kThreads>(tile_out + q * (kBM * kOutStride), out, m, n, ldo, m0 + 128 * half, n0 + 128 * q, tid);
+      store_tile<EPI, kThreads>(tile_out + q * (kBM * kOutStride), out, m, n, m0 + 128 * half, n0 + 128 * q, tid);
   }
 }
 
 template <int EPI>
-int launch_wide(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, int k, long ldo, hipStream_t s) {
+int launch_wide(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, int k, long m_blocks, long n_blocks,
+                hipStream_t s) {
   auto kernel = gemm_mfma_wide_kernel<EPI>;
   static bool raised = false;   // per instantiation: allow more than the default dynamic LDS
   if (!raised) {
@@ -561,56 +563,39 @@ int launch_wide(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, int
       return fail("gemm_mfma: cannot raise the dynamic LDS limit");
     raised = true;
   }
-  const long m_blocks = (m + kWide - 1) / kWide, n_blocks = (n + kWide - 1) / kWide;
   kernel<<<dim3(static_cast<unsigned>(m_blocks * n_blocks)), dim3(512), kWideLdsBytes, s>>>(
-      ap, wp, out, m, n, k, ldo, static_cast<int>(m_blocks), static_cast<int>(n_blocks));
+      ap, wp, out, m, n, k, static_cast<int>(m_blocks), static_cast<int>(n_blocks));
   return 0;
 }
 
-// Columns of the output (elements of `out` a row) that n columns of the product make.
-template <int EPI>
-constexpr long out_columns(long n) { return EPI == kSwigluBf16 ? n / 2 : n; }
 
-// ldo: elements between rows of `out` (the product may be a range of columns of a wider output).
 template <int EPI>
-int launch_tiled(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, int k, long ldo, hipStream_t s) {
-  const int cus = compute_units();
+int launch_tiled(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, int k, long m_blocks, long n_blocks,
+                 hipStream_t s) {
   // Where 256 x 256 tiles fill the CUs round after round (nine tenths of the rounds' places taken),
   // the form with those tiles; with fewer, the idle places of its last round cost more than it gains
   // (measured: 2048 x 28672 x 4096, 3.5 rounds, 633 against 576 us).
-  const long wide_rows = (m + kWide - 1) / kWide;
-  const long wide_blocks = wide_rows * ((n + kWide - 1) / kWide);
-  const long rounds = (wide_blocks + cus - 1) / cus;
-  if (wide_blocks * 10 >= rounds * cus * 9) return launch_wide<EPI>(ap, wp, out, m, n, k, ldo, s);
-  // Else, with more than a round of them: the columns that fill whole rounds go to that form, and
-  // the rest, a product of its own over the remaining rows of w, to whichever form suits it
-  // (measured: 2048 x 11264 x 2048 as 8192 + 3072 columns, 127 -> 121 us; 8192 x 2560 x 2048, 119 -> 102).
-  const long round_columns = (cus / wide_rows) * kWide;
-  if (wide_rows <= cus && n > round_columns && round_columns >= 8 * kWide) {
-    const int n_wide = static_cast<int>((n / round_columns) * round_columns);
-    if (int e = launch_wide<EPI>(ap, wp, out, m, n_wide, k, ldo, s)) return e;
-    const long elem = EPI == kStoreBf16 || EPI == kSwigluBf16 ? 2 : 4;
-    return launch_tiled<EPI>(ap, wp + static_cast<long>(n_wide) * k,
-                             static_cast<char*>(out) + out_columns<EPI>(n_wide) * elem, m, n - n_wide, k, ldo, s);
-  }
-  const long m_blocks = (m + kBM - 1) / kBM, n_blocks = (n + kBN - 1) / kBN;
+  const long wide_blocks = ((m + kWide - 1) / kWide) * ((n + kWide - 1) / kWide);
+  const long rounds = (wide_blocks + compute_units() - 1) / compute_units();
+  if (wide_blocks * 10 >= rounds * compute_units() * 9)
+    return launch_wide<EPI>(ap, wp, out, m, n, k, (m + kWide - 1) / kWide, (n + kWide - 1) / kWide, s);
   // With tiles enough for every CU to have two of them and more, the 256 x 128 tile: a quarter less
   // traffic per FLOP, which is what bounds this kernel.
   const long tall_blocks = (m + 255) / 256;
-  if (tall_blocks * n_blocks >= 2L * cus) {
+  if (tall_blocks * n_blocks >= 2L * compute_units()) {
     gemm_mfma_kernel<EPI, 2, 4><<<dim3(static_cast<unsigned>(tall_blocks * n_blocks)), dim3(512), 0, s>>>(
-        ap, wp, out, m, n, k, ldo, static_cast<int>(tall_blocks), static_cast<int>(n_blocks));
+        ap, wp, out, m, n, k, static_cast<int>(tall_blocks), static_cast<int>(n_blocks));
     return 0;
   }
   dim3 grid(static_cast<unsigned>(m_blocks * n_blocks)), block(256);
   // With at most one tile a CU nothing else runs beside a workgroup: then the split form, whose
   // moving and multiplying waves overlap, is the faster one (measured: 29 against 35 us for
   // 2048 x 2048 x 2048); with more tiles two workgroups of the plain form share a CU and do better.
-  if (m_blocks * n_blocks <= cus) {
-    gemm_mfma_split_kernel<EPI><<<grid, dim3(kSplitThreads), 0, s>>>(ap, wp, out, m, n, k, ldo, m_blocks, n_blocks);
+  if (m_blocks * n_blocks <= compute_units()) {
+    gemm_mfma_split_kernel<EPI><<<grid, dim3(kSplitThreads), 0, s>>>(ap, wp, out, m, n, k, m_blocks, n_blocks);
     return 0;
   }
-  gemm_mfma_kernel<EPI, 2, 2><<<grid, block, 0, s>>>(ap, wp, out, m, n, k, ldo, m_blocks, n_blocks);
+  gemm_mfma_kernel<EPI, 2, 2><<<grid, block, 0, s>>>(ap, wp, out, m, n, k, m_blocks, n_blocks);
   return 0;
 }
 
@@ -631,12 +616,12 @@ extern "C" int bc4g_gemm_mfma(const void* a, const void* w, void* out, int epilo
   const bf16_t* wp = static_cast<const bf16_t*>(w);
   int e = 0;
   switch (epilogue) {
-    case kStoreBf16: e = launch_tiled<kStoreBf16>(ap, wp, out, m, n, k, n, s); break;
-    case kStoreF32: e = launch_tiled<kStoreF32>(ap, wp, out, m, n, k, n, s); break;
-    case kAccumF32: e = launch_tiled<kAccumF32>(ap, wp, out, m, n, k, n, s); break;
+    case kStoreBf16: e = launch_tiled<kStoreBf16>(ap, wp, out, m, n, k, m_blocks, n_blocks, s); break;
+    case kStoreF32: e = launch_tiled<kStoreF32>(ap, wp, out, m, n, k, m_blocks, n_blocks, s); break;
+    case kAccumF32: e = launch_tiled<kAccumF32>(ap, wp, out, m, n, k, m_blocks, n_blocks, s); break;
     case kSwigluBf16:
       BC4G_REQUIRE(n % 16 == 0, "gemm_mfma: SwiGLU needs blocks of eight gate and eight up rows, N=%d is no multiple of 16", n);
-      e = launch_tiled<kSwigluBf16>(ap, wp, out, m, n, k, n / 2, s);
+      e = launch_tiled<kSwigluBf16>(ap, wp, out, m, n, k, m_blocks, n_blocks, s);
       break;
     default: return fail("gemm_mfma: unknown epilogue %d", epilogue);
   }

@@ -191,29 +191,6 @@ def test_gemm_mfma_wide_tiles_agree_bit_for_bit(ops):
     close(g, P.swiglu(gu[:, :1920], gu[:, 1920:]), 8e-3, 3e-2, "wide tiles, SwiGLU")
 
 
-def test_gemm_mfma_columns_shared_out_between_two_forms(ops):
-    """More than one round of 256 x 256 tiles, but the last round mostly empty: the columns that fill
-    whole rounds go to that form and the rest to another launch over the remaining rows of w, into the
-    same output (here 16,384 + 304 columns at 4 rows of tiles).  Same bits as with fewer rows, which
-    one form serves; SwiGLU pairs and the accumulating epilogue keep their places."""
-    n, k = 64 * 256 + 304, 72
-    a, w = bf(rnd(1000, k, seed=45)), bf(rnd(n, k, seed=46, scale=0.3))
-    ad, wd = a.to(DEV), w.to(DEV)
-    both = ops.gemm_fast(ad, wd, torch.float32)
-    close(both, a.double() @ w.double().T, 1e-4, 1e-3, "columns in two launches")
-    few = ops.gemm_fast(ad[:200].contiguous(), wd, torch.float32)       # one row of wide tiles: 66 of them, one form
-    assert torch.equal(few, both[:200])
-    acc, acc_few = torch.ones(1000, n, device=DEV), torch.ones(200, n, device=DEV)
-    ops.gemm_fast(ad, wd, accumulate_into=acc)
-    ops.gemm_fast(ad[:200].contiguous(), wd, accumulate_into=acc_few)
-    assert torch.equal(acc_few, acc[:200])
-    assert torch.equal(ops.gemm_fast(ad[:200].contiguous(), wd, torch.bfloat16), ops.gemm_fast(ad, wd, torch.bfloat16)[:200])
-    g = ops.gemm_swiglu(ad, wd, interleaved=True)
-    assert torch.equal(ops.gemm_swiglu(ad[:200].contiguous(), wd, interleaved=True), g[:200])
-    gu = (a.double() @ w.double().T).view(1000, n // 16, 2, 8)
-    close(g, P.swiglu(gu[:, :, 0].reshape(1000, -1), gu[:, :, 1].reshape(1000, -1)), 8e-3, 3e-2, "SwiGLU over both launches")
-
-
 @pytest.mark.parametrize("m,n", [(1024, 1024), (2304, 640), (1280 + 5, 384), (4352, 256)])
 def test_gemm_mfma_tile_numbering_covers_every_tile(ops, m, n):
     """Tiles are dealt to the XCDs and walked in bands of eight rows of tiles: every tile is computed
