@@ -97,6 +97,7 @@ __global__ __launch_bounds__(kThreads, XMODE != kPlain ? 6 : 4) void gemm_skinny
   constexpr int kPieces = 4 * U;                       // 16-byte pieces of a row in one batch of k-steps
   static_assert(!kNormed || MT == 1, "the fused norm handles one tile of rows");
   static_assert(!kTurned || 64 % kPieces == 0, "a load instruction covers whole rows of a batch");
+  static_assert(!kTurned || kPieces >= 8, "the buffer's swizzle (piece ^ row % 8) must stay inside a row's pieces");
   // The waves' partial sums, and before them (kTurned) every wave's buffer for x: the same memory.
   typedef float Red[MT][16][kRedPad];
   constexpr int kRedBytes = kWaves * static_cast<int>(sizeof(Red));
