@@ -352,76 +352,120 @@ __global__ void argmax_pick_kernel(const float* __restrict__ part_v, const int32
 }
 
 // ---- temperature sampling --------------------------------------------------
-// Thread t owns the contiguous slice [t*chunk, (t+1)*chunk) of the vocabulary, so that the
-// walk "subtract weights in vocabulary order until the target goes negative" can be done
-// as: per-slice sums, a serial scan over the 256 slice sums, then a walk inside one slice.
-__global__ void sample_kernel(const float* __restrict__ logits, const float* __restrict__ temperature,
-                              const double* __restrict__ u, int32_t* __restrict__ out, int vocab) {
-  __shared__ float fscratch[16];
-  __shared__ double slice_sum[kBlock];
-  __shared__ float best_v[kBlock];
-  __shared__ int best_i[kBlock];
-  const float* row = logits + static_cast<size_t>(blockIdx.x) * vocab;
-  const int chunk = (vocab + kBlock - 1) / kBlock;
-  const int begin = min(vocab, static_cast<int>(threadIdx.x) * chunk);
-  const int end = min(vocab, begin + chunk);
+// The law: weights w_i = exp((l_i - max) / T) in float, summed in double; the token is the first i,
+// in vocabulary order, at which u * total - (w_0 + ... + w_i) turns negative.  One workgroup a row.
+// The vocabulary is cut into groups of 64 consecutive tokens (64 * per_lane beyond 262,144 tokens,
+// so that the groups' sums fit LDS): a wave takes a group at a time, a lane a token, so every pass
+// over the row reads whole cache lines; the groups' sums, a running sum over them (one wave, 64
+// groups a step) and a last look inside the one group where the target is crossed find the token.
+// (Sums in another order than the host's one-by-one walk: a boundary may move by one token when u
+// falls within rounding of it.)
+constexpr int kSampleThreads = 512;
+constexpr int kSampleMaxGroups = 4096;
 
+__device__ inline double wave_sum_f64(double v) {
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+  return v;
+}
+// inclusive running sum over the wave's lanes, in lane order
+__device__ inline double wave_scan_f64(double v, int lane) {
+#pragma unroll
+  for (int off = 1; off < kWave; off <<= 1) {
+    const double up = __shfl_up(v, off, kWave);
+    if (lane >= off) v += up;
+  }
+  return v;
+}
+
+__global__ __launch_bounds__(kSampleThreads) void sample_kernel(const float* __restrict__ logits,
+                                                               const float* __restrict__ temperature,
+                                                               const double* __restrict__ u, int32_t* __restrict__ out,
+                                                               int vocab) {
+  __shared__ double group_sum[kSampleMaxGroups];      // then: the running sum up to and with each group
+  __shared__ float best_v[kSampleThreads];
+  __shared__ int best_i[kSampleThreads];
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  constexpr int kWaves = kSampleThreads / kWave;
+  const float* row = logits + static_cast<size_t>(blockIdx.x) * vocab;
+
+  // the maximum and where it stands first
   float v = -FLT_MAX;
   int idx = vocab;
-  for (int i = begin; i < end; ++i) {
-    if (row[i] > v) {
-      v = row[i];
-      idx = i;
-    }
-  }
+  for (int i = threadIdx.x; i < vocab; i += kSampleThreads) better(v, idx, row[i], i);
   best_v[threadIdx.x] = v;
   best_i[threadIdx.x] = idx;
   __syncthreads();
-  for (int h = kBlock / 2; h > 0; h >>= 1) {
-    if (threadIdx.x < h) {
-      const float ov = best_v[threadIdx.x + h];
-      const int oi = best_i[threadIdx.x + h];
-      if (ov > best_v[threadIdx.x] || (ov == best_v[threadIdx.x] && oi < best_i[threadIdx.x])) {
-        best_v[threadIdx.x] = ov;
-        best_i[threadIdx.x] = oi;
-      }
-    }
+  for (int h = kSampleThreads / 2; h > 0; h >>= 1) {
+    if (threadIdx.x < h) better(best_v[threadIdx.x], best_i[threadIdx.x], best_v[threadIdx.x + h], best_i[threadIdx.x + h]);
     __syncthreads();
   }
   const float row_max = best_v[0];
   const int arg = best_i[0] < vocab ? best_i[0] : 0;
-  (void)fscratch;
   const float temp = temperature[blockIdx.x];
   if (!(temp > 0.f)) {
     if (threadIdx.x == 0) out[blockIdx.x] = arg;
     return;
   }
   const float inv_t = 1.0f / temp;
-  double s = 0.0;
-  for (int i = begin; i < end; ++i) s += static_cast<double>(expf((row[i] - row_max) * inv_t));
-  slice_sum[threadIdx.x] = s;
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    double total = 0.0;
-    for (int t = 0; t < kBlock; ++t) total += slice_sum[t];
-    double target = u[blockIdx.x] * total;
-    int result = arg;  // rounding may leave the target a hair above zero after the last token
-    for (int t = 0; t < kBlock; ++t) {
-      if (target - slice_sum[t] < 0.0) {
-        const int b = min(vocab, t * chunk), e = min(vocab, b + chunk);
-        for (int i = b; i < e; ++i) {
-          target -= static_cast<double>(expf((row[i] - row_max) * inv_t));
-          if (target < 0.0) {
-            result = i;
-            break;
-          }
-        }
-        break;
-      }
-      target -= slice_sum[t];
+  const int per_lane = (vocab + kWave * kSampleMaxGroups - 1) / (kWave * kSampleMaxGroups);   // 1 for usual vocabularies
+  const int group_size = kWave * per_lane;
+  const int n_groups = (vocab + group_size - 1) / group_size;
+  auto lane_weight_sum = [&](int g) {      // this lane's tokens of group g, in order
+    double s = 0.0;
+    const int first = g * group_size + lane * per_lane;
+    for (int j = 0; j < per_lane; ++j) {
+      const int i = first + j;
+      if (i < vocab) s += static_cast<double>(expf((row[i] - row_max) * inv_t));
     }
-    out[blockIdx.x] = result;
+    return s;
+  };
+  for (int g = wave; g < n_groups; g += kWaves) {
+    const double s = wave_sum_f64(lane_weight_sum(g));
+    if (lane == 0) group_sum[g] = s;
   }
+  __syncthreads();
+  if (wave != 0) return;
+
+  // one wave: running sums over the groups, 64 at a step; then the first group they cross the target in
+  double carry = 0.0;
+  for (int c = 0; c < n_groups; c += kWave) {
+    const int g = c + lane;
+    const double incl = carry + wave_scan_f64(g < n_groups ? group_sum[g] : 0.0, lane);
+    if (g < n_groups) group_sum[g] = incl;
+    carry = __shfl(incl, kWave - 1, kWave);
+  }
+  const double target = u[blockIdx.x] * carry;
+  int found = n_groups;
+  for (int c = 0; c < n_groups && found == n_groups; c += kWave) {
+    const int g = c + lane;
+    const unsigned long long over = __ballot(g < n_groups && target - group_sum[g] < 0.0);
+    if (over != 0ull) found = c + __ffsll(static_cast<long long>(over)) - 1;
+  }
+  int result = arg;        // rounding may leave the target a hair above zero after the last token
+  if (found < n_groups) {
+    const double before = found > 0 ? group_sum[found - 1] : 0.0;
+    const double mine = lane_weight_sum(found);
+    const double upto = before + wave_scan_f64(mine, lane);              // with this lane's tokens
+    const unsigned long long over = __ballot(target - upto < 0.0);
+    if (over != 0ull) {
+      const int at = __ffsll(static_cast<long long>(over)) - 1;          // the lane whose tokens cross it
+      double left = target - (upto - mine);
+      const int first = found * group_size + lane * per_lane;
+      int hit = min(vocab - 1, first + per_lane - 1);
+      for (int j = 0; j < per_lane; ++j) {
+        const int i = first + j;
+        if (i >= vocab) break;
+        left -= static_cast<double>(expf((row[i] - row_max) * inv_t));
+        if (left < 0.0) {
+          hit = i;
+          break;
+        }
+      }
+      result = __shfl(hit, at, kWave);
+    }
+  }
+  if (lane == 0) out[blockIdx.x] = result;
 }
 
 int grid_for(long total) {
@@ -587,6 +631,6 @@ extern "C" int bc4g_sample(const float* logits, const float* temperature, const 
                            int n_rows, int vocab, void* stream) {
   BC4G_REQUIRE(n_rows >= 0 && vocab > 0, "sample: bad sizes rows=%d V=%d", n_rows, vocab);
   if (n_rows == 0) return 0;
-  sample_kernel<<<n_rows, kBlock, 0, static_cast<hipStream_t>(stream)>>>(logits, temperature, u, out, vocab);
+  sample_kernel<<<n_rows, kSampleThreads, 0, static_cast<hipStream_t>(stream)>>>(logits, temperature, u, out, vocab);
   return check_launch("sample");
 }

@@ -487,6 +487,30 @@ def test_argmax_ties_and_sampling(ops):
             assert abs(got[i] - want) == 1 and edge < 1e-3 * cum[-1], (i, got[i], want)
 
 
+@pytest.mark.parametrize("vocab", [97, 1000, 128256, 300001])
+def test_sampling_follows_the_law_at_other_vocabularies(ops, vocab):
+    """The device's draw against the host's walk through the vocabulary for the same uniform numbers:
+    vocabularies that are no multiple of the 64-token groups, one as large as Llama 3's, and one beyond
+    262,144 tokens (a lane then takes several tokens of a group); u near 0 and near 1 reach the ends."""
+    from bare_cuda_4gib_amd.sampling import SamplingParams, sample_token
+    row = rnd(1, vocab, seed=21, scale=2.0).float()
+    us = [0.0, 1e-12, 0.25, 0.5, 0.731, 0.999999, 0.9999999999]
+    temps = [1.0, 0.7, 1.3, 0.2, 2.0, 1.0, 1.0]
+    got = ops.sample(row.expand(len(us), -1).contiguous().to(DEV), torch.tensor(temps, device=DEV),
+                     torch.tensor(us, dtype=torch.float64, device=DEV)).tolist()
+
+    class Fixed:
+        def __init__(self, u): self.u = u
+        def uniform(self): return self.u
+    for i, (uu, t) in enumerate(zip(us, temps)):
+        want = sample_token(row[0].numpy(), SamplingParams(temperature=t), Fixed(uu))
+        if got[i] != want:   # sums in another order may move a boundary by one token at most
+            w = np.exp((row[0].numpy() - row[0].numpy().max()) / t)
+            cum = np.cumsum(w.astype(np.float64))
+            edge = abs(uu * cum[-1] - cum[min(got[i], want)])
+            assert abs(got[i] - want) == 1 and edge < 1e-6 * cum[-1], (vocab, i, got[i], want)
+
+
 @pytest.mark.parametrize("m", [1, 7, 16])
 @pytest.mark.parametrize("n,k", [(130, 304), (2560, 2048), (301, 80)])
 @pytest.mark.parametrize("gdt", [torch.bfloat16, torch.float32])
