@@ -140,8 +140,24 @@ extern "C" {
 // epilogue (see gemm_skinny.hip).  x: bfloat16 [m, k] with g null (m <= 64), or the float32 residual
 // stream with RMSNorm fused (g given, m <= 16).  w: [(heads + 2 kv heads) * head_dim, k] with every
 // head's rows reordered in blocks of 16.  q_out: bfloat16 [m, heads * head_dim].
-int bc4g_gemm_skinny_qkv(const void* x, const void* g, int g_dtype, float eps, const void* w, void* q_out,
+// With ssq_parts (g null) x is bfloat16(residual * g) and the rows' scales come from the parts, as
+// in bc4g_gemm_skinny_prenormed.
+int bc4g_gemm_skinny_qkv(const void* x, const void* g, int g_dtype, float eps, const float* ssq_parts, int ssq_blocks,
+                         int ssq_stride, const void* w, void* q_out,
                          const int32_t* positions, const int32_t* slot_map, void* k_cache, void* v_cache,
                          int m, int k, int n_heads, int n_kv_heads, int head_dim, int rotary_dim, float theta,
                          int page_tokens, int write_kv, void* stream);
+}
+
+extern "C" {
+// The adding product that prepares the RMSNorm after it: out (the float32 residual stream, [m, n])
+// += x w^T; emit_x [m, n] = bfloat16(new residual * g) (g: that norm's scale, g_dtype 0 float32, 1
+// bfloat16); emit_ssq [ceil(n / 16)][emit_stride]: block b's part (16 columns) of every row's sum of
+// squares.  bc4g_gemm_skinny_prenormed takes such an x (k = this n) and the parts instead of a norm:
+// out = rmsnorm(residual) w^T, the row's rsqrt(sum of the parts / k + eps) applied to the finished
+// sums; epilogues of bc4g_gemm_skinny except the adding one.
+int bc4g_gemm_skinny_emit(const void* x, const void* w, float* out, const void* g, int g_dtype, void* emit_x,
+                          float* emit_ssq, int emit_stride, int m, int n, int k, void* stream);
+int bc4g_gemm_skinny_prenormed(const void* x, const float* ssq_parts, int ssq_blocks, int ssq_stride, float eps,
+                               const void* w, void* out, int epilogue, int m, int n, int k, void* stream);
 }

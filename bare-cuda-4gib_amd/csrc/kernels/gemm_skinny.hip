@@ -25,11 +25,18 @@
 //            workgroup writes bf16(x * g) into LDS and sums x^2 per row; the MFMAs read their B
 //            operand from LDS, and the row's rsqrt(mean(x^2) + eps) -- a factor common to the
 //            whole row -- multiplies the finished sum.
+//   prenormed  x is bfloat16(residual * g), written by the product that last added to the residual
+//            (below), together with parts of every row's sum of squares: the row's scale is worked out
+//            from the parts while the weights are on their way and multiplies the finished sum -- the
+//            norm costs neither a kernel of its own nor the staging of the float rows.
 // What goes out (EPI): bfloat16 or float stored; float added into the residual stream; SwiGLU,
 // when every 16 rows of w are eight gate rows followed by the eight up rows of the same outputs; or
 // rotary positions and the cache write, when w holds query, key and value heads with every head's
 // rows reordered in blocks of 16 (eight dimensions, then their rotation partners): queries are
-// stored rotated, keys rotated into their page, values into theirs.
+// stored rotated, keys rotated into their page, values into theirs.  The epilogue that adds into the
+// residual stream can prepare the RMSNorm that follows (emit): it also stores bfloat16(new residual * g)
+// and, per row, the sum of squares over its 16 columns -- parts that the next product adds up in
+// block order, so the result does not depend on timing.
 #include <math.h>
 
 #include "api.h"
@@ -66,6 +73,14 @@ struct SkinnyArgs {
   int rows_per_block;       // plain mode: blockIdx.y takes rows y * rows_per_block .. of x and out (0: all rows)
   int m_stage;              // normed modes: rows of x staged in LDS (m rounded up to 4)
   float eps;
+  // prenormed x (plain mode): parts [ssq_blocks][ssq_stride] of the rows' sums of squares (null: x as it is)
+  const float* ssq_parts;
+  int ssq_blocks, ssq_stride;
+  // kAccumF32: what the RMSNorm after this product needs (emit_g null: nothing)
+  const void* emit_g;       // [n] its scale, bfloat16 or float (emit_g_f32)
+  bf16_t* emit_x;           // [m, n] bfloat16(new residual * g)
+  float* emit_ssq;          // [ceil(n / 16)][emit_stride]: block b's part of row r's sum of squares
+  int emit_g_f32, emit_stride;
   RopeKvArgs rope;          // kRopeKvBf16 only
 };
 
@@ -92,6 +107,11 @@ __global__ __launch_bounds__(kThreads, XMODE != kPlain ? 6 : 4) void gemm_skinny
       a.rope.positions = args.rope.positions ? args.rope.positions + row0 : nullptr;
       a.rope.slot_map = args.rope.slot_map ? args.rope.slot_map + row0 : nullptr;
     } else a.out = static_cast<float*>(args.out) + row0 * args.n;
+    if (args.ssq_parts) a.ssq_parts = args.ssq_parts + row0;
+    if (EPI == kAccumF32 && args.emit_g) {
+      a.emit_x = args.emit_x + row0 * args.n;
+      a.emit_ssq = args.emit_ssq + row0;
+    }
   }
   constexpr bool kTurned = !kNormed;                      // x reaches operand order through LDS
   constexpr int kPieces = 4 * U;                       // 16-byte pieces of a row in one batch of k-steps
@@ -104,7 +124,7 @@ __global__ __launch_bounds__(kThreads, XMODE != kPlain ? 6 : 4) void gemm_skinny
   constexpr int kTurnBytes = kTurned ? kWaves * MT * 16 * kPieces * 16 : 0;
   __shared__ __align__(16) unsigned char pool[kRedBytes > kTurnBytes ? kRedBytes : kTurnBytes];
   Red* red = reinterpret_cast<Red*>(pool);
-  __shared__ float ssq_row[16];
+  __shared__ float ssq_row[MT * 16];
   extern __shared__ __align__(16) unsigned char stage_raw[];   // normed: bf16 [m_stage][k + kStagePad]
   const int lane = threadIdx.x % kWave;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);   // uniform: k ranges and bases stay scalar
@@ -179,6 +199,19 @@ __global__ __launch_bounds__(kThreads, XMODE != kPlain ? 6 : 4) void gemm_skinny
         sincosf(static_cast<float>(r.positions[row]) * inv_freq, &rope_sn[j], &rope_cs[j]);
       }
       rope_slot[j] = (live && head >= r.n_heads && r.write_kv) ? r.slot_map[row] : 0;
+    }
+  }
+
+  // prenormed x: every row's sum of squares from its parts, in block order (threads take rows; a
+  // block's parts of neighbouring rows lie next to each other)
+  const bool prenormed = !kNormed && a.ssq_parts != nullptr;
+  if (prenormed) {
+    for (int row = threadIdx.x; row < MT * 16; row += kThreads) {
+      float ss = 0.f;
+      if (row < m) {
+        for (int b = 0; b < a.ssq_blocks; ++b) ss += a.ssq_parts[static_cast<long>(b) * a.ssq_stride + row];
+      }
+      ssq_row[row] = ss;
     }
   }
 
@@ -340,19 +373,22 @@ __global__ __launch_bounds__(kThreads, XMODE != kPlain ? 6 : 4) void gemm_skinny
 #pragma unroll
   for (int j = 0; j < kItems; ++j) {
     const int idx = threadIdx.x + j * kThreads;
-    if (idx >= MT * 16 * kCols) continue;
     const int nl = idx % kCols, row = idx / kCols;
     const int gn = n0 + nl;
-    if (row >= m || gn >= a.n) continue;
+    const bool live = idx < MT * 16 * kCols && row < m && gn < a.n;
+    // (the adding epilogue goes on with every lane: its lanes may have sums of squares to exchange)
+    if (EPI != kAccumF32 && !live) continue;
     float sum = 0.f, partner = 0.f;
+    if (live) {
 #pragma unroll
-    for (int wv = 0; wv < kWaves; ++wv) sum += red[wv][row / 16][nl][row % 16];
-    if constexpr (kPaired) {
+      for (int wv = 0; wv < kWaves; ++wv) sum += red[wv][row / 16][nl][row % 16];
+      if constexpr (kPaired) {
 #pragma unroll
-      for (int wv = 0; wv < kWaves; ++wv) partner += red[wv][row / 16][nl + 8][row % 16];
+        for (int wv = 0; wv < kWaves; ++wv) partner += red[wv][row / 16][nl + 8][row % 16];
+      }
     }
-    if constexpr (kNormed) {
-      const float scale = 1.0f / sqrtf(ssq_row[row] / static_cast<float>(k) + a.eps);
+    if (kNormed || prenormed) {
+      const float scale = live ? 1.0f / sqrtf(ssq_row[row] / static_cast<float>(k) + a.eps) : 0.f;
       sum *= scale;
       partner *= scale;
     }
@@ -361,7 +397,22 @@ __global__ __launch_bounds__(kThreads, XMODE != kPlain ? 6 : 4) void gemm_skinny
     } else if constexpr (EPI == kStoreF32) {
       static_cast<float*>(a.out)[static_cast<long>(row) * a.n + gn] = sum;
     } else if constexpr (EPI == kAccumF32) {
-      static_cast<float*>(a.out)[static_cast<long>(row) * a.n + gn] = prev[j] + sum;
+      const float nv = prev[j] + sum;
+      if (live) static_cast<float*>(a.out)[static_cast<long>(row) * a.n + gn] = nv;
+      if (a.emit_g != nullptr) {
+        // for the RMSNorm that follows: bf16(new residual * g), and this block's part of the row's sum
+        // of squares (a row's 16 columns lie in 16 neighbouring lanes)
+        float sq = 0.f;
+        if (live) {
+          const float g = a.emit_g_f32 ? static_cast<const float*>(a.emit_g)[gn]
+                                       : to_float(static_cast<const bf16_t*>(a.emit_g)[gn]);
+          a.emit_x[static_cast<long>(row) * a.n + gn] = from_float<bf16_t>(nv * g);
+          sq = nv * nv;
+        }
+#pragma unroll
+        for (int off = 1; off < 16; off <<= 1) sq += __shfl_xor(sq, off, kWave);
+        if (nl == 0 && idx < MT * 256 && row < m) a.emit_ssq[static_cast<long>(blockIdx.x) * a.emit_stride + row] = sq;
+      }
     } else if constexpr (EPI == kSwigluBf16) {
       // block b = n0 / 16 holds gates and ups of outputs 8b .. 8b + 7
       const long o = static_cast<long>(row) * (a.n / 2) + (n0 / 2 + nl);
@@ -491,12 +542,71 @@ int check_rope(const char* what, const RopeKvArgs& r, int n) {
 
 using namespace bc4g;
 
+namespace bc4g {
+namespace {
+SkinnyArgs plain_args(const void* x, const void* w, void* out, int m, int n, int k) {
+  SkinnyArgs a{};
+  a.x = x;
+  a.w = static_cast<const bf16_t*>(w);
+  a.out = out;
+  a.m = m;
+  a.n = n;
+  a.k = k;
+  a.n_out = n;
+  return a;
+}
+
+int check_parts(const char* what, const float* ssq_parts, int ssq_blocks, int ssq_stride, int m, float eps) {
+  BC4G_REQUIRE(ssq_parts != nullptr && ssq_blocks > 0 && ssq_stride >= m, "%s: the sums of squares need %d parts of at least %d rows",
+               what, ssq_blocks, m);
+  BC4G_REQUIRE(eps >= 0.f, "%s: eps must not be negative", what);
+  return 0;
+}
+}  // namespace
+}  // namespace bc4g
+
 extern "C" int bc4g_gemm_skinny(const void* x, const void* w, void* out, int epilogue, int m, int n, int k,
                                 void* stream) {
   if (int e = check_common("gemm_skinny", m, 64, n, k, epilogue)) return e;
   BC4G_REQUIRE(epilogue != kRopeKvBf16, "gemm_skinny: use bc4g_gemm_skinny_qkv for the rotary epilogue");
   if (m == 0) return 0;
-  SkinnyArgs a{x, nullptr, nullptr, static_cast<const bf16_t*>(w), out, m, n, k, n, 0, 0, 0.f, {}};
+  SkinnyArgs a = plain_args(x, w, out, m, n, k);
+  return launch_epilogue<kPlain>(a, epilogue, static_cast<hipStream_t>(stream));
+}
+
+// out (the float residual stream, [m, n]) += x w^T, and what the RMSNorm after it needs: emit_x
+// [m, n] = bfloat16(new residual * g) and emit_ssq [ceil(n / 16)][emit_stride], block b's part of
+// every row's sum of squares.
+extern "C" int bc4g_gemm_skinny_emit(const void* x, const void* w, float* out, const void* g, int g_dtype, void* emit_x,
+                                     float* emit_ssq, int emit_stride, int m, int n, int k, void* stream) {
+  if (int e = check_common("gemm_skinny_emit", m, 64, n, k, kAccumF32)) return e;
+  BC4G_REQUIRE(g && emit_x && emit_ssq && emit_stride >= m, "gemm_skinny_emit: the norm's scale and both outputs are needed");
+  BC4G_REQUIRE(g_dtype == kBF16 || g_dtype == kF32, "gemm_skinny_emit: unknown norm scale dtype %d", g_dtype);
+  if (m == 0) return 0;
+  SkinnyArgs a = plain_args(x, w, out, m, n, k);
+  a.emit_g = g;
+  a.emit_g_f32 = g_dtype == kF32 ? 1 : 0;
+  a.emit_x = static_cast<bf16_t*>(emit_x);
+  a.emit_ssq = emit_ssq;
+  a.emit_stride = emit_stride;
+  return launch<kAccumF32, kPlain>(a, static_cast<hipStream_t>(stream));
+}
+
+// x is bfloat16(residual * g) and ssq_parts the parts of the rows' sums of squares, as
+// bc4g_gemm_skinny_emit leaves them: out = rmsnorm(residual) w^T with the epilogues of bc4g_gemm_skinny
+// except the adding one.
+extern "C" int bc4g_gemm_skinny_prenormed(const void* x, const float* ssq_parts, int ssq_blocks, int ssq_stride, float eps,
+                                          const void* w, void* out, int epilogue, int m, int n, int k, void* stream) {
+  if (int e = check_common("gemm_skinny_prenormed", m, 64, n, k, epilogue)) return e;
+  if (int e = check_parts("gemm_skinny_prenormed", ssq_parts, ssq_blocks, ssq_stride, m, eps)) return e;
+  BC4G_REQUIRE(epilogue != kAccumF32 && epilogue != kRopeKvBf16, "gemm_skinny_prenormed: epilogue %d is not supported here",
+               epilogue);
+  if (m == 0) return 0;
+  SkinnyArgs a = plain_args(x, w, out, m, n, k);
+  a.ssq_parts = ssq_parts;
+  a.ssq_blocks = ssq_blocks;
+  a.ssq_stride = ssq_stride;
+  a.eps = eps;
   return launch_epilogue<kPlain>(a, epilogue, static_cast<hipStream_t>(stream));
 }
 
@@ -507,7 +617,11 @@ extern "C" int bc4g_gemm_skinny_normed(const float* x, const int32_t* rows, cons
   BC4G_REQUIRE(epilogue != kAccumF32 && epilogue != kRopeKvBf16, "gemm_skinny_normed: epilogue %d is not supported here",
                epilogue);
   if (m == 0) return 0;
-  SkinnyArgs a{x, rows, g, static_cast<const bf16_t*>(w), out, m, n, k, n, 0, ((m + 3) / 4) * 4, eps, {}};
+  SkinnyArgs a = plain_args(x, w, out, m, n, k);
+  a.rows = rows;
+  a.g = g;
+  a.m_stage = ((m + 3) / 4) * 4;
+  a.eps = eps;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (g_dtype == kBF16) return launch_epilogue<kNormedG16>(a, epilogue, s);
   if (g_dtype == kF32) return launch_epilogue<kNormedG32>(a, epilogue, s);
@@ -515,9 +629,12 @@ extern "C" int bc4g_gemm_skinny_normed(const float* x, const int32_t* rows, cons
 }
 
 // The query/key/value product of a decode step with rotary positions and the cache write in its
-// epilogue.  x: bfloat16 [m, k] (g null), or the float residual stream with RMSNorm fused (g given,
-// m <= 16).  q_out: bfloat16 [m, n_heads * head_dim], rotated, in the reordered head layout.
-extern "C" int bc4g_gemm_skinny_qkv(const void* x, const void* g, int g_dtype, float eps, const void* w, void* q_out,
+// epilogue.  x: bfloat16 [m, k] (g null) -- with ssq_parts given it is bfloat16(residual * g) and the
+// rows' scales come from the parts, as in bc4g_gemm_skinny_prenormed -- or the float residual stream
+// with RMSNorm fused (g given, m <= 16).  q_out: bfloat16 [m, n_heads * head_dim], rotated, in the
+// reordered head layout.
+extern "C" int bc4g_gemm_skinny_qkv(const void* x, const void* g, int g_dtype, float eps, const float* ssq_parts,
+                                    int ssq_blocks, int ssq_stride, const void* w, void* q_out,
                                     const int32_t* positions, const int32_t* slot_map, void* k_cache, void* v_cache,
                                     int m, int k, int n_heads, int n_kv_heads, int head_dim, int rotary_dim,
                                     float theta, int page_tokens, int write_kv, void* stream) {
@@ -527,9 +644,20 @@ extern "C" int bc4g_gemm_skinny_qkv(const void* x, const void* g, int g_dtype, f
   const int n = (n_heads + 2 * n_kv_heads) * head_dim;
   if (int e = check_common("gemm_skinny_qkv", m, g ? 16 : 64, n, k, kRopeKvBf16)) return e;
   if (int e = check_rope("gemm_skinny_qkv", r, n)) return e;
+  BC4G_REQUIRE(!(g && ssq_parts), "gemm_skinny_qkv: the norm is either fused or prepared, not both");
+  if (ssq_parts) {
+    if (int e = check_parts("gemm_skinny_qkv", ssq_parts, ssq_blocks, ssq_stride, m, eps)) return e;
+  }
   if (m == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  SkinnyArgs a{x, nullptr, g, static_cast<const bf16_t*>(w), q_out, m, n, k, n, 0, g ? ((m + 3) / 4) * 4 : 0, eps, r};
+  SkinnyArgs a = plain_args(x, w, q_out, m, n, k);
+  a.g = g;
+  a.m_stage = g ? ((m + 3) / 4) * 4 : 0;
+  a.eps = eps;
+  a.rope = r;
+  a.ssq_parts = ssq_parts;
+  a.ssq_blocks = ssq_blocks;
+  a.ssq_stride = ssq_stride;
   if (!g) return launch<kRopeKvBf16, kPlain>(a, s);
   if (g_dtype == kBF16) return launch<kRopeKvBf16, kNormedG16>(a, s);
   if (g_dtype == kF32) return launch<kRopeKvBf16, kNormedG32>(a, s);

@@ -443,6 +443,74 @@ def gemm_swiglu(a: torch.Tensor, w_gate_up, interleaved: bool = False) -> torch.
     return swiglu(gu, interleaved)
 
 
+class Prenormed:
+    """What a product that added into the residual stream left for the RMSNorm after it
+    (gemm_accumulate_emit): ``xb`` = bfloat16(residual * g) [m, width] and ``parts`` [blocks, m], block
+    b's share (16 columns) of every row's sum of squares.  A product that takes it
+    (gemm_prenormed, gemm_qkv_rope) applies the row's rsqrt(sum of parts / width + eps) to its sums."""
+
+    def __init__(self, xb: torch.Tensor, parts: torch.Tensor, eps: float):
+        self.xb, self.parts, self.eps = xb, parts, float(eps)
+
+
+def gemm_emit_supported(a: torch.Tensor, w, residual: torch.Tensor, g: torch.Tensor) -> bool:
+    """Whether the adding product of these operands can prepare the next RMSNorm: the
+    weight-streaming kernel serves it (bfloat16, up to SKINNY_PASSES_ROWS rows)."""
+    w, _ = _weight(w)
+    return (_fast_operands(a, w) and 0 < a.shape[0] <= SKINNY_PASSES_ROWS and residual.dtype == torch.float32
+            and g.dtype in _CODE and tuple(g.shape) == (w.shape[0],))
+
+
+def gemm_accumulate_emit(a: torch.Tensor, w, residual: torch.Tensor, g: torch.Tensor, eps: float) -> Prenormed:
+    """residual += a w^T, and the next RMSNorm (scale g, eps) prepared: see Prenormed."""
+    w, packed = _weight(w)
+    packed = packed if packed is not None else pack_weight(w)
+    _dev("gemm_accumulate_emit", a, w, residual, g)
+    m, k = a.shape
+    n = w.shape[0]
+    if tuple(residual.shape) != (m, n) or residual.dtype != torch.float32 or not residual.is_contiguous():
+        raise KernelError(f"gemm_accumulate_emit: the residual must be contiguous float32 [{m}, {n}]")
+    if tuple(g.shape) != (n,):
+        raise KernelError(f"gemm_accumulate_emit: norm scale must be [{n}], got {tuple(g.shape)}")
+    xb = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
+    parts = torch.empty((-(-n // 16), m), dtype=torch.float32, device=a.device)
+    for r0 in range(0, m, SKINNY_MAX_ROWS):
+        rows = min(SKINNY_MAX_ROWS, m - r0)
+        library.call("bc4g_gemm_skinny_emit", _ptr(a[r0:]), _ptr(packed), _ptr(residual[r0:]), _ptr(g),
+                     _code(g, "gemm_accumulate_emit"), _ptr(xb[r0:]), _ptr(parts[:, r0:]), m, rows, n, k, _stream(),
+                     cost=_gemm_cost(rows, n, k, 2, 2, 10))
+    return Prenormed(xb, parts, eps)
+
+
+def gemm_prenormed_supported(pre: Prenormed, w) -> bool:
+    w, _ = _weight(w)
+    return _fast_operands(pre.xb, w) and pre.xb.shape[0] <= SKINNY_PASSES_ROWS
+
+
+def gemm_prenormed(pre: Prenormed, w, epilogue: int) -> torch.Tensor:
+    """rmsnorm(residual) w^T from what gemm_accumulate_emit left: epilogue EPI_STORE_BF16,
+    EPI_STORE_F32 or EPI_SWIGLU (w in blocks of eight gate and eight up rows)."""
+    w, packed = _weight(w)
+    packed = packed if packed is not None else pack_weight(w)
+    _dev("gemm_prenormed", pre.xb, pre.parts, w)
+    m, k = pre.xb.shape
+    n = w.shape[0]
+    if epilogue == EPI_SWIGLU:
+        out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=w.device)
+    elif epilogue == EPI_STORE_BF16:
+        out = torch.empty((m, n), dtype=torch.bfloat16, device=w.device)
+    elif epilogue == EPI_STORE_F32:
+        out = torch.empty((m, n), dtype=torch.float32, device=w.device)
+    else:
+        raise KernelError(f"gemm_prenormed: epilogue {epilogue} is not supported")
+    for r0 in range(0, m, SKINNY_MAX_ROWS):
+        rows = min(SKINNY_MAX_ROWS, m - r0)
+        library.call("bc4g_gemm_skinny_prenormed", _ptr(pre.xb[r0:]), _ptr(pre.parts[:, r0:]), pre.parts.shape[0], m,
+                     pre.eps, _ptr(packed), _ptr(out[r0:]), epilogue, rows, n, k, _stream(),
+                     cost=_gemm_cost(rows, n, k, 2, 2, out.element_size() * out.shape[1] / n))
+    return out
+
+
 def gemm_qkv_rope_supported(x: torch.Tensor, n_rows: int, normed: bool, w, head_dim: int,
                             rotary_dim: int) -> bool:
     """Whether the q|k|v product of these rows can rotate and write the cache in its epilogue."""
@@ -456,10 +524,11 @@ def gemm_qkv_rope_supported(x: torch.Tensor, n_rows: int, normed: bool, w, head_
 def gemm_qkv_rope(x: torch.Tensor, g: Optional[torch.Tensor], eps: float, w,
                   positions: torch.Tensor, slot_map: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
                   v_cache: Optional[torch.Tensor], n_heads: int, n_kv_heads: int, head_dim: int, rotary_dim: int,
-                  theta: float, write_kv: bool = True) -> torch.Tensor:
+                  theta: float, write_kv: bool = True, pre: Optional[Prenormed] = None) -> torch.Tensor:
     """The q|k|v product of a decode step with rotary positions and the cache write in its
     epilogue (w in the reordered head layout).  With g the input is the float residual stream
-    and RMSNorm is fused.  Returns the rotated queries [M, heads * head_dim]."""
+    and RMSNorm is fused; with ``pre`` (x = pre.xb) the norm was prepared by the product before.
+    Returns the rotated queries [M, heads * head_dim]."""
     w, packed = _weight(w)
     packed = packed if packed is not None else pack_weight(w)
     _dev("gemm_qkv_rope", x, g, w, positions, slot_map, k_cache, v_cache)
@@ -476,10 +545,14 @@ def gemm_qkv_rope(x: torch.Tensor, g: Optional[torch.Tensor], eps: float, w,
     if g is not None and (tuple(g.shape) != (k,) or x.dtype != torch.float32):
         raise KernelError("gemm_qkv_rope: the fused norm needs a float32 input and a scale of its width")
     q = torch.empty((m, n_heads * head_dim), dtype=torch.bfloat16, device=x.device)
+    if pre is not None and (g is not None or x is not pre.xb):
+        raise KernelError("gemm_qkv_rope: a prepared norm comes with its own rows and without a scale")
+    parts = pre.parts if pre is not None else None
     library.call("bc4g_gemm_skinny_qkv", _ptr(x), _ptr(g), _code(g, "gemm_qkv_rope") if g is not None else 0,
-                 float(eps), _ptr(packed), _ptr(q), _ptr(positions), _ptr(slot_map), _ptr(k_cache), _ptr(v_cache),
-                 m, k, n_heads, n_kv_heads, head_dim, int(rotary_dim), float(theta), page_tokens,
-                 1 if write_kv else 0, _stream(), cost=_gemm_cost(m, n, k, x.element_size(), 2, 2))
+                 float(pre.eps if pre is not None else eps), _ptr(parts), parts.shape[0] if pre is not None else 0,
+                 parts.shape[1] if pre is not None else 0, _ptr(packed), _ptr(q), _ptr(positions), _ptr(slot_map),
+                 _ptr(k_cache), _ptr(v_cache), m, k, n_heads, n_kv_heads, head_dim, int(rotary_dim), float(theta),
+                 page_tokens, 1 if write_kv else 0, _stream(), cost=_gemm_cost(m, n, k, x.element_size(), 2, 2))
     return q
 
 

@@ -597,6 +597,65 @@ def test_qkv_product_with_rotation_and_cache_write(ops, nh, nkv, d, m, normed, r
         close(buf.view(m, nh + 2 * nkv, d)[:, :nh], q.view(m, nh, d), 1e-2, 2e-2, "unfused queries")
 
 
+@pytest.mark.parametrize("m", [1, 5, 8, 9, 16, 33, 64, 100])
+@pytest.mark.parametrize("width,k,gdt", [(96, 40, torch.bfloat16), (2048, 256, torch.bfloat16), (200, 72, torch.float32)])
+def test_adding_product_prepares_the_next_norm(ops, m, width, k, gdt):
+    """The product that adds into the residual stream also leaves bfloat16(new residual * g) and, per
+    block of 16 columns, every row's part of its sum of squares; the product after it takes both
+    instead of a norm.  The residual is the same bits as without the extra outputs; what is left is
+    exactly what the definition says; and the next product equals rmsnorm(residual) w^T computed from
+    the residual it saw -- with every epilogue, the q|k|v one with rotation and cache write included."""
+    a, w = bf(rnd(m, k, seed=70)), bf(rnd(width, k, seed=71, scale=0.3))
+    g = (1.0 + 0.2 * rnd(width, seed=72)).to(gdt)
+    base = rnd(m, width, seed=73, scale=2.0).float()
+    res, res_plain = base.clone().to(DEV), base.clone().to(DEV)
+    assert ops.gemm_emit_supported(a.to(DEV), w.to(DEV), res, g.to(DEV))
+    pre = ops.gemm_accumulate_emit(a.to(DEV), w.to(DEV), res, g.to(DEV), 1e-5)
+    ops.gemm_fast(a.to(DEV), w.to(DEV), accumulate_into=res_plain)
+    assert torch.equal(res, res_plain)
+    r = res.cpu()
+    assert torch.equal(pre.xb.cpu(), (r * g.float()).to(torch.bfloat16))
+    assert tuple(pre.parts.shape) == (-(-width // 16), m)
+    pad = torch.zeros(m, 16 * pre.parts.shape[0])
+    pad[:, :width] = r
+    close(pre.parts.cpu().T, (pad.double() ** 2).view(m, -1, 16).sum(-1), 1e-5, 1e-6, "parts of the sums of squares")
+    # the product after it
+    hb = pre.xb.cpu().double() / torch.sqrt((r.double() ** 2).mean(-1, keepdim=True) + 1e-5)
+    n2 = 176
+    w2 = bf(rnd(n2, width, seed=74, scale=0.3))
+    scale = math.sqrt(width)
+    close(ops.gemm_prenormed(pre, w2.to(DEV), ops.EPI_STORE_F32), hb @ w2.double().T, 1e-4, 1e-4 * scale, "prenormed -> f32")
+    close(ops.gemm_prenormed(pre, w2.to(DEV), ops.EPI_STORE_BF16), hb @ w2.double().T, 8e-3, 1e-3 * scale, "prenormed -> bf16")
+    gu = hb @ w2.double().T
+    wi = interleave8(w2[:n2 // 2], w2[n2 // 2:])
+    close(ops.gemm_prenormed(pre, wi.to(DEV), ops.EPI_SWIGLU), P.swiglu(gu[:, :n2 // 2], gu[:, n2 // 2:]), 8e-3, 3e-2,
+          "prenormed, SwiGLU")
+    if m <= 8 and width % 8 == 0:   # the norm fused into the product instead: the same up to rounding
+        fused = ops.gemm_normed(res, None, m, g.to(DEV), 1e-5, w2.to(DEV), ops.EPI_STORE_F32)
+        close(ops.gemm_prenormed(pre, w2.to(DEV), ops.EPI_STORE_F32), fused, 1e-4, 1e-4 * scale, "against the fused norm")
+    if m <= 64:
+        nh, nkv, d, page, pages, theta = 3, 1, 32, 16, 8, 10000.0
+        order = block_order(d)
+        wq = bf(rnd((nh + 2 * nkv) * d, width, seed=75, scale=0.3))
+        wp = wq.view(nh + 2 * nkv, d, width)[:, order, :].reshape(-1, width).contiguous()
+        positions = [2 + 3 * i for i in range(m)]
+        slots = random.Random(2).sample(range(pages * page), m)
+        kc = torch.full((pages, nkv, page, d), -7.5, dtype=torch.bfloat16, device=DEV)
+        vc = torch.full((pages, nkv, d, page), -7.5, dtype=torch.bfloat16, device=DEV)
+        q = ops.gemm_qkv_rope(pre.xb, None, 0.0, wp.to(DEV), torch.tensor(positions, dtype=torch.int32, device=DEV),
+                              torch.tensor(slots, dtype=torch.int32, device=DEV), kc, vc, nh, nkv, d, d, theta, pre=pre)
+        qkv = (hb @ wq.double().T).view(m, nh + 2 * nkv, d)
+        pos = torch.tensor(positions)
+        tol = dict(rtol=2e-2, atol=3e-2)
+        close(q.view(m, nh, d), P.rope(qkv[:, :nh], pos, theta)[:, :, order], what="q after a prepared norm", **tol)
+        kc_c, vc_c = (c.cpu().double() for c in ops.cache_to_plain(kc, vc))
+        k_want = P.rope(qkv[:, nh:nh + nkv], pos, theta)
+        for i, sl in enumerate(slots):
+            pg, off = divmod(sl, page)
+            close(kc_c[pg, :, off, :], k_want[i][:, order], what=f"k row {i} after a prepared norm", **tol)
+            close(vc_c[pg, :, :, off], qkv[i, nh + nkv:][:, order], what=f"v row {i} after a prepared norm", **tol)
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("m,n,k", [(1, 48, 64), (7, 100, 200), (33, 272, 1000), (64, 16, 8)])
 def test_streamed_weight_packing(ops, m, n, k):
