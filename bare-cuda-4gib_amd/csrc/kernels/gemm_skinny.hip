@@ -124,7 +124,7 @@ __global__ __launch_bounds__(kThreads, XMODE != kPlain ? 6 : 4) void gemm_skinny
   constexpr int kTurnBytes = kTurned ? kWaves * MT * 16 * kPieces * 16 : 0;
   __shared__ __align__(16) unsigned char pool[kRedBytes > kTurnBytes ? kRedBytes : kTurnBytes];
   Red* red = reinterpret_cast<Red*>(pool);
-  __shared__ float ssq_row[MT * 16];
+  __shared__ float ssq_row[16];
   extern __shared__ __align__(16) unsigned char stage_raw[];   // normed: bf16 [m_stage][k + kStagePad]
   const int lane = threadIdx.x % kWave;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);   // uniform: k ranges and bases stay scalar
@@ -202,18 +202,31 @@ __global__ __launch_bounds__(kThreads, XMODE != kPlain ? 6 : 4) void gemm_skinny
     }
   }
 
-  // prenormed x: every row's sum of squares from its parts, in block order (threads take rows; a
-  // block's parts of neighbouring rows lie next to each other)
+  // prenormed x: every row's sum of squares from its parts.  Eight threads a row, thread j adding
+  // the parts of blocks j, j + 8, ... in ascending order (its loads all in flight together); the eight
+  // sums meet in LDS and are added in order of j after the product: the order of the additions, and
+  // so the rounding, is the same for every number of rows.  (After the first weights have been asked for.)
+  constexpr int kPartSums = 8;
+  __shared__ float part_sum[kPartSums][MT * 16];
   const bool prenormed = !kNormed && a.ssq_parts != nullptr;
-  if (prenormed) {
-    for (int row = threadIdx.x; row < MT * 16; row += kThreads) {
+  auto sum_parts = [&]() {
+    if (prenormed && threadIdx.x < kPartSums * MT * 16) {
+      const int row = threadIdx.x % (MT * 16), j0 = threadIdx.x / (MT * 16);
       float ss = 0.f;
       if (row < m) {
-        for (int b = 0; b < a.ssq_blocks; ++b) ss += a.ssq_parts[static_cast<long>(b) * a.ssq_stride + row];
+        const float* p = a.ssq_parts + row;
+        int b = j0;
+        for (; b + 3 * kPartSums < a.ssq_blocks; b += 4 * kPartSums) {
+          const float p0 = p[static_cast<long>(b) * a.ssq_stride], p1 = p[static_cast<long>(b + kPartSums) * a.ssq_stride];
+          const float p2 = p[static_cast<long>(b + 2 * kPartSums) * a.ssq_stride];
+          const float p3 = p[static_cast<long>(b + 3 * kPartSums) * a.ssq_stride];
+          ss = (((ss + p0) + p1) + p2) + p3;
+        }
+        for (; b < a.ssq_blocks; b += kPartSums) ss += p[static_cast<long>(b) * a.ssq_stride];
       }
-      ssq_row[row] = ss;
+      part_sum[j0][row] = ss;
     }
-  }
+  };
 
   // kTurned: load i of a batch brings piece (i * 64 + lane) % kPieces of row (i * 64 + lane) / kPieces;
   // in the wave's buffer piece p of row r lies at r * kPieces + (p ^ (r % 8)), which keeps both the
@@ -350,6 +363,7 @@ __global__ __launch_bounds__(kThreads, XMODE != kPlain ? 6 : 4) void gemm_skinny
     lds_barrier();                                         // (the weights stay in flight)
   } else {
     if (k_begin < k_end) load(cur, k_begin);
+    sum_parts();
   }
 
   for (int k0 = k_begin; k0 < k_end; k0 += kStep) {
@@ -388,7 +402,16 @@ __global__ __launch_bounds__(kThreads, XMODE != kPlain ? 6 : 4) void gemm_skinny
       }
     }
     if (kNormed || prenormed) {
-      const float scale = live ? 1.0f / sqrtf(ssq_row[row] / static_cast<float>(k) + a.eps) : 0.f;
+      float ssq = 0.f;
+      if (live) {
+        if (prenormed) {
+#pragma unroll
+          for (int j2 = 0; j2 < kPartSums; ++j2) ssq += part_sum[j2][row];
+        } else {
+          ssq = ssq_row[row];
+        }
+      }
+      const float scale = live ? 1.0f / sqrtf(ssq / static_cast<float>(k) + a.eps) : 0.f;
       sum *= scale;
       partner *= scale;
     }

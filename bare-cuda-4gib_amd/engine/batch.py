@@ -39,6 +39,14 @@ class StepContext:
     tiles: Dict[int, Any] = dataclasses.field(default_factory=dict)
     made: Dict[Any, Any] = dataclasses.field(default_factory=dict)      # see shared()
     fixed_attention_splits: int = 0      # non-zero: the key split count is fixed (a captured step)
+    # The norm that reads the residual stream next, while a part that adds into the stream runs (set by
+    # the block around the part; by the model: the norm the next schedule entry begins with).  A product
+    # that adds into the stream may then prepare that norm and leave the result in ``prepared`` under
+    # id(norm part); the block hands it to the norm's consumer.  Nothing prepared outlives the entry
+    # after the one that made it.
+    norm_after: Any = None
+    next_entry_norm: Any = None
+    prepared: Dict[int, Any] = dataclasses.field(default_factory=dict)
 
     def cache(self, stream: Optional[Hashable]):
         return None if stream is None else self.cache_views.get(stream)

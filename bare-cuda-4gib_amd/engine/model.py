@@ -133,8 +133,20 @@ class Model:
         """Run the batch through every schedule entry; float32 logits at the
         wanted rows ([n_logits, vocab]), or None if none are wanted."""
         x = self.embedding.part.forward(ctx)
-        for e in self.schedule:
-            self.layers[e.layer].forward(x, ctx, ctx.cache(e.cache), e.writes)
+        ctx.prepared.clear()
+        for i, e in enumerate(self.schedule):
+            layer = self.layers[e.layer]
+            # what the entry before prepared for this entry's first norm stays; nothing else does
+            first = layer.first_norm(ctx.n_tokens) if hasattr(layer, "first_norm") else None
+            kept = ctx.prepared.pop(id(first), None) if first is not None else None
+            ctx.prepared.clear()
+            if kept is not None:
+                ctx.prepared[id(first)] = kept
+            following = self.layers[self.schedule[i + 1].layer] if i + 1 < len(self.schedule) else None
+            ctx.next_entry_norm = following.first_norm(ctx.n_tokens) if hasattr(following, "first_norm") else None
+            layer.forward(x, ctx, ctx.cache(e.cache), e.writes)
+        ctx.prepared.clear()
+        ctx.next_entry_norm = None
         if ctx.n_logits == 0:
             return None
         norm, head = self.final_norm.part, self.head.part

@@ -18,15 +18,36 @@ class PreNormBlock(Part):
         return [self.mixer_norm, self.mixer, self.ffn_norm, self.ffn]
 
     def forward(self, x, ctx, cache, writes: bool = True) -> None:
+        # Each part is told which norm reads the stream after it, so that its last product can
+        # prepare that norm: the feed-forward's after the mixer, the next entry's first after the
+        # feed-forward.
+        after = ctx.next_entry_norm
+        ctx.norm_after = self.ffn_norm if self._wants_prepared(self.ffn, x.shape[0]) else None
         self.mixer.forward(self._normed(self.mixer, self.mixer_norm, x, ctx), ctx, cache, x, writes)
+        ctx.norm_after = after
         self.ffn.forward(self._normed(self.ffn, self.ffn_norm, x, ctx), ctx, x)
+        ctx.norm_after = None
+
+    def first_norm(self, n_rows: int):
+        """The norm this block begins with, if the entry before should prepare it for a step of
+        ``n_rows`` rows (else None)."""
+        return self.mixer_norm if self._wants_prepared(self.mixer, n_rows) else None
+
+    @staticmethod
+    def _wants_prepared(part, n_rows: int) -> bool:
+        """Whether the part's first product is better served by a prepared norm than by fusing the
+        norm or running it (parts that do not say are not: nothing is prepared for them)."""
+        wants = getattr(part, "wants_prepared_norm", None)
+        return bool(wants(n_rows)) if wants is not None else False
 
     @staticmethod
     def _normed(part, norm, x, ctx):
         """The part's input: the norm's result, or -- for a part that says it takes one -- the
-        norm not yet computed, so that the part's first product can absorb it."""
+        norm not yet computed, so that the part's first product can absorb it (or take what the
+        product before has prepared for it)."""
+        pre = ctx.prepared.pop(id(norm), None)
         if getattr(part, "accepts_lazy_norm", False):
-            return Normed(x, norm, ctx)
+            return Normed(x, norm, ctx, pre=pre)
         return norm.forward(x, ctx)
 
 

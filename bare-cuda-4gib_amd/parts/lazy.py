@@ -2,8 +2,9 @@
 
 A block hands ``Normed(x, norm)`` to a mixer or feed-forward that declares
 ``accepts_lazy_norm``; :func:`parts.linear.linear` then fuses the norm into the
-product where a kernel can, and otherwise calls :meth:`tensor`, which runs the
-norm once and keeps the result.
+product where a kernel can -- or takes what the product before has prepared for
+this norm (``pre``) -- and otherwise calls :meth:`tensor`, which runs the norm
+once and keeps the result.
 """
 from __future__ import annotations
 
@@ -14,8 +15,10 @@ import torch
 
 class Normed:
     def __init__(self, x: torch.Tensor, norm, ctx=None, rows: Optional[torch.Tensor] = None,
-                 n_rows: Optional[int] = None):
+                 n_rows: Optional[int] = None, pre=None):
         self.x, self.norm, self.ctx, self.rows = x, norm, ctx, rows
+        # what the product that last added into x left for this norm (ops.Prenormed), if anything
+        self.pre = pre if rows is None else None
         self.n_rows = x.shape[0] if rows is None and n_rows is None else (n_rows if n_rows is not None else rows.numel())
         self._tensor: Optional[torch.Tensor] = None
 

@@ -23,17 +23,34 @@ def _fused_norm(x: Normed, w, epilogue: int) -> Optional[torch.Tensor]:
     return ops.gemm_normed(x.x, x.rows, x.n_rows, scale[0], scale[1], w, epilogue)
 
 
+def _prepared_norm(x: Normed, w, epilogue: int) -> Optional[torch.Tensor]:
+    """The product from what the product before left for this norm, where there is such a thing."""
+    if x.pre is None or x._tensor is not None or not ops.gemm_prenormed_supported(x.pre, w):
+        return None
+    return ops.gemm_prenormed(x.pre, w, epilogue)
+
+
 def linear(x: Union[torch.Tensor, Normed], w, out_dtype: Optional[torch.dtype] = None,
-           accumulate_into: Optional[torch.Tensor] = None) -> torch.Tensor:
+           accumulate_into: Optional[torch.Tensor] = None, ctx=None) -> torch.Tensor:
     """x [M, K] times w [N, K] transposed (w a tensor or an ops.StreamedWeight).  With
-    ``accumulate_into`` (the float32 residual stream) the product is added to it in place."""
+    ``accumulate_into`` (the float32 residual stream) the product is added to it in place; with
+    ``ctx`` too, and a norm named there as the next reader of the stream (``ctx.norm_after``), the
+    product prepares that norm where its kernel can and leaves the result in ``ctx.prepared``."""
     if isinstance(x, Normed):
         if accumulate_into is None and out_dtype in (torch.bfloat16, torch.float32):
             epi = ops.EPI_STORE_BF16 if out_dtype == torch.bfloat16 else ops.EPI_STORE_F32
-            fused = _fused_norm(x, w, epi)
+            fused = _prepared_norm(x, w, epi)
+            if fused is None:
+                fused = _fused_norm(x, w, epi)
             if fused is not None:
                 return fused
         x = x.tensor()
+    if accumulate_into is not None and ctx is not None and ctx.norm_after is not None:
+        norm = ctx.norm_after
+        scale = norm.fusable() if hasattr(norm, "fusable") else None
+        if scale is not None and ops.gemm_emit_supported(x, w, accumulate_into, scale[0]):
+            ctx.prepared[id(norm)] = ops.gemm_accumulate_emit(x, w, accumulate_into, scale[0], scale[1])
+            return accumulate_into
     fast = ops.gemm_fast(x, w, out_dtype, accumulate_into)
     if fast is not None:
         return fast
@@ -44,7 +61,11 @@ def linear_swiglu(x: Union[torch.Tensor, Normed], w_gate_up, interleaved: bool =
     """silu(x Wg^T) * (x Wu^T) for w_gate_up = gate rows followed by up rows, or (interleaved)
     blocks of eight gate rows and the eight up rows of the same outputs."""
     if isinstance(x, Normed):
-        fused = _fused_norm(x, w_gate_up, ops.EPI_SWIGLU) if interleaved and w_gate_up.shape[0] % 16 == 0 else None
+        fused = None
+        if interleaved and w_gate_up.shape[0] % 16 == 0:
+            fused = _prepared_norm(x, w_gate_up, ops.EPI_SWIGLU)
+            if fused is None:
+                fused = _fused_norm(x, w_gate_up, ops.EPI_SWIGLU)
         if fused is not None:
             return fused
         x = x.tensor()

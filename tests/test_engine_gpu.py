@@ -52,6 +52,52 @@ def test_long_decoding(folders, dtype):
     helpers.compare_with_plain({(0, p): got[p] for p in range(400)}, where, {"r": plain}, label=f"long {dtype}", **TOL[dtype])
 
 
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_norms_prepared_by_the_product_before(folders, monkeypatch, name):
+    """In bfloat16 the product that adds into the residual stream prepares the norm that the next
+    attention begins with (and, from 64 rows on, the feed-forward's): the path is taken -- the
+    preparing kernel runs once a layer and step, none where no layer follows -- and the logits are
+    those of the path without it up to rounding, and the plain implementation's, for decoded tokens
+    alone, for 70 rows in a step (both norms prepared) and for portions beside decoded tokens."""
+    from bare_cuda_4gib_amd.csrc import ops
+    from bare_cuda_4gib_amd.engine import Executor, load_model
+    from bare_cuda_4gib_amd.parts.attention import CausalAttention
+    from bare_cuda_4gib_amd.parts.feedforward import SwiGLU
+    cfg = helpers.TINY[name][0]
+    folder = folders(name, "bfloat16")
+    requests = {f"r{i}": helpers.random_ids(n, cfg["vocab_size"], 500 + i) for i, n in enumerate([75, 20, 9])}
+    plain = PlainLlama(folder)
+    plain_logits = {rid: plain.logits(ids).numpy() for rid, ids in requests.items()}
+    model, _ = load_model(folder, "bfloat16")
+    at = {rid: 0 for rid in requests}
+
+    def entry(rid, n):
+        e = {"id": rid, "tokens": requests[rid][at[rid]:at[rid] + n], "want": list(range(n)), "_start": at[rid]}
+        at[rid] += n
+        return e
+    plan = [[("r0", 70)], [("r0", 1)], [("r0", 1), ("r1", 18)], [("r0", 1), ("r1", 1), ("r2", 9)], [("r0", 1), ("r1", 1)], [("r0", 1)]]
+    steps = [{"step": i, "entries": [entry(rid, n) for rid, n in group], "end": []} for i, group in enumerate(plan)]
+    steps, where = helpers._finish(steps)
+    calls = []
+    real = ops.gemm_accumulate_emit
+    monkeypatch.setattr(ops, "gemm_accumulate_emit", lambda *a, **k: (calls.append(a[0].shape[0]), real(*a, **k))[1])
+
+    def run():
+        ex = Executor(model, num_pages=12, max_requests=4, max_tokens=128, page_tokens=16, poison=True, use_graphs=False)
+        return helpers.replay_in_process(ex, steps)
+    with_prepared = run()
+    layers = cfg["num_hidden_layers"]
+    assert len(calls) >= len(steps) * (layers - 1) and any(m >= 64 for m in calls) and any(m == 1 for m in calls)
+    n_with = len(calls)
+    monkeypatch.setattr(CausalAttention, "wants_prepared_norm", lambda self, n: False)
+    monkeypatch.setattr(SwiGLU, "wants_prepared_norm", lambda self, n: False)
+    without = run()
+    assert len(calls) == n_with, "nothing is prepared for parts that do not want it"
+    helpers.compare_with_plain(with_prepared, where, plain_logits, label=f"prepared norms {name}", **TOL["bfloat16"])
+    for key in with_prepared:
+        torch.testing.assert_close(torch.from_numpy(with_prepared[key]), torch.from_numpy(without[key]), rtol=2e-2, atol=4e-3)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_decoded_tokens_at_long_contexts_beside_prompt_portions(folders, dtype):
     """Requests with hundreds of cached tokens decode one token each in the same step in which others
