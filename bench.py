@@ -161,6 +161,26 @@ def run_prefill(model, cfg, tokens, runs=3, seed=2):
     return best
 
 
+def run_gemm(m, n, k, runs=20):
+    """One product of the linear maps' kernels alone (operands drawn as the model's are)."""
+    import torch
+    from bare_cuda_4gib_amd.csrc import ops
+    gen = torch.Generator(device="cuda").manual_seed(4)
+    a = torch.randn(m, k, device="cuda", generator=gen).bfloat16()
+    w = (torch.randn(n, k, device="cuda", generator=gen) * 0.02).bfloat16()
+    for _ in range(3):
+        ops.gemm_fast(a, w, torch.bfloat16)
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(runs):
+        ops.gemm_fast(a, w, torch.bfloat16)
+    end.record()
+    torch.cuda.synchronize()
+    us = start.elapsed_time(end) / runs * 1e3
+    return {"only": "gemm", "m": m, "n": n, "k": k, "us": round(us, 1), "tflops": round(2.0 * m * n * k / us / 1e6, 1),
+            "frac": round(2.0 * m * n * k / us / 1e6 / PEAK_TFLOPS["bf16"], 4)}
+
+
 def run_serve(model, cfg, n_requests, new_tokens, chunk, seed=3):
     """A mixed batch through the scheduler: n_requests submitted at once, prompt lengths uniform in
     [128, max context - new_tokens], prompts cut into portions of `chunk` tokens beside the decoded
@@ -221,8 +241,10 @@ def main() -> int:
     ap.add_argument("--requests", type=int, default=64, help="--only serve: requests submitted at once")
     ap.add_argument("--new-tokens", type=int, default=256, help="--only serve: tokens generated per request")
     ap.add_argument("--chunk", type=int, default=512, help="--only serve: prompt portion size")
-    ap.add_argument("--only", choices=["decode", "prefill", "serve"], default=None,
+    ap.add_argument("--only", choices=["decode", "prefill", "serve", "gemm"], default=None,
                     help="run one part only and print its own short line (for profiling)")
+    ap.add_argument("--mnk", default="2048,11264,2048",
+                    help="--only gemm: rows, outputs and k of one bfloat16 product x w^T (the tiled matrix-core kernel)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -232,6 +254,9 @@ def main() -> int:
     from bare_cuda_4gib_amd.csrc import library
     library.load()
     assert torch.cuda.is_available(), "bench.py needs a GPU"
+    if args.only == "gemm":
+        print(json.dumps(run_gemm(*(int(v) for v in args.mnk.split(",")))), flush=True)
+        return 0
     dtype = "bfloat16" if args.dtype == "bf16" else "float32"
     elem = 2 if args.dtype == "bf16" else 4
     shape = SHAPES[args.shape]
