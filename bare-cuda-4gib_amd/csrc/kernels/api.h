@@ -112,12 +112,14 @@ extern "C" {
 // merges into out.  A request without pieces (tile_start[s + 1] == tile_start[s]) is left out: its
 // rows of out are not written, provided row_seq ([T]: each row's request) is given for the merge
 // to see which rows those are -- so two launches of different forms can share one out.
+// single_rows (form 1): every request brings exactly one row, so request s is tile s and row s and the
+// kernel looks nothing up before it asks for the block table and the query (a decode step).
 int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, float* part_o, float* part_ml, const void* k_cache,
                         const void* v_cache, const int32_t* block_table, int table_stride,
                         const int32_t* seq_start, const int32_t* seq_ctx, const int32_t* tile_start,
                         int n_seqs, int n_tiles, int n_tokens, int n_heads, int n_kv_heads, int head_dim,
                         int page_tokens, int window, float scale, int tokens_per_tile, int q_tiles,
-                        int form, int n_splits, const int32_t* row_seq, void* stream);
+                        int form, int n_splits, int single_rows, const int32_t* row_seq, void* stream);
 }
 
 extern "C" {

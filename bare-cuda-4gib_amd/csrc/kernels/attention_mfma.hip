@@ -99,6 +99,7 @@ struct AttnArgs {
   int n_heads, n_kv_heads, head_dim, page_tokens, window;
   int hg, tpt, n_sub;          // heads per tile, tokens per tile, head sub-groups per kv head
   int n_splits;
+  int single_rows;             // every request brings exactly one row (a decode step): request s is tile s and row s
   float scale_log2;            // softmax scale times log2(e)
 };
 
@@ -129,7 +130,12 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, 2) void att
   // Which request this tile belongs to, and that request's rows and context.  Up to 63 requests
   // are looked at by one lane each (three loads, all at once, and a vote); more by bisection.
   int s, row0, q_len, ctx, tile0;
-  if (a.n_seqs < kWave) {
+  if (a.single_rows) {
+    // nothing to look up but the context: the block table, the query and the context are asked for together
+    s = tile0 = row0 = tile;
+    q_len = 1;
+    ctx = a.seq_ctx[tile];
+  } else if (a.n_seqs < kWave) {
     const int ts = lane <= a.n_seqs ? a.tile_start[lane] : 0;
     const int ss = lane <= a.n_seqs ? a.seq_start[lane] : 0;
     const int sc = lane < a.n_seqs ? a.seq_ctx[lane] : 0;
@@ -656,7 +662,7 @@ extern "C" int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, flo
                                    const int32_t* seq_start, const int32_t* seq_ctx, const int32_t* tile_start,
                                    int n_seqs, int n_tiles, int n_tokens, int n_heads, int n_kv_heads, int head_dim,
                                    int page_tokens, int window, float scale, int tokens_per_tile, int q_tiles,
-                                   int form, int n_splits, const int32_t* row_seq, void* stream) {
+                                   int form, int n_splits, int single_rows, const int32_t* row_seq, void* stream) {
   BC4G_REQUIRE(n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0, "attention_mfma: bad heads %d/%d",
                n_heads, n_kv_heads);
   BC4G_REQUIRE(head_dim >= 16 && head_dim <= 256 && head_dim % 16 == 0,
@@ -695,6 +701,10 @@ extern "C" int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, flo
   a.tpt = tokens_per_tile;
   a.n_sub = (group + a.hg - 1) / a.hg;
   a.n_splits = n_splits;
+  a.single_rows = single_rows ? 1 : 0;
+  BC4G_REQUIRE(!single_rows || (form == 1 && n_tiles == n_seqs && n_tokens == n_seqs),
+               "attention_mfma: single rows means one row and one tile a request in the decode form (%d requests, %d "
+               "tiles, %d rows)", n_seqs, n_tiles, n_tokens);
   a.scale_log2 = scale * kLog2e;
   BC4G_REQUIRE(a.tpt >= 1 && a.tpt * a.hg <= 16, "attention_mfma: %d tokens x %d heads do not fit a 16-row tile",
                a.tpt, a.hg);

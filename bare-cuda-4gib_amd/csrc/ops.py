@@ -614,12 +614,15 @@ def attention_mfma(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
                    seq_start: torch.Tensor, seq_ctx: torch.Tensor, tile_start: torch.Tensor, n_tiles: int,
                    n_heads: int, n_kv_heads: int, head_dim: int, window: int, scale: float,
                    n_splits: int, q_tiles: int = 1, form: int = 0, work=None,
-                   out: Optional[torch.Tensor] = None, row_seq: Optional[torch.Tensor] = None) -> torch.Tensor:
+                   out: Optional[torch.Tensor] = None, row_seq: Optional[torch.Tensor] = None,
+                   single_rows: bool = False) -> torch.Tensor:
     """form 0: four independent waves a workgroup, tile_start counts pieces of q_tiles tiles; 1: one
     tile a workgroup, its waves share the keys (q_tiles 1); 2: four waves a workgroup that walk their
     keys together through LDS, tile_start counts pieces of 4 * q_tiles tiles (ATTENTION_STAGED_WAVES).
     Requests without pieces are left out; with ``out`` (the result of another launch over the other
-    requests) and ``row_seq`` (each row's request) their rows of it stay as they are."""
+    requests) and ``row_seq`` (each row's request) their rows of it stay as they are.
+    ``single_rows`` (form 1): the caller knows that every request brings exactly one row (a decode
+    step), and the kernel then looks nothing up before it asks for the block table and the query."""
     _dev("attention_mfma", qkv, k_cache, v_cache, block_table, seq_start, seq_ctx, tile_start)
     t = qkv.shape[0]
     _check_queries("attention_mfma", qkv, n_heads, n_kv_heads, head_dim)
@@ -647,7 +650,7 @@ def attention_mfma(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
                  _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(seq_start), _ptr(seq_ctx),
                  _ptr(tile_start), n_seqs, n_tiles, t, n_heads, n_kv_heads, head_dim, k_cache.shape[2],
                  int(window), float(scale), attention_tile_tokens(n_heads, n_kv_heads), int(q_tiles),
-                 int(form), int(n_splits), _ptr(row_seq), _stream(), cost=work)
+                 int(form), int(n_splits), 1 if single_rows else 0, _ptr(row_seq), _stream(), cost=work)
     return out
 
 
@@ -667,7 +670,8 @@ def attention(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, b
             tile_start, n_tiles = ctx.attention_tiles(tpt)
             n_splits = ctx.fixed_attention_splits or attention_splits(
                 n_tiles, n_heads, n_kv_heads, ctx.max_kv_len, attention_shared_waves(head_dim))
-            return attention_mfma(*args, tile_start, n_tiles, *sizes, n_splits, 1, 1, work=work)
+            return attention_mfma(*args, tile_start, n_tiles, *sizes, n_splits, 1, 1, work=work,
+                                  single_rows=ctx.max_q_len == 1 and ctx.n_tokens == ctx.n_seqs)
         # Else four waves with consecutive tiles of a request walk their keys together -- but a
         # request that brings a single tile beside them (a decoded token in a step with prompt
         # portions) would walk its whole context with one wave: those requests get a launch of their

@@ -404,6 +404,29 @@ def test_attention_mfma(ops, nh, nkv, d, page, window, n_splits):
           what="mfma, keys shared between a workgroup's waves")
 
 
+@pytest.mark.parametrize("n_splits", [1, 3])
+def test_attention_of_a_decode_step_without_looking_requests_up(ops, n_splits):
+    """Every request brings exactly one row: told so, the kernel takes request s for tile s and row s
+    and asks for nothing before the block table and the query -- the same bits as with the lookup, for
+    few requests and for more than a wave's lanes hold (70)."""
+    for n_req in (5, 70):
+        seqs = [(3 + 17 * i % 190, 1) for i in range(n_req)]
+        case = paged_case(seqs, 8, 2, 32, 16, torch.bfloat16, seed=12)
+        kc, vc = ops.cache_from_plain(case["kc"], case["vc"])
+        dev = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
+        args = (case["qkv"], kc, vc, case["table"], dev(case["seq_start"]), dev(case["seq_ctx"]),
+                dev(list(range(n_req + 1))), n_req, 8, 2, 32, 0, 1.0 / math.sqrt(32), n_splits, 1, 1)
+        looked_up = ops.attention_mfma(*args)
+        told = ops.attention_mfma(*args, single_rows=True)
+        assert torch.equal(told, looked_up)
+        close(told, plain_result(case), rtol=2e-2, atol=2e-2, what=f"{n_req} single rows")
+    with pytest.raises(Exception, match="single rows"):
+        two = paged_case([(4, 2), (9, 1)], 8, 2, 32, 16, torch.bfloat16, seed=13)
+        kc, vc = ops.cache_from_plain(two["kc"], two["vc"])
+        ops.attention_mfma(two["qkv"], kc, vc, two["table"], dev(two["seq_start"]), dev(two["seq_ctx"]), dev([0, 1, 2]), 2,
+                           8, 2, 32, 0, 1.0 / math.sqrt(32), 1, 1, 1, single_rows=True)
+
+
 @pytest.mark.parametrize("n_splits", [1, 5])
 def test_attention_far_key_among_hundreds(ops, n_splits):
     """The last query of each request looks at one key far back (position 3 of 400+): softmax puts
