@@ -91,7 +91,7 @@ __device__ inline uint32_t pack2(float a, float b) {
 template <int MT, int EPI, int XMODE, int U>
 // (The normed form keeps to 80 registers, so that three workgroups share a CU and all the blocks of
 // a 5,632 x 2 wide gate-up matrix are in flight at once.)
-__global__ __launch_bounds__(kThreads, XMODE != kPlain ? 6 : 4) void gemm_skinny_kernel(const SkinnyArgs args) {
+__global__ __launch_bounds__(kThreads, (XMODE != kPlain || (MT == 1 && U == 2)) ? 6 : 4) void gemm_skinny_kernel(const SkinnyArgs args) {
   constexpr bool kNormed = XMODE != kPlain;
   // Where the weight blocks are too few to occupy the CUs, the rows are shared out over blockIdx.y:
   // such a workgroup sees its own rows only, as if they were the whole batch.
@@ -515,7 +515,13 @@ int launch(const SkinnyArgs& a, hipStream_t s) {
     }
     switch (tiles) {
       // k-steps per batch chosen so that two batches of operands fit 128 registers (two workgroups a CU)
-      case 1: gemm_skinny_kernel<1, EPI, XMODE, 4><<<grid, block, 0, s>>>(b); break;
+      case 1:
+        // (a wide product's many workgroups, more than two a CU: with fewer k-steps in flight each they
+        // need half the registers, and all of them are on the CUs at once -- the gate-up product of 8
+        // rows after a prepared norm: a decode step 1.020 -> 0.990 ms)
+        if (static_cast<int>(grid.x) > 2 * compute_units()) gemm_skinny_kernel<1, EPI, XMODE, 2><<<grid, block, 0, s>>>(b);
+        else gemm_skinny_kernel<1, EPI, XMODE, 4><<<grid, block, 0, s>>>(b);
+        break;
       case 2: gemm_skinny_kernel<2, EPI, XMODE, 2><<<grid, block, 0, s>>>(b); break;
       case 3: gemm_skinny_kernel<3, EPI, XMODE, 2><<<grid, block, 0, s>>>(b); break;
       case 4: gemm_skinny_kernel<4, EPI, XMODE, 2><<<grid, block, 0, s>>>(b); break;

@@ -45,12 +45,14 @@ class SwiGLU(Part):
         self.act_dtype = rt.act_dtype
 
     def wants_prepared_norm(self, n_rows: int) -> bool:
-        """Only from 64 rows on.  Below, the norm fused into the gate-up product (up to
-        ops.NORMED_MAX_ROWS rows; that kernel keeps all of a wide product's workgroups on the CUs at
-        once) or a norm kernel of its own is the faster way: every one of the product's many
-        workgroups has to add up the prepared parts (measured at TinyLlama's sizes, a decode step:
-        1.085 against 1.072 ms at 16 rows, 1.269 against 1.252 at 32, 1.558 against 1.565 at 64)."""
-        return self.interleaved and n_rows >= 64
+        """From 5 to 8 rows and from 64 on.  With fewer rows the norm fused into the gate-up product
+        costs little (few float rows to stage); from 5 on reading prepared bfloat16 rows beats staging
+        float ones in every one of the product's many workgroups (a decode step at TinyLlama's sizes:
+        1.020 -> 0.990 ms at 8 rows, no difference at 4, 0.918 -> 0.948 at one).  From 9 rows on the
+        fused norm is out of reach and the choice is a norm kernel of its own: that is the faster way
+        up to 63 rows, because every workgroup of the product has to add up the prepared parts (1.085
+        against 1.072 ms at 16 rows, 1.269 against 1.252 at 32, 1.558 against 1.565 at 64)."""
+        return self.interleaved and (5 <= n_rows <= ops.NORMED_MAX_ROWS or n_rows >= 64)
 
     def forward(self, h, ctx, residual) -> None:
         act = linear_swiglu(h, self.w_gu, self.interleaved)
