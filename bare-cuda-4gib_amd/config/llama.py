@@ -117,4 +117,5 @@ def describe_llama(cfg: LlamaConfig):
 
 LLAMA = register_architecture(Architecture(
     name="LlamaForCausalLM", model_type="llama",
-    config_class=LlamaConfig, describe=describe_llama))
+    config_class=LlamaConfig, describe=describe_llama,
+    ignored_tensors=("*.rotary_emb.inv_freq",)))      # a buffer some checkpoints carry; the angles are computed here

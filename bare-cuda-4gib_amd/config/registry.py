@@ -10,7 +10,7 @@ function, scheduler and the programs never name an architecture.
 from __future__ import annotations
 
 import dataclasses
-from typing import Any, Callable, Dict, List, Type
+from typing import Any, Callable, Dict, List, Tuple, Type
 
 from ..errors import ConfigError
 from .base import ModelConfig, read_config_json
@@ -22,6 +22,9 @@ class Architecture:
     model_type: str                # config.json "model_type"
     config_class: Type[ModelConfig]
     describe: Callable[[ModelConfig], Any]   # config -> engine.ModelSpec
+    # glob patterns of tensor names that this architecture's checkpoints may carry and the engine
+    # does not need (buffers that are recomputed): passed over without a warning
+    ignored_tensors: Tuple[str, ...] = ()
 
 
 _BY_NAME: Dict[str, Architecture] = {}

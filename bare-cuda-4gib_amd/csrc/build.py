@@ -21,7 +21,6 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 SRC_DIR = os.path.join(HERE, "kernels")
 BUILD_DIR = os.path.join(HERE, "_build")
 LIB_PATH = os.path.join(HERE, "libbc4g.so")
-HASH_PATH = LIB_PATH + ".sources"
 
 ARCH = "gfx950"
 # -packed-fp32-ops is switched off: the compiler must not form packed float32
@@ -57,17 +56,42 @@ def is_built() -> bool:
     return os.path.exists(LIB_PATH)
 
 
-def is_stale() -> bool:
+_MARKER = b"bc4g-sources-digest:"
+
+
+def built_digest() -> str:
+    """The digest of the sources the library file was built from, read from the file itself (it
+    carries it behind a marker), without loading it; empty if there is none."""
+    import mmap
     try:
-        with open(HASH_PATH, "r") as fh:
-            return fh.read().strip() != sources_digest()
-    except OSError:
+        with open(LIB_PATH, "rb") as fh, mmap.mmap(fh.fileno(), 0, access=mmap.ACCESS_READ) as mm:
+            at = mm.find(_MARKER)
+            if at < 0:
+                return ""
+            raw = mm[at + len(_MARKER):at + len(_MARKER) + 64]
+            return raw.split(b"\0", 1)[0].decode("ascii", "replace")
+    except (OSError, ValueError):
+        return ""
+
+
+def is_stale() -> bool:
+    """Whether the built library comes from other sources (or flags) than those beside it."""
+    return built_digest() != sources_digest()
+
+
+def can_build() -> bool:
+    try:
+        _hipcc()
         return True
+    except KernelError:
+        return False
 
 
-def _compile_one(hipcc: str, name: str) -> str:
+def _compile_one(hipcc: str, name: str, digest: str) -> str:
     obj = os.path.join(BUILD_DIR, name[:-4] + ".o")
     cmd = [hipcc, *HIPCC_FLAGS, "-I", SRC_DIR, "-c", os.path.join(SRC_DIR, name), "-o", obj]
+    if name == "common.hip":      # the library carries the digest of what it was built from
+        cmd.insert(1, f'-DBC4G_SOURCES_DIGEST="{digest}"')
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise KernelError(f"hipcc failed on {name}:\n{proc.stderr[-4000:]}")
@@ -79,6 +103,7 @@ def build(verbose: bool = True, jobs: int = 0) -> str:
     hipcc = _hipcc()
     os.makedirs(BUILD_DIR, exist_ok=True)
     names = sources()
+    digest = sources_digest()
     jobs = jobs or min(len(names), max(1, min(16, os.cpu_count() or 1)))
     t0 = time.time()
     out = sys.stderr
@@ -86,7 +111,7 @@ def build(verbose: bool = True, jobs: int = 0) -> str:
         print(f"[bc4g] compiling {len(names)} kernel sources for {ARCH} with {jobs} jobs ...", file=out, flush=True)
     objs = []
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
-        futs = {pool.submit(_compile_one, hipcc, n): n for n in names}
+        futs = {pool.submit(_compile_one, hipcc, n, digest): n for n in names}
         for fut in concurrent.futures.as_completed(futs):
             objs.append(fut.result())
             if verbose:
@@ -97,8 +122,6 @@ def build(verbose: bool = True, jobs: int = 0) -> str:
     if proc.returncode != 0:
         raise KernelError(f"linking libbc4g.so failed:\n{proc.stderr[-4000:]}")
     os.replace(tmp, LIB_PATH)
-    with open(HASH_PATH, "w") as fh:
-        fh.write(sources_digest())
     if verbose:
         print(f"[bc4g] built {LIB_PATH} in {time.time() - t0:.0f} s", file=out, flush=True)
     return LIB_PATH

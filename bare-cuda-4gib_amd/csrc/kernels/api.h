@@ -12,6 +12,7 @@ extern "C" {
 
 const char* bc4g_last_error();
 int bc4g_version();
+const char* bc4g_sources_digest();   // digest of the sources and flags the library was built from
 
 // x[t, :] = float(table[ids[t], :])            (reference: embedding_lookup.cu:16-31)
 int bc4g_embed_gather(const void* table, int table_dtype, const int32_t* ids, float* out,

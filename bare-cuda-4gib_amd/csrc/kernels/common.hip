@@ -37,5 +37,15 @@ int compute_units() {
 
 }  // namespace bc4g
 
+#ifndef BC4G_SOURCES_DIGEST
+#define BC4G_SOURCES_DIGEST "unknown"
+#endif
+
 extern "C" const char* bc4g_last_error() { return bc4g::g_error; }
-extern "C" int bc4g_version() { return 1; }
+extern "C" int bc4g_version() { return 2; }
+// The digest of the kernel sources and compiler flags this library was built from (the build passes it
+// in): whoever loads the library compares it with the sources beside it, so that signatures declared
+// for new sources are never bound to an old binary.
+// (behind a marker, so that it can also be found in the file without loading it)
+static const char kSourcesDigest[] = "bc4g-sources-digest:" BC4G_SOURCES_DIGEST;
+extern "C" const char* bc4g_sources_digest() { return kSourcesDigest + sizeof("bc4g-sources-digest:") - 1; }

@@ -52,8 +52,14 @@ def load(build_if_missing: bool = True) -> ctypes.CDLL:
             raise KernelError(f"{_build.LIB_PATH} is not built; run __graft_entry__.build()")
         _build.build(verbose=True)
     elif _build.is_stale():
-        print(f"[bc4g] warning: {_build.LIB_PATH} is older than its sources; "
-              "run __graft_entry__.build() to rebuild", file=sys.stderr, flush=True)
+        # A library built from other sources than those beside it would be called with the wrong
+        # arguments (entry points gain parameters): it is built again, or refused.
+        if not (build_if_missing and _build.can_build()):
+            raise KernelError(f"{_build.LIB_PATH} was built from other sources than those in {_build.SRC_DIR} "
+                              "and cannot be rebuilt here; run __graft_entry__.build()")
+        print(f"[bc4g] {_build.LIB_PATH} was built from other sources than those beside it: building it again",
+              file=sys.stderr, flush=True)
+        _build.build(verbose=True)
     # PyTorch first: it brings a HIP runtime of its own, and the library must bind to that one.  Loaded
     # before torch, the library pulls in the system's runtime instead, the process then holds two, and
     # the library's launches fail ("no ROCm-capable device is detected").
@@ -62,6 +68,10 @@ def load(build_if_missing: bool = True) -> ctypes.CDLL:
         lib = ctypes.CDLL(_build.LIB_PATH)
     except OSError as e:
         raise KernelError(f"cannot load {_build.LIB_PATH}: {e}") from None
+    lib.bc4g_sources_digest.restype = c_char_p
+    lib.bc4g_sources_digest.argtypes = []
+    if (lib.bc4g_sources_digest() or b"").decode("ascii", "replace") != _build.sources_digest():
+        raise KernelError(f"{_build.LIB_PATH} does not carry the digest of the sources beside it")
     lib.bc4g_last_error.restype = c_char_p
     lib.bc4g_last_error.argtypes = []
     lib.bc4g_version.restype = c_int

@@ -159,14 +159,11 @@ def expected_weights(spec: ModelSpec) -> Dict[str, WeightSpec]:
     return Model(spec).expected_weights()
 
 
-IGNORED_TENSORS = ("*.rotary_emb.inv_freq",)   # a buffer some checkpoints carry; recomputed here
-
-
 def load_model(model_dir: str, dtype, device="cuda:0") -> Tuple[Model, object]:
     """(model with weights on the device, typed configuration) of a model folder."""
     from .runtime import parse_dtype
     arch, cfg = load_config(model_dir)
     model = Model(arch.describe(cfg))
-    tensors = load_weights(model_dir, model.expected_weights(), ignore=IGNORED_TENSORS)
+    tensors = load_weights(model_dir, model.expected_weights(), ignore=arch.ignored_tensors)
     model.bind(tensors, Runtime(torch.device(device), parse_dtype(dtype)))
     return model, cfg

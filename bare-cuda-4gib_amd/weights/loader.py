@@ -1,15 +1,19 @@
 """Loading weights by tensor name against what the model's parts declare.
 
 The reference validates every tensor by name, dtype and element count and
-names the tensor in the message (engine/src/model.cpp:24-74,
-engine/src/loader.cpp:137-148).  Here all problems of a model folder are
-collected and reported in one error: missing tensors, unexpected tensors and
-wrong shapes.
+names the tensor in the message (engine/src/model.cpp:24-74), and it only
+looks up the names it needs: a tensor nobody asks for is ignored
+(engine/src/loader.cpp:137-148).  Here all problems of a model folder are
+collected and reported in one error that lists missing tensors, wrong shapes
+and, beside them, the unexpected tensors (a misspelt name shows up as one
+missing and one unexpected).  A folder whose only oddity is unexpected tensors
+loads, with one warning on standard error that lists them.
 """
 from __future__ import annotations
 
 import dataclasses
 import fnmatch
+import sys
 from typing import Dict, Iterable, Tuple
 
 import torch
@@ -47,8 +51,10 @@ def load_weights(model_dir: str, expected: Dict[str, WeightSpec],
     Returns name -> CPU tensor (bfloat16 stays bfloat16, 32-bit stays 32-bit, float16 stays
     float16 until it is placed on the device, where the 16-bit path keeps it in bfloat16,
     integers are int32).  ``ignore`` holds glob patterns of tensor names a file
-    may carry that the engine does not need.  Raises one WeightError that lists
-    every missing tensor, unexpected tensor and wrong shape.
+    may carry that the engine does not need (an architecture names them); they are
+    passed over in silence.  Raises one WeightError that lists every missing tensor
+    and wrong shape, and the unexpected tensors beside them; unexpected tensors alone
+    are a warning.
     """
     available = open_model_tensors(model_dir)
     ignore = tuple(ignore)
@@ -68,7 +74,10 @@ def load_weights(model_dir: str, expected: Dict[str, WeightSpec],
     for name in available:
         if name not in expected and not any(fnmatch.fnmatchcase(name, pat) for pat in ignore):
             unexpected.append(name)
-    if missing or wrong or unexpected:
+    if unexpected and not (missing or wrong):
+        print(f"[weights] warning: {model_dir} holds {len(unexpected)} tensors the configuration does not "
+              f"ask for (ignored): " + ", ".join(sorted(unexpected)), file=sys.stderr, flush=True)
+    if missing or wrong:
         lines = [f"weights in {model_dir} do not fit the configuration:"]
         if missing:
             lines.append(f"  missing tensors ({len(missing)}): " + ", ".join(sorted(missing)))

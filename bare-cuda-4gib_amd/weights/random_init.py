@@ -5,13 +5,18 @@ values are drawn in float32 from torch's CPU generator seeded with ``seed``,
 tensor after tensor in the order the model's parts declare them, and rounded
 to bfloat16 (to nearest, ties to even) when ``dtype`` is bfloat16.  (The
 reference only has random weights in its Python fixture generator,
-tools/references/reference_forward.py:301-321.)
+tools/references/reference_forward.py:301-321: matrices randn * 0.05, norm
+scales 1 + 0.05 * randn.)  Two options make folders on which more can go
+wrong: ``norm_std`` draws every norm scale as 1 + norm_std * randn, a draw of
+its own for every norm, and ``scales`` multiplies the tensors whose names match
+a pattern by a factor (larger query and key weights make attention peaked).
 """
 from __future__ import annotations
 
+import fnmatch
 import json
 import os
-from typing import Any, Dict, Union
+from typing import Any, Dict, Optional, Union
 
 import torch
 
@@ -24,17 +29,23 @@ _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16,
            "float32": torch.float32, "fp32": torch.float32, "f32": torch.float32}
 
 
-def random_tensor(spec, gen: torch.Generator, std: float, dtype: torch.dtype) -> torch.Tensor:
+def random_tensor(spec, gen: torch.Generator, std: float, dtype: torch.dtype, norm_std: float = 0.0,
+                  factor: float = 1.0) -> torch.Tensor:
     if spec.init == "ones":
-        return torch.ones(spec.shape, dtype=dtype)
+        if norm_std == 0.0:
+            return torch.full(spec.shape, factor, dtype=dtype)
+        return ((1.0 + norm_std * torch.randn(spec.shape, generator=gen, dtype=torch.float32)) * factor).to(dtype)
     if spec.kind == "int_table":
         return torch.zeros(spec.shape, dtype=torch.int32)
-    return (torch.randn(spec.shape, generator=gen, dtype=torch.float32) * std).to(dtype)
+    return (torch.randn(spec.shape, generator=gen, dtype=torch.float32) * (std * factor)).to(dtype)
 
 
 def write_random_model(config: Union[Dict[str, Any], ModelConfig], seed: int, out_dir: str,
-                       dtype: str = "bfloat16", std: float = 0.02) -> str:
-    """Write ``out_dir/config.json`` and ``out_dir/model.safetensors``; returns out_dir."""
+                       dtype: str = "bfloat16", std: float = 0.02, norm_std: float = 0.0,
+                       scales: Optional[Dict[str, float]] = None) -> str:
+    """Write ``out_dir/config.json`` and ``out_dir/model.safetensors``; returns out_dir.
+    ``norm_std``: spread of the norm scales around 1.0 (0: exactly 1.0).  ``scales``: glob pattern
+    of tensor names -> factor on what is drawn for them (the first pattern that matches)."""
     from ..engine.model import expected_weights
 
     if dtype not in _DTYPES:
@@ -54,10 +65,17 @@ def write_random_model(config: Union[Dict[str, Any], ModelConfig], seed: int, ou
         json.dump(raw, fh, indent=1)
     layout = [(n, s.shape, torch.int32 if s.kind == "int_table" else tdtype) for n, s in expected.items()]
     writer = SafetensorsWriter(os.path.join(out_dir, "model.safetensors"), layout,
-                               metadata={"format": "pt", "seed": seed, "std": std})
+                               metadata={"format": "pt", "seed": seed, "std": std, "norm_std": norm_std})
     gen = torch.Generator(device="cpu")
     gen.manual_seed(int(seed))
+    scales = scales or {}
+
+    def factor(name: str) -> float:
+        for pattern, f in scales.items():
+            if fnmatch.fnmatchcase(name, pattern):
+                return float(f)
+        return 1.0
     for name, s in expected.items():
-        writer.write(name, random_tensor(s, gen, std, tdtype))
+        writer.write(name, random_tensor(s, gen, std, tdtype, norm_std, factor(name)))
     writer.close()
     return out_dir

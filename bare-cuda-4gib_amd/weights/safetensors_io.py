@@ -56,10 +56,20 @@ class SafetensorsFile:
         self._data_start = 8 + n
         self._mm = mmap.mmap(self._fh.fileno(), 0, access=mmap.ACCESS_READ) if size else None
         self.entries: Dict[str, dict] = {}
+        if not isinstance(header, dict):
+            raise WeightError(f"{path}: header is not a JSON object")
         for name, e in header.items():
-            dt, shape, (b, end) = e.get("dtype"), e.get("shape"), e.get("data_offsets", (0, 0))
+            if not isinstance(e, dict):
+                raise WeightError(f"{path}: header entry of tensor '{name}' is not an object")
+            dt, shape, offsets = e.get("dtype"), e.get("shape"), e.get("data_offsets")
             if dt not in _NP_VIEW:
                 raise WeightError(f"{path}: tensor '{name}' has unsupported dtype {dt}")
+            if not isinstance(shape, list) or any(not isinstance(d, int) or isinstance(d, bool) or d < 0 for d in shape):
+                raise WeightError(f"{path}: tensor '{name}' has a bad shape {shape!r} (a list of non-negative integers is needed)")
+            if (not isinstance(offsets, list) or len(offsets) != 2
+                    or any(not isinstance(o, int) or isinstance(o, bool) for o in offsets) or not 0 <= offsets[0] <= offsets[1]):
+                raise WeightError(f"{path}: tensor '{name}' has bad data_offsets {offsets!r} (a pair 0 <= begin <= end is needed)")
+            b, end = offsets
             count = int(np.prod(shape, dtype=np.int64)) if len(shape) else 1
             if end - b != count * _NP_VIEW[dt][1]:
                 raise WeightError(f"{path}: tensor '{name}' of shape {shape} and dtype {dt} "

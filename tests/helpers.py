@@ -32,13 +32,34 @@ TINY_C = dict(architectures=["LlamaForCausalLM"], model_type="llama", vocab_size
 TINY = {"A": (TINY_A, 0), "B": (TINY_B, 2), "C": (TINY_C, 5)}   # name -> (config, weight seed)
 
 
-def make_model_dir(tmp_path, name: str, dtype: str = "float32", std: float = 0.02) -> str:
+# How a model folder's weights are drawn.  "ones": every matrix N(0, 0.02), every norm scale exactly
+# 1.0 (what the benchmark's configurations say).  "spread": every norm scale 1 + 0.1 * randn, a draw of
+# its own for each norm (the reference's fixture draws 1 + 0.05 * randn,
+# tools/references/reference_forward.py:306-318) -- a scale handed to the wrong norm, or dropped,
+# then changes the logits -- and query and key weights several times as large, so that the scores
+# have a spread of about one to two and attention is peaked rather than near-uniform: a wrong key or a
+# wrong score shows.  (Configuration B, with three layers, gets the smaller factor: peaked attention
+# multiplies whatever error the layers before have left in its input -- the plain implementation itself,
+# with its activations rounded to bfloat16 where the engine rounds them, is off by more than the
+# bfloat16 tolerance at a factor of eight there, and by half of it at five.)
+QK_FACTOR = {"A": 8.0, "B": 5.0, "C": 8.0}
+
+
+def variant_args(name: str, variant: str) -> dict:
+    if variant == "ones":
+        return {}
+    assert variant == "spread"
+    f = QK_FACTOR[name]
+    return dict(norm_std=0.1, scales={"*.q_proj.weight": f, "*.k_proj.weight": f})
+
+
+def make_model_dir(tmp_path, name: str, dtype: str = "float32", std: float = 0.02, variant: str = "ones") -> str:
     """A model folder with random weights, written by the framework's own random-weights mode."""
     from bare_cuda_4gib_amd.weights import write_random_model
     cfg, seed = TINY[name]
-    out = os.path.join(str(tmp_path), f"tiny_{name}_{dtype}")
+    out = os.path.join(str(tmp_path), f"tiny_{name}_{dtype}_{variant}")
     if not os.path.exists(os.path.join(out, "model.safetensors")):
-        write_random_model(cfg, seed, out, dtype, std=std)
+        write_random_model(cfg, seed, out, dtype, std=std, **variant_args(name, variant))
     return out
 
 
@@ -199,9 +220,12 @@ def replay_subprocess(model_dir: str, dtype: str, steps, out_dir: str, max_token
     return out
 
 
-def compare_with_plain(got, where, plain_logits: Dict[str, np.ndarray], rtol: float, atol: float, label: str):
+def compare_with_plain(got, where, plain_logits: Dict[str, np.ndarray], rtol: float, atol: float, label: str,
+                       row_rms: float = 0.0):
     """Every logits row the replay produced against the plain implementation's row at the same
-    request and position; reports the first wrong place."""
+    request and position; reports the first wrong place.  ``row_rms`` (if not 0): moreover the root
+    mean square of a row's errors may be at most this fraction of the root mean square of the row's
+    logits -- rounding noise averages out over a vocabulary, a fault in a scale or a sum does not."""
     assert set(got) == set(where), f"{label}: rows produced {len(got)}, rows expected {len(where)}"
     worst = 0.0
     for key in sorted(where):
@@ -210,6 +234,10 @@ def compare_with_plain(got, where, plain_logits: Dict[str, np.ndarray], rtol: fl
         row = got[key]
         assert np.all(np.isfinite(row)), f"{label}: non-finite logits at step {key[0]} request {rid} position {pos}"
         err = np.abs(row - ref)
+        if row_rms:
+            e, r = float(np.sqrt(np.mean(err * err))), float(np.sqrt(np.mean(ref * ref)))
+            assert e <= row_rms * r, (f"{label}: step {key[0]}, request {rid}, position {pos}: the row's errors have a "
+                                      f"root mean square of {e:.3g}, {e / r:.3g} of the logits' {r:.3g} (limit {row_rms:.3g})")
         bound = atol + rtol * np.abs(ref)
         if np.any(err > bound):
             i = int(np.argmax(err - bound))

@@ -4,6 +4,7 @@ import os
 import subprocess
 import sys
 
+import numpy as np
 import pytest
 import torch
 
@@ -17,7 +18,7 @@ TOL = {"float32": dict(rtol=1e-4, atol=2e-6), "bfloat16": dict(rtol=2e-2, atol=6
 @pytest.fixture(scope="module")
 def folders(tmp_path_factory):
     tmp = tmp_path_factory.mktemp("models")
-    return lambda name, dtype: helpers.make_model_dir(tmp, name, dtype)
+    return lambda name, dtype, variant="ones": helpers.make_model_dir(tmp, name, dtype, variant=variant)
 
 
 def follow_with_plain(plain, prompt, tokens, margin):
@@ -32,11 +33,12 @@ def follow_with_plain(plain, prompt, tokens, margin):
         assert gap <= margin, f"token {i} ({tok}) lies {gap:.4g} below the plain best {argmax_lowest(row)}"
 
 
+@pytest.mark.parametrize("variant", ["ones", "spread"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_long_decoding(folders, dtype):
+def test_long_decoding(folders, dtype, variant):
     """A short prompt, then several hundred tokens one by one (captured graphs, many pages)."""
     from bare_cuda_4gib_amd.engine import Executor, StepEntry, load_model
-    folder = folders("C", dtype)
+    folder = folders("C", dtype, variant)
     ids = helpers.random_ids(400, helpers.TINY_C["vocab_size"], 77)
     plain = PlainLlama(folder).logits(ids).numpy()
     model, _ = load_model(folder, dtype)
@@ -52,8 +54,9 @@ def test_long_decoding(folders, dtype):
     helpers.compare_with_plain({(0, p): got[p] for p in range(400)}, where, {"r": plain}, label=f"long {dtype}", **TOL[dtype])
 
 
+@pytest.mark.parametrize("variant", ["ones", "spread"])
 @pytest.mark.parametrize("name", ["A", "B"])
-def test_norms_prepared_by_the_product_before(folders, monkeypatch, name):
+def test_norms_prepared_by_the_product_before(folders, monkeypatch, name, variant):
     """In bfloat16 the product that adds into the residual stream prepares the norm that the next
     attention begins with (and, from 64 rows on, the feed-forward's): the path is taken -- the
     preparing kernel runs once a layer and step, none where no layer follows -- and the logits are
@@ -64,7 +67,7 @@ def test_norms_prepared_by_the_product_before(folders, monkeypatch, name):
     from bare_cuda_4gib_amd.parts.attention import CausalAttention
     from bare_cuda_4gib_amd.parts.feedforward import SwiGLU
     cfg = helpers.TINY[name][0]
-    folder = folders(name, "bfloat16")
+    folder = folders(name, "bfloat16", variant)
     requests = {f"r{i}": helpers.random_ids(n, cfg["vocab_size"], 500 + i) for i, n in enumerate([75, 20, 9])}
     plain = PlainLlama(folder)
     plain_logits = {rid: plain.logits(ids).numpy() for rid, ids in requests.items()}
@@ -278,11 +281,76 @@ def test_entry_point_statuses_and_failure_path(folders):
     assert engine.submit(9, [1], 1)[0] == "unavailable"
 
 
+def follow_sampled_with_plain(plain, prompt, tokens, temperature, seed, logit_tol):
+    """The engine's sampled tokens, checked step by step against the law (engine/src/sampler.cpp:39-61)
+    applied to the plain logits of the engine's own sequence: weights exp((l - max) / T), their running
+    sum in vocabulary order, and u * total with u from a fresh generator of the request's seed.  The
+    engine's token must be the one in whose stretch of the running sum u * total falls -- or one next
+    to it when u * total lies so close to the stretch's edge that the rounding of the engine's logits
+    (logit_tol: rtol and atol of the logits in this precision) can move the edge across it.  Returns how
+    many tokens were exactly the plain choice."""
+    from bare_cuda_4gib_amd.sampling import MT19937_64
+    rng = MT19937_64(seed)
+    full = plain.logits(list(prompt) + list(tokens)).numpy()
+    exact = 0
+    for i, tok in enumerate(tokens):
+        row = full[len(prompt) - 1 + i]
+        w = np.exp((row - row.max()) / temperature)
+        cum = np.cumsum(w)
+        total = cum[-1]
+        target = rng.uniform() * total
+        want = int(np.nonzero(target - cum < 0.0)[0][0])
+        exact += tok == want
+        # a logit off by e moves its weight by a factor exp(e / T): every edge of the running sum by at most
+        # 2 e / T of the total (the maximum's own error included)
+        margin = 2.0 * (logit_tol["rtol"] * float(np.abs(row).max()) + logit_tol["atol"]) / temperature * total
+        low = cum[tok - 1] if tok > 0 else 0.0
+        assert low - margin <= target < cum[tok] + margin, (
+            f"token {i}: the engine drew {tok}, the law gives {want} (u * total = {target:.6g}, the engine's token "
+            f"spans [{low:.6g}, {cum[tok]:.6g}), margin {margin:.3g})")
+    return exact
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_sampled_tokens_follow_the_law_on_the_plain_logits(folders, dtype):
+    """Configuration B's workload -- prompts of 5, 64 and 130 tokens as one mixed batch with 32-token
+    portions, 24 tokens each at temperature 0.8: every token the engine draws is the one the sampling
+    law gives on the plain implementation's logits for the request's own generator (the k-th token
+    uses the generator's k-th number, whatever else is in the batch).  In 32-bit the check is sharp
+    (a token spans 1/384 of the running sum, the margin is a fifteenth of that): a draw from another
+    request's row, with another request's generator or with the temperature applied twice gives
+    other tokens, which the test shows.  In bfloat16 the logits' tolerance makes the margin wider
+    than a token, so there the check only says that the draw follows the running sum."""
+    from bare_cuda_4gib_amd.engine import Engine
+    folder = folders("B", dtype, "spread")
+    plain = PlainLlama(folder)
+    prompts = [helpers.random_ids(n, 384, 40 + n) for n in (5, 64, 130)]
+    engine = Engine(folder, max_tokens=256, max_seqs=3, kv_pages=0, dtype=dtype, page_tokens=16, prefill_chunk=32,
+                    max_batch_tokens=96)
+    for i, p in enumerate(prompts):
+        assert engine.submit(i, p, 24, temperature=0.8, seed=4 + i)[0] == "ok"
+    out = {}
+    while len(out) < 3 or any(len(v) < 24 for v in out.values()):
+        for id, tok, idx, fin in engine.poll():
+            out.setdefault(id, []).append(tok)
+    exact = sum(follow_sampled_with_plain(plain, prompts[i], out[i], 0.8, 4 + i, TOL[dtype]) for i in range(3))
+    if dtype == "float32":
+        assert exact >= 66, f"only {exact} of 72 tokens are the plain choice"
+        # the check bites: the same tokens against another request's generator, a temperature applied
+        # twice, or another request's tokens (its rows) fail
+        with pytest.raises(AssertionError):
+            follow_sampled_with_plain(plain, prompts[1], out[1], 0.8, 4 + 2, TOL[dtype])
+        with pytest.raises(AssertionError):
+            follow_sampled_with_plain(plain, prompts[1], out[1], 0.8 * 0.8, 4 + 1, TOL[dtype])
+        with pytest.raises(AssertionError):
+            follow_sampled_with_plain(plain, prompts[1], out[2], 0.8, 4 + 2, TOL[dtype])
+
+
 def test_sampling_and_preemption_on_the_device(folders):
     """Temperature sampling on the device: a seed gives the same tokens alone, batched, and when the
     pool is so small that requests are preempted and recomputed."""
     from bare_cuda_4gib_amd.engine import Engine, generate_batch
-    folder = folders("B", "float32")
+    folder = folders("B", "float32", "spread")
     prompts = [helpers.random_ids(n, 384, 40 + n) for n in (5, 64, 130)]            # BASELINE's workload for B
     def run(kv_pages, which):
         engine = Engine(folder, max_tokens=256, max_seqs=3, kv_pages=kv_pages, dtype="float32", page_tokens=16,

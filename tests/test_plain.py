@@ -133,6 +133,99 @@ def test_model_reduces_to_embedding_norm_head_without_layers_output(plain_a):
     assert torch.allclose(m.logits(ids), want, atol=1e-12)
 
 
+# --- each branch of a layer against library routines ---------------------------------------------
+# One layer of configuration B (three heads, not grouped) with norm scales drawn around 1.0, a
+# different draw for each norm, and peaked attention.  With one branch's output projection zeroed
+# the layer is the other branch alone, which is written here with library routines only.  Each
+# check is shown to bite: the same comparison on a model whose weights are swapped the way a
+# plausible mistake would swap them (the two norms' scales, gate and up, no scale at all) fails.
+
+@pytest.fixture(scope="module")
+def one_layer(tmp_path_factory):
+    from bare_cuda_4gib_amd.weights import write_random_model
+    cfg = dict(helpers.TINY_B, num_hidden_layers=1)
+    folder = write_random_model(cfg, 7, str(tmp_path_factory.mktemp("one") / "m"), "float32", **helpers.variant_args("B", "spread"))
+    return P.PlainLlama(folder)
+
+
+def _with(m, **replaced):
+    import copy
+    out = copy.copy(m)
+    out.w = dict(m.w)
+    for name, t in replaced.items():
+        out.w["model.layers.0." + name.replace("__", ".")] = t
+    return out
+
+
+def _library_attention_branch(m, x):
+    """x + o_proj(SDPA(rope(q), rope(k), v)) on F.rms_norm(x, input_layernorm): heads not grouped."""
+    w, t = m.w, x.shape[0]
+    h = F.rms_norm(x, (m.hidden,), w["model.layers.0.input_layernorm.weight"], m.eps)
+    q, k, v = (F.linear(h, w[f"model.layers.0.self_attn.{n}_proj.weight"]).view(t, m.heads, m.head_dim) for n in "qkv")
+    pos = torch.arange(t)
+    q, k = P.rope(q, pos, m.theta), P.rope(k, pos, m.theta)
+    o = F.scaled_dot_product_attention(q.transpose(0, 1), k.transpose(0, 1), v.transpose(0, 1), is_causal=True)
+    return x + F.linear(o.transpose(0, 1).reshape(t, -1), w["model.layers.0.self_attn.o_proj.weight"])
+
+
+def _library_ffn_branch(m, x):
+    """x + down(F.silu(gate(h)) * up(h)) on h = F.rms_norm(x, post_attention_layernorm)."""
+    w = m.w
+    h = F.rms_norm(x, (m.hidden,), w["model.layers.0.post_attention_layernorm.weight"], m.eps)
+    a = F.silu(F.linear(h, w["model.layers.0.mlp.gate_proj.weight"])) * F.linear(h, w["model.layers.0.mlp.up_proj.weight"])
+    return x + F.linear(a, w["model.layers.0.mlp.down_proj.weight"])
+
+
+def test_attention_branch_reads_its_own_norm(one_layer):
+    m = one_layer
+    assert m.heads == m.kv_heads and m.layers == 1
+    ids = helpers.random_ids(23, m.vocab, 4)
+    x = m.w["model.embed_tokens.weight"][torch.tensor(ids)]
+    w1, w2 = m.w["model.layers.0.input_layernorm.weight"], m.w["model.layers.0.post_attention_layernorm.weight"]
+    assert not torch.allclose(w1, w2) and float((w1 - 1).abs().max()) > 0.05
+    alone = _with(m, mlp__down_proj__weight=torch.zeros_like(m.w["model.layers.0.mlp.down_proj.weight"]))
+    want = _library_attention_branch(alone, x)
+    assert torch.allclose(alone.hidden_states(ids), want, atol=1e-12)
+    assert float((want - x).abs().max()) > 1e-3                       # the branch is really there
+    # mistakes that must not pass: the other norm's scale, no scale, no norm at all
+    swapped = _with(alone, input_layernorm__weight=w2, post_attention_layernorm__weight=w1)
+    assert not torch.allclose(swapped.hidden_states(ids), want, atol=1e-6)
+    unscaled = _with(alone, input_layernorm__weight=torch.ones_like(w1))
+    assert not torch.allclose(unscaled.hidden_states(ids), want, atol=1e-6)
+    qkv_of_x = [F.linear(x, m.w[f"model.layers.0.self_attn.{n}_proj.weight"]) for n in "qkv"]
+    assert not torch.allclose(qkv_of_x[0], F.linear(F.rms_norm(x, (m.hidden,), w1, m.eps), m.w["model.layers.0.self_attn.q_proj.weight"]), atol=1e-3)
+
+
+def test_feed_forward_branch_reads_its_own_norm_and_gates_with_gate(one_layer):
+    m = one_layer
+    ids = helpers.random_ids(17, m.vocab, 5)
+    x = m.w["model.embed_tokens.weight"][torch.tensor(ids)]
+    w1, w2 = m.w["model.layers.0.input_layernorm.weight"], m.w["model.layers.0.post_attention_layernorm.weight"]
+    alone = _with(m, self_attn__o_proj__weight=torch.zeros_like(m.w["model.layers.0.self_attn.o_proj.weight"]))
+    want = _library_ffn_branch(alone, x)
+    assert torch.allclose(alone.hidden_states(ids), want, atol=1e-12)
+    assert float((want - x).abs().max()) > 1e-3
+    # mistakes that must not pass: silu on the up projection, the attention's norm, no scale
+    g, u = m.w["model.layers.0.mlp.gate_proj.weight"], m.w["model.layers.0.mlp.up_proj.weight"]
+    gate_up_swapped = _with(alone, mlp__gate_proj__weight=u, mlp__up_proj__weight=g)
+    assert not torch.allclose(gate_up_swapped.hidden_states(ids), want, atol=1e-6)
+    norms_swapped = _with(alone, input_layernorm__weight=w2, post_attention_layernorm__weight=w1)
+    assert not torch.allclose(norms_swapped.hidden_states(ids), want, atol=1e-6)
+    unscaled = _with(alone, post_attention_layernorm__weight=torch.ones_like(w2))
+    assert not torch.allclose(unscaled.hidden_states(ids), want, atol=1e-6)
+
+
+def test_both_branches_chain_through_the_residual_stream(one_layer):
+    """The whole layer is the feed-forward branch applied to the attention branch's result (not to x)."""
+    m = one_layer
+    ids = helpers.random_ids(11, m.vocab, 6)
+    x = m.w["model.embed_tokens.weight"][torch.tensor(ids)]
+    want = _library_ffn_branch(m, _library_attention_branch(m, x))
+    assert torch.allclose(m.hidden_states(ids), want, atol=1e-12)
+    parallel = _library_attention_branch(m, x) + _library_ffn_branch(m, x) - x
+    assert not torch.allclose(m.hidden_states(ids), parallel, atol=1e-6)
+
+
 def test_greedy_recomputes_whole_sequence(plain_a):
     ids = helpers.random_ids(5, 256, 3)
     out = plain_a.greedy(ids, 3)

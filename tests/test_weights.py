@@ -68,24 +68,73 @@ def test_integer_tables_become_int32(tmp_path):
     assert f.tensor("t").dtype == torch.int32 and f.tensor("t").tolist() == [[1, 2], [3, 40000]]
 
 
-def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
+def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path, capsys):
     folder = write_random_model(helpers.TINY_A, 0, str(tmp_path / "m"), "float32")
     path = os.path.join(folder, "model.safetensors")
-    tensors = load_file(path)
+    good = load_file(path)
+    tensors = dict(good)
     del tensors["model.layers.1.self_attn.k_proj.weight"]
     del tensors["model.norm.weight"]
     tensors["model.layers.0.mlp.down_proj.weight"] = torch.zeros(64, 175)
     tensors["model.layers.7.extra.weight"] = torch.zeros(3)
     tensors["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(8)            # tolerated buffer
     save_file(tensors, path)
-    from bare_cuda_4gib_amd.engine.model import IGNORED_TENSORS
+    ignored = load_config(folder)[0].ignored_tensors
+    assert ignored                                                # the architecture names what its checkpoints may carry
     with pytest.raises(WeightError) as e:
-        load_weights(folder, _expected(folder), ignore=IGNORED_TENSORS)
+        load_weights(folder, _expected(folder), ignore=ignored)
     msg = str(e.value)
     assert "model.layers.1.self_attn.k_proj.weight" in msg and "model.norm.weight" in msg and "missing tensors (2)" in msg
     assert "model.layers.7.extra.weight" in msg and "unexpected tensors (1)" in msg
     assert "model.layers.0.mlp.down_proj.weight" in msg and "[64, 175]" in msg and "[64, 176]" in msg
     assert "inv_freq" not in msg
+
+
+def test_unexpected_tensors_alone_are_a_warning(tmp_path, capsys):
+    """A folder that holds everything the configuration needs, and more, loads: the tensors nobody
+    asks for are listed once on standard error (the reference only looks up the names it needs,
+    engine/src/loader.cpp:137-148); what the architecture says its checkpoints carry is not even listed."""
+    folder = write_random_model(helpers.TINY_A, 0, str(tmp_path / "m"), "float32")
+    path = os.path.join(folder, "model.safetensors")
+    tensors = load_file(path)
+    tensors["model.layers.7.extra.weight"] = torch.zeros(3)
+    tensors["optimizer.step"] = torch.zeros(1)
+    tensors["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(8)
+    save_file(tensors, path)
+    capsys.readouterr()
+    w = load_weights(folder, _expected(folder), ignore=load_config(folder)[0].ignored_tensors)
+    err = capsys.readouterr().err
+    assert set(w) == set(_expected(folder)) and "model.layers.7.extra.weight" not in w
+    assert err.count("warning") == 1 and "model.layers.7.extra.weight" in err and "optimizer.step" in err
+    assert "inv_freq" not in err and "2 tensors" in err
+
+
+def test_malformed_header_entries_name_the_tensor(tmp_path):
+    p = tmp_path / "model.safetensors"
+    for entry, word in (({"dtype": "F32", "data_offsets": [0, 16]}, "shape"),
+                        ({"dtype": "F32", "shape": [4], "data_offsets": [0]}, "data_offsets"),
+                        ({"dtype": "F32", "shape": [-4], "data_offsets": [0, 16]}, "shape"),
+                        ({"dtype": "F32", "shape": [4], "data_offsets": [16, 0]}, "data_offsets"),
+                        ("nonsense", "object")):
+        header = json.dumps({"bad.tensor": entry}).encode()
+        p.write_bytes(len(header).to_bytes(8, "little") + header + b"\0" * 16)
+        with pytest.raises(WeightError) as e:
+            SafetensorsFile(str(p))
+        assert "bad.tensor" in str(e.value) and word in str(e.value)
+
+
+def test_norm_spread_and_scaled_tensors(tmp_path):
+    """The random-weights mode's two options: norm scales drawn around 1.0, a different draw for
+    every norm, and tensors scaled by name."""
+    a = load_file(os.path.join(write_random_model(helpers.TINY_A, 0, str(tmp_path / "a"), "float32", norm_std=0.1,
+                                                  scales={"*.q_proj.weight": 8.0}), "model.safetensors"))
+    plain = load_file(os.path.join(write_random_model(helpers.TINY_A, 0, str(tmp_path / "p"), "float32"), "model.safetensors"))
+    n1, n2 = a["model.layers.0.input_layernorm.weight"], a["model.layers.0.post_attention_layernorm.weight"]
+    assert not torch.equal(n1, n2) and abs(float(n1.mean()) - 1.0) < 0.05 and 0.05 < float(n1.std()) < 0.15
+    assert not torch.equal(a["model.norm.weight"], a["model.layers.1.input_layernorm.weight"])
+    assert abs(float(a["model.layers.0.self_attn.q_proj.weight"].std()) - 0.16) < 0.02
+    assert abs(float(a["model.layers.0.self_attn.k_proj.weight"].std()) - 0.02) < 0.003
+    assert torch.equal(plain["model.norm.weight"], torch.ones(64))
 
 
 def test_file_errors(tmp_path):
