@@ -3,6 +3,8 @@
 #include <float.h>
 #include <math.h>
 
+#include <mutex>
+
 #include "api.h"
 #include "common.h"
 
@@ -621,6 +623,62 @@ extern "C" int bc4g_argmax(const float* logits, int32_t* out, float* part_v, int
   if (n_rows == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   static_assert(kArgmaxSlices == kWave, "one lane per slice in the second stage");
+  argmax_slices_kernel<<<dim3(n_rows, kArgmaxSlices), kBlock, 0, s>>>(logits, part_v, part_i, vocab);
+  if (int e = check_launch("argmax_slices")) return e;
+  argmax_pick_kernel<<<n_rows, kWave, 0, s>>>(part_v, part_i, out, vocab);
+  return check_launch("argmax_pick");
+}
+
+// ---- argmax for callers that cannot allocate ------------------------------------------------
+// The two stages of bc4g_argmax hand the slices' bests over through device memory that the caller
+// brings as a workspace.  Here that memory is an array of the library's own: every GPU the library
+// runs on holds a copy of it (512 KiB) at an address of its own until the process ends, and all calls
+// on a GPU share it.  In host code the array's name is a stand-in, not a device address: the address
+// is asked for once per device (hipGetSymbolAddress, with that device current) and kept, and only
+// that pointer is ever handed to a kernel.
+constexpr int kArgmaxStaticMaxRows = 1024;
+constexpr size_t kArgmaxStaticValueBytes = static_cast<size_t>(kArgmaxStaticMaxRows) * kArgmaxSlices * sizeof(float);
+constexpr size_t kArgmaxStaticBytes = kArgmaxStaticValueBytes + static_cast<size_t>(kArgmaxStaticMaxRows) * kArgmaxSlices * sizeof(int32_t);
+static __device__ __align__(256) unsigned char scratch[kArgmaxStaticBytes];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {nullptr};
+
+// The address of `scratch` on the current device (asked for at the first call on that device).
+int scratch_on_current_device(unsigned char** ptr) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail("argmax_static: no current device: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices) return fail("argmax_static: device %d is beyond the %d this library keeps track of", dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr)
+      return fail("argmax_static: cannot find the scratch array on device %d: %s", dev, hipGetErrorString(e));
+    g_scratch_ptr[dev] = p;
+  }
+  *ptr = static_cast<unsigned char*>(g_scratch_ptr[dev]);
+  return 0;
+}
+}  // namespace
+
+extern "C" int bc4g_argmax_static_max_rows() { return kArgmaxStaticMaxRows; }
+
+extern "C" int bc4g_argmax_static(const float* logits, int32_t* out, int n_rows, int vocab, void* stream) {
+  BC4G_REQUIRE(n_rows >= 0 && vocab > 0, "argmax_static: bad sizes rows=%d V=%d", n_rows, vocab);
+  BC4G_REQUIRE(n_rows <= kArgmaxStaticMaxRows, "argmax_static: %d rows are more than the %d the library's own scratch memory holds; "
+               "use bc4g_argmax with a workspace of the caller's", n_rows, kArgmaxStaticMaxRows);
+  BC4G_REQUIRE(logits && out, "argmax_static: logits and out are needed");
+  if (n_rows == 0) return 0;
+  unsigned char* base = nullptr;
+  if (int e = scratch_on_current_device(&base)) return e;
+  // nothing in the array has to start at zero: the first stage writes every slot the second reads
+  float* part_v = reinterpret_cast<float*>(base);
+  int32_t* part_i = reinterpret_cast<int32_t*>(base + kArgmaxStaticValueBytes);
+  hipStream_t s = static_cast<hipStream_t>(stream);
   argmax_slices_kernel<<<dim3(n_rows, kArgmaxSlices), kBlock, 0, s>>>(logits, part_v, part_i, vocab);
   if (int e = check_launch("argmax_slices")) return e;
   argmax_pick_kernel<<<n_rows, kWave, 0, s>>>(part_v, part_i, out, vocab);

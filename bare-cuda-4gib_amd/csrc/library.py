@@ -26,6 +26,7 @@ _SIGNATURES = {
     "bc4g_attention_generic": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _P],
     "bc4g_argmax": [_P, _P, _P, _P, _I, _I, _P],
     "bc4g_sample": [_P, _P, _P, _P, _I, _I, _P],
+    "bc4g_argmax_static": [_P, _P, _I, _I, _P],
     "bc4g_gemm_skinny": [_P, _P, _P, _I, _I, _I, _I, _P],
     "bc4g_gemm_mfma": [_P, _P, _P, _I, _I, _I, _I, _P],
     "bc4g_gemm_skinny_normed": [_P, _P, _P, _I, _F, _P, _P, _I, _I, _I, _I, _P],
