@@ -2,16 +2,18 @@
 request, and slots for per-request state of fixed size.
 
 A model's cache *streams* (one per schedule entry that caches, or shared
-between entries) each declare a spec.  Streams whose spec is :class:`PagedKV`
-are put into *groups* by their window: all streams that keep every key share
-one page pool and one block table per request; streams with a window of W
-tokens share another, whose pages are given back once a request's window has
-passed them.  Within a group one page index stands for the same ``page_tokens``
-tokens in every stream of the group, each stream having storage of its own
-shape ``[pages, kv_heads, page_tokens, head_dim]`` for keys and, transposed,
-``[pages, kv_heads, head_dim, page_tokens]`` for values.
-Streams whose spec is :class:`FixedState` get a tensor ``[max_requests,
-*shape]``; a request's row is its slot, zeroed at admission.
+between entries) each declare a spec, which says what it keeps and in which
+tensors (see ``specs.py``; the manager knows no spec by name).  Streams that keep
+something per token are put into *groups* by their window: all streams that keep
+every token share one page pool and one block table per request; streams with a
+window of W tokens share another, whose pages are given back once a request's
+window has passed them.  Within a group one page index stands for the same
+``page_tokens`` tokens in every stream of the group, each stream having tensors
+of its own, ``[pages, *shape of one page]`` (for keys and values:
+``[pages, kv_heads, page_tokens, head_dim]`` and, transposed,
+``[pages, kv_heads, head_dim, page_tokens]``).
+Streams that keep something per request get tensors ``[max_requests, *shape]``;
+a request's row is its slot, zeroed at admission.
 
 (Reference: KVCache, engine/include/llm/kv_cache.h:14-88 and
 engine/src/kv_cache.cpp:17-153 -- one group, 64-token pages, one page table row
@@ -31,25 +33,56 @@ import torch
 
 from ..errors import EngineError, OutOfPages
 from .page_pool import PagePool
-from .specs import FixedState, PagedKV
 
-_STATE_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "int32": torch.int32}
-
-
-@dataclasses.dataclass
-class PagedView:
-    """What a mixer sees of its paged stream."""
-    k: torch.Tensor            # [pages, kv_heads, page_tokens, head_dim]
-    v: torch.Tensor            # [pages, kv_heads, head_dim, page_tokens]
-    group: Hashable            # key of the group whose block table addresses it
-    page_tokens: int
-    window: int
+_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "int32": torch.int32}
 
 
-@dataclasses.dataclass
-class StateView:
-    """What a mixer sees of its fixed-size state stream: row = request slot."""
-    state: torch.Tensor        # [max_requests, *shape]
+def _shape_and_dtype(entry, default: torch.dtype):
+    """A spec names a tensor as a shape (in the cache's dtype) or as (shape, dtype name)."""
+    if len(entry) == 2 and isinstance(entry[1], str):
+        dt = _DTYPES.get(entry[1])
+        if dt is None:
+            raise EngineError(f"cache: dtype {entry[1]!r} is not one of {sorted(_DTYPES)}")
+        return tuple(int(d) for d in entry[0]), dt
+    return tuple(int(d) for d in entry), default
+
+
+class View:
+    """What a mixer sees of its cache stream: the stream's tensors by name (``view.k``, ``view.v``
+    for keys and values; ``view.state`` for a state slot, row = request slot), and for a paged
+    stream the key of the group whose block table addresses it, the page size and the window."""
+
+    def __init__(self, tensors: Dict[str, torch.Tensor], group: Optional[Hashable] = None, page_tokens: int = 0,
+                 window: int = 0):
+        self.tensors = dict(tensors)
+        self.group, self.page_tokens, self.window = group, page_tokens, window
+
+    def __getattr__(self, name: str) -> torch.Tensor:
+        try:
+            return self.__dict__["tensors"][name]
+        except KeyError:
+            raise AttributeError(f"this cache stream has no tensor '{name}' (it has {sorted(self.__dict__.get('tensors', {}))})") from None
+
+    @property
+    def paged(self) -> bool:
+        return self.group is not None
+
+
+PagedView = StateView = View     # (the two kinds of view were classes of their own once)
+
+
+def bytes_per_page(specs: Iterable[Any], page_tokens: int, dtype: torch.dtype) -> int:
+    """Device bytes that one page index stands for, over all streams that keep something per token."""
+    total = 0
+    for spec in specs:
+        if spec is not None and getattr(spec, "per_token", False):
+            for entry in spec.page_tensors(page_tokens).values():
+                shape, dt = _shape_and_dtype(entry, dtype)
+                n = 1
+                for d in shape:
+                    n *= d
+                total += n * torch.empty((), dtype=dt).element_size()
+    return total
 
 
 class _Group:
@@ -86,29 +119,32 @@ class CacheManager:
         self.groups: Dict[Hashable, _Group] = {}
         self._views: Dict[Hashable, Any] = {}
         for sid, spec in self.specs.items():
-            if isinstance(spec, PagedKV):
-                key = ("window", spec.window)
+            if spec is None:
+                continue
+            if getattr(spec, "per_token", None) is True and hasattr(spec, "page_tensors"):
+                window = int(getattr(spec, "window", 0))
+                key = ("window", window)
                 group = self.groups.get(key)
                 if group is None:
-                    group = self.groups[key] = _Group(spec.window, num_pages)
+                    group = self.groups[key] = _Group(window, num_pages)
                 group.streams.append(sid)
-                k = torch.empty((num_pages, spec.num_kv_heads, page_tokens, spec.head_dim),
-                                dtype=dtype, device=self.device)
-                # values are kept transposed (consecutive tokens of one dimension lie together)
-                v = torch.empty((num_pages, spec.num_kv_heads, spec.head_dim, page_tokens),
-                                dtype=dtype, device=self.device)
-                if poison:
-                    k.fill_(float("nan"))
-                    v.fill_(float("nan"))
-                self._views[sid] = PagedView(k=k, v=v, group=key, page_tokens=page_tokens, window=spec.window)
-            elif isinstance(spec, FixedState):
-                sdt = _STATE_DTYPES.get(spec.dtype)
-                if sdt is None:
-                    raise EngineError(f"cache: state dtype {spec.dtype!r} is not one of {sorted(_STATE_DTYPES)}")
-                self._views[sid] = StateView(state=torch.zeros((max_requests, *spec.shape), dtype=sdt,
-                                                               device=self.device))
-            elif spec is not None:
-                raise EngineError(f"cache: stream {sid!r} has an unknown spec {spec!r}")
+                tensors = {}
+                for name, entry in spec.page_tensors(page_tokens).items():
+                    shape, dt = _shape_and_dtype(entry, dtype)
+                    t = torch.empty((num_pages, *shape), dtype=dt, device=self.device)
+                    if poison and t.is_floating_point():
+                        t.fill_(float("nan"))
+                    tensors[name] = t
+                self._views[sid] = View(tensors, group=key, page_tokens=page_tokens, window=window)
+            elif getattr(spec, "per_token", None) is False and hasattr(spec, "slot_tensors"):
+                tensors = {}
+                for name, entry in spec.slot_tensors().items():
+                    shape, dt = _shape_and_dtype(entry, dtype)
+                    tensors[name] = torch.zeros((max_requests, *shape), dtype=dt, device=self.device)
+                self._views[sid] = View(tensors)
+            else:
+                raise EngineError(f"cache: stream {sid!r} has a spec that says neither what it keeps per token "
+                                  f"(per_token = True, page_tensors) nor per request (per_token = False, slot_tensors): {spec!r}")
         self._requests: Dict[Hashable, _Request] = {}
         self._free_slots: List[int] = list(range(max_requests - 1, -1, -1))
         # The same bookkeeping as arrays by request slot, for whoever describes a batch of many
@@ -139,8 +175,9 @@ class CacheManager:
         self._requests[request] = _Request(slot, self.groups)
         self.lengths_by_slot[slot] = 0
         for view in self._views.values():
-            if isinstance(view, StateView):
-                view.state[slot].zero_()
+            if not view.paged:
+                for t in view.tensors.values():
+                    t[slot].zero_()
         return slot
 
     def _req(self, request: Hashable) -> _Request:
@@ -249,10 +286,9 @@ class CacheManager:
             raise EngineError(f"cache: page {page} of group {group} was freed twice or never held")
         if self.poison:
             for sid in self.groups[group].streams:
-                view = self._views[sid]
-                if view.k.is_floating_point():
-                    view.k[page].fill_(float("nan"))
-                    view.v[page].fill_(float("nan"))
+                for t in self._views[sid].tensors.values():
+                    if t.is_floating_point():
+                        t[page].fill_(float("nan"))
 
     def release(self, request: Hashable) -> None:
         """The request has ended: its pages and its slot are given back."""
@@ -290,10 +326,4 @@ class CacheManager:
             g.pool.shuffle_free_list(seed + i)
 
     def storage_bytes(self) -> int:
-        total = 0
-        for view in self._views.values():
-            if isinstance(view, PagedView):
-                total += view.k.numel() * view.k.element_size() * 2
-            else:
-                total += view.state.numel() * view.state.element_size()
-        return total
+        return sum(t.numel() * t.element_size() for view in self._views.values() for t in view.tensors.values())

@@ -654,40 +654,74 @@ def attention_mfma(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     return out
 
 
+_DECODE_TILE_STARTS: dict = {}
+
+
+def attention_plan(batch, n_heads: int, n_kv_heads: int, head_dim: int):
+    """What the matrix-core attention kernel needs to know about a batch before it is launched, worked
+    out on the host when the batch is described (``batch``: the step's HostBatch): how every request's
+    rows are cut into pieces.  Returns (int32 arrays to go up with the batch, notes for attention()).
+
+    While every request brings one tile of rows at most (decoded tokens), a workgroup is one tile and
+    its waves share the tile's keys.  Else four waves with consecutive tiles of a request walk their
+    keys together -- but a request that brings a single tile beside them (a decoded token in a step with
+    prompt portions) would walk its whole context with one wave: from ATTENTION_APART_CONTEXT cached
+    tokens on those requests get a launch of their own in the other form, into the same output."""
+    tpt = attention_tile_tokens(n_heads, n_kv_heads)
+    S, start = batch.n_seqs, batch.seq_start
+    if batch.max_q_len <= tpt:
+        if batch.n_tokens == S:                       # one row a request: the same array for every such step
+            tiles = _DECODE_TILE_STARTS.get(S)
+            if tiles is None:
+                tiles = _DECODE_TILE_STARTS[S] = list(range(S + 1))
+            return {"tiles": tiles}, dict(form="decode", n_tiles=S)
+        return {"tiles": list(range(S + 1))}, dict(form="decode", n_tiles=S)
+    piece = tpt * attention_q_tiles(head_dim) * ATTENTION_STAGED_WAVES
+    new = [start[s + 1] - start[s] for s in range(S)]
+    short = [s for s in range(S) if new[s] <= tpt]
+    apart = bool(short) and max(batch.seq_ctx[s] for s in short) >= ATTENTION_APART_CONTEXT
+    long_starts, short_starts = [0], [0]
+    for s in range(S):
+        is_short = new[s] <= tpt
+        long_starts.append(long_starts[-1] + (0 if apart and is_short else -(-new[s] // piece)))
+        short_starts.append(short_starts[-1] + (-(-new[s] // tpt) if apart and is_short else 0))
+    arrays = {"tiles": long_starts}
+    notes = dict(form="prompt", n_tiles=long_starts[-1], apart=apart)
+    if apart:
+        arrays["short_tiles"] = short_starts
+        notes.update(n_short=short_starts[-1], longest_short=max(batch.seq_ctx[s] for s in short) + tpt)
+    return arrays, notes
+
+
 def attention(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
-              ctx, n_heads: int, n_kv_heads: int, head_dim: int, window: int, scale: float) -> torch.Tensor:
+              ctx, plan, n_heads: int, n_kv_heads: int, head_dim: int, window: int, scale: float) -> torch.Tensor:
     """Attention of a step's rows over the cache: the matrix-core kernel where it takes the
     sizes (bfloat16, head size a multiple of 16 up to 256, pages of a multiple of 16 tokens),
-    else the plain float kernel."""
+    else the plain float kernel.  ``plan``: (device arrays, notes) of attention_plan() for this
+    batch.  The number of parts the keys are cut into follows from ctx.max_kv_len: in a captured
+    step that is the bound of the graph's context bucket, so the choice holds for every replay."""
     work = lambda: attention_work(ctx, n_heads, n_kv_heads, head_dim, window, qkv.element_size())
     if attention_mfma_supported(qkv, k_cache, head_dim):
-        tpt = attention_tile_tokens(n_heads, n_kv_heads)
+        if plan is None:
+            raise KernelError("attention: the matrix-core kernel needs the batch's attention_plan()")
+        arrays, notes = plan
         args = (qkv, k_cache, v_cache, block_table, ctx.seq_start_dev, ctx.seq_ctx_dev)
         sizes = (n_heads, n_kv_heads, head_dim, window, scale)
-        # While every request brings one tile of rows at most (decoded tokens), a workgroup is one
-        # tile and its waves share the tile's keys.
-        if ctx.max_q_len <= tpt:
-            tile_start, n_tiles = ctx.attention_tiles(tpt)
-            n_splits = ctx.fixed_attention_splits or attention_splits(
-                n_tiles, n_heads, n_kv_heads, ctx.max_kv_len, attention_shared_waves(head_dim))
-            return attention_mfma(*args, tile_start, n_tiles, *sizes, n_splits, 1, 1, work=work,
+        if notes["form"] == "decode":
+            n_tiles = notes["n_tiles"]
+            n_splits = attention_splits(n_tiles, n_heads, n_kv_heads, ctx.max_kv_len, attention_shared_waves(head_dim))
+            return attention_mfma(*args, arrays["tiles"], n_tiles, *sizes, n_splits, 1, 1, work=work,
                                   single_rows=ctx.max_q_len == 1 and ctx.n_tokens == ctx.n_seqs)
-        # Else four waves with consecutive tiles of a request walk their keys together -- but a
-        # request that brings a single tile beside them (a decoded token in a step with prompt
-        # portions) would walk its whole context with one wave: those requests get a launch of their
-        # own in the other form, into the same output.
         q_tiles = attention_q_tiles(head_dim)
-        short = [s for s in range(ctx.n_seqs) if ctx.seq_start[s + 1] - ctx.seq_start[s] <= tpt]
-        apart = bool(short) and max(ctx.seq_ctx[s] for s in short) >= ATTENTION_APART_CONTEXT
-        long_tiles = ctx.attention_tiles(tpt * q_tiles * ATTENTION_STAGED_WAVES, *((False, tpt) if apart else ()))
-        n_splits = attention_splits(long_tiles[1] * ATTENTION_STAGED_WAVES, n_heads, n_kv_heads, ctx.max_kv_len)
-        out = attention_mfma(*args, long_tiles[0], long_tiles[1], *sizes, n_splits, q_tiles, 2, work=work,
+        apart = notes["apart"]
+        n_splits = attention_splits(notes["n_tiles"] * ATTENTION_STAGED_WAVES, n_heads, n_kv_heads, ctx.max_kv_len)
+        out = attention_mfma(*args, arrays["tiles"], notes["n_tiles"], *sizes, n_splits, q_tiles, 2, work=work,
                              row_seq=ctx.row_seq if apart else None)
         if apart:
-            short_tiles = ctx.attention_tiles(tpt, True, tpt)
-            longest = max(ctx.seq_ctx[s] for s in short) + tpt
-            n_splits = attention_splits(short_tiles[1], n_heads, n_kv_heads, longest, attention_shared_waves(head_dim))
-            attention_mfma(*args, short_tiles[0], short_tiles[1], *sizes, n_splits, 1, 1, out=out, row_seq=ctx.row_seq)
+            n_splits = attention_splits(notes["n_short"], n_heads, n_kv_heads, notes["longest_short"],
+                                        attention_shared_waves(head_dim))
+            attention_mfma(*args, arrays["short_tiles"], notes["n_short"], *sizes, n_splits, 1, 1, out=out,
+                           row_seq=ctx.row_seq)
         return out
     return attention_generic(qkv, k_cache, v_cache, block_table, ctx.row_seq, ctx.positions,
                              n_heads, n_kv_heads, head_dim, window, scale, work=work)

@@ -2,11 +2,28 @@
 from __future__ import annotations
 
 import dataclasses
-from typing import Any, Dict, Hashable, List, Optional
+from typing import Any, Dict, Hashable, List, Optional, Sequence, Tuple
 
 import torch
 
 from .runtime import Runtime
+
+
+@dataclasses.dataclass
+class HostBatch:
+    """A step's batch as the host knows it, before anything is on the device: request s (in batch
+    order) brings ``seq_start[s+1] - seq_start[s]`` tokens after ``seq_ctx[s]`` cached ones.  What a
+    part's ``prepare_step`` is given.  ``captured``: the step is (or will be replayed from) a captured
+    graph -- then ``max_kv_len`` is not this step's longest context but the bound of the graph's context
+    bucket, so that whatever launch geometry a part derives from it holds for every replay."""
+    n_tokens: int
+    n_seqs: int
+    seq_start: Sequence[int]             # [S+1]
+    seq_ctx: Sequence[int]               # [S] tokens cached before this step
+    seq_slots: Sequence[int]             # [S] state slot of each request
+    max_q_len: int
+    max_kv_len: int
+    captured: bool = False
 
 
 @dataclasses.dataclass
@@ -35,10 +52,12 @@ class StepContext:
     max_q_len: int
     max_kv_len: int
     cache_views: Dict[Hashable, Any] = dataclasses.field(default_factory=dict)
-    # tokens per attention tile -> (device int32 [S+1] first tile of each request, number of tiles)
-    tiles: Dict[int, Any] = dataclasses.field(default_factory=dict)
     made: Dict[Any, Any] = dataclasses.field(default_factory=dict)      # see shared()
-    fixed_attention_splits: int = 0      # non-zero: the key split count is fixed (a captured step)
+    # What the parts' prepare_step made of this batch, by the part's step_signature: (int32 device
+    # tensors by name -- they came up with the batch's own arrays, in the same copy --, whatever else
+    # the part noted for itself on the host).
+    step_data: Dict[Hashable, Tuple[Dict[str, torch.Tensor], Any]] = dataclasses.field(default_factory=dict)
+    captured: bool = False               # see HostBatch
     # The norm that reads the residual stream next, while a part that adds into the stream runs (set by
     # the block around the part; by the model: the norm the next schedule entry begins with).  A product
     # that adds into the stream may then prepare that norm and leave the result in ``prepared`` under
@@ -57,20 +76,3 @@ class StepContext:
         if key not in self.made:
             self.made[key] = make()
         return self.made[key]
-
-    def attention_tiles(self, tokens_per_tile: int, short: Optional[bool] = None, short_max: int = 0):
-        """Each request's rows cut into tiles of ``tokens_per_tile`` tokens: (first tile of each
-        request as a device tensor, total).  With ``short`` given, only the requests that bring at
-        most ``short_max`` rows (True) or more than that (False) get tiles; the others get none.
-        Made once per step, tile size and choice."""
-        key = tokens_per_tile if short is None else (tokens_per_tile, short, short_max)
-        if key not in self.tiles:
-            starts = [0]
-            for s in range(self.n_seqs):
-                n = self.seq_start[s + 1] - self.seq_start[s]
-                if short is not None and (n <= short_max) != short:
-                    n = 0
-                starts.append(starts[-1] + -(-n // tokens_per_tile))
-            dev = torch.tensor(starts, dtype=torch.int32).to(self.token_ids.device, non_blocking=True)
-            self.tiles[key] = (dev, starts[-1])
-        return self.tiles[key]

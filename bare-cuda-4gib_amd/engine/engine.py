@@ -26,21 +26,30 @@ from .scheduler import (FINISH_CANCELLED, FINISH_ERROR, Request, Scheduler, Toke
 Event = Tuple[int, int, int, str]
 
 
+def working_memory_estimate(model, max_seqs: int, max_batch_tokens: int, graphs: int) -> int:
+    """Device bytes the engine will take beyond weights and cache while it serves: a step's activations
+    (a few rows of the widest activation per token) and, for every captured decode graph, its own
+    logits [requests, vocab] in float and activations."""
+    per_token = 64 * model.hidden_size                      # residual stream, products' outputs, attention parts
+    step = max(max_batch_tokens, max_seqs) * (per_token + 4 * model.vocab_size // 8)
+    graph = max_seqs * (4 * model.vocab_size + per_token)
+    return step + graphs * graph
+
+
 def fit_kv_pages(model, max_tokens: int, max_seqs: int, page_tokens: int, dtype: torch.dtype,
-                 device, headroom_bytes: int = 1 << 30) -> int:
-    """Pages for every request to reach max_tokens, or as many as free memory
-    (less a headroom) holds (reference: fit_kv_pages, engine/src/model.cpp:259-277)."""
+                 device, headroom_bytes: int = 1 << 30, working_bytes: int = 0) -> int:
+    """Pages for every request to reach max_tokens, or as many as free memory holds (less a headroom
+    and what the engine will need to work: ``working_bytes``).  The weights -- both copies of every
+    linear map -- are on the device already when this is asked, so free memory accounts for them.
+    (Reference: fit_kv_pages, engine/src/model.cpp:259-277.)"""
+    from ..cache import bytes_per_page
     per_request = -(-max_tokens // page_tokens)
     want = per_request * max_seqs
-    elem = 2 if dtype == torch.bfloat16 else 4
-    per_page = 0
-    for spec in model.cache_streams().values():
-        if hasattr(spec, "num_kv_heads"):
-            per_page += 2 * spec.num_kv_heads * spec.head_dim * page_tokens * elem
+    per_page = bytes_per_page(model.cache_streams().values(), page_tokens, dtype)
     if per_page == 0:
         return want
     free, _ = torch.cuda.mem_get_info(device)
-    fit = max(0, (free - headroom_bytes)) // per_page
+    fit = max(0, (free - headroom_bytes - working_bytes)) // per_page
     if fit < per_request:
         raise EngineError(f"free GPU memory holds {fit} cache pages, one request of {max_tokens} tokens "
                           f"needs {per_request}")
@@ -58,7 +67,9 @@ class Engine:
             raise EngineError(f"max_tokens {max_tokens} is beyond the model's {self.model.max_seq_len} positions")
         rt = self.model.rt
         if kv_pages <= 0:
-            kv_pages = fit_kv_pages(self.model, max_tokens, max_seqs, page_tokens, rt.act_dtype, rt.device)
+            working = working_memory_estimate(self.model, max_seqs, max_batch_tokens, Executor.MAX_GRAPHS)
+            kv_pages = fit_kv_pages(self.model, max_tokens, max_seqs, page_tokens, rt.act_dtype, rt.device,
+                                    working_bytes=working)
         self.executor = Executor(self.model, num_pages=kv_pages, max_requests=max_seqs,
                                  max_tokens=max_tokens, page_tokens=page_tokens,
                                  max_batch_tokens=max_batch_tokens)

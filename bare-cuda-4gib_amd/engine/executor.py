@@ -15,16 +15,12 @@ from typing import Hashable, List, Optional, Sequence
 import numpy as np
 import torch
 
+import collections
+
 from ..cache.manager import CacheManager
 from ..errors import EngineError
-from .batch import StepContext
+from .batch import HostBatch, StepContext
 from .model import Model
-
-
-def _walk_parts(part):
-    yield part
-    for child in part.children():
-        yield from _walk_parts(child)
 
 
 @dataclasses.dataclass
@@ -43,7 +39,21 @@ class Executor:
     pool.  max_requests: requests that can be live at once.  max_tokens: the
     most tokens one request may hold.  max_batch_tokens: the most rows one
     step may bring (0: no limit but memory).
+
+    What a part may add to a step (both optional; the executor knows no part by name):
+      prepare_step(batch: HostBatch) -> (arrays, notes)   called once a step before anything is launched,
+          also before every replay of a captured step.  ``arrays``: name -> ints, which go up to the
+          device in the batch's one copy; ``notes``: anything the part wants to find again.  forward()
+          finds both in ``ctx.step_data[part.step_signature]`` (parts with equal ``step_signature``
+          share one call; a part without the attribute is its own).  In a captured step only the
+          arrays' values may change from replay to replay, not their lengths, and forward() is not run.
+      prepare_capture(n_seqs, max_context)                  called once before a decode step of n_seqs
+          requests is captured for contexts up to max_context: launch geometry of the part's own is
+          fixed here (what forward() derives from ctx.max_kv_len is fixed by itself: that is
+          max_context while capturing).
     """
+    MAX_GRAPHS = 16       # captured decode graphs kept (each owns its logits and activations); the least
+                          # recently used one goes when another is captured
 
     def __init__(self, model: Model, *, num_pages: int, max_requests: int, max_tokens: int,
                  page_tokens: int = 64, max_batch_tokens: int = 0, poison: bool = False,
@@ -57,15 +67,18 @@ class Executor:
                                   max_requests=max_requests, max_tokens=max_tokens,
                                   dtype=self.rt.act_dtype, device=self.rt.device, poison=poison)
         self._views = {sid: self.cache.view(sid) for sid in self.cache.specs}
-        # attention tile sizes the model's mixers ask for (made once per step, with the batch)
-        parts = [p for layer in model.layers for p in _walk_parts(layer)]
-        self._attention_parts = [p for p in parts if hasattr(p, "attention_tile_tokens")]
-        self._tile_sizes = sorted({size for p in self._attention_parts for size in p.attention_tile_tokens()})
+        parts = model.all_parts()
+        # parts that prepare something of their own for every step, one per signature
+        self._preparers = {}
+        for p in parts:
+            if hasattr(p, "prepare_step"):
+                self._preparers.setdefault(getattr(p, "step_signature", id(p)), p)
+        self._capture_parts = [p for p in parts if hasattr(p, "prepare_capture")]
         # decode steps are replayed from captured graphs if every part of the model allows it
         self.use_graphs = bool(use_graphs) and all(getattr(p, "graph_safe", False) for p in parts) \
             and self.rt.device.type == "cuda"
         self.graph_max_batch = graph_max_batch
-        self._graphs = {}
+        self._graphs = collections.OrderedDict()
 
     # ---- requests -----------------------------------------------------------
     def admit(self, request: Hashable) -> int:
@@ -107,9 +120,11 @@ class Executor:
             raise EngineError(f"step: {total} rows are more than max_batch_tokens={self.max_batch_tokens}")
         return total
 
-    def _host_arrays(self, entries: Sequence[StepEntry], table_width: int = 0, all_logits: bool = False):
+    def _host_arrays(self, entries: Sequence[StepEntry], table_width: int = 0, all_logits: bool = False,
+                     max_kv_bound: int = 0):
         """The batch as one flat list of int32 and the layout of its parts.  ``table_width`` 0
-        makes block tables as wide as the batch needs; ``all_logits`` asks for every row."""
+        makes block tables as wide as the batch needs; ``all_logits`` asks for every row;
+        ``max_kv_bound`` (a step about to be captured): the context bound the parts are to plan for."""
         cache, P = self.cache, self.cache.page_tokens
         token_ids: List[int] = []
         positions: List[int] = []
@@ -131,14 +146,14 @@ class Executor:
         flat = token_ids + positions + row_seq + seq_start + seq_ctx + seq_slots + logit_rows
         layout = [("token_ids", T), ("positions", T), ("row_seq", T), ("seq_start", S + 1), ("seq_ctx", S),
                   ("seq_slots", S), ("logit_rows", len(logit_rows))]
-        tiles = {}
-        for tpt in self._tile_sizes:
-            starts = [0]
-            for s in range(S):
-                starts.append(starts[-1] + -(-(seq_start[s + 1] - seq_start[s]) // tpt))
-            flat.extend(starts)
-            layout.append((("tiles", tpt), S + 1))
-            tiles[tpt] = starts[-1]
+        batch = HostBatch(n_tokens=T, n_seqs=S, seq_start=seq_start, seq_ctx=seq_ctx, seq_slots=seq_slots,
+                          max_q_len=max_q, max_kv_len=max_kv_bound or max_kv, captured=bool(max_kv_bound))
+        notes = {}
+        for sig, part in self._preparers.items():
+            arrays, notes[sig] = part.prepare_step(batch)
+            for name, values in arrays.items():
+                flat.extend(values)
+                layout.append(((sig, name), len(values)))
         group_layout = []
         for g in cache.groups:
             tables = [cache.table(g, e.request) for e in entries]
@@ -151,10 +166,10 @@ class Executor:
                 flat.extend(t[p // P] * P + p % P for p in range(ctx_len, ctx_len + len(e.tokens)))
             group_layout.append((g, width))
         host = dict(seq_start=seq_start, seq_ctx=seq_ctx, seq_slots=seq_slots, n_logits=len(logit_rows),
-                    max_q=max_q, max_kv=max_kv, tiles=tiles, T=T, S=S)
+                    max_q=max_q, max_kv=max_kv_bound or max_kv, notes=notes, T=T, S=S, captured=bool(max_kv_bound))
         return flat, layout, group_layout, host
 
-    def _context_from(self, dev: torch.Tensor, layout, group_layout, host, fixed_splits: int = 0) -> StepContext:
+    def _context_from(self, dev: torch.Tensor, layout, group_layout, host) -> StepContext:
         off = 0
         parts = {}
         for name, n in layout:
@@ -167,14 +182,17 @@ class Executor:
             off += S * width
             slot_maps[g] = dev[off:off + T]
             off += T
-        tiles = {tpt: (parts[("tiles", tpt)], n) for tpt, n in host["tiles"].items()}
+        step_data = {sig: ({}, note) for sig, note in host["notes"].items()}
+        for name in parts:
+            if isinstance(name, tuple):
+                step_data[name[0]][0][name[1]] = parts[name]
         return StepContext(
             rt=self.rt, n_tokens=T, n_seqs=S, token_ids=parts["token_ids"], positions=parts["positions"],
             row_seq=parts["row_seq"], seq_start=host["seq_start"], seq_ctx=host["seq_ctx"],
             seq_slots=host["seq_slots"], seq_start_dev=parts["seq_start"], seq_ctx_dev=parts["seq_ctx"],
             seq_slots_dev=parts["seq_slots"], logit_rows=parts["logit_rows"], n_logits=host["n_logits"],
             block_tables=block_tables, slot_maps=slot_maps, max_q_len=host["max_q"], max_kv_len=host["max_kv"],
-            cache_views=self._views, tiles=tiles, fixed_attention_splits=fixed_splits)
+            cache_views=self._views, step_data=step_data, captured=host["captured"])
 
     def build_context(self, entries: Sequence[StepEntry]) -> StepContext:
         """Host arrays of the batch, uploaded in one copy."""
@@ -203,8 +221,11 @@ class Executor:
         key = (S, bucket)
         slot = self._graphs.get(key)
         if slot is None:
-            flat, layout, group_layout, host = self._host_arrays(entries, table_width=width, all_logits=True)
+            flat, layout, group_layout, host = self._host_arrays(entries, table_width=width, all_logits=True,
+                                                                 max_kv_bound=bucket)
             slot = self._capture(key, flat, layout, group_layout, host, bucket)
+        else:
+            self._graphs.move_to_end(key)
         # a ring of pinned staging buffers, each with an event that says its copy has been done
         ring = slot["ring"]
         buf, view, event = ring[slot["next"] % len(ring)]
@@ -223,6 +244,16 @@ class Executor:
             tables = cache.tables_by_slot[g][slots]
             view[tables_at:tables_at + S * width] = tables.reshape(-1)
             view[slots_at:slots_at + S] = tables[rows, ctx // P] * P + ctx % P
+        if self._preparers:
+            batch = HostBatch(n_tokens=S, n_seqs=S, seq_start=slot["seq_start"], seq_ctx=ctx, seq_slots=slots,
+                              max_q_len=1, max_kv_len=bucket, captured=True)
+            for sig, part in self._preparers.items():
+                for name, values in part.prepare_step(batch)[0].items():
+                    off, n = at[(sig, name)]
+                    if len(values) != n:
+                        raise EngineError(f"step: a captured step's array '{name}' of {type(part).__name__} changed its "
+                                          f"length from {n} to {len(values)}")
+                    view[off:off + n] = values
         slot["dev"].copy_(buf, non_blocking=True)
         event.record()
         if device_tokens is not None:
@@ -231,14 +262,15 @@ class Executor:
         return slot["logits"]
 
     def _capture(self, key, flat, layout, group_layout, host, bucket):
-        from ..csrc import ops
         S = key[0]
+        while len(self._graphs) >= self.MAX_GRAPHS:  # the graph used longest ago makes room (its memory goes with it)
+            self._graphs.popitem(last=False)
         dev = torch.tensor(flat, dtype=torch.int32).to(self.rt.device)
-        # the key split count is frozen into the graph: chosen for the bucket's longest context
-        splits = max((ops.attention_splits(S, m.num_heads, m.num_kv_heads, bucket,
-                                           ops.attention_shared_waves(m.head_dim))
-                      for m in self._attention_parts), default=1)
-        ctx = self._context_from(dev, layout, group_layout, dict(host, max_kv=bucket), fixed_splits=splits)
+        # Whatever the parts derive from the context is derived from the bucket's bound (host["max_kv"]), so
+        # the launch geometry frozen into the graph holds for every context of the bucket.
+        for part in self._capture_parts:
+            part.prepare_capture(S, bucket)
+        ctx = self._context_from(dev, layout, group_layout, host)
         self.model.forward(ctx)                      # once outside the graph: first-use work happens here
         torch.cuda.synchronize()
         ctx.made.clear()                             # what layers share is made again inside the graph
@@ -255,13 +287,14 @@ class Executor:
         # where the parts that change between steps lie in the flat array
         at, off = {}, 0
         for name, n in layout:
-            at[name] = off
+            at[name] = (off, n) if isinstance(name, tuple) else off
             off += n
         at["groups"] = []
         for g, width in group_layout:
             at["groups"].append((g, off, off + S * width))
             off += S * width + host["T"]
-        slot = dict(graph=graph, dev=dev, logits=logits, ring=ring, next=0, at=at, rows=np.arange(S))
+        slot = dict(graph=graph, dev=dev, logits=logits, ring=ring, next=0, at=at, rows=np.arange(S),
+                    seq_start=list(range(S + 1)))
         self._graphs[key] = slot
         return slot
 

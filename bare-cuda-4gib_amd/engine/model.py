@@ -58,6 +58,12 @@ class Model:
         self.max_seq_len = spec.max_seq_len
         self.rt: Optional[Runtime] = None
 
+    def all_parts(self) -> List[Part]:
+        """Every part of the model, nested ones included: embedding, each layer's block with its norms,
+        mixer and feed-forward, final norm, head."""
+        tops = [self.embedding.part, *self.layers, self.final_norm.part, self.head.part]
+        return [p for top in tops for p in _walk(top)]
+
     # ---- weights ------------------------------------------------------------
     def _all_bound(self) -> List[_Bound]:
         out = [self.embedding]
@@ -80,6 +86,8 @@ class Model:
         """Place the loaded tensors on the device and hand each part its own."""
         self.rt = rt
         placed: Dict[str, torch.Tensor] = {}
+        cuda = rt.device.type == "cuda"
+        before = torch.cuda.memory_allocated(rt.device) if cuda else 0
 
         def get(name: str) -> Optional[torch.Tensor]:
             if name not in placed and name in tensors:
@@ -97,7 +105,10 @@ class Model:
                         raise ConfigError(f"tensor '{name}' was not loaded")
                 mine[local] = t
             b.part.bind(mine, rt)
+        # the tensors as loaded, and what they take on the device once the parts have packed them
+        # (a linear map's weight is kept in two orders, one for each family of kernels)
         self.weight_bytes = sum(t.numel() * t.element_size() for t in placed.values())
+        self.device_weight_bytes = torch.cuda.memory_allocated(rt.device) - before if cuda else self.weight_bytes
 
     # ---- cache --------------------------------------------------------------
     def cache_streams(self) -> Dict[Hashable, object]:
@@ -127,6 +138,20 @@ class Model:
                 raise ConfigError(f"layers sharing cache stream {e.cache!r} keep a head's dimensions in "
                                   "different orders (their position encodings or dtypes differ)")
         return streams
+
+    # ---- what a step costs -----------------------------------------------------
+    def step_work(self, batch, n_logits: int, elem: int):
+        """(floating-point operations, bytes that have to be read at least) of one step over ``batch``
+        (a HostBatch) with logits at ``n_logits`` rows: every weight the step uses once, the cache of
+        the live requests, as the parts state them; a layer that the schedule names twice counts twice."""
+        flops, nbytes = self.embedding.part.step_work(batch, batch.n_tokens, elem)
+        for e in self.schedule:
+            f, b = self.layers[e.layer].step_work(batch, batch.n_tokens, elem)
+            flops, nbytes = flops + f, nbytes + b
+        for part in (self.final_norm.part, self.head.part):
+            f, b = part.step_work(batch, n_logits, elem)
+            flops, nbytes = flops + f, nbytes + b
+        return flops, nbytes
 
     # ---- forward ------------------------------------------------------------
     def forward(self, ctx: StepContext) -> Optional[torch.Tensor]:

@@ -49,11 +49,18 @@ class CausalAttention(Part):
         layers that share a cache stream must agree on it."""
         return getattr(self, "dim_order", None)
 
-    def attention_tile_tokens(self):
-        """The piece sizes (in tokens) the matrix-core kernel wants each request's rows cut into:
-        one 16-row tile for decoded tokens, four waves' tiles for prompt portions."""
-        tpt = ops.attention_tile_tokens(self.num_heads, self.num_kv_heads)
-        return (tpt, tpt * ops.attention_q_tiles(self.head_dim) * ops.ATTENTION_STAGED_WAVES)
+    @property
+    def step_signature(self):
+        """Attention parts of the same head counts and head size cut a batch alike: one preparation
+        a step serves them all."""
+        return ("attention", self.num_heads, self.num_kv_heads, self.head_dim)
+
+    def prepare_step(self, batch):
+        """How the matrix-core kernel will cut this batch's rows into pieces (nothing where the plain
+        kernel serves): arrays that go up with the batch, and notes for forward()."""
+        if getattr(self, "act_dtype", None) != torch.bfloat16 or self.head_dim % 16 or self.head_dim > 256:
+            return {}, None
+        return ops.attention_plan(batch, self.num_heads, self.num_kv_heads, self.head_dim)
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
         q, kv, h = self.num_heads * self.head_dim, self.num_kv_heads * self.head_dim, self.hidden_size
@@ -86,6 +93,22 @@ class CausalAttention(Part):
         self.w_o = ops.StreamedWeight(o)
         self.act_dtype = rt.act_dtype
 
+    def step_work(self, batch, rows: int, elem: int):
+        """The products' work, plus attention's own: two products of head_dim per query head and visible
+        key, and every visible key and value of every request read once."""
+        flops, nbytes = super().step_work(batch, rows, elem)
+        pairs = keys = 0
+        for s in range(batch.n_seqs):
+            cached, new = int(batch.seq_ctx[s]), int(batch.seq_start[s + 1] - batch.seq_start[s])
+            if self.window > 0:
+                pairs += sum(min(self.window, cached + i + 1) for i in range(new))
+                keys += min(cached + new, self.window + new - 1)
+            else:
+                pairs += new * cached + new * (new + 1) // 2
+                keys += cached + new
+        return (flops + 4.0 * pairs * self.num_heads * self.head_dim,
+                nbytes + 2.0 * keys * self.num_kv_heads * self.head_dim * elem)
+
     def wants_prepared_norm(self, n_rows: int) -> bool:
         """The q|k|v product reads bfloat16 rows faster than it stages float ones for a fused norm
         (6.1 against 8.7 us at TinyLlama's sizes), and beyond 8 rows a prepared norm saves the
@@ -116,7 +139,8 @@ class CausalAttention(Part):
             else:
                 ops.rope_kv_write(q, ctx.positions, slot_map, k_cache, v_cache, self.num_heads, self.num_kv_heads,
                                   self.head_dim, rotary_dim, theta, write_kv=writes, block_pairs=self.block_pairs)
-        o = ops.attention(q, cache.k, cache.v, ctx.block_tables[cache.group], ctx,
+        arrays, notes = ctx.step_data.get(self.step_signature, ({}, None))
+        o = ops.attention(q, cache.k, cache.v, ctx.block_tables[cache.group], ctx, (arrays, notes) if notes else None,
                           self.num_heads, self.num_kv_heads, self.head_dim, self.window, self.scale)
         linear(o, self.w_o, accumulate_into=residual, ctx=ctx)
 

@@ -48,6 +48,30 @@ class Part:
     def children(self) -> List["Part"]:
         return []
 
+    def step_work(self, batch, rows: int, elem: int):
+        """(floating-point operations, bytes that have to be read at least) of this part in a step
+        in which ``rows`` rows pass through it (``batch``: the step's HostBatch; ``elem``: bytes of a
+        stored element).  By default what the part's tensors say: a linear map's weight is read once
+        and takes two operations per row and element, a vector is read once, of a table one row per
+        row; nested parts add theirs.  A part with work beyond its tensors (attention over a cache)
+        adds it."""
+        flops = nbytes = 0.0
+        for spec in self.weight_specs().values():
+            n = 1
+            for d in spec.shape:
+                n *= d
+            if spec.kind == "matrix":
+                flops += 2.0 * rows * n
+                nbytes += n * elem
+            elif spec.kind == "vector":
+                nbytes += n * elem
+            else:
+                nbytes += rows * (n // max(spec.shape[0], 1)) * elem
+        for child in self.children():
+            f, b = child.step_work(batch, rows, elem)
+            flops, nbytes = flops + f, nbytes + b
+        return flops, nbytes
+
 
 def register_part(category: str, kind: str, factory: Callable[..., Part], *, replace: bool = False) -> None:
     """Make ``kind`` buildable: ``factory(**params)`` returns the part."""

@@ -15,6 +15,7 @@ class Embedding(Part):
     """x[t, :] = float(table[ids[t], :]); no scaling, nothing added
     (reference: engine/kernels/embedding_lookup.cu:16-31)."""
     category = "embedding"
+    graph_safe = True     # launches kernels only: may run inside a captured graph
 
     def __init__(self, vocab_size: int, hidden_size: int):
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
@@ -35,6 +36,7 @@ class LMHead(Part):
     ``tied_to`` names the embedding table's tensor and the file has no weight
     of the head's own, the table is used."""
     category = "head"
+    graph_safe = True     # launches kernels only: may run inside a captured graph
 
     def __init__(self, vocab_size: int, hidden_size: int, tied_to=None):
         self.vocab_size, self.hidden_size, self.tied_to = int(vocab_size), int(hidden_size), tied_to

@@ -57,27 +57,22 @@ def build_model(layers, dtype, seed=0, shape=TINYLLAMA):
     return model, cfg
 
 
-def linear_params(cfg):
-    """Weights of the linear maps of one layer, and of the output head."""
-    h, q, kv, i = cfg.hidden_size, cfg.num_heads * cfg.head_dim, cfg.num_kv_heads * cfg.head_dim, cfg.intermediate_size
-    return h * (q + 2 * kv) + q * h + 3 * h * i, cfg.vocab_size * h
-
-
-def decode_bytes(cfg, elem, contexts):
+def decode_bytes(model, elem, contexts):
     """Bytes one decode step has to read: every weight it uses once (linear maps, norms, the
-    embedding rows of the batch) and the cached keys and values of the live requests."""
-    per_layer, head = linear_params(cfg)
-    weights = (cfg.num_layers * (per_layer + 2 * cfg.hidden_size) + head + cfg.hidden_size) * elem
-    weights += len(contexts) * cfg.hidden_size * elem
-    kv = sum(contexts) * cfg.num_layers * 2 * cfg.num_kv_heads * cfg.head_dim * elem
-    return weights + kv
+    embedding rows of the batch) and the cached keys and values of the live requests -- as the model's
+    parts state them (Model.step_work), so another architecture's bytes need no formula here."""
+    from bare_cuda_4gib_amd.engine.batch import HostBatch
+    n = len(contexts)
+    batch = HostBatch(n_tokens=n, n_seqs=n, seq_start=list(range(n + 1)), seq_ctx=[c - 1 for c in contexts],
+                      seq_slots=list(range(n)), max_q_len=1, max_kv_len=max(contexts))
+    return model.step_work(batch, n, elem)[1]
 
 
-def prefill_flops(cfg, t):
-    per_layer, head = linear_params(cfg)
-    linear = 2.0 * t * cfg.num_layers * per_layer + 2.0 * head       # logits at the last place only
-    attn = cfg.num_layers * 4.0 * cfg.num_heads * cfg.head_dim * (t * (t + 1) / 2.0)
-    return linear + attn
+def prefill_flops(model, t):
+    """Operations of one prompt of t tokens with logits at its last place only (Model.step_work)."""
+    from bare_cuda_4gib_amd.engine.batch import HostBatch
+    batch = HostBatch(n_tokens=t, n_seqs=1, seq_start=[0, t], seq_ctx=[0], seq_slots=[0], max_q_len=t, max_kv_len=t)
+    return model.step_work(batch, 1, 2)[0]
 
 
 def run_decode(model, cfg, batch, prompt_len, steps, warmup, seed=1):
@@ -267,14 +262,14 @@ def main() -> int:
 
     if args.only == "decode":
         dt, contexts = run_decode(model, cfg, args.batch, args.prompt_len, args.steps, args.warmup)
-        gbs = decode_bytes(cfg, elem, contexts) / (dt / args.steps) / 1e9
+        gbs = decode_bytes(model, elem, contexts) / (dt / args.steps) / 1e9
         print(json.dumps({"only": "decode", "shape": args.shape, "batch": args.batch, "context": contexts[0],
                           "hbm_frac": round(gbs / HBM_PEAK_GBS, 4), "ms_per_step": round(dt / args.steps * 1e3, 4),
                           "tokens_per_s": round(args.batch * args.steps / dt, 1)}), flush=True)
         return 0
     if args.only == "prefill":
         pre_s = run_prefill(model, cfg, args.prefill_tokens)
-        frac = prefill_flops(cfg, args.prefill_tokens) / pre_s / (PEAK_TFLOPS[args.dtype] * 1e12)
+        frac = prefill_flops(model, args.prefill_tokens) / pre_s / (PEAK_TFLOPS[args.dtype] * 1e12)
         print(json.dumps({"only": "prefill", "shape": args.shape, "tokens": args.prefill_tokens,
                           "ms": round(pre_s * 1e3, 3), "frac": round(frac, 4),
                           "tokens_per_s": round(args.prefill_tokens / pre_s, 1)}), flush=True)
@@ -290,10 +285,10 @@ def main() -> int:
     dt, contexts = run_decode(model, cfg, args.batch, args.prompt_len, args.steps, args.warmup)
     ms_per_step = dt / args.steps * 1e3
     value = args.batch * args.steps / dt
-    achieved = decode_bytes(cfg, elem, contexts) / (dt / args.steps) / 1e9
+    achieved = decode_bytes(model, elem, contexts) / (dt / args.steps) / 1e9
 
     pre_s = run_prefill(model, cfg, args.prefill_tokens)
-    pre_frac = prefill_flops(cfg, args.prefill_tokens) / pre_s / (PEAK_TFLOPS[args.dtype] * 1e12)
+    pre_frac = prefill_flops(model, args.prefill_tokens) / pre_s / (PEAK_TFLOPS[args.dtype] * 1e12)
 
     points = {}
     if not args.no_points:

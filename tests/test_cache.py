@@ -179,3 +179,51 @@ def test_random_orders_of_requests(seed):
         _check_invariants(cm, lengths)
     cm.release_all()
     assert cm.pages_in_use() == 0 and cm.free_slots == 4
+
+
+def test_a_spec_says_its_own_storage():
+    """The manager allocates what a spec names and knows no spec by name: a spec of the test's own,
+    with one tensor per page in a dtype of its own and a window, gets its pages, its group and its
+    poison; a spec that says nothing of the kind is refused."""
+    import dataclasses
+    from bare_cuda_4gib_amd.cache import bytes_per_page
+    from bare_cuda_4gib_amd.errors import EngineError
+
+    @dataclasses.dataclass(frozen=True)
+    class Latent:
+        width: int
+        window: int = 0
+        per_token = True
+
+        def page_tensors(self, page_tokens):
+            return {"c": (page_tokens, self.width), "scale": ((page_tokens,), "float32")}
+
+    @dataclasses.dataclass(frozen=True)
+    class Counters:
+        per_token = False
+
+        def slot_tensors(self):
+            return {"hits": ((2,), "int32"), "sum": ((5,), "float32")}
+
+    cm = CacheManager({"kv": PagedKV(2, 8), "lat": Latent(6), "lat_w": Latent(3, window=9), "n": Counters()},
+                      page_tokens=4, num_pages=10, max_requests=3, max_tokens=40, dtype=torch.bfloat16, device="cpu",
+                      poison=True)
+    lat, lat_w, n = cm.view("lat"), cm.view("lat_w"), cm.view("n")
+    assert lat.c.shape == (10, 4, 6) and lat.c.dtype == torch.bfloat16 and lat.scale.dtype == torch.float32
+    assert lat.group == cm.view("kv").group == ("window", 0) and lat_w.group == ("window", 9) and lat_w.window == 9
+    assert torch.isnan(lat.c.float()).all() and torch.isnan(lat.scale).all()
+    assert n.hits.shape == (3, 2) and n.hits.dtype == torch.int32 and not n.paged and lat.paged
+    with pytest.raises(AttributeError, match="no tensor 'k'"):
+        lat.k
+    assert bytes_per_page(cm.specs.values(), 4, torch.bfloat16) == 2 * (2 * 4 * 8 * 2) + (4 * 6 * 2 + 4 * 4) + (4 * 3 * 2 + 4 * 4)
+    slot = cm.admit("a")
+    n.sum[slot] += 1.0
+    cm.reserve([("a", 6)])
+    cm.advance("a", 6)
+    lat.c[cm.table(("window", 0), "a")[0]] = 1.0
+    page = cm.table(("window", 0), "a")[0]
+    cm.release("a")
+    assert torch.isnan(lat.c[page].float()).all()                       # poisoned again when given back
+    assert cm.admit("b") == slot and float(n.sum[slot].sum()) == 0.0     # zeroed at admission
+    with pytest.raises(EngineError, match="neither"):
+        CacheManager({"x": object()}, page_tokens=4, num_pages=2, max_requests=1, max_tokens=8, dtype=torch.float32, device="cpu")

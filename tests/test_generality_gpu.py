@@ -424,3 +424,186 @@ def test_routed_feed_forward_and_another_position_encoding(tmp_path):
         got = helpers.replay_in_process(ex, st)
         helpers.compare_with_plain(got, wh, plain, label=f"routed toy {label}", rtol=2e-4, atol=2e-5)
         assert ex.cache.pages_in_use() == 0
+
+
+# --- a third toy: a mixer with a cache layout and a launch geometry of its own, inside captured graphs ---
+# Defined here and never leaving the tests.  It keeps, per token, the vector it was given (a cache spec
+# of its own: one float tensor per page, no keys or values) and gives every row the mean of its
+# request's vectors so far, times a matrix.  It walks the cache in chunks of 64 positions, as many as
+# the longest context needs -- a launch geometry of its own, which a captured step has to fix for the
+# graph's whole context bucket -- and it divides by counts that the host works out for every step and
+# sends up with the batch.  All of it through the part hooks; nothing under engine/ or cache/ knows it.
+
+G_CHUNK = 64
+
+
+def register_geometry_toy():
+    from bare_cuda_4gib_amd.config import Architecture, ModelConfig, field_from_json, register_architecture
+    from bare_cuda_4gib_amd.config.registry import unregister_architecture
+    from bare_cuda_4gib_amd.engine.spec import LayerSpec, ModelSpec, PartSpec, ScheduleEntry
+    from bare_cuda_4gib_amd.parts import Part, register_part
+    from bare_cuda_4gib_amd.weights import WeightSpec
+
+    @dataclasses.dataclass(frozen=True)
+    class PagedVectors:
+        """One float vector per token, in pages: a cache spec the framework has never heard of."""
+        width: int
+        window: int = 0
+        per_token = True
+
+        def page_tensors(self, page_tokens):
+            return {"h": ((page_tokens, self.width), "float32")}
+
+    class CausalMean(Part):
+        category = "mixer"
+        graph_safe = True                 # torch kernels on the current stream only, nothing read back
+        calls = {"forward": 0, "prepare_step": 0, "prepare_capture": []}
+
+        def __init__(self, hidden_size):
+            self.hidden = hidden_size
+            self.frozen_chunks = {}
+
+        def cache_spec(self):
+            return PagedVectors(self.hidden)
+
+        def weight_specs(self):
+            return {"mix.weight": WeightSpec((self.hidden, self.hidden))}
+
+        def bind(self, tensors, rt):
+            self.w = tensors["mix.weight"].float()
+
+        def prepare_step(self, batch):
+            CausalMean.calls["prepare_step"] += 1
+            counts = []
+            for s in range(batch.n_seqs):
+                n = int(batch.seq_start[s + 1] - batch.seq_start[s])
+                counts.extend(range(int(batch.seq_ctx[s]) + 1, int(batch.seq_ctx[s]) + n + 1))
+            return {"counts": counts}, dict(chunks=-(-batch.max_kv_len // G_CHUNK))
+
+        def prepare_capture(self, n_seqs, max_context):
+            CausalMean.calls["prepare_capture"].append((n_seqs, max_context))
+            self.frozen_chunks[n_seqs] = -(-max_context // G_CHUNK)
+
+        def forward(self, h, ctx, cache, residual, writes=True):
+            CausalMean.calls["forward"] += 1
+            arrays, notes = ctx.step_data[id(self)]
+            chunks = notes["chunks"]
+            if ctx.captured:                                    # the geometry fixed for the bucket, not this step's
+                assert chunks == self.frozen_chunks[ctx.n_seqs] == -(-ctx.max_kv_len // G_CHUNK)
+            P_, H_ = cache.page_tokens, self.hidden
+            store = cache.h.view(-1, H_)
+            if writes:
+                store[ctx.slot_maps[cache.group].long()] = h.float()
+            table = ctx.block_tables[cache.group][ctx.row_seq.long()].long()           # [T, pages]
+            positions = ctx.positions.long()
+            total = torch.zeros(ctx.n_tokens, H_, device=h.device)
+            for c in range(chunks):
+                pos = c * G_CHUNK + torch.arange(G_CHUNK, device=h.device)
+                seen = pos[None, :] <= positions[:, None]                                # [T, chunk]
+                page = torch.gather(table, 1, (pos // P_).clamp(max=table.shape[1] - 1)[None, :].expand(ctx.n_tokens, -1))
+                index = torch.where(seen, page * P_ + pos % P_, torch.zeros_like(page))
+                rows = store[index.clamp(min=0)]                                         # [T, chunk, H]
+                total += torch.where(seen[:, :, None], rows, torch.zeros_like(rows)).sum(dim=1)
+            mean = total / arrays["counts"].float()[:, None]
+            residual += mean @ self.w.T
+
+    @dataclasses.dataclass
+    class GeometryConfig(ModelConfig):
+        vocab_size: int = field_from_json("vocab_size")
+        hidden_size: int = field_from_json("hidden_size")
+
+    def describe(cfg):
+        norm = dict(size=cfg.hidden_size, eps=1e-5)
+        def layer(i, mixer):
+            p = f"blocks.{i}."
+            return LayerSpec("prenorm", mixer, PartSpec("swiglu", dict(hidden_size=cfg.hidden_size, intermediate_size=INTER),
+                                                        prefix=p + "ffn."),
+                             PartSpec("rmsnorm", dict(norm), prefix=p + "norm1."), PartSpec("rmsnorm", dict(norm), prefix=p + "norm2."))
+        layers = [layer(0, PartSpec("toy_causal_mean", dict(hidden_size=cfg.hidden_size), prefix="blocks.0.")),
+                  layer(1, PartSpec("attention", dict(hidden_size=cfg.hidden_size, num_heads=NH, num_kv_heads=NKV, head_dim=D,
+                                                      window=0, position=PartSpec("rotary", dict(theta=1000.0, dim=D))),
+                                    prefix="blocks.1.attn."))]
+        return ModelSpec(vocab_size=cfg.vocab_size, hidden_size=cfg.hidden_size, max_seq_len=4096,
+                         embedding=PartSpec("embedding", dict(vocab_size=cfg.vocab_size, hidden_size=cfg.hidden_size), prefix="embed."),
+                         layers=layers, schedule=[ScheduleEntry(0, "vectors"), ScheduleEntry(1, "kv")],
+                         final_norm=PartSpec("rmsnorm", dict(norm), prefix="final_norm."),
+                         head=PartSpec("lm_head", dict(vocab_size=cfg.vocab_size, hidden_size=cfg.hidden_size), prefix="head."))
+
+    register_part("mixer", "toy_causal_mean", CausalMean, replace=True)
+    unregister_architecture("ToyGeometryForTests")
+    register_architecture(Architecture("ToyGeometryForTests", "toy_geometry_for_tests", GeometryConfig, describe))
+    return CausalMean
+
+
+GEOMETRY_CONFIG = dict(architectures=["ToyGeometryForTests"], vocab_size=VOCAB, hidden_size=H)
+
+
+def plain_geometry_logits(folder, ids):
+    from safetensors import safe_open
+    with safe_open(os.path.join(folder, "model.safetensors"), "pt") as f:
+        w = {n: f.get_tensor(n).double() for n in f.keys()}
+    t = len(ids)
+    pos = torch.arange(t)
+    x = w["embed.weight"][torch.tensor(ids)]
+
+    def ffn(i, x):
+        p = f"blocks.{i}."
+        h = P.rmsnorm(x, w[p + "norm2.weight"], 1e-5)
+        return x + P.swiglu(h @ w[p + "ffn.gate_proj.weight"].T, h @ w[p + "ffn.up_proj.weight"].T) @ w[p + "ffn.down_proj.weight"].T
+    h = P.rmsnorm(x, w["blocks.0.norm1.weight"], 1e-5)
+    mean = torch.cumsum(h, 0) / torch.arange(1, t + 1, dtype=torch.float64)[:, None]
+    x = ffn(0, x + mean @ w["blocks.0.mix.weight"].T)
+    h = P.rmsnorm(x, w["blocks.1.norm1.weight"], 1e-5)
+    q = (h @ w["blocks.1.attn.q_proj.weight"].T).view(t, NH, D)
+    k = (h @ w["blocks.1.attn.k_proj.weight"].T).view(t, NKV, D)
+    v = (h @ w["blocks.1.attn.v_proj.weight"].T).view(t, NKV, D)
+    o = P.attention(P.rope(q, pos, 1000.0), P.rope(k, pos, 1000.0), v)
+    x = ffn(1, x + o.reshape(t, -1) @ w["blocks.1.attn.o_proj.weight"].T)
+    return P.rmsnorm(x, w["final_norm.weight"], 1e-5) @ w["head.weight"].T
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_mixer_with_its_own_cache_layout_and_step_geometry_runs_in_captured_graphs(tmp_path, dtype):
+    CausalMean = register_geometry_toy()
+    from bare_cuda_4gib_amd.cache import bytes_per_page
+    from bare_cuda_4gib_amd.engine import Executor, StepEntry, load_model
+    from bare_cuda_4gib_amd.weights import write_random_model
+    folder = write_random_model(GEOMETRY_CONFIG, 33, str(tmp_path / "geometry"), dtype, std=0.08, norm_std=0.1)
+    requests = {f"r{i}": helpers.random_ids(n, VOCAB, 700 + i) for i, n in enumerate([270, 90, 41])}
+    plain = {r: plain_geometry_logits(folder, ids).numpy() for r, ids in requests.items()}
+    model, _ = load_model(folder, dtype)
+    page = 16
+    streams = model.cache_streams()
+    elem = 4 if dtype == "float32" else 2
+    assert bytes_per_page(streams.values(), page, model.rt.act_dtype) == page * H * 4 + 2 * NKV * D * page * elem
+    tol = TOL[dtype]
+    # whole, portions, and mixed with few pages: the general path
+    steps_m, where_m, peak = helpers.trace_mixed(requests, seed=3, max_live=3, page_tokens=page)
+    for label, (steps, where), pages in (("whole", helpers.trace_whole(requests), 20),
+                                         ("portions", helpers.trace_portions(requests, seed=2), 20),
+                                         ("mixed", (steps_m, where_m), peak // page)):
+        ex = Executor(model, num_pages=pages, max_requests=3, max_tokens=304, page_tokens=page, poison=True)
+        assert ex.use_graphs                                          # every part here says it may be captured
+        ex.cache.shuffle_free_pages(6)
+        got = helpers.replay_in_process(ex, steps)
+        helpers.compare_with_plain(got, where, plain, label=f"geometry toy {label} {dtype}", **tol)
+    # decoding: three requests' last tokens one by one, all three in every step -- replayed from graphs
+    ex = Executor(model, num_pages=40, max_requests=3, max_tokens=304, page_tokens=page, poison=True)
+    ex.cache.shuffle_free_pages(8)
+    tail = 30
+    for r, ids in requests.items():
+        ex.admit(r)
+        ex.step([StepEntry(r, ids[:-tail], [])])
+    before = dict(CausalMean.calls, prepare_capture=list(CausalMean.calls["prepare_capture"]))
+    for i in range(tail):
+        rows = ex.step([StepEntry(r, [ids[len(ids) - tail + i]], [0]) for r, ids in requests.items()]).float().cpu().numpy()
+        for row, (r, ids) in zip(rows, requests.items()):
+            want = plain[r][len(ids) - tail + i]
+            assert np.all(np.abs(row - want) <= tol["atol"] + tol["rtol"] * np.abs(want)), f"decode step {i}, request {r}"
+    # the longest request crosses from the 256-token bucket into the 512-token one: two graphs, each captured once
+    # after the hook was told its request count and context bound; forward ran for the captures only (twice each),
+    # the step preparation for every step
+    assert sorted(ex._graphs) == [(3, 256), (3, 512)]
+    assert CausalMean.calls["prepare_capture"][len(before["prepare_capture"]):] == [(3, 256), (3, 512)]
+    assert CausalMean.calls["forward"] - before["forward"] == 4
+    assert CausalMean.calls["prepare_step"] - before["prepare_step"] >= tail
