@@ -156,6 +156,8 @@ class CausalAttention(Part):
             scale = h.fusable_scale() if h._tensor is None and h.rows is None else None
             if scale is not None and ops.gemm_qkv_rope_supported(h.x, h.n_rows, True, self.w_qkv, self.head_dim, rotary_dim):
                 return ops.gemm_qkv_rope(h.x, scale[0], scale[1], self.w_qkv, *args)
+            if h.n_rows > ops.SKINNY_MAX_ROWS:
+                return None       # beyond this kernel's rows: the plain product takes the norm as it comes, prepared or not
             h = h.tensor()
         if ops.gemm_qkv_rope_supported(h, h.shape[0], False, self.w_qkv, self.head_dim, rotary_dim):
             return ops.gemm_qkv_rope(h, None, 0.0, self.w_qkv, *args)
