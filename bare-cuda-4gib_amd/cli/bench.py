@@ -87,16 +87,23 @@ def kernel_report(engine, run, dtype: str) -> str:
     wall = (time.perf_counter() - start) * 1e3
     total = sum(s.ms for s in stats) or 1e-9
     peak_tf = PEAK_TFLOPS[dtype]
+    from ..csrc.peaks import measured_peaks
+    measured = measured_peaks()
     lines = [f"\nper-kernel breakdown of one profiled request ({wall:.1f} ms wall, {total:.1f} ms on device; "
              "steps launched kernel by kernel, no captured graphs)",
-             f"device peaks: {HBM_PEAK_GBS:.0f} GB/s memory, {peak_tf:.1f} TFLOP/s dense {dtype} (MI355X, published)\n",
-             f"  {'kernel':<24s} {'calls':>7s} {'ms':>9s} {'%':>6s} {'TFLOP/s':>9s} {'%peak':>6s} {'GB/s':>9s} {'%peak':>6s}"]
+             f"device peaks: {HBM_PEAK_GBS:.0f} GB/s memory, {peak_tf:.1f} TFLOP/s dense {dtype} (MI355X, published); measured "
+             f"on this device: {measured['hbm_gbs']:.0f} GB/s by a kernel that only reads, {measured['bf16_tflops']:.0f} TFLOP/s of "
+             "nothing but bfloat16 MFMAs\n",
+             f"  {'kernel':<24s} {'calls':>7s} {'ms':>9s} {'%':>6s} {'TFLOP/s':>9s} {'%peak':>6s} {'GB/s':>9s} {'%peak':>6s} "
+             f"{'%meas':>6s} {'req GB/s':>9s} {'re-read':>8s}"]
     for s in stats:
         sec = s.ms / 1e3
         tf = s.flops / sec / 1e12 if sec > 0 else 0.0
         gbs = s.bytes / sec / 1e9 if sec > 0 else 0.0
+        req = s.moved / sec / 1e9 if sec > 0 else 0.0
         lines.append(f"  {s.name:<24s} {s.calls:7d} {s.ms:9.2f} {100 * s.ms / total:6.1f} {tf:9.2f} {100 * tf / peak_tf:6.1f} "
-                     f"{gbs:9.1f} {100 * gbs / HBM_PEAK_GBS:6.1f}")
+                     f"{gbs:9.1f} {100 * gbs / HBM_PEAK_GBS:6.1f} {100 * gbs / measured['hbm_gbs']:6.1f} {req:9.1f} "
+                     f"{(s.moved / s.bytes if s.bytes > 0 else 0.0):8.1f}")
     slowest = max(stamps.values(), key=lambda t: t[-1])
     lines += [f"\n  {'host + gaps':<24s} {wall - total:9.2f} ms ({100 * (wall - total) / wall:.1f}% of wall) -- launches, "
               "token copies, the profiler's events",
@@ -104,7 +111,11 @@ def kernel_report(engine, run, dtype: str) -> str:
               "without the profiler)",
               "\n  ms       device time between the events around every launch, summed",
               "  TFLOP/s  floating-point work the result needs / device time",
-              "  GB/s     bytes that have to be moved at least (every operand once) / device time"]
+              "  GB/s     bytes that have to be moved at least (every operand once) / device time; %peak of the published",
+              "           bandwidth, %meas of what a kernel that only reads reaches on this device",
+              "  req      bytes the kernel's workgroups ask for in all / device time (what L2 has to deliver)",
+              "  re-read  asked for / moved at least: 1.0 means every byte is read once; the weight-streaming product reads",
+              "           all its rows of x in every block of 16 columns, prompt attention walks the keys once per piece of rows"]
     return "\n".join(lines)
 
 

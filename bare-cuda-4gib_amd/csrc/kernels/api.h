@@ -177,3 +177,12 @@ int bc4g_gemm_skinny_emit(const void* x, const void* w, float* out, const void* 
 int bc4g_gemm_skinny_prenormed(const void* x, const float* ssq_parts, int ssq_blocks, int ssq_stride, float eps,
                                const void* w, void* out, int epilogue, int m, int n, int k, void* stream);
 }
+
+extern "C" {
+// What the device delivers to a kernel that does nothing else (probes.hip): bc4g_probe_read reads
+// `bytes` of device memory once (sixteen 16-byte loads of a thread in flight); bc4g_probe_mfma runs
+// iters x 4 back-to-back 32x32x16 bfloat16 MFMAs in every one of its workgroups' four waves
+// (workgroups * 4 * iters * 4 * 32768 operations).  The caller times them.
+int bc4g_probe_read(const void* p, long bytes, float* sink, int workgroups, void* stream);
+int bc4g_probe_mfma(int iters, float* sink, int workgroups, void* stream);
+}

@@ -3,7 +3,7 @@ from __future__ import annotations
 
 import ctypes
 import sys
-from ctypes import c_char_p, c_float, c_int, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_long, c_void_p
 from typing import Optional
 
 from ..errors import KernelError
@@ -27,6 +27,8 @@ _SIGNATURES = {
     "bc4g_argmax": [_P, _P, _P, _P, _I, _I, _P],
     "bc4g_sample": [_P, _P, _P, _P, _I, _I, _P],
     "bc4g_argmax_static": [_P, _P, _I, _I, _P],
+    "bc4g_probe_read": [_P, c_long, _P, _I, _P],
+    "bc4g_probe_mfma": [_I, _P, _I, _P],
     "bc4g_gemm_skinny": [_P, _P, _P, _I, _I, _I, _I, _P],
     "bc4g_gemm_mfma": [_P, _P, _P, _I, _I, _I, _I, _P],
     "bc4g_gemm_skinny_normed": [_P, _P, _P, _I, _F, _P, _P, _I, _I, _I, _I, _P],

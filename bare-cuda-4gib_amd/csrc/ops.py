@@ -51,9 +51,23 @@ def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
     return None if t is None else t.data_ptr()
 
 
-def _gemm_cost(m: int, n: int, k: int, in_bytes: int, w_bytes: int, out_bytes: float):
-    """(operations, bytes moved at least) of an [m, k] x [n, k]^T product; out_bytes per output element."""
-    return lambda: (2.0 * m * n * k, m * k * in_bytes + n * k * w_bytes + m * n * out_bytes)
+def _gemm_cost(m: int, n: int, k: int, in_bytes: int, w_bytes: int, out_bytes: float, x_readers: int = 1,
+               w_readers: int = 1):
+    """(operations, bytes moved at least, bytes asked for in all) of an [m, k] x [n, k]^T product; out_bytes per
+    output element.  x_readers / w_readers: how many workgroups read every element of x / of w (the
+    weight-streaming kernel: every block of 16 columns reads all the rows; the tiled kernel: every row of
+    tiles reads all the weights, every column of tiles all the rows)."""
+    ideal = m * k * in_bytes + n * k * w_bytes + m * n * out_bytes
+    moved = x_readers * m * k * in_bytes + w_readers * n * k * w_bytes + m * n * out_bytes
+    return lambda: (2.0 * m * n * k, ideal, moved)
+
+
+def _skinny_cost(m: int, n: int, k: int, in_bytes: int, out_bytes: float):
+    return _gemm_cost(m, n, k, in_bytes, 2, out_bytes, x_readers=-(-n // 16))
+
+
+def _tiled_cost(m: int, n: int, k: int, out_bytes: float):
+    return _gemm_cost(m, n, k, 2, 2, out_bytes, x_readers=-(-n // 128), w_readers=-(-m // 128))
 
 
 def embed_gather(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -363,10 +377,10 @@ def gemm_fast(a: torch.Tensor, w, out_dtype=None,
         for r0 in range(0, m, SKINNY_MAX_ROWS):                        # the weights once for every 64 rows
             rows = min(SKINNY_MAX_ROWS, m - r0)
             library.call("bc4g_gemm_skinny", _ptr(a[r0:]), _ptr(packed), _ptr(out[r0:]), epi, rows, n, k, _stream(),
-                         cost=_gemm_cost(rows, n, k, 2, 2, out_bytes))
+                         cost=_skinny_cost(rows, n, k, 2, out_bytes))
     else:
         library.call("bc4g_gemm_mfma", _ptr(a), _ptr(w), _ptr(out), epi, m, n, k, _stream(),
-                     cost=_gemm_cost(m, n, k, 2, 2, out_bytes))
+                     cost=_tiled_cost(m, n, k, out_bytes))
     return out
 
 
@@ -412,7 +426,7 @@ def gemm_normed(x: torch.Tensor, rows: Optional[torch.Tensor], n_rows: int, g: t
         raise KernelError(f"gemm_normed: epilogue {epilogue} is not supported")
     library.call("bc4g_gemm_skinny_normed", _ptr(x), _ptr(rows), _ptr(g), _code(g, "gemm_normed"), float(eps),
                  _ptr(packed), _ptr(out), epilogue, n_rows, n, k, _stream(),
-                 cost=_gemm_cost(n_rows, n, k, 4, 2, out.element_size() * out.shape[1] / n))
+                 cost=_skinny_cost(n_rows, n, k, 4, out.element_size() * out.shape[1] / n))
     return out
 
 
@@ -432,10 +446,10 @@ def gemm_swiglu(a: torch.Tensor, w_gate_up, interleaved: bool = False) -> torch.
             for r0 in range(0, m, SKINNY_MAX_ROWS):
                 part = min(SKINNY_MAX_ROWS, m - r0)
                 library.call("bc4g_gemm_skinny", _ptr(a[r0:]), _ptr(packed), _ptr(out[r0:]), EPI_SWIGLU, part, n, k,
-                             _stream(), cost=_gemm_cost(part, n, k, 2, 2, 1))
+                             _stream(), cost=_skinny_cost(part, n, k, 2, 1))
         else:
             library.call("bc4g_gemm_mfma", _ptr(a), _ptr(rows), _ptr(out), EPI_SWIGLU, m, n, k, _stream(),
-                         cost=_gemm_cost(m, n, k, 2, 2, 1))
+                         cost=_tiled_cost(m, n, k, 1))
         return out
     gu = gemm_fast(a, w_gate_up, a.dtype)
     if gu is None:
@@ -478,7 +492,7 @@ def gemm_accumulate_emit(a: torch.Tensor, w, residual: torch.Tensor, g: torch.Te
         rows = min(SKINNY_MAX_ROWS, m - r0)
         library.call("bc4g_gemm_skinny_emit", _ptr(a[r0:]), _ptr(packed), _ptr(residual[r0:]), _ptr(g),
                      _code(g, "gemm_accumulate_emit"), _ptr(xb[r0:]), _ptr(parts[:, r0:]), m, rows, n, k, _stream(),
-                     cost=_gemm_cost(rows, n, k, 2, 2, 10))
+                     cost=_skinny_cost(rows, n, k, 2, 10))
     return Prenormed(xb, parts, eps)
 
 
@@ -507,7 +521,7 @@ def gemm_prenormed(pre: Prenormed, w, epilogue: int) -> torch.Tensor:
         rows = min(SKINNY_MAX_ROWS, m - r0)
         library.call("bc4g_gemm_skinny_prenormed", _ptr(pre.xb[r0:]), _ptr(pre.parts[:, r0:]), pre.parts.shape[0], m,
                      pre.eps, _ptr(packed), _ptr(out[r0:]), epilogue, rows, n, k, _stream(),
-                     cost=_gemm_cost(rows, n, k, 2, 2, out.element_size() * out.shape[1] / n))
+                     cost=_skinny_cost(rows, n, k, 2, out.element_size() * out.shape[1] / n))
     return out
 
 
@@ -552,7 +566,7 @@ def gemm_qkv_rope(x: torch.Tensor, g: Optional[torch.Tensor], eps: float, w,
                  float(pre.eps if pre is not None else eps), _ptr(parts), parts.shape[0] if pre is not None else 0,
                  parts.shape[1] if pre is not None else 0, _ptr(packed), _ptr(q), _ptr(positions), _ptr(slot_map),
                  _ptr(k_cache), _ptr(v_cache), m, k, n_heads, n_kv_heads, head_dim, int(rotary_dim), float(theta),
-                 page_tokens, 1 if write_kv else 0, _stream(), cost=_gemm_cost(m, n, k, x.element_size(), 2, 2))
+                 page_tokens, 1 if write_kv else 0, _stream(), cost=_skinny_cost(m, n, k, x.element_size(), 2))
     return q
 
 
@@ -728,17 +742,23 @@ def attention(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, b
 
 
 def attention_work(ctx, n_heads: int, n_kv_heads: int, head_dim: int, window: int, elem: int):
-    """(operations, bytes moved at least) of a step's attention, for the profiler: two products
-    of head_dim per query head and visible key; every visible key and value read once per
-    request, queries read and outputs written once."""
-    pairs = keys = 0
+    """(operations, bytes moved at least, bytes asked for in all) of a step's attention, for the profiler: two
+    products of head_dim per query head and visible key; every visible key and value read once per
+    request, queries read and outputs written once.  Asked for in all: every piece of a request's new
+    rows (the rows one workgroup of the matrix-core kernel's prompt form takes) walks the keys up to its
+    last row by itself."""
+    pairs = keys = walked = 0
+    piece = attention_tile_tokens(n_heads, n_kv_heads) * attention_q_tiles(head_dim) * ATTENTION_STAGED_WAVES
     for s in range(ctx.n_seqs):
         cached, new = ctx.seq_ctx[s], ctx.seq_start[s + 1] - ctx.seq_start[s]
         if window > 0:
             pairs += sum(min(window, cached + i + 1) for i in range(new))
             keys += min(cached + new, window + new - 1)
+            walked += sum(min(cached + min(new, j + piece), window + piece - 1) for j in range(0, new, piece))
         else:
             pairs += new * cached + new * (new + 1) // 2
             keys += cached + new
-    return (4.0 * pairs * n_heads * head_dim,
-            (2 * keys * n_kv_heads * head_dim + 2 * ctx.n_tokens * n_heads * head_dim) * elem)
+            walked += sum(cached + min(new, j + piece) for j in range(0, new, piece))
+    rows = 2 * ctx.n_tokens * n_heads * head_dim
+    return (4.0 * pairs * n_heads * head_dim, (2 * keys * n_kv_heads * head_dim + rows) * elem,
+            (2 * walked * n_kv_heads * head_dim + rows) * elem)

@@ -9,6 +9,10 @@ token for every request through the engine's step function, greedy choice on the
 chosen ids read back while the next step runs).  It prints ONE JSON line: decoded tokens a second, the prefill of one
 2,048-token prompt, the decode step against the HBM roofline, and decoding at batch 1 and 64.
 
+The prefill figure is the best of three runs, the decode figure the mean of K steps; both are also stated
+against what this device was measured to deliver (`--only peaks`: a kernel that only reads; nothing but
+matrix-core instructions).
+
 Beside the headline: `--shape` runs the same measurements at the sizes of Llama-2-7B or Llama-3-8B;
 `--only decode|prefill` runs one part and prints a short line of its own (what the profiles use);
 `--only serve` submits `--requests` requests of mixed lengths to the scheduler and times the whole
@@ -236,8 +240,9 @@ def main() -> int:
     ap.add_argument("--requests", type=int, default=64, help="--only serve: requests submitted at once")
     ap.add_argument("--new-tokens", type=int, default=256, help="--only serve: tokens generated per request")
     ap.add_argument("--chunk", type=int, default=512, help="--only serve: prompt portion size")
-    ap.add_argument("--only", choices=["decode", "prefill", "serve", "gemm"], default=None,
-                    help="run one part only and print its own short line (for profiling)")
+    ap.add_argument("--only", choices=["decode", "prefill", "serve", "gemm", "peaks"], default=None,
+                    help="run one part only and print its own short line (for profiling); peaks: what a kernel that only "
+                         "reads, and one of nothing but matrix-core instructions, reach on this device")
     ap.add_argument("--mnk", default="2048,11264,2048",
                     help="--only gemm: rows, outputs and k of one bfloat16 product x w^T (the tiled matrix-core kernel)")
     args = ap.parse_args()
@@ -252,6 +257,13 @@ def main() -> int:
     if args.only == "gemm":
         print(json.dumps(run_gemm(*(int(v) for v in args.mnk.split(",")))), flush=True)
         return 0
+    from bare_cuda_4gib_amd.csrc.peaks import measured_peaks
+    measured = measured_peaks()
+    if args.only == "peaks":
+        print(json.dumps({"only": "peaks", "hbm_gbs": measured["hbm_gbs"], "hbm_frac_of_published": round(measured["hbm_gbs"] / HBM_PEAK_GBS, 4),
+                          "bf16_tflops": measured["bf16_tflops"],
+                          "bf16_frac_of_published": round(measured["bf16_tflops"] / PEAK_TFLOPS["bf16"], 4)}), flush=True)
+        return 0
     dtype = "bfloat16" if args.dtype == "bf16" else "float32"
     elem = 2 if args.dtype == "bf16" else 4
     shape = SHAPES[args.shape]
@@ -264,14 +276,16 @@ def main() -> int:
         dt, contexts = run_decode(model, cfg, args.batch, args.prompt_len, args.steps, args.warmup)
         gbs = decode_bytes(model, elem, contexts) / (dt / args.steps) / 1e9
         print(json.dumps({"only": "decode", "shape": args.shape, "batch": args.batch, "context": contexts[0],
-                          "hbm_frac": round(gbs / HBM_PEAK_GBS, 4), "ms_per_step": round(dt / args.steps * 1e3, 4),
+                          "hbm_frac": round(gbs / HBM_PEAK_GBS, 4), "hbm_frac_of_measured": round(gbs / measured["hbm_gbs"], 4),
+                          "ms_per_step": round(dt / args.steps * 1e3, 4),
                           "tokens_per_s": round(args.batch * args.steps / dt, 1)}), flush=True)
         return 0
     if args.only == "prefill":
         pre_s = run_prefill(model, cfg, args.prefill_tokens)
         frac = prefill_flops(model, args.prefill_tokens) / pre_s / (PEAK_TFLOPS[args.dtype] * 1e12)
-        print(json.dumps({"only": "prefill", "shape": args.shape, "tokens": args.prefill_tokens,
+        print(json.dumps({"only": "prefill", "shape": args.shape, "tokens": args.prefill_tokens, "of": "best of 3",
                           "ms": round(pre_s * 1e3, 3), "frac": round(frac, 4),
+                          "frac_of_measured": round(frac * PEAK_TFLOPS[args.dtype] / measured["bf16_tflops"], 4) if args.dtype == "bf16" else None,
                           "tokens_per_s": round(args.prefill_tokens / pre_s, 1)}), flush=True)
         return 0
 
@@ -311,9 +325,12 @@ def main() -> int:
                    "page_tokens": 64, "parallelism": "single GPU",
                    "vs_baseline_is": "decode_b1 / 77.3 tok/s (reference, FP16, batch 1, RTX 3050)"},
         "prefill": {"value": round(args.prefill_tokens / pre_s, 1), "tokens": args.prefill_tokens,
-                    "ms": round(pre_s * 1e3, 3), "frac": round(pre_frac, 4)},
+                    "ms": round(pre_s * 1e3, 3), "frac": round(pre_frac, 4), "of": "best of 3",
+                    "frac_of_measured": round(pre_frac * PEAK_TFLOPS[args.dtype] / measured["bf16_tflops"], 4) if args.dtype == "bf16" else None,
+                    "measured_peak_tflops": measured["bf16_tflops"]},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4)},
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "measured_peak": measured["hbm_gbs"],
+                     "frac_of_measured": round(achieved / measured["hbm_gbs"], 4)},
         "points": points,
     }
     print(json.dumps(line), flush=True)

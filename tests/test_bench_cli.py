@@ -64,7 +64,11 @@ def test_profiler_accounting():
         prof.end(mark)
     mark = prof.begin("bare", None)
     prof.end(mark)
+    mark = prof.begin("reread", lambda: (8.0, 10.0, 25.0))        # operations, bytes at least, bytes asked for in all
+    prof.end(mark)
     stats = {s.name: s for s in prof.stats()}
+    assert stats["reread"].bytes == 10.0 and stats["reread"].moved == 25.0
+    assert stats["gemm"].moved == 40.0                              # nothing said: every byte once
     assert stats["gemm"].calls == 2 and stats["gemm"].flops == 400.0 and stats["gemm"].bytes == 40.0
     assert stats["gemm"].ms == pytest.approx(3.0) and stats["norm"].ms == pytest.approx(1.5)
     assert stats["bare"].calls == 1 and stats["bare"].flops == 0.0
@@ -93,10 +97,13 @@ def test_llm_bench_program(tmp_path):
     assert many.returncode == 0, many.stderr[-2000:]
     assert "TPS batch (dec)" in many.stdout and "3 sequences decoded together" in many.stdout
     table = many.stdout.split("per-kernel breakdown")[1]
-    rows = [l.split() for l in table.splitlines() if l.startswith("  ") and len(l.split()) == 8 and l.split()[1].isdigit()]
+    rows = [l.split() for l in table.splitlines() if l.startswith("  ") and len(l.split()) == 11 and l.split()[1].isdigit()]
     names = {r[0] for r in rows}
     assert {"gemm_skinny_qkv", "attention_mfma", "gemm_skinny", "argmax", "embed_gather"} <= names, names
     assert abs(sum(float(r[3]) for r in rows) - 100.0) < 1.0
-    assert "host + gaps" in table
+    assert "host + gaps" in table and "measured on this device" in table
+    by_name = {r[0]: r for r in rows}
+    assert float(by_name["gemm_skinny"][10]) > 1.5, "the weight-streaming product reads x once per block of columns"
+    assert float(by_name["argmax"][10]) == 1.0
     assert run("--prompt", "1,2", "--prompt-len", "4").returncode == 1          # two prompt sources
     assert run("--prompt-len", "4", "--tokens", "1").returncode == 1            # TPOT needs two tokens
