@@ -140,6 +140,9 @@ extern "C" {
 // bfloat16 a [m, k] times bfloat16 w [n, k] transposed on the matrix cores, any m.
 // epilogue: 0 store bfloat16; 1 store float32; 2 add into float32; 3 SwiGLU as in bc4g_gemm_skinny.
 int bc4g_gemm_mfma(const void* a, const void* w, void* out, int epilogue, int m, int n, int k, void* stream);
+// The output tile (rows, columns) bc4g_gemm_mfma takes for these operands: for the accounting of bytes and for
+// tests that want to meet every tile.  Launches nothing.
+int bc4g_gemm_mfma_tile(const void* a, const void* w, int m, int n, int k, int* rows, int* cols);
 }
 
 extern "C" {

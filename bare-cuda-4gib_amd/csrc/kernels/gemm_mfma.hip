@@ -1,22 +1,25 @@
 // out[m, n] (+)= sum_k a[m, k] * w[n, k], bfloat16 operands, float accumulation on the matrix
 // cores: the product of prompt portions (many rows).
 //
-// A workgroup of 4 waves computes a 128 x 128 tile of the output in k-steps of 64.  Both operands
-// are contiguous in k, so a tile of each is staged through LDS as [128 rows][64 k] with rows padded
-// to 144 bytes (which makes the 16-byte fragment reads of 8 consecutive lanes cover all banks), in
-// two buffers: while the waves feed 32x32x16 MFMAs from one, the next k-step is written to the other
-// and the two after it are in flight from memory, in registers.  Each wave owns a 64 x 64 quarter
-// (2 x 2 MFMA blocks).  The finished tile leaves through LDS in 16-byte pieces.
-// Rows and columns beyond the matrix are read as zero and not stored; k must be a multiple of 8.
-// Every output element is accumulated over k in ascending order, whatever the number of rows.
+// Both operands are contiguous in k.  A workgroup computes a tile of the output in k-steps of 64:
+// the rows of a and of w that the tile needs are staged in LDS, every wave reads its fragments there
+// and feeds 32x32x16 MFMAs.  Two forms:
+//  - gemm_mfma_direct_kernel: the operand tiles go from memory into LDS without passing registers
+//    (k a multiple of 64, operands on 16-byte boundaries).  Tiles of 256 x 256, 256 x 192,
+//    256 x 128, 128 x 64 or 64 x 64, whichever lets the busiest CU finish first.
+//  - gemm_mfma_staged_kernel: through registers, 128 x 128 tiles; any k that is a multiple of 8.
+// Every output element is accumulated over k in ascending order in both, whatever the number of
+// rows and the tile: the same bits whichever form and tile a shape selects.
+// Rows and columns beyond the matrix are not stored.
 //
-// What bounds this kernel is not the matrix cores but what a CU can pull through its cache: at
-// 128 x 128 a k-step of 64 brings 32 KB for 2 MFLOP, and 256 CUs doing so reach ~10 TB/s together
-// (measured: ~650 TFLOP/s).  Where the output has tiles enough, a workgroup of 8 waves therefore
-// takes a 256 x 128 tile (the same waves a CU, the same per-wave work, a quarter less traffic).
+// What bounds these kernels is not the matrix cores but how far a k-step's memory loads, LDS
+// traffic and MFMAs overlap: a 64 x 64 part of a wave reads 1 KB of LDS per 32-clock MFMA, which is
+// all that LDS delivers, and the memory path and LDS share their way into the CU.  More waves a CU
+// (the direct form spends no registers on staging) and larger tiles (less traffic per FLOP) help;
+// a deeper pipeline does not.
 //
-// Workgroups are numbered so that those sharing tiles of a and w run on the same XCD at the same
-// time (tile_of).  Where 256 x 256 tiles fill the CUs, a third form takes those (gemm_mfma_wide_kernel).
+// Workgroups are numbered so that those sharing rows of a and of w run on the same XCD at the same
+// time (tile_of).
 #include <math.h>
 
 #include "api.h"
@@ -30,9 +33,8 @@ constexpr int kLdsStride = kBK + 8;   // elements; 144 bytes
 constexpr int kXcds = 8;
 
 // kSwigluBf16: every 16 rows of w are eight gate rows and the eight up rows of the same outputs;
-// out [m, n / 2] = silu(gate) * up.  A gate and its up lie eight lanes apart in the MFMA result.
+// out [m, n / 2] = silu(gate) * up.  A gate and its up lie eight columns apart in the product.
 enum Epilogue : int { kStoreBf16 = 0, kStoreF32 = 1, kAccumF32 = 2, kSwigluBf16 = 3 };
-
 
 // Which tile a workgroup takes.  Workgroups are dealt to the 8 XCDs in turn, each with an L2 of its
 // own: consecutive logical ids stay on one XCD and walk the output in bands of kBand rows of tiles,
@@ -52,25 +54,18 @@ __device__ inline void tile_of(int block, int m_blocks, int n_blocks, int& bm, i
   bn = in_band / rows;
 }
 
-struct Tile {
-  bf16_t a[kBM][kLdsStride];
-  bf16_t w[kBN][kLdsStride];
-};
-
-// Stores a finished tile (float [128][kBN + 4] in LDS) with the epilogue, THREADS threads together.
-template <int EPI, int THREADS>
-__device__ inline void store_tile(const float* tile_out, void* __restrict__ out, int m, int n, long m0, long n0, int tid) {
-  constexpr int kOutStride = kBN + 4;
-  const bool vec = n % 4 == 0;      // rows of the output start on 16-byte (bfloat16: 8-byte) boundaries
+// Stores ROWS x COLS floats (stride COLS + 4) from LDS with the epilogue, THREADS threads together.
+template <int EPI, int THREADS, int ROWS, int COLS>
+__device__ inline void store_patch(const float* patch, void* __restrict__ out, int m, int n, long m0, long n0, int tid) {
+  constexpr int kStride = COLS + 4;
   if constexpr (EPI == kSwigluBf16) {
-    // every 16 columns: eight gates, then the eight ups of the same outputs; a thread takes four gates
     const long n_out = n / 2;
-    for (int c = tid; c < kBM * (kBN / 8); c += THREADS) {
-      const int row = c / (kBN / 8), q = c % (kBN / 8);           // q: group of four outputs
-      const int col = (q / 2) * 16 + (q % 2) * 4;                 // first gate column in the tile
+    for (int c = tid; c < ROWS * (COLS / 8); c += THREADS) {
+      const int row = c / (COLS / 8), q = c % (COLS / 8);
+      const int col = (q / 2) * 16 + (q % 2) * 4;
       const long gm = m0 + row, gn = n0 + col;
       if (gm >= m || gn >= n) continue;
-      const float* src = tile_out + row * kOutStride + col;
+      const float* src = patch + row * kStride + col;
       float v[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) v[e] = (src[e] / (1.0f + expf(-src[e]))) * src[e + 8];
@@ -86,11 +81,12 @@ __device__ inline void store_tile(const float* tile_out, void* __restrict__ out,
       }
     }
   } else {
-    for (int c = tid; c < kBM * (kBN / 4); c += THREADS) {
-      const int row = c / (kBN / 4), col = (c % (kBN / 4)) * 4;
+    const bool vec = n % 4 == 0;
+    for (int c = tid; c < ROWS * (COLS / 4); c += THREADS) {
+      const int row = c / (COLS / 4), col = (c % (COLS / 4)) * 4;
       const long gm = m0 + row, gn = n0 + col;
       if (gm >= m || gn >= n) continue;
-      const floatx4 v = *reinterpret_cast<const floatx4*>(tile_out + row * kOutStride + col);
+      const floatx4 v = *reinterpret_cast<const floatx4*>(patch + row * kStride + col);
       const long o = gm * n + gn;
       if (vec) {
         if constexpr (EPI == kStoreBf16) {
@@ -118,22 +114,26 @@ __device__ inline void store_tile(const float* tile_out, void* __restrict__ out,
   }
 }
 
-// SETS: register sets; SETS - 1 k-steps are in flight from memory while one is written to LDS.
-// WMS: rows of waves (64 output rows each) -- 2 for the 128 x 128 tile, 4 for the 256 x 128 one.
-template <int WMS>
-struct TileOf {
-  bf16_t a[64 * WMS][kLdsStride];
+// ---- operands through registers ---------------------------------------------------------------
+// A workgroup of 4 waves computes a 128 x 128 tile.  A tile of each operand is staged in LDS as
+// [128 rows][64 k] with rows padded to 144 bytes (which makes the 16-byte fragment reads of
+// consecutive lanes cover all banks), in two buffers: while the waves feed MFMAs from one, the next
+// k-step is written to the other and the one after it is in flight from memory, in registers.
+// Each wave owns a 64 x 64 quarter (2 x 2 MFMA blocks).  Rows, columns and k beyond the matrix are
+// read as zero.
+struct StagedTile {
+  bf16_t a[kBM][kLdsStride];
   bf16_t w[kBN][kLdsStride];
 };
 
-template <int EPI, int SETS, int WMS>
-__global__ __launch_bounds__(128 * WMS, WMS == 2 ? 2 : 1) void gemm_mfma_kernel(
+template <int EPI>
+__global__ __launch_bounds__(256, 2) void gemm_mfma_staged_kernel(
     const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, void* __restrict__ out, int m, int n, int k,
     int m_blocks, int n_blocks) {
-  constexpr int kRows = 64 * WMS, kThreads = 128 * WMS;
+  constexpr int SETS = 2, kRows = kBM, kThreads = 256;   // SETS register sets: SETS - 1 k-steps in flight while one is written
   constexpr int kChunkRows = kThreads / 8;           // rows one chunk of a thread's loads covers
   constexpr int kChunksA = kRows / kChunkRows, kChunksW = kBN / kChunkRows;
-  typedef TileOf<WMS> Tile;
+  typedef StagedTile Tile;
   __shared__ __align__(16) unsigned char lds_raw[sizeof(Tile) * 2];
   Tile* tiles = reinterpret_cast<Tile*>(lds_raw);
   const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
@@ -245,357 +245,259 @@ __global__ __launch_bounds__(128 * WMS, WMS == 2 ? 2 : 1) void gemm_mfma_kernel(
     }
   }
 
-  // The tile goes out through LDS (as float [128][128 + 4], 128 rows at a time), so that a thread
-  // stores four neighbouring columns of a row at once.  acc[i][j][r] is row wm*64 + i*32 + 8*(r/4) +
-  // 4*(lane/32) + r%4 and column wn*64 + j*32 + lane%32 of the tile.
+  // The tile goes out through LDS (as float [128][128 + 4]), so that a thread stores four
+  // neighbouring columns of a row at once.  acc[i][j][r] is row wm*64 + i*32 + 8*(r/4) + 4*(lane/32)
+  // + r%4 and column wn*64 + j*32 + lane%32 of the tile.
   constexpr int kOutStride = kBN + 4;
   static_assert(sizeof(float) * kBM * kOutStride <= sizeof(Tile) * 2, "the output tile must fit the operand buffers");
   float* tile_out = reinterpret_cast<float*>(lds_raw);
 #pragma unroll
-  for (int half = 0; half < WMS / 2; ++half) {
-    if (half > 0) lds_barrier();                      // the half before has been read
-    if (wm / 2 == half) {
+  for (int i = 0; i < 2; ++i)
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+    for (int j = 0; j < 2; ++j)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-          for (int r = 0; r < 16; ++r)
-            tile_out[((wm % 2) * 64 + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + r % 4) * kOutStride + wn * 64 + j * 32 +
-                     lane % 32] = acc[i][j][r];
-    }
-    lds_barrier();
-    store_tile<EPI, kThreads>(tile_out, out, m, n, m0 + 128 * half, n0, tid);
-  }
-}
-
-// The same product with the work split between waves: four waves only multiply, eight only move
-// operands (memory -> registers -> LDS).  A wave issues its instructions in order, so a wave that
-// does everything stands still at a full memory queue with its MFMAs behind it; here the
-// multiplying waves wait for data only.  The moving waves form two groups that take the k-steps in
-// turn: in a round one group writes its step into LDS while the other asks memory for a later one
-// -- writing a step takes about as long as asking for one (measured: 900 and 1,300 clocks for a
-// 48 KB step), and one group doing both in a row was what a round waited for.  LDS holds three
-// k-steps: while step t is multiplied, step t + 2 is written; each group has two more in flight
-// in registers.
-constexpr int kStages = 3, kSets = 2;
-constexpr int kSplitThreads = 768;
-
-template <int EPI>
-__global__ __launch_bounds__(kSplitThreads) void gemm_mfma_split_kernel(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
-                                                              void* __restrict__ out, int m, int n, int k,
-                                                              int m_blocks, int n_blocks) {
-  __shared__ __align__(16) unsigned char lds_raw[sizeof(Tile) * kStages];
-  Tile* tiles = reinterpret_cast<Tile*>(lds_raw);
-  const int tid = threadIdx.x, lane = tid % kWave;
-  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
-  const bool mover = wave >= 4;
-
-  int bm, bn;
-  tile_of(blockIdx.x, m_blocks, n_blocks, bm, bn);
-  const long m0 = static_cast<long>(bm) * kBM, n0 = static_cast<long>(bn) * kBN;
-  const int nk = (k + kBK - 1) / kBK;
-
-  floatx16 acc[2][2];
-  const int wm = (wave % 4) / 2, wn = wave % 2;   // a multiplying wave's 64 x 64 quarter
-
-  if (mover) {
-    // thread u of a group's 256 takes segment u % 8 of rows u / 8 + 32 i of both operands
-    const int group = (wave - 4) / 4;             // owns the k-steps s with s % 2 == group
-    const int u = tid - 256 - 256 * group, seg = u % 8, lrow = u / 8;
-    struct Staged {
-      uint4 a[4], w[4];
-    };
-    const bf16_t* arow[4];
-    const bf16_t* wrow[4];
-    bool a_ok[4], w_ok[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const long gm = m0 + lrow + 32 * i, gn = n0 + lrow + 32 * i;
-      a_ok[i] = gm < m;
-      w_ok[i] = gn < n;
-      arow[i] = a + (a_ok[i] ? gm : 0) * k + seg * 8;
-      wrow[i] = w + (w_ok[i] ? gn : 0) * k + seg * 8;
-    }
-    auto load_step = [&](Staged& r, int kt) {
-      const int kk = kt * kBK;
-      const bool k_ok = kk + seg * 8 < k;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        r.a[i] = (k_ok && a_ok[i]) ? load16(arow[i] + kk) : zero16();
-        r.w[i] = (k_ok && w_ok[i]) ? load16(wrow[i] + kk) : zero16();
-      }
-    };
-    auto store_step = [&](const Staged& r, int buf) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        *reinterpret_cast<uint4*>(&tiles[buf].a[lrow + 32 * i][seg * 8]) = r.a[i];
-        *reinterpret_cast<uint4*>(&tiles[buf].w[lrow + 32 * i][seg * 8]) = r.w[i];
-      }
-    };
-    // Step s lands in LDS buffer s % kStages; steps 0 and 1 before the first round, step t + 2 in
-    // round t.  A group's step s >= 2 travels in its register set (s / 2 - 1) % kSets.  In round t
-    // the group of step t + 2 (t % 2) stores it; the other group asks for step t + 1 + 2 kSets into
-    // the set its step t + 1 left the round before.
-    Staged r[kSets];
-    if (group < nk) {
-      load_step(r[0], group);
-      store_step(r[0], group);
-    }
-#pragma unroll
-    for (int i = 0; i < kSets; ++i)
-      if (2 + group + 2 * i < nk) load_step(r[i], 2 + group + 2 * i);
-    lds_barrier();
-    constexpr int kUnroll = 12;   // lcm(kStages, 2 groups x kSets)
-    for (int kt = 0; kt < nk; kt += kUnroll) {
-#pragma unroll
-      for (int j = 0; j < kUnroll; ++j) {
-        const int t = kt + j;
-        if (t >= nk) break;
-        if (group == j % 2) {
-          if (t + 2 < nk) store_step(r[(j / 2) % kSets], (j + 2) % kStages);
-        } else if (t >= 1) {
-          if (t + 1 + 2 * kSets < nk) load_step(r[((j + 1) / 2 + kSets - 1) % kSets], t + 1 + 2 * kSets);
-        }
-        lds_barrier();
-      }
-    }
-  } else {
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-      for (int j = 0; j < 2; ++j)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-    const int frow = lane % 32, fk = (lane / 32) * 8;
-    lds_barrier();
-    constexpr int kUnroll = 3;
-    for (int kt = 0; kt < nk; kt += kUnroll) {
-#pragma unroll
-      for (int j = 0; j < kUnroll; ++j) {
-        const int t = kt + j;
-        if (t >= nk) break;
-        const int cur = j % kStages;
-#pragma unroll
-        for (int ks = 0; ks < kBK / 16; ++ks) {
-          uint4 fa[2], fw[2];
-#pragma unroll
-          for (int i = 0; i < 2; ++i) {
-            fa[i] = *reinterpret_cast<const uint4*>(&tiles[cur].a[wm * 64 + i * 32 + frow][ks * 16 + fk]);
-            fw[i] = *reinterpret_cast<const uint4*>(&tiles[cur].w[wn * 64 + i * 32 + frow][ks * 16 + fk]);
-          }
-#pragma unroll
-          for (int i = 0; i < 2; ++i)
-#pragma unroll
-            for (int jj = 0; jj < 2; ++jj) acc[i][jj] = mfma_32x32x16(fa[i], fw[jj], acc[i][jj]);
-        }
-        lds_barrier();
-      }
-    }
-  }
-
-  // The tile goes out through LDS (as float [128][128 + 4]): all threads store it, four
-  // neighbouring columns of a row at once.
-  constexpr int kOutStride = kBN + 4;
-  float* tile_out = reinterpret_cast<float*>(lds_raw);
-  if (!mover) {
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-      for (int j = 0; j < 2; ++j)
-#pragma unroll
-        for (int r = 0; r < 16; ++r)
-          tile_out[(wm * 64 + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + r % 4) * kOutStride + wn * 64 + j * 32 + lane % 32] =
-              acc[i][j][r];
-  }
+      for (int r = 0; r < 16; ++r)
+        tile_out[(wm * 64 + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + r % 4) * kOutStride + wn * 64 + j * 32 + lane % 32] =
+            acc[i][j][r];
   lds_barrier();
-  store_tile<EPI, kSplitThreads>(tile_out, out, m, n, m0, n0, tid);
+  store_patch<EPI, kThreads, kBM, kBN>(tile_out, out, m, n, m0, n0, tid);
 }
 
-// The same product for outputs with very many tiles: a workgroup of 8 waves takes a 256 x 256 tile
-// and a wave a 128 x 64 part of it (4 x 2 MFMA blocks).  Per FLOP the tile brings two thirds of the
-// bytes of a 256 x 128 one through the CU's cache, which is what bounds these kernels, and a wave
-// reads three quarters of the fragments from LDS (measured, with the banded tile order:
-// 4096 x 4096 x 4096 833 -> 1,015 TFLOP/s, 8192 x 6144 x 4096 917 -> 1,044; no gain where k is long
-// and the output wide, 8192 x 28672 x 4096).  A k-step of 64 is 72 KB in LDS, in two buffers; the
-// step after the next is in flight in registers: between the MFMAs of each slice of 16 a quarter of it
-// is written to LDS and asked for again, two steps ahead, and the next slice's fragments are read
-// while this slice's MFMAs run.  The order of the additions over k is that of the other forms.
-constexpr int kWide = 256;
-struct WideTile {
-  bf16_t a[kWide][kLdsStride];
-  bf16_t w[kWide][kLdsStride];
-};
-constexpr size_t kWideLdsBytes = sizeof(WideTile) * 2;
+// ---- operands straight into LDS ---------------------------------------------------------------
+// The same product with the operand tiles going from memory into LDS without passing registers
+// (global_load_lds_dwordx4: a wave's 64 lanes bring 16 bytes each to 1 KB of consecutive LDS), in a
+// ring of STAGES buffers: step t + STAGES - 1 is asked for when step t's multiplication starts, one
+// barrier a step.  No registers are spent on staging and no instruction on writing LDS, so twice
+// the waves fit a CU, and the forms below are 15-30 % faster than those above on every shape measured
+// (2048 x 11264 x 2048: 104 against 131 us; 2048 x 2048 x 5632: 52 against 74; 4096^3: 1,139 against
+// 1,015 TFLOP/s).  What did not help: a deeper ring where the tiles fill the chip (three stages are
+// slower than two; with fewer tiles than CUs a step is as long as a load takes, and four stages of a
+// 64 x 64 tile halve that: 512 x 2048 x 5632 48 -> 28 us), raising the waves' priority around the MFMAs, 128 x 64 parts for a wave with half the waves.
+//
+// A tile's rows lie in LDS without padding, BK * 2 bytes each; the 16-byte segment s of row r lies in
+// slot s ^ (r % 8) (rows of 128 bytes and more) of its row, so that the fragment reads of eight
+// consecutive rows cover all banks.  A wave-wide load covers 1024 / (BK * 2) rows; which segment a lane
+// brings follows from where its 16 bytes land.
+//
+// WM x WN waves take TM x TN MFMA blocks of 32 x 32 each.  An output element is added up over k in
+// ascending order, as in the form above: the same bits whichever form the shape selects.
+// k must be a multiple of BK; rows beyond m or n are read from the last row and not stored.
+__device__ inline void load_to_lds_16(const void* global, unsigned lds_address) {
+  // The LDS base of a wave-wide load travels in m0, which the compiler reserves for such uses of its
+  // own and sets right before each (this file gives it none: no LDS load builtin, no register array
+  // indexed at run time).  The compiler does not know the instruction, so the waits for it are written
+  // by hand (wait_loads).
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(global), "s"(lds_address) : "memory");
+}
 
-template <int EPI>
-__global__ __launch_bounds__(512, 1) void gemm_mfma_wide_kernel(const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
-                                                                     void* __restrict__ out, int m, int n, int k,
-                                                                     int m_blocks, int n_blocks) {
-  constexpr int WN = 4;                         // waves along n (two rows of them along m)
-  constexpr int kThreads = 128 * WN;
-  constexpr int kWaveN = kWide / WN;            // columns of a wave's part
-  constexpr int kJ = kWaveN / 32;               // MFMA blocks along n
-  extern __shared__ __align__(16) unsigned char wide_raw[];
-  WideTile* tiles = reinterpret_cast<WideTile*>(wide_raw);
+// Waits until at most N of the wave's memory operations are outstanding (they finish in order).
+template <int N>
+__device__ inline void wait_loads() {
+  static_assert(N >= 0 && N < 64, "vmcnt has six bits");
+  // vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] at [15:14]; the other counters unconstrained
+  __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
+}
+template <int PER, int MAX>
+__device__ inline void wait_for_stage(int later) {
+  if constexpr (MAX == 0) {
+    wait_loads<0>();
+  } else {
+    if (later >= MAX) wait_loads<PER * MAX>();
+    else wait_for_stage<PER, MAX - 1>(later);
+  }
+}
+
+template <int WM, int WN, int TM, int TN, int BK, int STAGES>
+struct DirectShape {
+  static constexpr int kRowsA = 32 * TM * WM, kRowsW = 32 * TN * WN, kRowBytes = BK * 2;
+  static constexpr int kWaves = WM * WN, kThreads = 64 * kWaves;
+  static constexpr int kStageBytes = (kRowsA + kRowsW) * kRowBytes;
+  static constexpr int kPatchBytes = 32 * (32 * TN + 4) * 4;                   // a wave's 32 rows of output, as floats
+  static constexpr int kLdsBytes = STAGES * kStageBytes > kWaves * kPatchBytes ? STAGES * kStageBytes : kWaves * kPatchBytes;
+  static_assert(kLdsBytes <= 160 * 1024, "a workgroup's LDS");
+  static_assert(kRowBytes == 128 || kRowBytes == 256, "rows of 128 or 256 bytes (the slot rule)");
+};
+
+template <int EPI, int WM, int WN, int TM, int TN, int BK, int STAGES, int MINWG>
+__global__ __launch_bounds__(64 * WM * WN, MINWG) void gemm_mfma_direct_kernel(
+    const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, void* __restrict__ out, int m, int n, int k, int m_blocks,
+    int n_blocks) {
+  typedef DirectShape<WM, WN, TM, TN, BK, STAGES> S;
+  constexpr int RA = S::kRowsA, RW = S::kRowsW, RB = S::kRowBytes, NW = S::kWaves;
+  constexpr int kGroupRows = 1024 / RB;                    // rows a wave-wide load covers
+  constexpr int GA = RA / kGroupRows, GW = RW / kGroupRows, PER = (GA + GW + NW - 1) / NW;
+  extern __shared__ __align__(1024) unsigned char direct_lds[];
+  const unsigned lds_base = static_cast<unsigned>(
+      reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) unsigned char*)direct_lds));   // its LDS address
   const int tid = threadIdx.x, lane = tid % kWave;
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int wm = wave / WN, wn = wave % WN;
-
   int bm, bn;
   tile_of(blockIdx.x, m_blocks, n_blocks, bm, bn);
-  const long m0 = static_cast<long>(bm) * kWide, n0 = static_cast<long>(bn) * kWide;
+  const long m0 = static_cast<long>(bm) * RA, n0 = static_cast<long>(bn) * RW;
 
-  // global -> LDS: thread t moves segment t % 8 (16 bytes) of rows t / 8 + kChunkRows i of both operands
-  constexpr int kChunkRows = kThreads / 8;
-  constexpr int kChunks = kWide / kChunkRows;
-  constexpr int kPerSlice = kChunks / (kBK / 16);   // chunks written and asked for again per slice of k
-  static_assert(kPerSlice >= 1, "a slice moves at least one chunk");
-  const int seg = tid % 8, lrow = tid / 8;
-  uint4 ra[kChunks], rw[kChunks];
-  const bf16_t* arow[kChunks];
-  const bf16_t* wrow[kChunks];
-  bool a_ok[kChunks], w_ok[kChunks];
+  // the groups of rows this wave brings every step (a spare turn repeats the last group: the same
+  // bytes to the same place), and which of a row's segments this lane's 16 bytes are
+  const int lr = (lane * 16) / RB, ls = (lane * 16 % RB) / 16;
+  const unsigned char* src[PER];
+  unsigned dst[PER];
 #pragma unroll
-  for (int i = 0; i < kChunks; ++i) {
-    const long gm = m0 + lrow + kChunkRows * i, gn = n0 + lrow + kChunkRows * i;
-    a_ok[i] = gm < m;
-    w_ok[i] = gn < n;
-    arow[i] = a + (a_ok[i] ? gm : 0) * k + seg * 8;
-    wrow[i] = w + (w_ok[i] ? gn : 0) * k + seg * 8;
+  for (int i = 0; i < PER; ++i) {
+    int g = wave + NW * i;
+    if (g >= GA + GW) g = GA + GW - 1;
+    const bool of_a = g < GA;
+    const int trow = (of_a ? g : g - GA) * kGroupRows + lr;
+    const int seg = ls ^ (trow & 7);
+    long row = (of_a ? m0 : n0) + trow;
+    const long last = (of_a ? m : n) - 1;
+    if (row > last) row = last;
+    src[i] = reinterpret_cast<const unsigned char*>((of_a ? a : w) + row * k) + seg * 16;
+    dst[i] = (of_a ? 0 : RA * RB) + (of_a ? g : g - GA) * 1024;
   }
-  auto load_chunk = [&](int kt, int i) {
-    const int kk = kt * kBK;
-    const bool k_ok = kk + seg * 8 < k;
-    ra[i] = (k_ok && a_ok[i]) ? load16(arow[i] + kk) : zero16();
-    rw[i] = (k_ok && w_ok[i]) ? load16(wrow[i] + kk) : zero16();
-  };
-  auto store_chunk = [&](int buf, int i) {
-    *reinterpret_cast<uint4*>(&tiles[buf].a[lrow + kChunkRows * i][seg * 8]) = ra[i];
-    *reinterpret_cast<uint4*>(&tiles[buf].w[lrow + kChunkRows * i][seg * 8]) = rw[i];
+  auto ask = [&](int step) {
+    const unsigned base = lds_base + (step % STAGES) * S::kStageBytes;
+#pragma unroll
+    for (int i = 0; i < PER; ++i)
+      load_to_lds_16(src[i] + static_cast<size_t>(step) * RB, __builtin_amdgcn_readfirstlane(base + dst[i]));
   };
 
-  floatx16 acc[4][kJ];
+  floatx16 acc[TM][TN];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < kJ; ++j)
+    for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  const int frow = lane % 32, fk = (lane / 32) * 8;
-  const int nk = (k + kBK - 1) / kBK;
+  const int nk = k / BK;
 #pragma unroll
-  for (int i = 0; i < kChunks; ++i) load_chunk(0, i);
-#pragma unroll
-  for (int i = 0; i < kChunks; ++i) store_chunk(0, i);
-  if (nk > 1) {
-#pragma unroll
-    for (int i = 0; i < kChunks; ++i) load_chunk(1, i);
-  }
-  lds_barrier();
-  uint4 fa[2][4], fw[2][kJ];
-  auto read_fragments = [&](int set, int buf, int ks) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      fa[set][i] = *reinterpret_cast<const uint4*>(&tiles[buf].a[wm * 128 + i * 32 + frow][ks * 16 + fk]);
-#pragma unroll
-    for (int j = 0; j < kJ; ++j)
-      fw[set][j] = *reinterpret_cast<const uint4*>(&tiles[buf].w[wn * kWaveN + j * 32 + frow][ks * 16 + fk]);
-  };
-  for (int t = 0; t < nk; ++t) {
-    const int cur = t & 1;
-    const bool st = t + 1 < nk, ld = t + 2 < nk;
-    read_fragments(0, cur, 0);
-#pragma unroll
-    for (int ks = 0; ks < kBK / 16; ++ks) {
-      // the next slice's fragments are asked for before this slice's MFMAs, which hide the wait
-      if (ks + 1 < kBK / 16) read_fragments((ks + 1) % 2, cur, ks + 1);
-      // a part of the next step goes to the other buffer and is asked for again, two steps ahead
-#pragma unroll
-      for (int c = 0; c < kPerSlice; ++c) {
-        if (st) store_chunk(1 - cur, kPerSlice * ks + c);
-        if (ld) load_chunk(t + 2, kPerSlice * ks + c);
-      }
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < kJ; ++j) acc[i][j] = mfma_32x32x16(fa[ks % 2][i], fw[ks % 2][j], acc[i][j]);
-    }
-    lds_barrier();
-  }
+  for (int s = 0; s < STAGES - 1; ++s)
+    if (s < nk) ask(s);
 
-  // The tile goes out through LDS, its upper and its lower half in turn, each as two float
-  // [128][128 + 4] quarters.  acc[i][j][r] is row wm*128 + i*32 + 8*(r/4) + 4*(lane/32) + r%4 and
-  // column wn*kWaveN + j*32 + lane%32 of the tile.
-  constexpr int kOutStride = kBN + 4;
-  static_assert(2 * sizeof(float) * kBM * kOutStride <= kWideLdsBytes, "two output quarters must fit the operand buffers");
-  float* tile_out = reinterpret_cast<float*>(wide_raw);
+  const int frow = lane % 32, fhalf = lane / 32;
+  int aoff[TM], woff[TN], aswz[TM], wswz[TN];
 #pragma unroll
-  for (int half = 0; half < 2; ++half) {
-    if (half > 0) lds_barrier();
-    if (wm == half) {
-      const int col0 = wn * kWaveN;
-      float* mine = tile_out + (col0 / kBN) * (kBM * kOutStride) + col0 % kBN;
+  for (int i = 0; i < TM; ++i) {
+    const int r = (wm * TM + i) * 32 + frow;
+    aoff[i] = r * RB;
+    aswz[i] = r & 7;
+  }
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+  for (int j = 0; j < TN; ++j) {
+    const int r = (wn * TN + j) * 32 + frow;
+    woff[j] = RA * RB + r * RB;
+    wswz[j] = r & 7;
+  }
+  constexpr int kSlices = BK / 16;
+  uint4 fa[2][TM], fw[2][TN];
+  auto read_fragments = [&](int set, const unsigned char* stage, int slice) {
+    const int s = slice * 2 + fhalf;
 #pragma unroll
-        for (int j = 0; j < kJ; ++j)
+    for (int i = 0; i < TM; ++i) fa[set][i] = *reinterpret_cast<const uint4*>(stage + aoff[i] + ((s ^ aswz[i]) * 16));
 #pragma unroll
-          for (int r = 0; r < 16; ++r)
-            mine[(i * 32 + 8 * (r / 4) + 4 * (lane / 32) + r % 4) * kOutStride + j * 32 + lane % 32] = acc[i][j][r];
+    for (int j = 0; j < TN; ++j) fw[set][j] = *reinterpret_cast<const uint4*>(stage + woff[j] + ((s ^ wswz[j]) * 16));
+  };
+
+  for (int t = 0; t < nk; ++t) {
+    // step t has landed once only the steps asked for after it are outstanding
+    wait_for_stage<PER, STAGES - 2>(min(nk - 1, t + STAGES - 2) - t);
+    lds_barrier();          // everybody's part of step t is there, and nobody reads step t - 1 any more
+    if (t + STAGES - 1 < nk) ask(t + STAGES - 1);
+    const unsigned char* stage = direct_lds + (t % STAGES) * S::kStageBytes;
+    read_fragments(0, stage, 0);
+#pragma unroll
+    for (int ks = 0; ks < kSlices; ++ks) {
+      if (ks + 1 < kSlices) read_fragments((ks + 1) % 2, stage, ks + 1);   // asked for before this slice's MFMAs
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = mfma_32x32x16(fa[ks % 2][i], fw[ks % 2][j], acc[i][j]);
     }
-    lds_barrier();
+  }
+  lds_barrier();            // the last step has been read: LDS is free for the output
+
+  // The tile goes out through LDS so that a thread stores four neighbouring columns of a row at once:
+  // every wave for itself, 32 rows of its part at a time through a patch of its own (no barrier).
+  // acc[i][j][r] is row i 32 + 8 (r / 4) + 4 (lane / 32) + r % 4 and column j 32 + lane % 32 of the part.
+  constexpr int kStride = 32 * TN + 4;
+  float* patch = reinterpret_cast<float*>(direct_lds) + wave * (S::kPatchBytes / 4);
 #pragma unroll
-    for (int q = 0; q < 2; ++q)
-      store_tile<EPI, kThreads>(tile_out + q * (kBM * kOutStride), out, m, n, m0 + 128 * half, n0 + 128 * q, tid);
+  for (int i = 0; i < TM; ++i) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) patch[(8 * (r / 4) + 4 * (lane / 32) + r % 4) * kStride + j * 32 + lane % 32] = acc[i][j][r];
+    store_patch<EPI, kWave, 32, 32 * TN>(patch, out, m, n, m0 + (wm * TM + i) * 32, n0 + wn * TN * 32, lane);
   }
 }
 
-template <int EPI>
-int launch_wide(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, int k, long m_blocks, long n_blocks,
-                hipStream_t s) {
-  auto kernel = gemm_mfma_wide_kernel<EPI>;
+template <int EPI, int WM, int WN, int TM, int TN, int BK, int STAGES, int MINWG>
+int launch_direct(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, int k, hipStream_t s) {
+  typedef DirectShape<WM, WN, TM, TN, BK, STAGES> S;
+  auto kernel = gemm_mfma_direct_kernel<EPI, WM, WN, TM, TN, BK, STAGES, MINWG>;
   static bool raised = false;   // per instantiation: allow more than the default dynamic LDS
   if (!raised) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            static_cast<int>(kWideLdsBytes)) != hipSuccess)
+                            S::kLdsBytes) != hipSuccess)
       return fail("gemm_mfma: cannot raise the dynamic LDS limit");
     raised = true;
   }
-  kernel<<<dim3(static_cast<unsigned>(m_blocks * n_blocks)), dim3(512), kWideLdsBytes, s>>>(
+  const long m_blocks = (m + S::kRowsA - 1) / S::kRowsA, n_blocks = (n + S::kRowsW - 1) / S::kRowsW;
+  kernel<<<dim3(static_cast<unsigned>(m_blocks * n_blocks)), dim3(S::kThreads), S::kLdsBytes, s>>>(
       ap, wp, out, m, n, k, static_cast<int>(m_blocks), static_cast<int>(n_blocks));
   return 0;
 }
 
+// Which tile: the one with which the busiest CU finishes first.  A CU's tiles take their FLOPs over what
+// a CU sustains with that tile (TFLOP/s per CU, measured on shapes that fill the chip), and no tile is
+// faster than its k-steps follow each other when nothing else hides their latency (microseconds a step,
+// measured on shapes with fewer tiles than CUs: the small tile with four stages is for those).  A
+// function of (m, n, k) alone; every tile adds over k in the same order.
+struct DirectForm {
+  int rows, cols;
+  double tflops_a_cu, us_a_step;
+};
+constexpr int kDirectForms = 5;
+constexpr DirectForm kDirectForm[kDirectForms] = {
+    {256, 256, 4.45, 0.5}, {256, 192, 3.9, 0.5}, {256, 128, 3.7, 0.5}, {128, 64, 3.2, 0.5}, {64, 64, 2.2, 0.28}};
+
+int direct_form(int m, int n, int k) {
+  int best = 0;
+  double best_time = 0.0;
+  for (int f = 0; f < kDirectForms; ++f) {
+    const DirectForm& form = kDirectForm[f];
+    const long tiles = static_cast<long>((m + form.rows - 1) / form.rows) * ((n + form.cols - 1) / form.cols);
+    const long turns = (tiles + compute_units() - 1) / compute_units();
+    const double work = turns * (2.0e-6 * form.rows * form.cols * k) / form.tflops_a_cu;
+    const double chain = 3.0 + (k / 64) * form.us_a_step;
+    const double time = work > chain ? work : chain;
+    if (f == 0 || time < best_time) best = f, best_time = time;
+  }
+  return best;
+}
 
 template <int EPI>
-int launch_tiled(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, int k, long m_blocks, long n_blocks,
-                 hipStream_t s) {
-  // Where 256 x 256 tiles fill the CUs round after round (nine tenths of the rounds' places taken),
-  // the form with those tiles; with fewer, the idle places of its last round cost more than it gains
-  // (measured: 2048 x 28672 x 4096, 3.5 rounds, 633 against 576 us).
-  const long wide_blocks = ((m + kWide - 1) / kWide) * ((n + kWide - 1) / kWide);
-  const long rounds = (wide_blocks + compute_units() - 1) / compute_units();
-  if (wide_blocks * 10 >= rounds * compute_units() * 9)
-    return launch_wide<EPI>(ap, wp, out, m, n, k, (m + kWide - 1) / kWide, (n + kWide - 1) / kWide, s);
-  // With tiles enough for every CU to have two of them and more, the 256 x 128 tile: a quarter less
-  // traffic per FLOP, which is what bounds this kernel.
-  const long tall_blocks = (m + 255) / 256;
-  if (tall_blocks * n_blocks >= 2L * compute_units()) {
-    gemm_mfma_kernel<EPI, 2, 4><<<dim3(static_cast<unsigned>(tall_blocks * n_blocks)), dim3(512), 0, s>>>(
-        ap, wp, out, m, n, k, static_cast<int>(tall_blocks), static_cast<int>(n_blocks));
-    return 0;
+int launch_direct_form(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, int k, hipStream_t s) {
+  switch (direct_form(m, n, k)) {
+    case 0: return launch_direct<EPI, 4, 4, 2, 2, 64, 2, 1>(ap, wp, out, m, n, k, s);
+    case 1: return launch_direct<EPI, 4, 2, 2, 3, 64, 2, 1>(ap, wp, out, m, n, k, s);
+    case 2: return launch_direct<EPI, 4, 2, 2, 2, 64, 2, 1>(ap, wp, out, m, n, k, s);
+    case 3: return launch_direct<EPI, 2, 2, 2, 1, 64, 2, 4>(ap, wp, out, m, n, k, s);
+    default: return launch_direct<EPI, 2, 2, 1, 1, 64, 4, 2>(ap, wp, out, m, n, k, s);
   }
-  dim3 grid(static_cast<unsigned>(m_blocks * n_blocks)), block(256);
-  // With at most one tile a CU nothing else runs beside a workgroup: then the split form, whose
-  // moving and multiplying waves overlap, is the faster one (measured: 29 against 35 us for
-  // 2048 x 2048 x 2048); with more tiles two workgroups of the plain form share a CU and do better.
-  if (m_blocks * n_blocks <= compute_units()) {
-    gemm_mfma_split_kernel<EPI><<<grid, dim3(kSplitThreads), 0, s>>>(ap, wp, out, m, n, k, m_blocks, n_blocks);
-    return 0;
-  }
-  gemm_mfma_kernel<EPI, 2, 2><<<grid, block, 0, s>>>(ap, wp, out, m, n, k, m_blocks, n_blocks);
+}
+
+bool direct_operands(const void* ap, const void* wp, int k) {
+  // operands straight into LDS wherever k is whole steps of it and rows start on 16-byte boundaries
+  return k % 64 == 0 && reinterpret_cast<uintptr_t>(ap) % 16 == 0 && reinterpret_cast<uintptr_t>(wp) % 16 == 0;
+}
+
+template <int EPI>
+int launch_tiled(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, int k, hipStream_t s) {
+  if (direct_operands(ap, wp, k)) return launch_direct_form<EPI>(ap, wp, out, m, n, k, s);
+  const long m_blocks = (m + kBM - 1) / kBM, n_blocks = (n + kBN - 1) / kBN;
+  gemm_mfma_staged_kernel<EPI><<<dim3(static_cast<unsigned>(m_blocks * n_blocks)), dim3(256), 0, s>>>(
+      ap, wp, out, m, n, k, static_cast<int>(m_blocks), static_cast<int>(n_blocks));
   return 0;
 }
 
@@ -609,22 +511,32 @@ extern "C" int bc4g_gemm_mfma(const void* a, const void* w, void* out, int epilo
   BC4G_REQUIRE(m >= 0 && n > 0 && k > 0 && k % 8 == 0, "gemm_mfma: K=%d must be a positive multiple of 8 (M=%d N=%d)",
                k, m, n);
   if (m == 0) return 0;
-  const long m_blocks = (m + kBM - 1) / kBM, n_blocks = (n + kBN - 1) / kBN;
-  BC4G_REQUIRE(m_blocks * n_blocks <= 2147483647L, "gemm_mfma: too many tiles");
+  BC4G_REQUIRE(((m + 63L) / 64) * ((n + 63L) / 64) <= 2147483647L, "gemm_mfma: too many tiles");
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bf16_t* ap = static_cast<const bf16_t*>(a);
   const bf16_t* wp = static_cast<const bf16_t*>(w);
   int e = 0;
   switch (epilogue) {
-    case kStoreBf16: e = launch_tiled<kStoreBf16>(ap, wp, out, m, n, k, m_blocks, n_blocks, s); break;
-    case kStoreF32: e = launch_tiled<kStoreF32>(ap, wp, out, m, n, k, m_blocks, n_blocks, s); break;
-    case kAccumF32: e = launch_tiled<kAccumF32>(ap, wp, out, m, n, k, m_blocks, n_blocks, s); break;
+    case kStoreBf16: e = launch_tiled<kStoreBf16>(ap, wp, out, m, n, k, s); break;
+    case kStoreF32: e = launch_tiled<kStoreF32>(ap, wp, out, m, n, k, s); break;
+    case kAccumF32: e = launch_tiled<kAccumF32>(ap, wp, out, m, n, k, s); break;
     case kSwigluBf16:
       BC4G_REQUIRE(n % 16 == 0, "gemm_mfma: SwiGLU needs blocks of eight gate and eight up rows, N=%d is no multiple of 16", n);
-      e = launch_tiled<kSwigluBf16>(ap, wp, out, m, n, k, m_blocks, n_blocks, s);
+      e = launch_tiled<kSwigluBf16>(ap, wp, out, m, n, k, s);
       break;
     default: return fail("gemm_mfma: unknown epilogue %d", epilogue);
   }
   if (e) return e;
   return check_launch("gemm_mfma");
+}
+
+extern "C" int bc4g_gemm_mfma_tile(const void* a, const void* w, int m, int n, int k, int* rows, int* cols) {
+  BC4G_REQUIRE(rows != nullptr && cols != nullptr && m > 0 && n > 0 && k > 0, "gemm_mfma_tile: sizes and two places for the answer");
+  if (direct_operands(a, w, k)) {
+    const DirectForm& form = kDirectForm[direct_form(m, n, k)];
+    *rows = form.rows, *cols = form.cols;
+  } else {
+    *rows = kBM, *cols = kBN;
+  }
+  return 0;
 }

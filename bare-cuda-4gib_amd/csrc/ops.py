@@ -7,8 +7,9 @@ library, or on a CPU tensor, they raise.
 """
 from __future__ import annotations
 
+import ctypes
 import math
-from typing import Optional
+from typing import Optional, Tuple
 
 import torch
 
@@ -66,8 +67,17 @@ def _skinny_cost(m: int, n: int, k: int, in_bytes: int, out_bytes: float):
     return _gemm_cost(m, n, k, in_bytes, 2, out_bytes, x_readers=-(-n // 16))
 
 
+def tiled_tile(m: int, n: int, k: int, a_ptr: int = 0, w_ptr: int = 0) -> Tuple[int, int]:
+    """(rows, columns) of the output tile the tiled matrix-core kernel takes for an [m, k] x [n, k]^T product of
+    operands at these addresses (0: well aligned)."""
+    rows, cols = ctypes.c_int(0), ctypes.c_int(0)
+    library.call("bc4g_gemm_mfma_tile", a_ptr or None, w_ptr or None, m, n, k, ctypes.byref(rows), ctypes.byref(cols))
+    return rows.value, cols.value
+
+
 def _tiled_cost(m: int, n: int, k: int, out_bytes: float):
-    return _gemm_cost(m, n, k, 2, 2, out_bytes, x_readers=-(-n // 128), w_readers=-(-m // 128))
+    rows, cols = tiled_tile(m, n, k)
+    return _gemm_cost(m, n, k, 2, 2, out_bytes, x_readers=-(-n // cols), w_readers=-(-m // rows))
 
 
 def embed_gather(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -339,9 +349,17 @@ def _weight(w):
 
 
 SKINNY_MAX_ROWS = 64
-SKINNY_PASSES_ROWS = 128            # up to here the weights are streamed once per 64 rows rather than tiled: the
-                                    # tiled kernel has one row of tiles to give to 256 CUs (measured at 65 rows:
-                                    # 3.8 ms a step tiled)
+SKINNY_PASSES_ROWS = 128            # up to here the weights are streamed once per 64 rows rather than tiled, unless
+SKINNY_PASSES_MAX_N = 8192          # the output is at least this wide: with one or two rows of tiles a product is as
+                                    # long as its chain of k-steps, which the streaming kernel's eight waves cut
+                                    # into eight (measured at 128 rows: 2048 x 5632 20 against 27 us tiled, 4096 x
+                                    # 14336 66 against 64; but 11264 x 2048 34 against 16, 28672 x 4096 122 against 46)
+
+
+def _in_passes(m: int, n: int) -> bool:
+    return m <= SKINNY_MAX_ROWS or (m <= SKINNY_PASSES_ROWS and n < SKINNY_PASSES_MAX_N)
+
+
 EPI_STORE_BF16, EPI_STORE_F32, EPI_ACCUM_F32, EPI_SWIGLU = 0, 1, 2, 3
 
 
@@ -354,7 +372,8 @@ def gemm_fast(a: torch.Tensor, w, out_dtype=None,
               accumulate_into: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
     """The matrix-core product where a kernel takes these operands (bfloat16, k a multiple of
     8), else None (the caller then uses the plain float kernel).  Up to 64 rows the weights
-    are streamed once (a decode step); beyond that the tiled kernel runs."""
+    are streamed once (a decode step), up to 128 once per 64 rows unless the output is wide; beyond
+    that the tiled kernel runs."""
     w, packed = _weight(w)
     if not _fast_operands(a, w):
         return None
@@ -372,7 +391,7 @@ def gemm_fast(a: torch.Tensor, w, out_dtype=None,
         out = torch.empty((m, n), dtype=out_dtype, device=a.device)
         epi = EPI_STORE_BF16 if out_dtype == torch.bfloat16 else EPI_STORE_F32
     out_bytes = 8 if accumulate_into is not None else out.element_size()
-    if m <= SKINNY_PASSES_ROWS:
+    if _in_passes(m, n):
         packed = packed if packed is not None else pack_weight(w)      # (packing per call: tests only)
         for r0 in range(0, m, SKINNY_MAX_ROWS):                        # the weights once for every 64 rows
             rows = min(SKINNY_MAX_ROWS, m - r0)
@@ -441,7 +460,7 @@ def gemm_swiglu(a: torch.Tensor, w_gate_up, interleaved: bool = False) -> torch.
         m, k = a.shape
         n = rows.shape[0]
         out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=a.device)
-        if m <= SKINNY_PASSES_ROWS:
+        if _in_passes(m, n):
             packed = packed if packed is not None else pack_weight(rows)
             for r0 in range(0, m, SKINNY_MAX_ROWS):
                 part = min(SKINNY_MAX_ROWS, m - r0)
@@ -469,9 +488,9 @@ class Prenormed:
 
 def gemm_emit_supported(a: torch.Tensor, w, residual: torch.Tensor, g: torch.Tensor) -> bool:
     """Whether the adding product of these operands can prepare the next RMSNorm: the
-    weight-streaming kernel serves it (bfloat16, up to SKINNY_PASSES_ROWS rows)."""
+    weight-streaming kernel serves it (bfloat16, few rows: _in_passes)."""
     w, _ = _weight(w)
-    return (_fast_operands(a, w) and 0 < a.shape[0] <= SKINNY_PASSES_ROWS and residual.dtype == torch.float32
+    return (_fast_operands(a, w) and 0 < a.shape[0] and _in_passes(a.shape[0], w.shape[0]) and residual.dtype == torch.float32
             and g.dtype in _CODE and tuple(g.shape) == (w.shape[0],))
 
 
@@ -498,7 +517,7 @@ def gemm_accumulate_emit(a: torch.Tensor, w, residual: torch.Tensor, g: torch.Te
 
 def gemm_prenormed_supported(pre: Prenormed, w) -> bool:
     w, _ = _weight(w)
-    return _fast_operands(pre.xb, w) and pre.xb.shape[0] <= SKINNY_PASSES_ROWS
+    return _fast_operands(pre.xb, w) and _in_passes(pre.xb.shape[0], w.shape[0])
 
 
 def gemm_prenormed(pre: Prenormed, w, epilogue: int) -> torch.Tensor:

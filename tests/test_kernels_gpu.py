@@ -136,68 +136,71 @@ def test_gemm_mfma(ops, m, n, k):
     assert ops.gemm_fast(a.float().to(DEV), w.to(DEV)) is None                      # float operands: not taken
 
 
-def test_gemm_mfma_both_forms_agree_bit_for_bit(ops):
-    """Few tiles go to the form with moving and multiplying waves, many to the plain one (two
-    workgroups a CU), very many to the one with 256 x 128 tiles.  All add over k in the same order:
-    a row's result is the same bits whichever form the number of rows selects, also for sizes that
-    are no multiple of anything."""
-    n, k = 2060, 200                                    # 17 tiles across
-    a, w = bf(rnd(2500, k, seed=40)), bf(rnd(n, k, seed=41))
-    wd = w.to(DEV)
-    many = ops.gemm_fast(a.to(DEV), wd, torch.float32)                 # 20 x 17 = 340 tiles: plain form
-    few = ops.gemm_fast(a[:300].contiguous().to(DEV), wd, torch.float32)   # 3 x 17 tiles: split form
-    close(many, a.double() @ w.double().T, 1e-4, 2e-3, "many tiles")
-    assert torch.equal(few, many[:300])
-    gate_up = interleave8(w[:1024], w[1024:2048])
-    g = ops.gemm_swiglu(a.to(DEV), gate_up.to(DEV), interleaved=True)
-    assert torch.equal(ops.gemm_swiglu(a[:300].contiguous().to(DEV), gate_up.to(DEV), interleaved=True), g[:300])
-    acc_many, acc_few = torch.ones(2500, n, device=DEV), torch.ones(300, n, device=DEV)
-    ops.gemm_fast(a.to(DEV), wd, accumulate_into=acc_many)
-    ops.gemm_fast(a[:300].contiguous().to(DEV), wd, accumulate_into=acc_few)
-    assert torch.equal(acc_few, acc_many[:300])
-    # 7,700 rows: 31 x 17 tiles of 256 x 128, the last of them with 20 rows and 12 columns
-    big = torch.cat([a, bf(rnd(5200, k, seed=42))]).to(DEV)
-    most = ops.gemm_fast(big, wd, torch.float32)
-    assert torch.equal(most[:2500], many)
-    close(most[2500:], big[2500:].double().cpu() @ w.double().T, 1e-4, 2e-3, "very many tiles")
-    assert torch.equal(ops.gemm_swiglu(big, gate_up.to(DEV), interleaved=True)[:2500], g)
-    acc_most = torch.ones(7700, n, device=DEV)
-    ops.gemm_fast(big, wd, accumulate_into=acc_most)
-    assert torch.equal(acc_most[:2500], acc_many)
-    assert torch.equal(ops.gemm_fast(big, wd, torch.bfloat16)[:2500], ops.gemm_fast(a.to(DEV), wd, torch.bfloat16))
-
-
-def test_gemm_mfma_wide_tiles_agree_bit_for_bit(ops):
-    """Outputs that fill every CU with 256 x 256 tiles go to the form with those tiles (eight waves,
-    128 x 64 each): same order over k, same bits as the other forms, whose results for the first rows
-    are taken from a product with fewer rows; edges in both directions (20 rows, 12 columns) and a k
-    that is no multiple of the k-step."""
-    n, k = 16 * 256 - 244, 200                          # 16 tiles across, the last with 12 columns
-    a, w = bf(rnd(16 * 256 - 236, k, seed=43)), bf(rnd(n, k, seed=44))     # 16 tiles down, the last with 20 rows
+@pytest.mark.parametrize("m,n,k,tile", [(4096 - 236, 4096 - 244, 192, (256, 256)), (2048 - 20, 6144 - 12, 192, (256, 192)),
+                                        (2048 - 20, 4096 - 12, 192, (256, 128)), (2048 - 20, 2048 - 12, 1024, (128, 64))])
+def test_gemm_mfma_every_tile_agrees_bit_for_bit(ops, m, n, k, tile):
+    """Five tiles for the operands that go straight into LDS, chosen by the output's shape.  All add over k in
+    the same order: a row's result is the same bits whichever tile the number of rows selects (the first 300 rows
+    alone take the smallest), with edges in both directions, for every epilogue."""
+    if torch.cuda.get_device_properties(0).multi_processor_count != 256:
+        pytest.skip("the shapes are chosen for 256 CUs")
+    assert ops.tiled_tile(m, n, k) == tile and ops.tiled_tile(300, n, k) == (64, 64)
+    a, w = bf(rnd(m, k, seed=40)), bf(rnd(n, k, seed=41))
     ad, wd = a.to(DEV), w.to(DEV)
-    wide = ops.gemm_fast(ad, wd, torch.float32)                        # 256 tiles of 256 x 256
-    close(wide, a.double() @ w.double().T, 1e-4, 2e-3, "wide tiles")
-    few = ops.gemm_fast(ad[:700].contiguous(), wd, torch.float32)      # 3 x 16 wide tiles: the other forms
-    assert torch.equal(few, wide[:700])
-    assert torch.equal(ops.gemm_fast(ad[:700].contiguous(), wd, torch.bfloat16), ops.gemm_fast(ad, wd, torch.bfloat16)[:700])
-    acc_wide, acc_few = torch.ones(a.shape[0], n, device=DEV), torch.ones(700, n, device=DEV)
-    ops.gemm_fast(ad, wd, accumulate_into=acc_wide)
-    ops.gemm_fast(ad[:700].contiguous(), wd, accumulate_into=acc_few)
-    assert torch.equal(acc_few, acc_wide[:700])
-    gate_up = interleave8(w[:1920], w[1920:3840]).to(DEV)               # 15 tiles across: 240 of 256 places
+    full = ops.gemm_fast(ad, wd, torch.float32)
+    close(full, a.double() @ w.double().T, 1e-4, 2e-3, f"tile {tile}")
+    few = ops.gemm_fast(ad[:300].contiguous(), wd, torch.float32)
+    assert torch.equal(few, full[:300])
+    assert torch.equal(ops.gemm_fast(ad[:300].contiguous(), wd, torch.bfloat16), ops.gemm_fast(ad, wd, torch.bfloat16)[:300])
+    acc_full, acc_few = torch.ones(m, n, device=DEV), torch.ones(300, n, device=DEV)
+    ops.gemm_fast(ad, wd, accumulate_into=acc_full)
+    ops.gemm_fast(ad[:300].contiguous(), wd, accumulate_into=acc_few)
+    assert torch.equal(acc_few, acc_full[:300])
+    close(acc_full, a.double() @ w.double().T + 1.0, 1e-4, 2e-3, f"tile {tile}, added")
+    half = (n // 32) * 16                                           # gate and up rows in blocks of eight
+    gate_up = interleave8(w[:half], w[half:2 * half]).to(DEV)
+    assert ops.tiled_tile(m, 2 * half, k) == tile
     g = ops.gemm_swiglu(ad, gate_up, interleaved=True)
-    assert torch.equal(ops.gemm_swiglu(ad[:700].contiguous(), gate_up, interleaved=True), g[:700])
-    gu = a.double() @ w[:3840].double().T
-    close(g, P.swiglu(gu[:, :1920], gu[:, 1920:]), 8e-3, 3e-2, "wide tiles, SwiGLU")
+    assert torch.equal(ops.gemm_swiglu(ad[:300].contiguous(), gate_up, interleaved=True), g[:300])
+    gu = a.double() @ w[:2 * half].double().T
+    close(g, P.swiglu(gu[:, :half], gu[:, half:]), 8e-3, 3e-2, f"tile {tile}, SwiGLU")
+
+
+def test_gemm_mfma_both_forms_agree_bit_for_bit(ops):
+    """A k that is no multiple of 64 goes through registers, in 128 x 128 tiles; the same operands padded with
+    zeros to whole steps go straight into LDS.  Zeros add nothing, and both add over k in the same order: the
+    same bits, for every epilogue."""
+    m, n, k = 700, 2060, 200
+    a, w = bf(rnd(m, k, seed=42)), bf(rnd(n, k, seed=43))
+    pad = lambda t: torch.cat([t, torch.zeros(t.shape[0], 256 - k, dtype=t.dtype)], dim=1).contiguous()
+    ad, wd, ap, wp = a.to(DEV), w.to(DEV), pad(a).to(DEV), pad(w).to(DEV)
+    staged = ops.gemm_fast(ad, wd, torch.float32)
+    close(staged, a.double() @ w.double().T, 1e-4, 2e-3, "through registers")
+    assert torch.equal(staged, ops.gemm_fast(ap, wp, torch.float32))
+    assert torch.equal(ops.gemm_fast(ad, wd, torch.bfloat16), ops.gemm_fast(ap, wp, torch.bfloat16))
+    acc_staged, acc_direct = torch.ones(m, n, device=DEV), torch.ones(m, n, device=DEV)
+    ops.gemm_fast(ad, wd, accumulate_into=acc_staged)
+    ops.gemm_fast(ap, wp, accumulate_into=acc_direct)
+    assert torch.equal(acc_staged, acc_direct)
+    gate_up = interleave8(w[:1024], w[1024:2048])
+    assert torch.equal(ops.gemm_swiglu(ad, gate_up.to(DEV), interleaved=True),
+                       ops.gemm_swiglu(ap, pad(gate_up).to(DEV), interleaved=True))
+    # the form through registers with many tiles (20 x 17) and an operand that does not start on 16 bytes
+    big = bf(rnd(2500, k, seed=44))
+    close(ops.gemm_fast(big.to(DEV), wd, torch.float32), big.double() @ w.double().T, 1e-4, 2e-3, "many tiles")
+    shifted = torch.zeros(m * 256 + 4, dtype=torch.bfloat16, device=DEV)[4:].view(m, 256)     # 8 bytes off
+    shifted.copy_(ap)
+    assert torch.equal(ops.gemm_fast(shifted, wp, torch.float32), staged)
 
 
 @pytest.mark.parametrize("m,n", [(1024, 1024), (2304, 640), (1280 + 5, 384), (4352, 256)])
 def test_gemm_mfma_tile_numbering_covers_every_tile(ops, m, n):
     """Tiles are dealt to the XCDs and walked in bands of eight rows of tiles: every tile is computed
-    once, whether the rows of tiles are a multiple of the band or not (9, 11 and 17 or 34 rows of
-    tiles here) and whether the tile count is a multiple of the XCDs or not."""
-    a, w = bf(rnd(m, 64, seed=15)), bf(rnd(n, 64, seed=16))
-    close(ops.gemm_fast(a.to(DEV), w.to(DEV), torch.float32), a.double() @ w.double().T, 1e-4, 1e-3, "numbering")
+    once, whether the rows of tiles are a multiple of the band or not and whether the tile count is a multiple of
+    the XCDs or not; with operands straight into LDS (k = 64) and through registers (k = 72)."""
+    for k in (64, 72):
+        a, w = bf(rnd(m, k, seed=15)), bf(rnd(n, k, seed=16))
+        close(ops.gemm_fast(a.to(DEV), w.to(DEV), torch.float32), a.double() @ w.double().T, 1e-4, 1e-3, f"numbering, k={k}")
 
 
 def test_gemm_mfma_xcd_numbering_covers_every_tile(ops):
