@@ -133,7 +133,7 @@ int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, float* part_o,
                         const int32_t* seq_start, const int32_t* seq_ctx, const int32_t* tile_start,
                         int n_seqs, int n_tiles, int n_tokens, int n_heads, int n_kv_heads, int head_dim,
                         int page_tokens, int window, float scale, int tokens_per_tile, int q_tiles,
-                        int form, int n_splits, int single_rows, const int32_t* row_seq, void* stream);
+                        int form, int n_splits, int min_walk, int single_rows, const int32_t* row_seq, void* stream);
 }
 
 extern "C" {

@@ -99,6 +99,7 @@ struct AttnArgs {
   int n_heads, n_kv_heads, head_dim, page_tokens, window;
   int hg, tpt, n_sub;          // heads per tile, tokens per tile, head sub-groups per kv head
   int n_splits;
+  int min_walk;                // prompt forms: 32-key tiles a part of a walk holds at least (0: every walk in n_splits parts)
   int single_rows;             // every request brings exactly one row (a decode step): request s is tile s and row s
   float scale_log2;            // softmax scale times log2(e)
 };
@@ -122,8 +123,12 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, 2) void att
   const int col = lane % 16, grp = lane / 16;
   // what tile_start counts: a wave's tiles (WS == 1), or a workgroup's (one tile, or four waves' tiles)
   // (prompt forms: the last workgroups first -- under the causal mask a request's last rows walk
-  // the most keys, and the longest walks should not be the ones that start last)
-  const int block_x = WS > 1 ? blockIdx.x : gridDim.x - 1 - blockIdx.x;
+  // the most keys, and the longest walks should not be the ones that start last -- in every other
+  // (head, part of the keys), and the first ones first in those between: workgroups that are a grid's
+  // x extent apart tend to share a CU, and so a long walk meets a short one there; measured, a
+  // 2,048-token prompt with head size 64: 82 -> 68 us)
+  const bool last_first = ((blockIdx.y + blockIdx.z) & 1) == 0;
+  const int block_x = (WS > 1 || !last_first) ? blockIdx.x : gridDim.x - 1 - blockIdx.x;
   const int tile = WS == 1 ? block_x * kWavesPerBlock + wave : block_x;
   if (WS == 1 && tile >= a.n_tiles) return;   // (waves are independent there: no barrier below)
 
@@ -197,7 +202,12 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, 2) void att
   const int lo_min = (a.window > 0 && walk_min - a.window + 1 > 0) ? walk_min - a.window + 1 : 0;
   const int kt_first = lo_min / 32, kt_last = walk_max / 32;
   const int n_kt = kt_last - kt_first + 1;
-  const int n_parts = a.n_splits * (WS > 1 ? WS : 1);
+  // Into how many parts this walk is cut: all of them, or (prompt forms with min_walk) as many as keep
+  // min_walk tiles each -- under the causal mask the walks differ in length, and parts of about one
+  // length each, few for the short walks and n_splits for the longest, keep the workgroups alike.  The
+  // parts beyond those are empty: they leave their statistics (no keys) and nothing else.
+  int n_parts = a.n_splits * (WS > 1 ? WS : 1);
+  if (WS <= 1 && a.min_walk > 0) n_parts = max(1, min(n_parts, (n_kt + a.min_walk - 1) / a.min_walk));
   const int per_split = (n_kt + n_parts - 1) / n_parts;
   const int kt_begin = kt_first + (blockIdx.z * (WS > 1 ? WS : 1) + (WS > 1 ? wave : 0)) * per_split;
   const int kt_end = min(kt_last + 1, kt_begin + per_split);
@@ -411,7 +421,13 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, 2) void att
             sv[t][4 * h + r] = vis ? sc[t][h][r] : -INFINITY;
           }
     }
-    // the running maximum is kept over raw scores; the softmax scale (> 0) enters the exponent
+    // The exponents are taken against a reference per row, kept over raw scores (the softmax scale, > 0,
+    // enters the exponent): a maximum the row has seen, moved up to the tile's maximum only when that
+    // exceeds it by more than kSlack in the exponent.  Probabilities then reach 2^kSlack at most, which
+    // float sums and bfloat16 factors hold as well as values up to 1, and the quotient of the two sums
+    // does not depend on the reference -- but what has been summed is scaled down far less often (with
+    // the latest maximum as reference some row of a wave's 64 moves in most of a prompt's tiles).
+    constexpr float kSlack = 8.0f;
     float m_new[QT], psum[QT];
     uint4 pf[QT];
     bool moved = false;
@@ -421,7 +437,8 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, 2) void att
       m_tile = max3(m_tile, sv[t][3], sv[t][4]);
       m_tile = max3(m_tile, sv[t][5], sv[t][6]);
       m_tile = max_16_32(max2(m_tile, sv[t][7]));
-      m_new[t] = max2(m_run[t], m_tile);
+      const bool up = (m_tile - m_run[t]) * a.scale_log2 > kSlack;     // (from -inf: yes; nothing seen in the tile: no)
+      m_new[t] = up ? m_tile : m_run[t];
       const float m_safe = (m_new[t] == -INFINITY) ? 0.f : m_new[t];
       const float shift = -m_safe * a.scale_log2;
       float p[8];
@@ -430,11 +447,11 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, 2) void att
       psum[t] = ((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]));
       pf[t] = make_uint4(pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3]), pack_bf16x2(p[4], p[5]),
                          pack_bf16x2(p[6], p[7]));
-      moved = moved || m_new[t] != m_run[t];
+      moved = moved || up;
     }
     if (__any(moved)) {
-      // the running maximum moved for some row of the wave (early in a walk, rarely later): what has
-      // been summed so far is scaled down by 2^(old maximum - new maximum), 0 while nothing had been seen
+      // the reference moved for some row of the wave (early in a walk, rarely later): what has been
+      // summed so far is scaled down by 2^(old reference - new reference), 0 while nothing had been seen
 #pragma unroll
       for (int t = 0; t < QT; ++t) {
         const float m_safe = (m_new[t] == -INFINITY) ? 0.f : m_new[t];
@@ -530,10 +547,12 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, 2) void att
     } else {
       const long slot = (static_cast<long>(blockIdx.z) * a.n_tokens + row) * a.n_heads + q_head;
       float* dst = a.part_o + slot * d + 4 * grp;
+      if (a.min_walk == 0 || kt_begin < kt_end) {   // (an empty part of a walk with a least length: the merge does not look at its outputs)
 #pragma unroll
-      for (int b = 0; b < DB; ++b) {
-        if (!EXACT && 16 * b >= d) break;
-        *reinterpret_cast<floatx4*>(dst + 16 * b) = o[t][b];
+        for (int b = 0; b < DB; ++b) {
+          if (!EXACT && 16 * b >= d) break;
+          *reinterpret_cast<floatx4*>(dst + 16 * b) = o[t][b];
+        }
       }
       if (grp == 0) {
         a.part_ml[slot * 2] = m_run[t] * a.scale_log2;
@@ -599,7 +618,9 @@ __global__ __launch_bounds__(kWave) void attention_merge_kernel(const float* __r
 // short contexts into few): a thread takes four neighbouring output dimensions of one (row, head),
 // asks for every part's statistics and outputs at once -- one trip to memory, no LDS, no barrier --
 // and adds the parts in order of z.
-template <int MAXS>
+// SKIP: parts without keys (statistics -inf) may have left no outputs: those are not read (the
+// statistics first, then the outputs of the parts that have any).
+template <int MAXS, bool SKIP>
 __global__ __launch_bounds__(256) void attention_merge_few_kernel(const float* __restrict__ part_o,
                                                                   const float* __restrict__ part_ml,
                                                                   bf16_t* __restrict__ out, int n_splits,
@@ -621,7 +642,14 @@ __global__ __launch_bounds__(256) void attention_merge_few_kernel(const float* _
   for (int z = 0; z < MAXS; ++z) {
     const bool live = z < n_splits;
     ml[z] = live ? *reinterpret_cast<const float2*>(part_ml + (z * n_rows_heads + rh) * 2) : make_float2(-INFINITY, 0.f);
-    o[z] = live ? *reinterpret_cast<const floatx4*>(part_o + (z * n_rows_heads + rh) * d + c) : floatx4{0.f, 0.f, 0.f, 0.f};
+    if constexpr (!SKIP)
+      o[z] = live ? *reinterpret_cast<const floatx4*>(part_o + (z * n_rows_heads + rh) * d + c) : floatx4{0.f, 0.f, 0.f, 0.f};
+  }
+  if constexpr (SKIP) {
+#pragma unroll
+    for (int z = 0; z < MAXS; ++z)
+      o[z] = (z < n_splits && ml[z].x != -INFINITY) ? *reinterpret_cast<const floatx4*>(part_o + (z * n_rows_heads + rh) * d + c)
+                                                    : floatx4{0.f, 0.f, 0.f, 0.f};
   }
   float m = -INFINITY;
 #pragma unroll
@@ -662,7 +690,7 @@ extern "C" int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, flo
                                    const int32_t* seq_start, const int32_t* seq_ctx, const int32_t* tile_start,
                                    int n_seqs, int n_tiles, int n_tokens, int n_heads, int n_kv_heads, int head_dim,
                                    int page_tokens, int window, float scale, int tokens_per_tile, int q_tiles,
-                                   int form, int n_splits, int single_rows, const int32_t* row_seq, void* stream) {
+                                   int form, int n_splits, int min_walk, int single_rows, const int32_t* row_seq, void* stream) {
   BC4G_REQUIRE(n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0, "attention_mfma: bad heads %d/%d",
                n_heads, n_kv_heads);
   BC4G_REQUIRE(head_dim >= 16 && head_dim <= 256 && head_dim % 16 == 0,
@@ -672,6 +700,9 @@ extern "C" int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, flo
   BC4G_REQUIRE(n_splits >= 1 && n_splits <= kMaxSplits && (n_splits == 1 || (part_o && part_ml)),
                "attention_mfma: the split count %d must lie in 1..64", n_splits);
   BC4G_REQUIRE(window >= 0 && table_stride > 0 && n_seqs > 0, "attention_mfma: bad sizes");
+  BC4G_REQUIRE(min_walk >= 0 && (min_walk == 0 || (form != 1 && n_splits <= 8)),
+               "attention_mfma: a least walk (%d) goes with the prompt forms and at most 8 parts (form %d, %d parts)", min_walk,
+               form, n_splits);
   BC4G_REQUIRE(scale > 0.f, "attention_mfma: the softmax scale must be positive, got %g", static_cast<double>(scale));
   BC4G_REQUIRE(q_stride >= n_heads * head_dim && q_stride % 8 == 0, "attention_mfma: bad query row stride %d", q_stride);
   if (n_tiles == 0 || n_tokens == 0) return 0;
@@ -701,6 +732,7 @@ extern "C" int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, flo
   a.tpt = tokens_per_tile;
   a.n_sub = (group + a.hg - 1) / a.hg;
   a.n_splits = n_splits;
+  a.min_walk = min_walk;
   a.single_rows = single_rows ? 1 : 0;
   BC4G_REQUIRE(!single_rows || (form == 1 && n_tiles == n_seqs && n_tokens == n_seqs),
                "attention_mfma: single rows means one row and one tile a request in the decode form (%d requests, %d "
@@ -758,8 +790,13 @@ extern "C" int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, flo
     constexpr int kFew = 8;
     if (n_splits <= kFew) {
       const long items = rows_heads * (head_dim / 4);
-      attention_merge_few_kernel<kFew><<<static_cast<unsigned>((items + 255) / 256), 256, 0, s>>>(
-          part_o, part_ml, a.out, n_splits, rows_heads, head_dim, n_heads, row_seq, tile_start);
+      const unsigned blocks = static_cast<unsigned>((items + 255) / 256);
+      if (a.min_walk > 0 && form != 1)
+        attention_merge_few_kernel<kFew, true><<<blocks, 256, 0, s>>>(part_o, part_ml, a.out, n_splits, rows_heads, head_dim,
+                                                                     n_heads, row_seq, tile_start);
+      else
+        attention_merge_few_kernel<kFew, false><<<blocks, 256, 0, s>>>(part_o, part_ml, a.out, n_splits, rows_heads, head_dim,
+                                                                      n_heads, row_seq, tile_start);
     } else {
       attention_merge_kernel<<<static_cast<unsigned>(rows_heads), 64, 0, s>>>(part_o, part_ml, a.out, n_splits,
                                                                                rows_heads, head_dim, n_heads, row_seq,

@@ -610,8 +610,13 @@ def attention_q_tiles(head_dim: int) -> int:
 
 
 ATTENTION_MAX_SPLITS = 64
-ATTENTION_PROMPT_GROUPS = 512     # workgroups a prompt step should bring: the longest walks run first, and
-                                  # with two rounds of workgroups the short ones fill in behind them
+ATTENTION_PROMPT_GROUPS = 512     # workgroups a prompt step should bring if every walk were cut into the most parts
+ATTENTION_LONG_WALK = 16          # 32-key tiles from which on a prompt's longest walk is cut in two at least.
+                                  # Under the causal mask the walks differ in length; every walk is cut into parts
+                                  # of about the length of the longest walk's parts, the short ones into fewer
+                                  # (the kernel's min_walk), so that the workgroups are alike (measured, head size
+                                  # 64, attention and merge: 2,048 tokens 77 -> 69 us, 4,096 252 -> 212, 8,192
+                                  # 747 -> 597; head size 128: 8,192 tokens 1,113 -> 1,023)
 ATTENTION_MAX_PROMPT_SPLITS = 8
 ATTENTION_MIN_WALK = 4            # 32-key tiles a part of a prompt's keys should hold at least
 ATTENTION_APART_CONTEXT = 256     # cached tokens from which on a single-tile request beside prompt portions gets a
@@ -630,7 +635,8 @@ def attention_shared_waves(head_dim: int) -> int:
 def attention_splits(n_tiles: int, n_heads: int, n_kv_heads: int, max_kv_len: int, shared_waves: int = 0) -> int:
     """Into how many parts the keys are cut over workgroups so that the GPU has enough of them.
     n_tiles counts waves' tiles.  Prompt forms (four waves a workgroup): towards
-    ATTENTION_PROMPT_GROUPS workgroups, while a part keeps ATTENTION_MIN_WALK tiles of 32 keys.
+    ATTENTION_PROMPT_GROUPS workgroups, and two parts at least from ATTENTION_LONG_WALK tiles of 32 keys
+    on, while a part keeps ATTENTION_MIN_WALK tiles.
     With ``shared_waves`` a workgroup is one tile whose waves already cut the keys between them;
     the keys are cut further only while a wave would walk more than ATTENTION_SHARED_WALK tiles."""
     group = n_heads // n_kv_heads
@@ -641,8 +647,8 @@ def attention_splits(n_tiles: int, n_heads: int, n_kv_heads: int, max_kv_len: in
         return max(1, min(-(-walk // ATTENTION_SHARED_WALK), ATTENTION_ENOUGH_GROUPS // max(waves, 1),
                           ATTENTION_MAX_SPLITS))
     groups = max(1, -(-waves // ATTENTION_STAGED_WAVES))
-    return max(1, min(-(-ATTENTION_PROMPT_GROUPS // groups), ATTENTION_MAX_PROMPT_SPLITS,
-                      key_tiles // ATTENTION_MIN_WALK))
+    wanted = max(-(-ATTENTION_PROMPT_GROUPS // groups), 2 if key_tiles >= ATTENTION_LONG_WALK else 1)
+    return max(1, min(wanted, ATTENTION_MAX_PROMPT_SPLITS, key_tiles // ATTENTION_MIN_WALK))
 
 
 def attention_mfma(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
@@ -650,14 +656,16 @@ def attention_mfma(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
                    n_heads: int, n_kv_heads: int, head_dim: int, window: int, scale: float,
                    n_splits: int, q_tiles: int = 1, form: int = 0, work=None,
                    out: Optional[torch.Tensor] = None, row_seq: Optional[torch.Tensor] = None,
-                   single_rows: bool = False) -> torch.Tensor:
+                   single_rows: bool = False, min_walk: int = 0) -> torch.Tensor:
     """form 0: four independent waves a workgroup, tile_start counts pieces of q_tiles tiles; 1: one
     tile a workgroup, its waves share the keys (q_tiles 1); 2: four waves a workgroup that walk their
     keys together through LDS, tile_start counts pieces of 4 * q_tiles tiles (ATTENTION_STAGED_WAVES).
     Requests without pieces are left out; with ``out`` (the result of another launch over the other
     requests) and ``row_seq`` (each row's request) their rows of it stay as they are.
     ``single_rows`` (form 1): the caller knows that every request brings exactly one row (a decode
-    step), and the kernel then looks nothing up before it asks for the block table and the query."""
+    step), and the kernel then looks nothing up before it asks for the block table and the query.
+    ``min_walk`` (forms 0 and 2, up to 8 parts): a walk of n tiles of 32 keys is cut into
+    ceil(n / min_walk) parts, n_splits at most; the other parts of its rows stay empty."""
     _dev("attention_mfma", qkv, k_cache, v_cache, block_table, seq_start, seq_ctx, tile_start)
     t = qkv.shape[0]
     _check_queries("attention_mfma", qkv, n_heads, n_kv_heads, head_dim)
@@ -685,7 +693,7 @@ def attention_mfma(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
                  _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(seq_start), _ptr(seq_ctx),
                  _ptr(tile_start), n_seqs, n_tiles, t, n_heads, n_kv_heads, head_dim, k_cache.shape[2],
                  int(window), float(scale), attention_tile_tokens(n_heads, n_kv_heads), int(q_tiles),
-                 int(form), int(n_splits), 1 if single_rows else 0, _ptr(row_seq), _stream(), cost=work)
+                 int(form), int(n_splits), int(min_walk), 1 if single_rows else 0, _ptr(row_seq), _stream(), cost=work)
     return out
 
 
@@ -750,8 +758,10 @@ def attention(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, b
         q_tiles = attention_q_tiles(head_dim)
         apart = notes["apart"]
         n_splits = attention_splits(notes["n_tiles"] * ATTENTION_STAGED_WAVES, n_heads, n_kv_heads, ctx.max_kv_len)
+        # parts of about one length: the longest walk's, which is cut into all n_splits
+        min_walk = max(ATTENTION_MIN_WALK, -(-(-(-ctx.max_kv_len // 32)) // n_splits)) if n_splits > 1 else 0
         out = attention_mfma(*args, arrays["tiles"], notes["n_tiles"], *sizes, n_splits, q_tiles, 2, work=work,
-                             row_seq=ctx.row_seq if apart else None)
+                             row_seq=ctx.row_seq if apart else None, min_walk=min_walk)
         if apart:
             n_splits = attention_splits(notes["n_short"], n_heads, n_kv_heads, notes["longest_short"],
                                         attention_shared_waves(head_dim))

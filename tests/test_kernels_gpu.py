@@ -369,7 +369,7 @@ def test_attention_generic(ops, nh, nkv, d, page, window):
         close(got, plain_result(case, window), what=f"generic {dt}", **tol)
 
 
-def run_mfma(ops, case, window, n_splits, q_tiles=1, shared=False, staged=False):
+def run_mfma(ops, case, window, n_splits, q_tiles=1, shared=False, staged=False, min_walk=0):
     nh, nkv, d = case["nh"], case["nkv"], case["d"]
     tpt = ops.attention_tile_tokens(nh, nkv) * q_tiles * (ops.ATTENTION_STAGED_WAVES if staged else 1)
     starts = [0]
@@ -379,7 +379,28 @@ def run_mfma(ops, case, window, n_splits, q_tiles=1, shared=False, staged=False)
     kc, vc = ops.cache_from_plain(case["kc"], case["vc"])      # the layout the writers leave for these sizes
     return ops.attention_mfma(case["qkv"], kc, vc, case["table"], dev(case["seq_start"]),
                               dev(case["seq_ctx"]), dev(starts), starts[-1], nh, nkv, d, window,
-                              1.0 / math.sqrt(d), n_splits, q_tiles, 2 if staged else int(shared))
+                              1.0 / math.sqrt(d), n_splits, q_tiles, 2 if staged else int(shared), min_walk=min_walk)
+
+
+@pytest.mark.parametrize("nh,nkv,d,page", [(4, 2, 16, 16), (32, 4, 64, 64), (8, 1, 128, 16)])
+@pytest.mark.parametrize("window", [0, 40])
+@pytest.mark.parametrize("n_splits,min_walk", [(3, 1), (4, 2), (8, 2), (8, 5)])
+def test_attention_mfma_parts_of_a_least_length(ops, nh, nkv, d, page, window, n_splits, min_walk):
+    """Prompt forms with a least walk: a walk of n tiles of 32 keys is cut into ceil(n / min_walk) parts (here one
+    to five: contexts of 1 to 134 tokens), the other parts of its rows stay empty and leave no outputs.  The
+    partial outputs are allocated where a tensor of NaNs has just been freed, so a merge that read an empty
+    part's outputs would show."""
+    case = paged_case(SEQS, nh, nkv, d, page, torch.bfloat16, seed=5)
+    want = plain_result(case, window)
+    t = case["qkv"].shape[0]
+    for qt in sorted({1, ops.attention_q_tiles(d)}):
+        for staged in (False, True):
+            junk = torch.full((n_splits, t, nh, d), float("nan"), dtype=torch.float32, device=DEV)
+            del junk
+            got = run_mfma(ops, case, window, n_splits, qt, staged=staged, min_walk=min_walk)
+            close(got, want, rtol=2e-2, atol=2e-2, what=f"parts of at least {min_walk} tiles, {qt} tiles a wave, staged={staged}")
+    with pytest.raises(ops.KernelError):
+        run_mfma(ops, case, window, n_splits, shared=True, min_walk=min_walk)     # the decode form cuts every walk alike
 
 
 @pytest.mark.parametrize("nh,nkv,d,page", SHAPES)
