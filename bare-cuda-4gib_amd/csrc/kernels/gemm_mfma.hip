@@ -275,8 +275,11 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_staged_kernel(
 // 64 x 64 tile halve that: 512 x 2048 x 5632 48 -> 28 us), raising the waves' priority around the MFMAs, 128 x 64 parts for a wave with half the waves.
 //
 // A tile's rows lie in LDS without padding, BK * 2 bytes each; the 16-byte segment s of row r lies in
-// slot s ^ (r % 8) (rows of 128 bytes and more) of its row, so that the fragment reads of eight
-// consecutive rows cover all banks.  A wave-wide load covers 1024 / (BK * 2) rows; which segment a lane
+// slot s ^ key(r) of its row, key(r) = (r / 2) % 8 for rows of 128 bytes and r % 16 for rows of 256.  A
+// fragment read is served sixteen lanes (rows r .. r + 15, one segment) at a time from 64 banks of
+// four bytes: two rows of 128 bytes share the banks' span, so the eight rows of one parity must lie
+// in eight different slots (with r % 8 as the key rows r and r + 8 met in one bank: counted, half of
+// all LDS cycles were conflicts).  A wave-wide load covers 1024 / (BK * 2) rows; which segment a lane
 // brings follows from where its 16 bytes land.
 //
 // WM x WN waves take TM x TN MFMA blocks of 32 x 32 each.  An output element is added up over k in
@@ -305,6 +308,11 @@ __device__ inline void wait_for_stage(int later) {
     if (later >= MAX) wait_loads<PER * MAX>();
     else wait_for_stage<PER, MAX - 1>(later);
   }
+}
+
+template <int ROW_BYTES>
+__device__ inline int slot_key(int row) {
+  return ROW_BYTES == 128 ? (row >> 1) & 7 : row & 15;
 }
 
 template <int WM, int WN, int TM, int TN, int BK, int STAGES>
@@ -347,7 +355,7 @@ __global__ __launch_bounds__(64 * WM * WN, MINWG) void gemm_mfma_direct_kernel(
     if (g >= GA + GW) g = GA + GW - 1;
     const bool of_a = g < GA;
     const int trow = (of_a ? g : g - GA) * kGroupRows + lr;
-    const int seg = ls ^ (trow & 7);
+    const int seg = ls ^ slot_key<RB>(trow);
     long row = (of_a ? m0 : n0) + trow;
     const long last = (of_a ? m : n) - 1;
     if (row > last) row = last;
@@ -380,13 +388,13 @@ __global__ __launch_bounds__(64 * WM * WN, MINWG) void gemm_mfma_direct_kernel(
   for (int i = 0; i < TM; ++i) {
     const int r = (wm * TM + i) * 32 + frow;
     aoff[i] = r * RB;
-    aswz[i] = r & 7;
+    aswz[i] = slot_key<RB>(r);
   }
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
     const int r = (wn * TN + j) * 32 + frow;
     woff[j] = RA * RB + r * RB;
-    wswz[j] = r & 7;
+    wswz[j] = slot_key<RB>(r);
   }
   constexpr int kSlices = BK / 16;
   uint4 fa[2][TM], fw[2][TN];
