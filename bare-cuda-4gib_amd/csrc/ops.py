@@ -352,14 +352,21 @@ def _weight(w):
 
 SKINNY_MAX_ROWS = 64
 SKINNY_PASSES_ROWS = 128            # up to here the weights are streamed once per 64 rows rather than tiled, unless
-SKINNY_PASSES_MAX_N = 8192          # the output is at least this wide: with one or two rows of tiles a product is as
-                                    # long as its chain of k-steps, which the streaming kernel's eight waves cut
-                                    # into eight (measured at 128 rows: 2048 x 5632 20 against 27 us tiled, 4096 x
-                                    # 14336 66 against 64; but 11264 x 2048 34 against 16, 28672 x 4096 122 against 46)
+SKINNY_PASSES_MAX_N = 8192          # the output is at least this wide, and then only below SKINNY_WIDE_ROWS rows.
+SKINNY_WIDE_ROWS = 32               # With one or two rows of tiles a product is as long as its chain of k-steps,
+                                    # which the streaming kernel's eight waves cut into eight -- but a wide output
+                                    # has tiles enough for every CU (64 x 64 ones, four stages), while every one of
+                                    # the streaming kernel's many workgroups reads all the rows of x (measured,
+                                    # streamed against tiled, us: 128 rows 2048 x 5632 20 / 27, 4096 x 14336 66 / 64;
+                                    # 64 rows 11264 x 2048 16.9 / 12.3, 28672 x 4096 59 / 37, 32000 x 2048 37 / 22,
+                                    # 6144 x 4096 19.4 / 19.6; 32 rows 11264 x 2048 12.7 / 12.4; 16 rows 9.3 / 12.2)
 
 
-def _in_passes(m: int, n: int) -> bool:
-    return m <= SKINNY_MAX_ROWS or (m <= SKINNY_PASSES_ROWS and n < SKINNY_PASSES_MAX_N)
+def streams_weights(m: int, n: int, k: int) -> bool:
+    """Whether the weight-streaming kernel takes a product of m rows, n outputs and this k."""
+    if k % 64 or n < SKINNY_PASSES_MAX_N:       # (the tiled kernel's small tiles need k in steps of 64)
+        return m <= SKINNY_PASSES_ROWS
+    return m < SKINNY_WIDE_ROWS
 
 
 EPI_STORE_BF16, EPI_STORE_F32, EPI_ACCUM_F32, EPI_SWIGLU = 0, 1, 2, 3
@@ -374,8 +381,8 @@ def gemm_fast(a: torch.Tensor, w, out_dtype=None,
               accumulate_into: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
     """The matrix-core product where a kernel takes these operands (bfloat16, k a multiple of
     8), else None (the caller then uses the plain float kernel).  Up to 64 rows the weights
-    are streamed once (a decode step), up to 128 once per 64 rows unless the output is wide; beyond
-    that the tiled kernel runs."""
+    are streamed once (a decode step), up to 128 once per 64 rows; a wide output goes to the tiled
+    kernel from 32 rows on, everything from 129."""
     w, packed = _weight(w)
     if not _fast_operands(a, w):
         return None
@@ -393,7 +400,7 @@ def gemm_fast(a: torch.Tensor, w, out_dtype=None,
         out = torch.empty((m, n), dtype=out_dtype, device=a.device)
         epi = EPI_STORE_BF16 if out_dtype == torch.bfloat16 else EPI_STORE_F32
     out_bytes = 8 if accumulate_into is not None else out.element_size()
-    if _in_passes(m, n):
+    if streams_weights(m, n, k):
         packed = packed if packed is not None else pack_weight(w)      # (packing per call: tests only)
         for r0 in range(0, m, SKINNY_MAX_ROWS):                        # the weights once for every 64 rows
             rows = min(SKINNY_MAX_ROWS, m - r0)
@@ -462,7 +469,7 @@ def gemm_swiglu(a: torch.Tensor, w_gate_up, interleaved: bool = False) -> torch.
         m, k = a.shape
         n = rows.shape[0]
         out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=a.device)
-        if _in_passes(m, n):
+        if streams_weights(m, n, k):
             packed = packed if packed is not None else pack_weight(rows)
             for r0 in range(0, m, SKINNY_MAX_ROWS):
                 part = min(SKINNY_MAX_ROWS, m - r0)
@@ -490,9 +497,9 @@ class Prenormed:
 
 def gemm_emit_supported(a: torch.Tensor, w, residual: torch.Tensor, g: torch.Tensor) -> bool:
     """Whether the adding product of these operands can prepare the next RMSNorm: the
-    weight-streaming kernel serves it (bfloat16, few rows: _in_passes)."""
+    weight-streaming kernel serves it (bfloat16, few rows: streams_weights)."""
     w, _ = _weight(w)
-    return (_fast_operands(a, w) and 0 < a.shape[0] and _in_passes(a.shape[0], w.shape[0]) and residual.dtype == torch.float32
+    return (_fast_operands(a, w) and 0 < a.shape[0] and streams_weights(a.shape[0], w.shape[0], w.shape[1]) and residual.dtype == torch.float32
             and g.dtype in _CODE and tuple(g.shape) == (w.shape[0],))
 
 
@@ -519,7 +526,7 @@ def gemm_accumulate_emit(a: torch.Tensor, w, residual: torch.Tensor, g: torch.Te
 
 def gemm_prenormed_supported(pre: Prenormed, w) -> bool:
     w, _ = _weight(w)
-    return _fast_operands(pre.xb, w) and _in_passes(pre.xb.shape[0], w.shape[0])
+    return _fast_operands(pre.xb, w) and streams_weights(pre.xb.shape[0], w.shape[0], w.shape[1])
 
 
 def gemm_prenormed(pre: Prenormed, w, epilogue: int) -> torch.Tensor:

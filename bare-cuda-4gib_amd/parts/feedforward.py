@@ -52,7 +52,10 @@ class SwiGLU(Part):
         fused norm is out of reach and the choice is a norm kernel of its own: that is the faster way
         up to 63 rows, because every workgroup of the product has to add up the prepared parts (1.085
         against 1.072 ms at 16 rows, 1.269 against 1.252 at 32, 1.558 against 1.565 at 64)."""
-        return self.interleaved and (5 <= n_rows <= ops.NORMED_MAX_ROWS or n_rows >= 64)
+        if not self.interleaved:
+            return False
+        # (a wide gate-up product of 32 rows and more goes to the tiled kernel, which reads a finished norm)
+        return 5 <= n_rows <= ops.NORMED_MAX_ROWS or (n_rows >= 64 and ops.streams_weights(n_rows, *self.w_gu.shape))
 
     def forward(self, h, ctx, residual) -> None:
         act = linear_swiglu(h, self.w_gu, self.interleaved)
