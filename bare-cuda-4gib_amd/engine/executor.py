@@ -109,9 +109,13 @@ class Executor:
             n = len(e.tokens)
             if n == 0:
                 raise EngineError(f"step: request {e.request!r} brings no tokens")
-            for t in e.tokens:
-                if not (0 <= int(t) < vocab):
-                    raise EngineError(f"step: token id {t} of request {e.request!r} is outside [0, {vocab})")
+            if n <= 8:
+                bad = [t for t in e.tokens if not (0 <= int(t) < vocab)]
+            else:                                       # (a prompt portion: looked at as one array)
+                ids = np.asarray(e.tokens, dtype=np.int64)
+                bad = ids[(ids < 0) | (ids >= vocab)]
+            if len(bad):
+                raise EngineError(f"step: token id {bad[0]} of request {e.request!r} is outside [0, {vocab})")
             for w in e.want:
                 if not (0 <= int(w) < n):
                     raise EngineError(f"step: wanted place {w} of request {e.request!r} is outside its {n} tokens")
@@ -122,28 +126,32 @@ class Executor:
 
     def _host_arrays(self, entries: Sequence[StepEntry], table_width: int = 0, all_logits: bool = False,
                      max_kv_bound: int = 0):
-        """The batch as one flat list of int32 and the layout of its parts.  ``table_width`` 0
+        """The batch as one flat int32 array and the layout of its parts.  ``table_width`` 0
         makes block tables as wide as the batch needs; ``all_logits`` asks for every row;
         ``max_kv_bound`` (a step about to be captured): the context bound the parts are to plan for."""
         cache, P = self.cache, self.cache.page_tokens
-        token_ids: List[int] = []
-        positions: List[int] = []
-        row_seq: List[int] = []
-        seq_start, seq_ctx, seq_slots, logit_rows = [0], [], [], []
+        i32 = np.int32
+        token_ids, positions, row_seq, logit_rows = [], [], [], []
+        seq_start, seq_ctx, seq_slots = [0], [], []
         max_q = max_kv = 0
-        for s, e in enumerate(entries):
+        for s, e in enumerate(entries):                 # (whole arrays per request: no Python loop over tokens)
             n, ctx_len = len(e.tokens), cache.length(e.request)
             base = seq_start[-1]
-            token_ids.extend(int(t) for t in e.tokens)
-            positions.extend(range(ctx_len, ctx_len + n))
-            row_seq.extend([s] * n)
+            token_ids.append(np.asarray(e.tokens, dtype=np.int64).astype(i32))
+            positions.append(np.arange(ctx_len, ctx_len + n, dtype=i32))
+            row_seq.append(np.full(n, s, dtype=i32))
             seq_start.append(base + n)
             seq_ctx.append(ctx_len)
             seq_slots.append(cache.slot(e.request))
-            logit_rows.extend(range(base, base + n) if all_logits else (base + int(w) for w in e.want))
+            logit_rows.append(np.arange(base, base + n, dtype=i32) if all_logits
+                              else base + np.asarray(e.want, dtype=np.int64).astype(i32))
             max_q, max_kv = max(max_q, n), max(max_kv, ctx_len + n)
-        T, S = len(token_ids), len(entries)
-        flat = token_ids + positions + row_seq + seq_start + seq_ctx + seq_slots + logit_rows
+        T, S = seq_start[-1], len(entries)
+        empty = np.zeros(0, dtype=i32)
+        logit_rows = np.concatenate(logit_rows) if logit_rows else empty
+        chunks = [np.concatenate(token_ids) if token_ids else empty, np.concatenate(positions) if positions else empty,
+                  np.concatenate(row_seq) if row_seq else empty, np.asarray(seq_start, dtype=i32),
+                  np.asarray(seq_ctx, dtype=i32), np.asarray(seq_slots, dtype=i32), logit_rows]
         layout = [("token_ids", T), ("positions", T), ("row_seq", T), ("seq_start", S + 1), ("seq_ctx", S),
                   ("seq_slots", S), ("logit_rows", len(logit_rows))]
         batch = HostBatch(n_tokens=T, n_seqs=S, seq_start=seq_start, seq_ctx=seq_ctx, seq_slots=seq_slots,
@@ -152,22 +160,22 @@ class Executor:
         for sig, part in self._preparers.items():
             arrays, notes[sig] = part.prepare_step(batch)
             for name, values in arrays.items():
-                flat.extend(values)
+                chunks.append(np.asarray(values, dtype=i32).reshape(-1))
                 layout.append(((sig, name), len(values)))
         group_layout = []
         for g in cache.groups:
-            tables = [cache.table(g, e.request) for e in entries]
+            tables = [np.asarray(cache.table(g, e.request), dtype=i32) for e in entries]
             width = table_width or max(1, max(len(t) for t in tables))
-            for t in tables:
-                flat.extend(t)
-                flat.extend([-1] * (width - len(t)))
-            for e, t in zip(entries, tables):
-                ctx_len = cache.length(e.request)
-                flat.extend(t[p // P] * P + p % P for p in range(ctx_len, ctx_len + len(e.tokens)))
+            padded = np.full((S, width), -1, dtype=i32)
+            for row, t in zip(padded, tables):
+                row[:len(t)] = t
+            chunks.append(padded.reshape(-1))
+            for e, t, where in zip(entries, tables, positions):       # where every new token's key and value go
+                chunks.append(t[where // P] * P + where % P if len(where) else empty)
             group_layout.append((g, width))
         host = dict(seq_start=seq_start, seq_ctx=seq_ctx, seq_slots=seq_slots, n_logits=len(logit_rows),
                     max_q=max_q, max_kv=max_kv_bound or max_kv, notes=notes, T=T, S=S, captured=bool(max_kv_bound))
-        return flat, layout, group_layout, host
+        return np.concatenate(chunks), layout, group_layout, host
 
     def _context_from(self, dev: torch.Tensor, layout, group_layout, host) -> StepContext:
         off = 0
@@ -197,7 +205,7 @@ class Executor:
     def build_context(self, entries: Sequence[StepEntry]) -> StepContext:
         """Host arrays of the batch, uploaded in one copy."""
         flat, layout, group_layout, host = self._host_arrays(entries)
-        dev = torch.tensor(flat, dtype=torch.int32).to(self.rt.device, non_blocking=True)
+        dev = torch.from_numpy(flat).to(self.rt.device, non_blocking=True)
         return self._context_from(dev, layout, group_layout, host)
 
     # ---- decode steps as captured graphs ------------------------------------------
@@ -265,7 +273,7 @@ class Executor:
         S = key[0]
         while len(self._graphs) >= self.MAX_GRAPHS:  # the graph used longest ago makes room (its memory goes with it)
             self._graphs.popitem(last=False)
-        dev = torch.tensor(flat, dtype=torch.int32).to(self.rt.device)
+        dev = torch.from_numpy(flat).to(self.rt.device)
         # Whatever the parts derive from the context is derived from the bucket's bound (host["max_kv"]), so
         # the launch geometry frozen into the graph holds for every context of the bucket.
         for part in self._capture_parts:

@@ -200,7 +200,7 @@ def test_decode_step_description_from_the_arrays_by_slot(folders):
         order = [r for r in ("e", "a", "f", "d", "c") if not (r == "d" and step % 3 == 0)]
         entries = [StepEntry(r, [(7 * step + j) % vocab], [0]) for j, r in enumerate(order)]
         ex.cache.reserve([(e.request, 1) for e in entries])
-        want = ex._host_arrays(entries, table_width=width, all_logits=True)[0]
+        want = ex._host_arrays(entries, table_width=width, all_logits=True)[0].tolist()
         ex.step(entries)
         used = [slot for slot in ex._graphs.values() if slot["next"] and len(slot["rows"]) == len(entries)]
         latest = [s["ring"][(s["next"] - 1) % len(s["ring"])][1].tolist() for s in used]
