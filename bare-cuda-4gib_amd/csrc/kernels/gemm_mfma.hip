@@ -413,13 +413,20 @@ __global__ __launch_bounds__(64 * WM * WN, MINWG) void gemm_mfma_direct_kernel(
     if (t + STAGES - 1 < nk) ask(t + STAGES - 1);
     const unsigned char* stage = direct_lds + (t % STAGES) * S::kStageBytes;
     read_fragments(0, stage, 0);
+    __builtin_amdgcn_sched_group_barrier(0x100, TM + TN, 0);
 #pragma unroll
     for (int ks = 0; ks < kSlices; ++ks) {
-      if (ks + 1 < kSlices) read_fragments((ks + 1) % 2, stage, ks + 1);   // asked for before this slice's MFMAs
+      // the next slice's fragments are asked for before this slice's MFMAs, which hide the wait (the
+      // order is pinned: left alone, the compiler moves the reads down to where their registers come free)
+      if (ks + 1 < kSlices) {
+        read_fragments((ks + 1) % 2, stage, ks + 1);
+        __builtin_amdgcn_sched_group_barrier(0x100, TM + TN, 0);
+      }
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j) acc[i][j] = mfma_32x32x16(fa[ks % 2][i], fw[ks % 2][j], acc[i][j]);
+      __builtin_amdgcn_sched_group_barrier(0x008, TM * TN, 0);
     }
   }
   lds_barrier();            // the last step has been read: LDS is free for the output
