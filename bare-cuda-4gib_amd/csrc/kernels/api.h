@@ -126,6 +126,10 @@ extern "C" {
 // merges into out.  A request without pieces (tile_start[s + 1] == tile_start[s]) is left out: its
 // rows of out are not written, provided row_seq ([T]: each row's request) is given for the merge
 // to see which rows those are -- so two launches of different forms can share one out.
+// items (form 2): a work list instead of the grid's own order -- n_items entries, piece | part << 20 | parts << 24, in
+// the order in which the workgroups are to start (the host puts the longest walks first and cuts a piece's keys
+// into as many parts as balances the walks); row_parts [T] then says for every row into how many parts its keys
+// were cut (rows with one part are written at once and left alone by the merge).
 // single_rows (form 1): every request brings exactly one row, so request s is tile s and row s and the
 // kernel looks nothing up before it asks for the block table and the query (a decode step).
 int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, float* part_o, float* part_ml, const void* k_cache,
@@ -133,7 +137,8 @@ int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, float* part_o,
                         const int32_t* seq_start, const int32_t* seq_ctx, const int32_t* tile_start,
                         int n_seqs, int n_tiles, int n_tokens, int n_heads, int n_kv_heads, int head_dim,
                         int page_tokens, int window, float scale, int tokens_per_tile, int q_tiles,
-                        int form, int n_splits, int min_walk, int single_rows, const int32_t* row_seq, void* stream);
+                        int form, int n_splits, const int32_t* items, int n_items, const int32_t* row_parts,
+                        int single_rows, const int32_t* row_seq, void* stream);
 }
 
 extern "C" {

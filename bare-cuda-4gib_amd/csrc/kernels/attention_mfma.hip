@@ -99,7 +99,9 @@ struct AttnArgs {
   int n_heads, n_kv_heads, head_dim, page_tokens, window;
   int hg, tpt, n_sub;          // heads per tile, tokens per tile, head sub-groups per kv head
   int n_splits;
-  int min_walk;                // prompt forms: 32-key tiles a part of a walk holds at least (0: every walk in n_splits parts)
+  const int32_t* items;        // prompt form with a work list: workgroup y takes piece items[y] % 2^20, part (items[y] >> 20) % 16 of
+                               // items[y] >> 24 parts of that piece's keys (nullptr: the grid's x is the piece, z the part of n_splits)
+  const int32_t* row_parts;    // with items: into how many parts each row's keys were cut ([T]; 1: the row is written as it is)
   int single_rows;             // every request brings exactly one row (a decode step): request s is tile s and row s
   float scale_log2;            // softmax scale times log2(e)
 };
@@ -121,14 +123,18 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, 2) void att
   const int lane = threadIdx.x % kWave;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int col = lane % 16, grp = lane / 16;
-  // what tile_start counts: a wave's tiles (WS == 1), or a workgroup's (one tile, or four waves' tiles)
-  // (prompt forms: the last workgroups first -- under the causal mask a request's last rows walk
-  // the most keys, and the longest walks should not be the ones that start last -- in every other
-  // (head, part of the keys), and the first ones first in those between: workgroups that are a grid's
-  // x extent apart tend to share a CU, and so a long walk meets a short one there; measured, a
-  // 2,048-token prompt with head size 64: 82 -> 68 us)
+  // what tile_start counts: a wave's tiles (WS == 1), or a workgroup's (one tile, or four waves' tiles).
+  // Prompt forms without a work list: the last workgroups first -- under the causal mask a request's last
+  // rows walk the most keys, and the longest walks should not be the ones that start last -- in every
+  // other (head, part of the keys), and the first ones first in those between: workgroups that are a
+  // grid's x extent apart tend to share a CU, and so a long walk meets a short one there.
+  // With a work list the host has put the longest walks first and says which piece and part this is.
+  const bool listed = kStaged && a.items != nullptr;
+  const int item = listed ? a.items[blockIdx.y] : 0;
+  const int head_block = listed ? blockIdx.x : blockIdx.y;
+  const int part = listed ? (item >> 20) & 15 : blockIdx.z;
   const bool last_first = ((blockIdx.y + blockIdx.z) & 1) == 0;
-  const int block_x = (WS > 1 || !last_first) ? blockIdx.x : gridDim.x - 1 - blockIdx.x;
+  const int block_x = listed ? (item & 0xfffff) : ((WS > 1 || !last_first) ? blockIdx.x : gridDim.x - 1 - blockIdx.x);
   const int tile = WS == 1 ? block_x * kWavesPerBlock + wave : block_x;
   if (WS == 1 && tile >= a.n_tiles) return;   // (waves are independent there: no barrier below)
 
@@ -166,7 +172,7 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, 2) void att
   const int tok0_wg = (tile - tile0) * a.tpt * QT * (kStaged ? kWavesPerBlock : 1);
   const int tok0 = tok0_wg + (kStaged ? wave * a.tpt * QT : 0);
   const int ntok = max(0, min(a.tpt * QT, q_len - tok0));     // (0: a wave past the request's rows)
-  const int kvh = blockIdx.y / a.n_sub, hsub = blockIdx.y % a.n_sub;
+  const int kvh = head_block / a.n_sub, hsub = head_block % a.n_sub;
   const int group = a.n_heads / a.n_kv_heads;
   const int d = EXACT ? 16 * DB : a.head_dim, P = a.page_tokens;
   const int32_t* table = a.block_table + static_cast<long>(s) * a.table_stride;
@@ -202,14 +208,11 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, 2) void att
   const int lo_min = (a.window > 0 && walk_min - a.window + 1 > 0) ? walk_min - a.window + 1 : 0;
   const int kt_first = lo_min / 32, kt_last = walk_max / 32;
   const int n_kt = kt_last - kt_first + 1;
-  // Into how many parts this walk is cut: all of them, or (prompt forms with min_walk) as many as keep
-  // min_walk tiles each -- under the causal mask the walks differ in length, and parts of about one
-  // length each, few for the short walks and n_splits for the longest, keep the workgroups alike.  The
-  // parts beyond those are empty: they leave their statistics (no keys) and nothing else.
-  int n_parts = a.n_splits * (WS > 1 ? WS : 1);
-  if (WS <= 1 && a.min_walk > 0) n_parts = max(1, min(n_parts, (n_kt + a.min_walk - 1) / a.min_walk));
+  // Into how many parts this walk is cut: n_splits (times the waves that share a tile's keys), or what
+  // the work list says for this piece.
+  const int n_parts = listed ? (item >> 24) : a.n_splits * (WS > 1 ? WS : 1);
   const int per_split = (n_kt + n_parts - 1) / n_parts;
-  const int kt_begin = kt_first + (blockIdx.z * (WS > 1 ? WS : 1) + (WS > 1 ? wave : 0)) * per_split;
+  const int kt_begin = kt_first + (part * (WS > 1 ? WS : 1) + (WS > 1 ? wave : 0)) * per_split;
   const int kt_end = min(kt_last + 1, kt_begin + per_split);
   // kStaged: the tiles of the walk that hold keys of this wave's rows
   const int own_lo = (a.window > 0 && pos_min - a.window + 1 > 0) ? pos_min - a.window + 1 : 0;
@@ -517,7 +520,7 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, 2) void att
       if (a.n_splits == 1) {
         a.out[(row * a.n_heads + head) * d + c] = from_float<bf16_t>(acc / l);
       } else {
-        const long slot = (static_cast<long>(blockIdx.z) * a.n_tokens + row) * a.n_heads + head;
+        const long slot = (static_cast<long>(part) * a.n_tokens + row) * a.n_heads + head;
         a.part_o[slot * d + c] = acc;
         if (c == 0) {
           a.part_ml[slot * 2] = m;
@@ -533,7 +536,7 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, 2) void att
     const float l_tot = sum_16_32(l_run[t]);
     if (!q_ok[t]) continue;
     const long row = row0 + tok0 + q_tok[t];
-    if (a.n_splits == 1) {
+    if (a.n_splits == 1 || (listed && n_parts == 1)) {      // (a walk that was not cut: nothing to merge)
       const float inv = 1.0f / l_tot;
       bf16_t* dst = a.out + (row * a.n_heads + q_head) * d + 4 * grp;
 #pragma unroll
@@ -545,14 +548,12 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, 2) void att
         *reinterpret_cast<uint2*>(dst + 16 * b) = pack;
       }
     } else {
-      const long slot = (static_cast<long>(blockIdx.z) * a.n_tokens + row) * a.n_heads + q_head;
+      const long slot = (static_cast<long>(part) * a.n_tokens + row) * a.n_heads + q_head;
       float* dst = a.part_o + slot * d + 4 * grp;
-      if (a.min_walk == 0 || kt_begin < kt_end) {   // (an empty part of a walk with a least length: the merge does not look at its outputs)
 #pragma unroll
-        for (int b = 0; b < DB; ++b) {
-          if (!EXACT && 16 * b >= d) break;
-          *reinterpret_cast<floatx4*>(dst + 16 * b) = o[t][b];
-        }
+      for (int b = 0; b < DB; ++b) {
+        if (!EXACT && 16 * b >= d) break;
+        *reinterpret_cast<floatx4*>(dst + 16 * b) = o[t][b];
       }
       if (grp == 0) {
         a.part_ml[slot * 2] = m_run[t] * a.scale_log2;
@@ -618,15 +619,16 @@ __global__ __launch_bounds__(kWave) void attention_merge_kernel(const float* __r
 // short contexts into few): a thread takes four neighbouring output dimensions of one (row, head),
 // asks for every part's statistics and outputs at once -- one trip to memory, no LDS, no barrier --
 // and adds the parts in order of z.
-// SKIP: parts without keys (statistics -inf) may have left no outputs: those are not read (the
-// statistics first, then the outputs of the parts that have any).
-template <int MAXS, bool SKIP>
+// row_parts (with a work list): how many parts row t's keys were cut into; a row with one part has been
+// written by the attention kernel and is left alone.
+template <int MAXS>
 __global__ __launch_bounds__(256) void attention_merge_few_kernel(const float* __restrict__ part_o,
                                                                   const float* __restrict__ part_ml,
                                                                   bf16_t* __restrict__ out, int n_splits,
                                                                   long n_rows_heads, int d, int n_heads,
                                                                   const int32_t* __restrict__ row_seq,
-                                                                  const int32_t* __restrict__ tile_start) {
+                                                                  const int32_t* __restrict__ tile_start,
+                                                                  const int32_t* __restrict__ row_parts) {
   const long item = blockIdx.x * 256L + threadIdx.x;
   const int per = d / 4;
   const long rh = item / per;
@@ -636,20 +638,17 @@ __global__ __launch_bounds__(256) void attention_merge_few_kernel(const float* _
     const int s = row_seq[rh / n_heads];
     if (tile_start[s + 1] == tile_start[s]) return;
   }
+  if (row_parts != nullptr) {
+    n_splits = row_parts[rh / n_heads];
+    if (n_splits <= 1) return;
+  }
   float2 ml[MAXS];
   floatx4 o[MAXS];
 #pragma unroll
   for (int z = 0; z < MAXS; ++z) {
     const bool live = z < n_splits;
     ml[z] = live ? *reinterpret_cast<const float2*>(part_ml + (z * n_rows_heads + rh) * 2) : make_float2(-INFINITY, 0.f);
-    if constexpr (!SKIP)
-      o[z] = live ? *reinterpret_cast<const floatx4*>(part_o + (z * n_rows_heads + rh) * d + c) : floatx4{0.f, 0.f, 0.f, 0.f};
-  }
-  if constexpr (SKIP) {
-#pragma unroll
-    for (int z = 0; z < MAXS; ++z)
-      o[z] = (z < n_splits && ml[z].x != -INFINITY) ? *reinterpret_cast<const floatx4*>(part_o + (z * n_rows_heads + rh) * d + c)
-                                                    : floatx4{0.f, 0.f, 0.f, 0.f};
+    o[z] = live ? *reinterpret_cast<const floatx4*>(part_o + (z * n_rows_heads + rh) * d + c) : floatx4{0.f, 0.f, 0.f, 0.f};
   }
   float m = -INFINITY;
 #pragma unroll
@@ -690,7 +689,8 @@ extern "C" int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, flo
                                    const int32_t* seq_start, const int32_t* seq_ctx, const int32_t* tile_start,
                                    int n_seqs, int n_tiles, int n_tokens, int n_heads, int n_kv_heads, int head_dim,
                                    int page_tokens, int window, float scale, int tokens_per_tile, int q_tiles,
-                                   int form, int n_splits, int min_walk, int single_rows, const int32_t* row_seq, void* stream) {
+                                   int form, int n_splits, const int32_t* items, int n_items, const int32_t* row_parts,
+                                   int single_rows, const int32_t* row_seq, void* stream) {
   BC4G_REQUIRE(n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0, "attention_mfma: bad heads %d/%d",
                n_heads, n_kv_heads);
   BC4G_REQUIRE(head_dim >= 16 && head_dim <= 256 && head_dim % 16 == 0,
@@ -700,9 +700,10 @@ extern "C" int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, flo
   BC4G_REQUIRE(n_splits >= 1 && n_splits <= kMaxSplits && (n_splits == 1 || (part_o && part_ml)),
                "attention_mfma: the split count %d must lie in 1..64", n_splits);
   BC4G_REQUIRE(window >= 0 && table_stride > 0 && n_seqs > 0, "attention_mfma: bad sizes");
-  BC4G_REQUIRE(min_walk >= 0 && (min_walk == 0 || (form != 1 && n_splits <= 8)),
-               "attention_mfma: a least walk (%d) goes with the prompt forms and at most 8 parts (form %d, %d parts)", min_walk,
-               form, n_splits);
+  BC4G_REQUIRE(items == nullptr || (form == 2 && row_parts != nullptr && n_items > 0 && n_items <= 65535 && n_splits <= 8 &&
+                                    n_tiles < (1 << 20)),
+               "attention_mfma: a work list goes with the staged prompt form, the rows' part counts, at most 65535 items, "
+               "8 parts and 2^20 pieces (form %d, %d items, %d parts, %d pieces)", form, n_items, n_splits, n_tiles);
   BC4G_REQUIRE(scale > 0.f, "attention_mfma: the softmax scale must be positive, got %g", static_cast<double>(scale));
   BC4G_REQUIRE(q_stride >= n_heads * head_dim && q_stride % 8 == 0, "attention_mfma: bad query row stride %d", q_stride);
   if (n_tiles == 0 || n_tokens == 0) return 0;
@@ -732,7 +733,8 @@ extern "C" int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, flo
   a.tpt = tokens_per_tile;
   a.n_sub = (group + a.hg - 1) / a.hg;
   a.n_splits = n_splits;
-  a.min_walk = min_walk;
+  a.items = items;
+  a.row_parts = items ? row_parts : nullptr;
   a.single_rows = single_rows ? 1 : 0;
   BC4G_REQUIRE(!single_rows || (form == 1 && n_tiles == n_seqs && n_tokens == n_seqs),
                "attention_mfma: single rows means one row and one tile a request in the decode form (%d requests, %d "
@@ -751,7 +753,9 @@ extern "C" int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, flo
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (form == 2) {
     // four waves' tiles per workgroup (n_tiles counts workgroups), key tiles staged in LDS twice over
+    // (with a work list: heads fastest, so that the items start in the list's order, longest first)
     dim3 grid(n_tiles, n_kv_heads * a.n_sub, n_splits);
+    if (items) grid = dim3(n_kv_heads * a.n_sub, n_items, 1);
     dim3 block(kWavesPerBlock * kWave);
     const size_t lds = static_cast<size_t>(2) * 128 * head_dim;
     if (dj <= 2 && db <= 4) {
@@ -789,14 +793,9 @@ extern "C" int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, flo
     BC4G_REQUIRE(rows_heads <= 2147483647L, "attention_mfma: too many rows to merge");
     constexpr int kFew = 8;
     if (n_splits <= kFew) {
-      const long items = rows_heads * (head_dim / 4);
-      const unsigned blocks = static_cast<unsigned>((items + 255) / 256);
-      if (a.min_walk > 0 && form != 1)
-        attention_merge_few_kernel<kFew, true><<<blocks, 256, 0, s>>>(part_o, part_ml, a.out, n_splits, rows_heads, head_dim,
-                                                                     n_heads, row_seq, tile_start);
-      else
-        attention_merge_few_kernel<kFew, false><<<blocks, 256, 0, s>>>(part_o, part_ml, a.out, n_splits, rows_heads, head_dim,
-                                                                      n_heads, row_seq, tile_start);
+      const long work = rows_heads * (head_dim / 4);
+      attention_merge_few_kernel<kFew><<<static_cast<unsigned>((work + 255) / 256), 256, 0, s>>>(
+          part_o, part_ml, a.out, n_splits, rows_heads, head_dim, n_heads, row_seq, tile_start, a.row_parts);
     } else {
       attention_merge_kernel<<<static_cast<unsigned>(rows_heads), 64, 0, s>>>(part_o, part_ml, a.out, n_splits,
                                                                                rows_heads, head_dim, n_heads, row_seq,

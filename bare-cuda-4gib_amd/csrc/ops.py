@@ -617,13 +617,8 @@ def attention_q_tiles(head_dim: int) -> int:
 
 
 ATTENTION_MAX_SPLITS = 64
-ATTENTION_PROMPT_GROUPS = 512     # workgroups a prompt step should bring if every walk were cut into the most parts
-ATTENTION_LONG_WALK = 16          # 32-key tiles from which on a prompt's longest walk is cut in two at least.
-                                  # Under the causal mask the walks differ in length; every walk is cut into parts
-                                  # of about the length of the longest walk's parts, the short ones into fewer
-                                  # (the kernel's min_walk), so that the workgroups are alike (measured, head size
-                                  # 64, attention and merge: 2,048 tokens 77 -> 69 us, 4,096 252 -> 212, 8,192
-                                  # 747 -> 597; head size 128: 8,192 tokens 1,113 -> 1,023)
+ATTENTION_PROMPT_GROUPS = 512     # workgroups a prompt step should bring where the caller cuts every walk alike
+ATTENTION_SLOTS = 512             # workgroups of the prompt form the GPU holds at a time (two a CU: the kernel's registers)
 ATTENTION_MAX_PROMPT_SPLITS = 8
 ATTENTION_MIN_WALK = 4            # 32-key tiles a part of a prompt's keys should hold at least
 ATTENTION_APART_CONTEXT = 256     # cached tokens from which on a single-tile request beside prompt portions gets a
@@ -642,8 +637,8 @@ def attention_shared_waves(head_dim: int) -> int:
 def attention_splits(n_tiles: int, n_heads: int, n_kv_heads: int, max_kv_len: int, shared_waves: int = 0) -> int:
     """Into how many parts the keys are cut over workgroups so that the GPU has enough of them.
     n_tiles counts waves' tiles.  Prompt forms (four waves a workgroup): towards
-    ATTENTION_PROMPT_GROUPS workgroups, and two parts at least from ATTENTION_LONG_WALK tiles of 32 keys
-    on, while a part keeps ATTENTION_MIN_WALK tiles.
+    ATTENTION_PROMPT_GROUPS workgroups, while a part keeps ATTENTION_MIN_WALK tiles of 32 keys (the
+    engine's steps bring a work list instead: prompt_work_list).
     With ``shared_waves`` a workgroup is one tile whose waves already cut the keys between them;
     the keys are cut further only while a wave would walk more than ATTENTION_SHARED_WALK tiles."""
     group = n_heads // n_kv_heads
@@ -654,8 +649,8 @@ def attention_splits(n_tiles: int, n_heads: int, n_kv_heads: int, max_kv_len: in
         return max(1, min(-(-walk // ATTENTION_SHARED_WALK), ATTENTION_ENOUGH_GROUPS // max(waves, 1),
                           ATTENTION_MAX_SPLITS))
     groups = max(1, -(-waves // ATTENTION_STAGED_WAVES))
-    wanted = max(-(-ATTENTION_PROMPT_GROUPS // groups), 2 if key_tiles >= ATTENTION_LONG_WALK else 1)
-    return max(1, min(wanted, ATTENTION_MAX_PROMPT_SPLITS, key_tiles // ATTENTION_MIN_WALK))
+    return max(1, min(-(-ATTENTION_PROMPT_GROUPS // groups), ATTENTION_MAX_PROMPT_SPLITS,
+                      key_tiles // ATTENTION_MIN_WALK))
 
 
 def attention_mfma(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
@@ -663,7 +658,8 @@ def attention_mfma(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
                    n_heads: int, n_kv_heads: int, head_dim: int, window: int, scale: float,
                    n_splits: int, q_tiles: int = 1, form: int = 0, work=None,
                    out: Optional[torch.Tensor] = None, row_seq: Optional[torch.Tensor] = None,
-                   single_rows: bool = False, min_walk: int = 0) -> torch.Tensor:
+                   single_rows: bool = False, items: Optional[torch.Tensor] = None, n_items: int = 0,
+                   row_parts: Optional[torch.Tensor] = None) -> torch.Tensor:
     """form 0: four independent waves a workgroup, tile_start counts pieces of q_tiles tiles; 1: one
     tile a workgroup, its waves share the keys (q_tiles 1); 2: four waves a workgroup that walk their
     keys together through LDS, tile_start counts pieces of 4 * q_tiles tiles (ATTENTION_STAGED_WAVES).
@@ -671,8 +667,9 @@ def attention_mfma(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     requests) and ``row_seq`` (each row's request) their rows of it stay as they are.
     ``single_rows`` (form 1): the caller knows that every request brings exactly one row (a decode
     step), and the kernel then looks nothing up before it asks for the block table and the query.
-    ``min_walk`` (forms 0 and 2, up to 8 parts): a walk of n tiles of 32 keys is cut into
-    ceil(n / min_walk) parts, n_splits at most; the other parts of its rows stay empty."""
+    ``items`` (form 2; prompt_work_list): a work list of n_items workgroups in the order in which they
+    are to start, each a piece, a part and the number of parts of that piece's keys; ``row_parts`` [T]:
+    into how many parts each row's keys are cut; n_splits is then the most parts of any piece."""
     _dev("attention_mfma", qkv, k_cache, v_cache, block_table, seq_start, seq_ctx, tile_start)
     t = qkv.shape[0]
     _check_queries("attention_mfma", qkv, n_heads, n_kv_heads, head_dim)
@@ -692,6 +689,10 @@ def attention_mfma(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     if row_seq is not None:
         _dev("attention_mfma", row_seq)
         _i32("attention_mfma", "row_seq", row_seq, t)
+    if items is not None:
+        _dev("attention_mfma", items, row_parts)
+        _i32("attention_mfma", "items", items, n_items)
+        _i32("attention_mfma", "row_parts", row_parts, t)
     part_o = part_ml = None
     if n_splits > 1:
         part_o = torch.empty((n_splits, t, n_heads, head_dim), dtype=torch.float32, device=qkv.device)
@@ -700,14 +701,49 @@ def attention_mfma(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
                  _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(seq_start), _ptr(seq_ctx),
                  _ptr(tile_start), n_seqs, n_tiles, t, n_heads, n_kv_heads, head_dim, k_cache.shape[2],
                  int(window), float(scale), attention_tile_tokens(n_heads, n_kv_heads), int(q_tiles),
-                 int(form), int(n_splits), int(min_walk), 1 if single_rows else 0, _ptr(row_seq), _stream(), cost=work)
+                 int(form), int(n_splits), _ptr(items), int(n_items), _ptr(row_parts), 1 if single_rows else 0,
+                 _ptr(row_seq), _stream(), cost=work)
     return out
 
 
 _DECODE_TILE_STARTS: dict = {}
 
 
-def attention_plan(batch, n_heads: int, n_kv_heads: int, head_dim: int):
+def prompt_work_list(batch, piece_starts, piece: int, head_blocks: int, window: int):
+    """The prompt form's workgroups for a batch, in the order in which they should start, and into how many parts
+    each row's keys are cut: (packed items, parts per row, most parts).  ``piece_starts`` [S + 1]: the first piece
+    of every request (a piece = the ``piece`` consecutive rows a workgroup takes); ``head_blocks``: workgroups
+    that take the same piece for different heads.
+
+    Under the causal mask a piece's walk over the keys is as long as its position: walks of 1 to 64 tiles of
+    32 keys in a 2,048-token prompt.  A workgroup takes about as long as its walk (1.6-1.9 us a tile, with a
+    second workgroup beside it on the CU or without, plus 6 us before and after), and a CU holds two at a
+    time.  So the walks are cut into parts of at most a quarter more than an even share of all tiles per place
+    (eight parts at most: every part of a row leaves float partial outputs), and the list starts with the
+    longest: what is short fills in behind them (list scheduling).  Measured against every walk in two parts
+    in the grid's own order, attention and merge: head size 64, 2,048 tokens 69 -> 57 us, 4,096 212 -> 180, 8,192
+    (no walk cut, no merge) 597 -> 512; head size 128, 2,048 tokens 126 -> 98, 8,192 1,027 -> 890."""
+    start = batch.seq_start
+    pieces = []                                        # (tiles of 32 keys, piece, request, first row, rows)
+    for s in range(batch.n_seqs):
+        ctx0, new = batch.seq_ctx[s], start[s + 1] - start[s]
+        for j in range(piece_starts[s + 1] - piece_starts[s]):
+            first, last = ctx0 + j * piece, ctx0 + min(new, (j + 1) * piece) - 1
+            lo = max(0, first - window + 1) if window > 0 else 0
+            pieces.append((last // 32 - lo // 32 + 1, piece_starts[s] + j, start[s] + j * piece, min(new, (j + 1) * piece) - j * piece))
+    share = sum(p[0] for p in pieces) * head_blocks / ATTENTION_SLOTS
+    longest = max(ATTENTION_MIN_WALK, -(-5 * share // 4))
+    items, row_parts, most = [], [1] * batch.n_tokens, 1
+    for tiles, index, row, rows in pieces:
+        parts = int(max(1, min(ATTENTION_MAX_PROMPT_SPLITS, -(-tiles // longest))))
+        most = max(most, parts)
+        row_parts[row:row + rows] = [parts] * rows
+        items.extend((-(-tiles // parts), index | (z << 20) | (parts << 24)) for z in range(parts))
+    items.sort(key=lambda it: -it[0])
+    return [it[1] for it in items], row_parts, most
+
+
+def attention_plan(batch, n_heads: int, n_kv_heads: int, head_dim: int, window: int = 0):
     """What the matrix-core attention kernel needs to know about a batch before it is launched, worked
     out on the host when the batch is described (``batch``: the step's HostBatch): how every request's
     rows are cut into pieces.  Returns (int32 arrays to go up with the batch, notes for attention()).
@@ -737,6 +773,12 @@ def attention_plan(batch, n_heads: int, n_kv_heads: int, head_dim: int):
         short_starts.append(short_starts[-1] + (-(-new[s] // tpt) if apart and is_short else 0))
     arrays = {"tiles": long_starts}
     notes = dict(form="prompt", n_tiles=long_starts[-1], apart=apart)
+    if 0 < long_starts[-1] < (1 << 20):
+        group = n_heads // n_kv_heads
+        items, row_parts, most = prompt_work_list(batch, long_starts, piece, n_kv_heads * -(-group // 16), window)
+        if len(items) <= 65535:
+            arrays.update(items=items, row_parts=row_parts)
+            notes.update(n_items=len(items), most_parts=most)
     if apart:
         arrays["short_tiles"] = short_starts
         notes.update(n_short=short_starts[-1], longest_short=max(batch.seq_ctx[s] for s in short) + tpt)
@@ -764,11 +806,14 @@ def attention(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, b
                                   single_rows=ctx.max_q_len == 1 and ctx.n_tokens == ctx.n_seqs)
         q_tiles = attention_q_tiles(head_dim)
         apart = notes["apart"]
-        n_splits = attention_splits(notes["n_tiles"] * ATTENTION_STAGED_WAVES, n_heads, n_kv_heads, ctx.max_kv_len)
-        # parts of about one length: the longest walk's, which is cut into all n_splits
-        min_walk = max(ATTENTION_MIN_WALK, -(-(-(-ctx.max_kv_len // 32)) // n_splits)) if n_splits > 1 else 0
-        out = attention_mfma(*args, arrays["tiles"], notes["n_tiles"], *sizes, n_splits, q_tiles, 2, work=work,
-                             row_seq=ctx.row_seq if apart else None, min_walk=min_walk)
+        if "items" in arrays:       # the pieces' parts in the order the host chose, longest walks first
+            out = attention_mfma(*args, arrays["tiles"], notes["n_tiles"], *sizes, notes["most_parts"], q_tiles, 2, work=work,
+                                 row_seq=ctx.row_seq if apart else None, items=arrays["items"], n_items=notes["n_items"],
+                                 row_parts=arrays["row_parts"])
+        else:
+            n_splits = attention_splits(notes["n_tiles"] * ATTENTION_STAGED_WAVES, n_heads, n_kv_heads, ctx.max_kv_len)
+            out = attention_mfma(*args, arrays["tiles"], notes["n_tiles"], *sizes, n_splits, q_tiles, 2, work=work,
+                                 row_seq=ctx.row_seq if apart else None)
         if apart:
             n_splits = attention_splits(notes["n_short"], n_heads, n_kv_heads, notes["longest_short"],
                                         attention_shared_waves(head_dim))

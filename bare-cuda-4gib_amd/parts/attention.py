@@ -51,16 +51,16 @@ class CausalAttention(Part):
 
     @property
     def step_signature(self):
-        """Attention parts of the same head counts and head size cut a batch alike: one preparation
-        a step serves them all."""
-        return ("attention", self.num_heads, self.num_kv_heads, self.head_dim)
+        """Attention parts of the same head counts, head size and window cut a batch alike: one
+        preparation a step serves them all."""
+        return ("attention", self.num_heads, self.num_kv_heads, self.head_dim, self.window)
 
     def prepare_step(self, batch):
         """How the matrix-core kernel will cut this batch's rows into pieces (nothing where the plain
         kernel serves): arrays that go up with the batch, and notes for forward()."""
         if getattr(self, "act_dtype", None) != torch.bfloat16 or self.head_dim % 16 or self.head_dim > 256:
             return {}, None
-        return ops.attention_plan(batch, self.num_heads, self.num_kv_heads, self.head_dim)
+        return ops.attention_plan(batch, self.num_heads, self.num_kv_heads, self.head_dim, self.window)
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
         q, kv, h = self.num_heads * self.head_dim, self.num_kv_heads * self.head_dim, self.hidden_size

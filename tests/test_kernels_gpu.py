@@ -369,7 +369,7 @@ def test_attention_generic(ops, nh, nkv, d, page, window):
         close(got, plain_result(case, window), what=f"generic {dt}", **tol)
 
 
-def run_mfma(ops, case, window, n_splits, q_tiles=1, shared=False, staged=False, min_walk=0):
+def run_mfma(ops, case, window, n_splits, q_tiles=1, shared=False, staged=False):
     nh, nkv, d = case["nh"], case["nkv"], case["d"]
     tpt = ops.attention_tile_tokens(nh, nkv) * q_tiles * (ops.ATTENTION_STAGED_WAVES if staged else 1)
     starts = [0]
@@ -379,28 +379,44 @@ def run_mfma(ops, case, window, n_splits, q_tiles=1, shared=False, staged=False,
     kc, vc = ops.cache_from_plain(case["kc"], case["vc"])      # the layout the writers leave for these sizes
     return ops.attention_mfma(case["qkv"], kc, vc, case["table"], dev(case["seq_start"]),
                               dev(case["seq_ctx"]), dev(starts), starts[-1], nh, nkv, d, window,
-                              1.0 / math.sqrt(d), n_splits, q_tiles, 2 if staged else int(shared), min_walk=min_walk)
+                              1.0 / math.sqrt(d), n_splits, q_tiles, 2 if staged else int(shared))
 
 
 @pytest.mark.parametrize("nh,nkv,d,page", [(4, 2, 16, 16), (32, 4, 64, 64), (8, 1, 128, 16)])
 @pytest.mark.parametrize("window", [0, 40])
-@pytest.mark.parametrize("n_splits,min_walk", [(3, 1), (4, 2), (8, 2), (8, 5)])
-def test_attention_mfma_parts_of_a_least_length(ops, nh, nkv, d, page, window, n_splits, min_walk):
-    """Prompt forms with a least walk: a walk of n tiles of 32 keys is cut into ceil(n / min_walk) parts (here one
-    to five: contexts of 1 to 134 tokens), the other parts of its rows stay empty and leave no outputs.  The
-    partial outputs are allocated where a tensor of NaNs has just been freed, so a merge that read an empty
-    part's outputs would show."""
+@pytest.mark.parametrize("slots,least", [(512, 1000), (512, 1), (100000, 2)])
+def test_attention_mfma_from_a_work_list(ops, nh, nkv, d, page, window, slots, least, monkeypatch):
+    """The prompt form from a work list: every piece's walk cut into as many parts as the host says (none with a
+    least walk beyond these contexts of 1 to 134 tokens; up to five otherwise, by an even share of 512 or of very
+    many places for workgroups), items in the host's order, rows with one part written at once and left alone by the
+    merge.  The partial outputs are allocated where a tensor of NaNs has just been freed: a merge that read a
+    part that no workgroup wrote would show."""
+    import types
+    monkeypatch.setattr(ops, "ATTENTION_SLOTS", slots)
+    monkeypatch.setattr(ops, "ATTENTION_MIN_WALK", least)
     case = paged_case(SEQS, nh, nkv, d, page, torch.bfloat16, seed=5)
     want = plain_result(case, window)
     t = case["qkv"].shape[0]
-    for qt in sorted({1, ops.attention_q_tiles(d)}):
-        for staged in (False, True):
-            junk = torch.full((n_splits, t, nh, d), float("nan"), dtype=torch.float32, device=DEV)
-            del junk
-            got = run_mfma(ops, case, window, n_splits, qt, staged=staged, min_walk=min_walk)
-            close(got, want, rtol=2e-2, atol=2e-2, what=f"parts of at least {min_walk} tiles, {qt} tiles a wave, staged={staged}")
-    with pytest.raises(ops.KernelError):
-        run_mfma(ops, case, window, n_splits, shared=True, min_walk=min_walk)     # the decode form cuts every walk alike
+    qt = ops.attention_q_tiles(d)
+    piece = ops.attention_tile_tokens(nh, nkv) * qt * ops.ATTENTION_STAGED_WAVES
+    starts = [0]
+    for s in range(len(case["seq_ctx"])):
+        starts.append(starts[-1] + -(-(case["seq_start"][s + 1] - case["seq_start"][s]) // piece))
+    batch = types.SimpleNamespace(n_seqs=len(case["seq_ctx"]), n_tokens=t, seq_start=case["seq_start"], seq_ctx=case["seq_ctx"])
+    items, row_parts, most = ops.prompt_work_list(batch, starts, piece, nkv * -(-(nh // nkv) // 16), window)
+    assert sorted(i & 0xfffff for i in items if (i >> 20) & 15 == 0) == list(range(starts[-1])), "every piece once"
+    assert all(sum(1 for i in items if i & 0xfffff == p) == next(i >> 24 for i in items if i & 0xfffff == p) for p in range(starts[-1]))
+    assert (most > 1) == (least < 1000) and max(row_parts) == most
+    dev = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
+    kc, vc = ops.cache_from_plain(case["kc"], case["vc"])
+    junk = torch.full((most, t, nh, d), float("nan"), dtype=torch.float32, device=DEV)
+    del junk
+    got = ops.attention_mfma(case["qkv"], kc, vc, case["table"], dev(case["seq_start"]), dev(case["seq_ctx"]), dev(starts),
+                             starts[-1], nh, nkv, d, window, 1.0 / math.sqrt(d), most, qt, 2, items=dev(items),
+                             n_items=len(items), row_parts=dev(row_parts))
+    close(got, want, rtol=2e-2, atol=2e-2, what=f"work list, {len(items)} items, up to {most} parts")
+    if most == 1:        # nothing cut: the same keys in the same order as the grid's own order gives
+        assert torch.equal(got, run_mfma(ops, case, window, 1, qt, staged=True))
 
 
 @pytest.mark.parametrize("nh,nkv,d,page", SHAPES)
