@@ -12,11 +12,13 @@
 // rows and the tile: the same bits whichever form and tile a shape selects.
 // Rows and columns beyond the matrix are not stored.
 //
-// What bounds these kernels is not the matrix cores but how far a k-step's memory loads, LDS
-// traffic and MFMAs overlap: a 64 x 64 part of a wave reads 1 KB of LDS per 32-clock MFMA, which is
-// all that LDS delivers, and the memory path and LDS share their way into the CU.  More waves a CU
-// (the direct form spends no registers on staging) and larger tiles (less traffic per FLOP) help;
-// a deeper pipeline does not.
+// What bounds these kernels (clock reads per workgroup, hardware counters): the loop over k is 85-90 %
+// of a tile's time, with the matrix cores busy 40-50 % of it -- a step's loads, fragment reads and
+// MFMAs overlap only so far between two barriers, although LDS (no bank conflicts, a third of its
+// cycles in use) and memory (a ring of three stages is no faster than one of two) both have room;
+// the small tiles are bound by what all CUs pull from L2 together (19 TB/s for 128 x 64); the rest
+// is the stores after the loop, which all CUs issue at the same time.  More waves a CU (this form
+// spends no registers on staging) and larger tiles (less traffic per FLOP) are what helped.
 //
 // Workgroups are numbered so that those sharing rows of a and of w run on the same XCD at the same
 // time (tile_of).
