@@ -95,13 +95,14 @@ _entry: dict = {}
 _profiler = profiler()
 
 
-def call(name: str, *args, cost=None) -> None:
+def call(name: str, *args, cost=None, launches: bool = True) -> None:
     """Calls an entry point of the library.  ``cost``: a function that gives (floating-point
-    operations, bytes to move at least) of this call, asked only while the profiler is on."""
+    operations, bytes to move at least) of this call, asked only while the profiler is on.
+    ``launches`` False: a question to the library that starts no kernel (the profiler leaves it out)."""
     fn = _entry.get(name)
     if fn is None:
         fn = _entry[name] = getattr(load(), name)
-    if _profiler.enabled:
+    if _profiler.enabled and launches:
         mark = _profiler.begin(name[5:] if name.startswith("bc4g_") else name, cost)
         status = fn(*args)
         _profiler.end(mark)

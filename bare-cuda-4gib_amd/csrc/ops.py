@@ -71,7 +71,8 @@ def tiled_tile(m: int, n: int, k: int, a_ptr: int = 0, w_ptr: int = 0) -> Tuple[
     """(rows, columns) of the output tile the tiled matrix-core kernel takes for an [m, k] x [n, k]^T product of
     operands at these addresses (0: well aligned)."""
     rows, cols = ctypes.c_int(0), ctypes.c_int(0)
-    library.call("bc4g_gemm_mfma_tile", a_ptr or None, w_ptr or None, m, n, k, ctypes.byref(rows), ctypes.byref(cols))
+    library.call("bc4g_gemm_mfma_tile", a_ptr or None, w_ptr or None, m, n, k, ctypes.byref(rows), ctypes.byref(cols),
+                 launches=False)
     return rows.value, cols.value
 
 
