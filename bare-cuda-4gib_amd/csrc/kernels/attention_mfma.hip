@@ -367,7 +367,9 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, 2) void att
         v1 = cur.v[1][b];
       }
       if (edge) {
-        const int kb = key0 + 4 * grp;
+        int kb = key0 + 4 * grp;
+        // (pinned here: left alone, the compiler works the masks out in every tile, before the branch)
+        asm volatile("" : "+v"(kb));
         v0.x &= (kb <= walk_max ? 0xffffu : 0u) | (kb + 1 <= walk_max ? 0xffff0000u : 0u);
         v0.y &= (kb + 2 <= walk_max ? 0xffffu : 0u) | (kb + 3 <= walk_max ? 0xffff0000u : 0u);
         v1.x &= (kb + 16 <= walk_max ? 0xffffu : 0u) | (kb + 17 <= walk_max ? 0xffff0000u : 0u);
