@@ -14,10 +14,11 @@
 //                 from the value pages, stored in that operand's order too (8-byte loads of 4
 //                 consecutive tokens, the 64 lanes' loads contiguous)
 // Prompt portions bring many tiles of one request: there a workgroup is four waves with
-// consecutive tiles that walk their keys together (WS == 0) -- all threads copy a key tile from the
-// cache into LDS once (a straight copy: the pages are in operand order already) and every wave
-// takes its operands from there, so a key is fetched once for 4 * QT * 16 query rows; the next
-// tile's loads are in flight during the arithmetic, and there is one barrier a tile.  (WS == 1 is
+// consecutive tiles that walk their keys together (WS == 0) -- a key tile goes from the cache into LDS
+// once (a straight copy: the pages are in operand order already; from memory into LDS without passing
+// registers) and every wave takes its operands from there, so a key is fetched once for 4 * QT * 16
+// query rows; the tiles up to three ahead are in flight during the arithmetic, and there is one
+// barrier a tile.  (WS == 1 is
 // the same without LDS, four independent waves each fetching its own keys: the simpler form, kept as
 // a cross-check -- both give the same bits.)
 // Decoded tokens bring few tiles and long key walks: there a workgroup is one tile and its WS
@@ -84,6 +85,9 @@ __device__ inline float sum_16_32(float x) {
   return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
+// What a tile's loads bring for blocks of keys that no row of the walk sees.
+__device__ __align__(16) const unsigned char kZeroLine[16] = {0};
+
 struct AttnArgs {
   const bf16_t* qkv;           // queries: row t, head h at qkv + t * q_stride + h * d
   bf16_t* out;                 // [T, n_heads * d]               (n_splits == 1)
@@ -118,7 +122,7 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, 2) void att
     const AttnArgs a) {
   static_assert(WS <= 1 || QT == 1, "waves share a tile's keys for single query tiles only");
   constexpr bool kStaged = WS == 0;
-  // WS > 1: [WS][16][d + pad] outputs, [WS][16][2] statistics; WS == 0: two key tiles of 128 * d bytes
+  // WS > 1: [WS][16][d + pad] outputs, [WS][16][2] statistics; WS == 0: a ring of key tiles of 128 * d bytes
   extern __shared__ __align__(16) float merge_raw[];
   const int lane = threadIdx.x % kWave;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
@@ -297,56 +301,63 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, 2) void att
   };
 
   // kStaged: a tile in LDS is four segments of 16 * d elements -- keys of its first and second 16
-  // tokens, then their values -- each a copy of the block in the cache.  A thread copies the same
-  // 16-byte pieces of every tile: piece c = threadIdx.x + 256 * r lies in segment c / (2 * d).
+  // tokens, then their values -- each a copy of the block in the cache, brought straight from memory into
+  // a ring of kStages tiles (no register and no LDS write is spent on it): the tile kStages - 1 ahead is
+  // asked for when a tile's arithmetic starts, which hides the way from memory behind several tiles' work.
+  // A thread brings the same 16-byte pieces of every tile: piece c = threadIdx.x + 256 * r lies in segment
+  // c / (2 * d) and lands at byte 16 * c of the tile; a wave's 64 pieces are one load.  Pieces beyond the
+  // tile (small heads) are whole waves' and are left out; blocks beyond the walk or before the window are
+  // brought from a line of zeros.
+  constexpr int kStages = !kStaged ? 1 : (DB <= 8 ? 4 : 2);
   constexpr int kPieces = kStaged ? (4 * 2 * 16 * DB + 255) / 256 : 1;    // per thread, for the largest d of this form
   int piece_seg[kPieces], piece_off[kPieces];
+  int pieces_a_tile = 0;                                                  // this wave's loads per tile
   if constexpr (kStaged) {
 #pragma unroll
     for (int r = 0; r < kPieces; ++r) {
       const int c = threadIdx.x + 256 * r;
       piece_seg[r] = c < 8 * d ? c / (2 * d) : -1;
       piece_off[r] = (c % (2 * d)) * 8;
+      if (wave * kWave + 256 * r < 8 * d) ++pieces_a_tile;                // (8 * d is a multiple of 128: whole waves)
     }
   }
-  uint4 staged[kPieces];
-  bool staged_ok[2];
-  auto stage_load = [&](int kt) {               // cache -> registers
-    locate(staged_ok, kt);
+  bf16_t* tiles = reinterpret_cast<bf16_t*>(merge_raw);
+  const unsigned tiles_lds = static_cast<unsigned>(
+      reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) float*)merge_raw));   // its LDS address
+  auto stage_ask = [&](int kt, int stage) {     // cache -> LDS; tiles are asked for in order, from kt_begin on
+    bool ok[2];
+    locate(ok, kt);
 #pragma unroll
     for (int r = 0; r < kPieces; ++r) {
       const int seg = piece_seg[r];
-      const bool live = seg >= 0 && staged_ok[seg & 1];
-      const bf16_t* base = (seg >= 2 ? a.v_cache : a.k_cache) + block_at[seg & 1];
-      staged[r] = live ? load16(base + piece_off[r]) : zero16();
+      if (wave * kWave + 256 * r >= 8 * d) continue;
+      const bf16_t* from = (seg >= 2 ? a.v_cache : a.k_cache) + block_at[seg & 1] + piece_off[r];
+      const void* src = ok[seg & 1] ? static_cast<const void*>(from) : static_cast<const void*>(kZeroLine);
+      load_to_lds_16(src, __builtin_amdgcn_readfirstlane(tiles_lds + stage * (128 * d) + (wave * kWave + 256 * r) * 16));
     }
-  };
-  bf16_t* tiles = reinterpret_cast<bf16_t*>(merge_raw);
-  auto stage_store = [&](int buf) {             // registers -> LDS
-#pragma unroll
-    for (int r = 0; r < kPieces; ++r)
-      if (piece_seg[r] >= 0)
-        *reinterpret_cast<uint4*>(tiles + buf * (64 * d) + piece_seg[r] * (16 * d) + piece_off[r]) = staged[r];
   };
 
   // (the fragments of the largest heads leave no room for a second tile)
   constexpr bool kAhead = DB <= 8;
   KeyTile cur, nxt;
   if constexpr (kStaged) {
-    if (kt_begin < kt_end) stage_load(kt_begin);
+#pragma unroll
+    for (int ahead = 0; ahead < kStages - 1; ++ahead)
+      if (kt_begin + ahead < kt_end) stage_ask(kt_begin + ahead, ahead);
   } else {
     if (kAhead && kt_begin < kt_end) fetch(cur, kt_begin);
   }
   for (int kt = kt_begin; kt < kt_end; ++kt) {
-    const bf16_t* tile_lds = tiles + ((kt - kt_begin) & 1) * (64 * d);
+    const bf16_t* tile_lds = tiles + ((kt - kt_begin) % kStages) * (64 * d);
     if constexpr (kStaged) {
-      // This tile goes into the buffer that the tile before the last was read from: every wave has
-      // passed the last barrier, so it has finished with that one.  The next tile's loads start now.
-      stage_store((kt - kt_begin) & 1);
-      cur.ok[0] = staged_ok[0];
-      cur.ok[1] = staged_ok[1];
-      if (kt + 1 < kt_end) stage_load(kt + 1);
+      // This tile has landed once only the tiles asked for after it are outstanding (loads finish in order).
+      // After the barrier everybody's pieces of it are there and nobody reads the tile before it any more,
+      // whose place the tile kStages - 1 ahead takes.
+      wait_loads_at_most<kPieces * (kStages - 2 > 0 ? kStages - 2 : 0)>(pieces_a_tile * min(kStages - 2, kt_end - 1 - kt));
       lds_barrier();
+      if (kt + kStages - 1 < kt_end) stage_ask(kt + kStages - 1, (kt - kt_begin + kStages - 1) % kStages);
+#pragma unroll
+      for (int h = 0; h < 2; ++h) cur.ok[h] = kt * 32 + 16 * h <= walk_max && kt * 32 + 16 * h + 15 >= lo_min;
       if (kt < own_first || kt > own_last) continue;      // no key of this wave's rows in the tile
     } else if constexpr (kAhead) {
       if (kt + 1 < kt_end) fetch(nxt, kt + 1);
@@ -754,12 +765,12 @@ extern "C" int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, flo
   BC4G_REQUIRE(form != 1 || q_tiles == 1, "attention_mfma: waves share the keys of single query tiles only");
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (form == 2) {
-    // four waves' tiles per workgroup (n_tiles counts workgroups), key tiles staged in LDS twice over
+    // four waves' tiles per workgroup (n_tiles counts workgroups), key tiles staged in a ring in LDS
     // (with a work list: heads fastest, so that the items start in the list's order, longest first)
     dim3 grid(n_tiles, n_kv_heads * a.n_sub, n_splits);
     if (items) grid = dim3(n_kv_heads * a.n_sub, n_items, 1);
     dim3 block(kWavesPerBlock * kWave);
-    const size_t lds = static_cast<size_t>(2) * 128 * head_dim;
+    const size_t lds = static_cast<size_t>(db <= 8 ? 4 : 2) * 128 * head_dim;      // (the kernel's ring of key tiles)
     if (dj <= 2 && db <= 4) {
       if (q_tiles == 4) launch_attention<2, 4, 4, 0>(a, grid, block, lds, s);
       else launch_attention<2, 4, 1, 0>(a, grid, block, lds, s);

@@ -287,21 +287,6 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_staged_kernel(
 // WM x WN waves take TM x TN MFMA blocks of 32 x 32 each.  An output element is added up over k in
 // ascending order, as in the form above: the same bits whichever form the shape selects.
 // k must be a multiple of BK; rows beyond m or n are read from the last row and not stored.
-__device__ inline void load_to_lds_16(const void* global, unsigned lds_address) {
-  // The LDS base of a wave-wide load travels in m0, which the compiler reserves for such uses of its
-  // own and sets right before each (this file gives it none: no LDS load builtin, no register array
-  // indexed at run time).  The compiler does not know the instruction, so the waits for it are written
-  // by hand (wait_loads).
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(global), "s"(lds_address) : "memory");
-}
-
-// Waits until at most N of the wave's memory operations are outstanding (they finish in order).
-template <int N>
-__device__ inline void wait_loads() {
-  static_assert(N >= 0 && N < 64, "vmcnt has six bits");
-  // vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] at [15:14]; the other counters unconstrained
-  __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
-}
 template <int PER, int MAX>
 __device__ inline void wait_for_stage(int later) {
   if constexpr (MAX == 0) {

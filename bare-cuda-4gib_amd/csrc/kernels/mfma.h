@@ -29,4 +29,32 @@ __device__ inline floatx16 mfma_32x32x16(uint4 a, uint4 b, floatx16 acc) {
 __device__ inline uint4 load16(const void* p) { return *reinterpret_cast<const uint4*>(p); }
 __device__ inline uint4 zero16() { return make_uint4(0u, 0u, 0u, 0u); }
 
+// Memory to LDS without passing registers: every lane of the wave brings the 16 bytes at its `global` to
+// lds_address (the same in all lanes) + 16 * lane -- 1 KB of consecutive LDS a wave.
+__device__ inline void load_to_lds_16(const void* global, unsigned lds_address) {
+  // The LDS base of a wave-wide load travels in m0, which the compiler reserves for such uses of its
+  // own and sets right before each (the kernels that call this give it none: no LDS load builtin, no
+  // register array indexed at run time).  The compiler does not know the instruction, so the waits for it are written
+  // by hand (wait_loads).
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(global), "s"(lds_address) : "memory");
+}
+
+// Waits until at most N of the wave's memory operations are outstanding (they finish in order).
+template <int N>
+__device__ inline void wait_loads() {
+  static_assert(N >= 0 && N < 64, "vmcnt has six bits");
+  // vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] at [15:14]; the other counters unconstrained
+  __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
+}
+// The same for a number known at run time only (the same in all lanes), up to kMost.
+template <int kMost>
+__device__ inline void wait_loads_at_most(int n) {
+  if constexpr (kMost == 0) {
+    wait_loads<0>();
+  } else {
+    if (n >= kMost) wait_loads<kMost>();
+    else wait_loads_at_most<kMost - 1>(n);
+  }
+}
+
 }  // namespace bc4g
