@@ -32,6 +32,8 @@
 // whatever lies in those places (NaN included) cannot reach the sums.
 #include <math.h>
 
+#include <type_traits>
+
 #include "api.h"
 #include "mfma.h"
 
@@ -86,7 +88,7 @@ __device__ inline float sum_16_32(float x) {
 }
 
 // What a tile's loads bring for blocks of keys that no row of the walk sees.
-__device__ __align__(16) const unsigned char kZeroLine[16] = {0};
+__device__ __align__(16) const unsigned char kZeroLine[1024] = {0};     // (a wave's load wide)
 
 struct AttnArgs {
   const bf16_t* qkv;           // queries: row t, head h at qkv + t * q_stride + h * d
@@ -232,15 +234,22 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, 2) void att
     for (int b = 0; b < DB; ++b) o[t][b] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
 
-  // The request's block table, held across the wave's lanes (entry i in lane i % 64 of register
-  // i / 64), so that finding a tile's page is a lane read and not a trip to memory.
+  // Where a tile's pages are.  The forms without LDS staging hold the request's block table across the wave's
+  // lanes (entry i in lane i % 64 of register i / 64), so that finding a tile's page is a lane read and not a trip
+  // to memory.  The staged form walks many tiles, and every instruction a wave issues for a tile counts there (a
+  // wave issues one every four clocks at best: the lane reads, selects and address arithmetic per half tile were a
+  // quarter of a tile's time): it copies the walk's part of the table into LDS first (behind the ring of tiles; a
+  // walk over more than kLdsEntries pages reads the rest from memory), looks a page up once, when the walk enters it
+  // -- the entry asked of LDS one page ahead -- and keeps the page's place in the cache.
   constexpr int kTableRegs = 4;
   int32_t tbl[kTableRegs];
   const int pages_needed = walk_max / P + 1;
+  if constexpr (!kStaged) {
 #pragma unroll
-  for (int r = 0; r < kTableRegs; ++r) {
-    const int idx = r * kWave + lane;
-    tbl[r] = (idx < pages_needed && idx < a.table_stride) ? table[idx] : 0;
+    for (int r = 0; r < kTableRegs; ++r) {
+      const int idx = r * kWave + lane;
+      tbl[r] = (idx < pages_needed && idx < a.table_stride) ? table[idx] : 0;
+    }
   }
   auto page_of = [&](int page_index) -> long {       // page_index is the same in every lane
     if (page_index >= kTableRegs * kWave) return table[page_index];
@@ -252,6 +261,9 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, 2) void att
       if (reg == r) v = w;
     }
     return v;
+  };
+  auto place_of = [&](int32_t page) -> long {   // of the page's keys or values of this key/value head, in elements
+    return (static_cast<long>(page) * a.n_kv_heads + kvh) * P * static_cast<long>(d);
   };
 
   // one tile of 32 keys: key fragments (A operand of the scores) and value fragments (A operand
@@ -268,17 +280,44 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, 2) void att
   const int k_lane = lane * 8, v_lane = lane * 4;
   int next_page = (kt_begin * 32) / P, next_off = (kt_begin * 32) % P;
   long block_at[2];                              // where the tile's two blocks of 16 keys lie in the cache
+  // kStaged: the place of page next_page in the cache, and the table's entry after it (asked for, not yet waited for)
+  constexpr int kLdsEntries = 1024;
+  int32_t* walk_table = reinterpret_cast<int32_t*>(merge_raw) + (!kStaged ? 0 : (DB <= 8 ? 4 : 2) * 32 * d);     // behind the ring
+  long page_at = 0;
+  int32_t entry_ahead = 0;
+  const int first_page = next_page, last_entry = min(pages_needed, a.table_stride) - 1;
+  typedef __attribute__((address_space(3))) int32_t lds_int;
+  auto entry = [&](int page_index) -> int32_t {       // page_index is the same in every lane
+    const int at = min(page_index, last_entry) - first_page;
+    if (__builtin_expect(at >= kLdsEntries, 0)) return __builtin_amdgcn_readfirstlane(table[first_page + at]);
+    return __builtin_amdgcn_readfirstlane(((lds_int*)walk_table)[at]);
+  };
+  if constexpr (kStaged) {
+    for (int i = threadIdx.x; i < kLdsEntries && first_page + i <= last_entry; i += kWavesPerBlock * kWave)
+      walk_table[i] = table[first_page + i];
+    __syncthreads();
+    page_at = place_of(entry(next_page));
+    entry_ahead = entry(next_page + 1);
+  }
   auto locate = [&](bool (&ok)[2], int kt) {    // tiles are located in order, from kt_begin on
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       const int kb = kt * 32 + 16 * h;
       ok[h] = kb <= walk_max && kb + 15 >= lo_min;
-      const long page = ok[h] ? page_of(next_page) : 0;
-      block_at[h] = ((page * a.n_kv_heads + kvh) * P + next_off) * static_cast<long>(d);
+      if constexpr (kStaged) {
+        block_at[h] = page_at + next_off * d;   // (a block that no row sees is never read: wherever this points)
+      } else {
+        const long page = ok[h] ? page_of(next_page) : 0;
+        block_at[h] = ((page * a.n_kv_heads + kvh) * P + next_off) * static_cast<long>(d);
+      }
       next_off += 16;                           // pages hold a multiple of 16 tokens
       if (next_off >= P) {
         next_off = 0;
         ++next_page;
+        if constexpr (kStaged) {
+          page_at = place_of(entry_ahead);
+          entry_ahead = entry(next_page + 1);
+        }
       }
     }
   };
@@ -310,15 +349,21 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, 2) void att
   // brought from a line of zeros.
   constexpr int kStages = !kStaged ? 1 : (DB <= 8 ? 4 : 2);
   constexpr int kPieces = kStaged ? (4 * 2 * 16 * DB + 255) / 256 : 1;    // per thread, for the largest d of this form
+  // (With heads of a multiple of 32 -- the sizes built EXACT -- a wave's 64 pieces lie in one segment: their load
+  // is one base address for the wave, worked out in scalar registers, plus 16 bytes a lane.)
+  constexpr bool kWholeChunks = EXACT && DB % 2 == 0;
   int piece_seg[kPieces], piece_off[kPieces];
+  int chunk_seg[kPieces], chunk_off[kPieces];                             // kWholeChunks: the wave's, not the lane's
   int pieces_a_tile = 0;                                                  // this wave's loads per tile
   if constexpr (kStaged) {
 #pragma unroll
     for (int r = 0; r < kPieces; ++r) {
-      const int c = threadIdx.x + 256 * r;
+      const int c = threadIdx.x + 256 * r, c0 = (wave * kPieces + r) * kWave;   // (whole chunks: a wave's lie side by side)
       piece_seg[r] = c < 8 * d ? c / (2 * d) : -1;
       piece_off[r] = (c % (2 * d)) * 8;
-      if (wave * kWave + 256 * r < 8 * d) ++pieces_a_tile;                // (8 * d is a multiple of 128: whole waves)
+      chunk_seg[r] = c0 / (2 * d);
+      chunk_off[r] = (c0 % (2 * d)) * 8;
+      if (kWholeChunks || wave * kWave + 256 * r < 8 * d) ++pieces_a_tile;   // (8 * d is a multiple of 128: whole waves)
     }
   }
   bf16_t* tiles = reinterpret_cast<bf16_t*>(merge_raw);
@@ -327,13 +372,39 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, 2) void att
   auto stage_ask = [&](int kt, int stage) {     // cache -> LDS; tiles are asked for in order, from kt_begin on
     bool ok[2];
     locate(ok, kt);
+    if constexpr (kWholeChunks) {
+      // the wave's kPieces chunks of 1 KB go side by side: one LDS address for all, in the middle of the stretch
+      constexpr int kMid = kPieces / 2;
+      set_lds_base(__builtin_amdgcn_readfirstlane(tiles_lds + stage * (128 * d) + (wave * kPieces + kMid) * 1024));
+      auto ask_chunk = [&](auto index) {
+        constexpr int r = decltype(index)::value;
+        const int seg = chunk_seg[r];
+        const bf16_t* from = (seg >= 2 ? a.v_cache : a.k_cache) + block_at[seg & 1] + chunk_off[r];
+        load_to_lds_16_at<(r - kMid) * 1024>(ok[seg & 1] ? static_cast<const void*>(from) : static_cast<const void*>(kZeroLine),
+                                             lane * 16u);
+      };
+      static_assert(kPieces == 1 || kPieces == 2 || kPieces == 4 || kPieces == 8, "chunks a wave brings");
+      ask_chunk(std::integral_constant<int, 0>{});
+      if constexpr (kPieces >= 2) ask_chunk(std::integral_constant<int, 1>{});
+      if constexpr (kPieces >= 4) {
+        ask_chunk(std::integral_constant<int, 2>{});
+        ask_chunk(std::integral_constant<int, 3>{});
+      }
+      if constexpr (kPieces >= 8) {
+        ask_chunk(std::integral_constant<int, 4>{});
+        ask_chunk(std::integral_constant<int, 5>{});
+        ask_chunk(std::integral_constant<int, 6>{});
+        ask_chunk(std::integral_constant<int, 7>{});
+      }
+    } else {
 #pragma unroll
-    for (int r = 0; r < kPieces; ++r) {
-      const int seg = piece_seg[r];
-      if (wave * kWave + 256 * r >= 8 * d) continue;
-      const bf16_t* from = (seg >= 2 ? a.v_cache : a.k_cache) + block_at[seg & 1] + piece_off[r];
-      const void* src = ok[seg & 1] ? static_cast<const void*>(from) : static_cast<const void*>(kZeroLine);
-      load_to_lds_16(src, __builtin_amdgcn_readfirstlane(tiles_lds + stage * (128 * d) + (wave * kWave + 256 * r) * 16));
+      for (int r = 0; r < kPieces; ++r) {
+        if (wave * kWave + 256 * r >= 8 * d) continue;
+        const unsigned to = __builtin_amdgcn_readfirstlane(tiles_lds + stage * (128 * d) + (wave * kWave + 256 * r) * 16);
+        const int seg = piece_seg[r];
+        const bf16_t* from = (seg >= 2 ? a.v_cache : a.k_cache) + block_at[seg & 1] + piece_off[r];
+        load_to_lds_16(ok[seg & 1] ? static_cast<const void*>(from) : static_cast<const void*>(kZeroLine + lane * 16), to);
+      }
     }
   };
 
@@ -353,7 +424,13 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, 2) void att
       // This tile has landed once only the tiles asked for after it are outstanding (loads finish in order).
       // After the barrier everybody's pieces of it are there and nobody reads the tile before it any more,
       // whose place the tile kStages - 1 ahead takes.
-      wait_loads_at_most<kPieces * (kStages - 2 > 0 ? kStages - 2 : 0)>(pieces_a_tile * min(kStages - 2, kt_end - 1 - kt));
+      if constexpr (kWholeChunks && kStages == 4) {       // (every wave brings kPieces loads a tile)
+        if (kt + 2 < kt_end) wait_loads<2 * kPieces>();
+        else if (kt + 1 < kt_end) wait_loads<kPieces>();
+        else wait_loads<0>();
+      } else {
+        wait_loads_at_most<kPieces * (kStages - 2 > 0 ? kStages - 2 : 0)>(pieces_a_tile * min(kStages - 2, kt_end - 1 - kt));
+      }
       lds_barrier();
       if (kt + kStages - 1 < kt_end) stage_ask(kt + kStages - 1, (kt - kt_begin + kStages - 1) % kStages);
 #pragma unroll
@@ -691,6 +768,14 @@ namespace bc4g {
 namespace {
 template <int DJ, int DB, int QT, int WS>
 void launch_attention(const AttnArgs& a, dim3 grid, dim3 block, size_t lds, hipStream_t s) {
+  static bool raised = false;   // per instantiation: the staged form's ring may need more than the default dynamic LDS
+  if (!raised && lds > 48 * 1024) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(attention_mfma_kernel<DJ, DB, QT, WS, true>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(attention_mfma_kernel<DJ, DB, QT, WS, false>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    raised = true;
+  }
   if (a.head_dim == 16 * DB) attention_mfma_kernel<DJ, DB, QT, WS, true><<<grid, block, lds, s>>>(a);
   else attention_mfma_kernel<DJ, DB, QT, WS, false><<<grid, block, lds, s>>>(a);
 }
@@ -770,7 +855,7 @@ extern "C" int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, flo
     dim3 grid(n_tiles, n_kv_heads * a.n_sub, n_splits);
     if (items) grid = dim3(n_kv_heads * a.n_sub, n_items, 1);
     dim3 block(kWavesPerBlock * kWave);
-    const size_t lds = static_cast<size_t>(db <= 8 ? 4 : 2) * 128 * head_dim;      // (the kernel's ring of key tiles)
+    const size_t lds = static_cast<size_t>(db <= 8 ? 4 : 2) * 128 * head_dim + 1024 * 4;   // (the kernel's ring of key tiles and its part of the block table)
     if (dj <= 2 && db <= 4) {
       if (q_tiles == 4) launch_attention<2, 4, 4, 0>(a, grid, block, lds, s);
       else launch_attention<2, 4, 1, 0>(a, grid, block, lds, s);

@@ -39,6 +39,34 @@ __device__ inline void load_to_lds_16(const void* global, unsigned lds_address) 
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(global), "s"(lds_address) : "memory");
 }
 
+// The same from one base address for the whole wave (in scalar registers) plus each lane's offset in bytes.
+__device__ inline void load_to_lds_16(const void* wave_base, unsigned lane_offset, unsigned lds_address) {
+  // (the base is the same in every lane; said so, half by half, it is kept in scalar registers)
+  const uintptr_t bits = reinterpret_cast<uintptr_t>(wave_base);
+  const unsigned lo = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(bits));
+  const unsigned hi = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(bits >> 32));
+  wave_base = reinterpret_cast<const void*>((static_cast<uintptr_t>(hi) << 32) | lo);
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_offset), "s"(wave_base), "s"(lds_address)
+               : "memory");
+}
+
+// The same in two steps, for several loads to one stretch of LDS: the LDS address is set once, and each load adds
+// OFFSET bytes (-4096 .. 4095) to it -- and to its memory address, so the caller takes OFFSET off that one.  (Setting
+// the LDS address anew for every load costs the wave hundreds of clocks a load: the write to m0 waits for the load
+// before it, which still needs the old value.)
+__device__ inline void set_lds_base(unsigned lds_address) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0" ::"s"(lds_address) : "memory");
+}
+template <int OFFSET>
+__device__ inline void load_to_lds_16_at(const void* wave_base, unsigned lane_offset) {
+  static_assert(OFFSET >= -4096 && OFFSET <= 4095, "the instruction's offset field");
+  const uintptr_t bits = reinterpret_cast<uintptr_t>(wave_base) - OFFSET;
+  const unsigned lo = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(bits));
+  const unsigned hi = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(bits >> 32));
+  wave_base = reinterpret_cast<const void*>((static_cast<uintptr_t>(hi) << 32) | lo);
+  asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" ::"v"(lane_offset), "s"(wave_base), "n"(OFFSET) : "memory");
+}
+
 // Waits until at most N of the wave's memory operations are outstanding (they finish in order).
 template <int N>
 __device__ inline void wait_loads() {
