@@ -224,11 +224,15 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, 2) void att
   const int own_lo = (a.window > 0 && pos_min - a.window + 1 > 0) ? pos_min - a.window + 1 : 0;
   const int own_first = own_lo / 32, own_last = ntok > 0 ? pos_max / 32 : -1;
 
-  float m_run[QT], l_run[QT];
+  // per row: the exponents' reference, the sum of the weights, and -- kept beside the reference so that a tile
+  // that moves nothing need not work them out -- the shift it makes in the exponent and the score beyond which it moves
+  float m_run[QT], l_run[QT], m_shift[QT], m_limit[QT];
   floatx4 o[QT][DB];
 #pragma unroll
   for (int t = 0; t < QT; ++t) {
     m_run[t] = -INFINITY;
+    m_shift[t] = 0.f;
+    m_limit[t] = -INFINITY;
     l_run[t] = 0.f;
 #pragma unroll
     for (int b = 0; b < DB; ++b) o[t][b] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -412,6 +416,10 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, 2) void att
   constexpr bool kAhead = DB <= 8;
   KeyTile cur, nxt;
   if constexpr (kStaged) {
+    // The loads the compiler knows of (the queries) are waited for here, where it sees it: left to itself it waits for
+    // them inside the loop, at the first use of a query, with a count of zero -- which would also wait, tile after tile,
+    // for the tile that has just been asked for.
+    wait_loads<0>();
 #pragma unroll
     for (int ahead = 0; ahead < kStages - 1; ++ahead)
       if (kt_begin + ahead < kt_end) stage_ask(kt_begin + ahead, ahead);
@@ -520,47 +528,51 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, 2) void att
     // float sums and bfloat16 factors hold as well as values up to 1, and the quotient of the two sums
     // does not depend on the reference -- but what has been summed is scaled down far less often (with
     // the latest maximum as reference some row of a wave's 64 moves in most of a prompt's tiles).
+    // A lane first looks at its own eight scores only: while none of the wave's lanes sees one beyond its row's
+    // reference by more than the slack -- every tile but a walk's first few -- the rows' maxima need not be
+    // found across lanes, nothing moves, and the exponents' shift is the one kept from before.
     constexpr float kSlack = 8.0f;
-    float m_new[QT], psum[QT];
-    uint4 pf[QT];
-    bool moved = false;
+    float lane_max[QT];
+    bool beyond = false;
 #pragma unroll
     for (int t = 0; t < QT; ++t) {
-      float m_tile = max3(sv[t][0], sv[t][1], sv[t][2]);
-      m_tile = max3(m_tile, sv[t][3], sv[t][4]);
-      m_tile = max3(m_tile, sv[t][5], sv[t][6]);
-      m_tile = max_16_32(max2(m_tile, sv[t][7]));
-      const bool up = (m_tile - m_run[t]) * a.scale_log2 > kSlack;     // (from -inf: yes; nothing seen in the tile: no)
-      m_new[t] = up ? m_tile : m_run[t];
-      const float m_safe = (m_new[t] == -INFINITY) ? 0.f : m_new[t];
-      const float shift = -m_safe * a.scale_log2;
-      float p[8];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) p[i] = fast_exp2(fmaf(sv[t][i], a.scale_log2, shift));
-      psum[t] = ((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]));
-      pf[t] = make_uint4(pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3]), pack_bf16x2(p[4], p[5]),
-                         pack_bf16x2(p[6], p[7]));
-      moved = moved || up;
+      float m_lane = max3(sv[t][0], sv[t][1], sv[t][2]);
+      m_lane = max3(m_lane, sv[t][3], sv[t][4]);
+      m_lane = max3(m_lane, sv[t][5], sv[t][6]);
+      lane_max[t] = max2(m_lane, sv[t][7]);
+      beyond = beyond || lane_max[t] > m_limit[t];                     // (from -inf: any score is)
     }
-    if (__any(moved)) {
-      // the reference moved for some row of the wave (early in a walk, rarely later): what has been
-      // summed so far is scaled down by 2^(old reference - new reference), 0 while nothing had been seen
+    if (__any(beyond)) {
+      // Some row of the wave may have to move its reference (early in a walk, rarely later): the rows' maxima
+      // are found, and what has been summed so far is scaled down by 2^(old reference - new reference), 0 while
+      // nothing had been seen.
 #pragma unroll
       for (int t = 0; t < QT; ++t) {
-        const float m_safe = (m_new[t] == -INFINITY) ? 0.f : m_new[t];
+        const float m_tile = max_16_32(lane_max[t]);
+        const bool up = (m_tile - m_run[t]) * a.scale_log2 > kSlack;   // (from -inf: yes; nothing seen in the tile: no)
+        const float m_new = up ? m_tile : m_run[t];
+        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
         const float alpha = fast_exp2((m_run[t] - m_safe) * a.scale_log2);
-        l_run[t] = l_run[t] * alpha + psum[t];
+        l_run[t] *= alpha;
 #pragma unroll
         for (int b = 0; b < DB; ++b)
 #pragma unroll
           for (int r = 0; r < 4; ++r) o[t][b][r] *= alpha;
+        m_run[t] = m_new;
+        m_shift[t] = -m_safe * a.scale_log2;
+        m_limit[t] = m_new + kSlack / a.scale_log2;                    // (-inf stays -inf)
       }
-    } else {
-#pragma unroll
-      for (int t = 0; t < QT; ++t) l_run[t] += psum[t];
     }
+    uint4 pf[QT];
 #pragma unroll
-    for (int t = 0; t < QT; ++t) m_run[t] = m_new[t];
+    for (int t = 0; t < QT; ++t) {
+      float p[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) p[i] = fast_exp2(fmaf(sv[t][i], a.scale_log2, m_shift[t]));
+      l_run[t] += ((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]));
+      pf[t] = make_uint4(pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3]), pack_bf16x2(p[4], p[5]),
+                         pack_bf16x2(p[6], p[7]));
+    }
     // (blocks past the head size hold zeros and are never stored)
 #pragma unroll
     for (int b = 0; b < DB; ++b) {
