@@ -292,7 +292,7 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, 2) void att
   const int first_page = next_page, last_entry = min(pages_needed, a.table_stride) - 1;
   typedef __attribute__((address_space(3))) int32_t lds_int;
   auto entry = [&](int page_index) -> int32_t {       // page_index is the same in every lane
-    const int at = min(page_index, last_entry) - first_page;
+    const int at = max(0, min(page_index, last_entry) - first_page);     // (an empty part may begin beyond the last page)
     if (__builtin_expect(at >= kLdsEntries, 0)) return __builtin_amdgcn_readfirstlane(table[first_page + at]);
     return __builtin_amdgcn_readfirstlane(((lds_int*)walk_table)[at]);
   };
