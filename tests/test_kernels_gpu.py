@@ -514,6 +514,19 @@ def test_attention_long_context(ops, nh, nkv, d, page):
                   what=f"shared keys, window {window}, {n_splits} parts")
 
 
+def test_attention_walk_over_more_pages_than_the_table_copy_holds(ops):
+    """The prompt form keeps a copy of its walk's part of the block table in LDS, 1,024 entries; a portion of 40 tokens
+    after 16,500 cached ones in pages of 16 walks 1,034 pages, the last of them looked up in memory -- with the keys in
+    one part and cut, and with a window that begins far into the walk."""
+    case = paged_case([(16500, 40), (3, 20)], 4, 1, 32, 16, torch.bfloat16, seed=15, poison=False)
+    qt = ops.attention_q_tiles(32)
+    for window in (0, 900):
+        want = plain_result(case, window)
+        for n_splits in (1, 3):
+            close(run_mfma(ops, case, window, n_splits, qt, staged=True), want, rtol=2e-2, atol=2e-2,
+                  what=f"staged, window {window}, {n_splits} parts")
+
+
 def test_attention_window_edge(ops):
     """Keys exactly at the window's edge: position p sees p - window + 1 but not p - window."""
     case = paged_case([(0, 50)], 2, 1, 32, 16, torch.bfloat16, seed=6, poison=False)
