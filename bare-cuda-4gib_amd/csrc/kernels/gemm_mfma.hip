@@ -70,7 +70,7 @@ __device__ inline void store_patch(const float* patch, void* __restrict__ out, i
       const float* src = patch + row * kStride + col;
       float v[4];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) v[e] = (src[e] / (1.0f + expf(-src[e]))) * src[e + 8];
+      for (int e = 0; e < 4; ++e) v[e] = silu_quick(src[e]) * src[e + 8];
       bf16_t* dst = static_cast<bf16_t*>(out) + gm * n_out + (gn / 16) * 8 + gn % 16;
       if (n_out % 4 == 0) {
         uint2 pk;

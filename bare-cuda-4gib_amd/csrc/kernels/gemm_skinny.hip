@@ -439,7 +439,7 @@ __global__ __launch_bounds__(kThreads, (XMODE != kPlain || (MT == 1 && U == 2)) 
     } else if constexpr (EPI == kSwigluBf16) {
       // block b = n0 / 16 holds gates and ups of outputs 8b .. 8b + 7
       const long o = static_cast<long>(row) * (a.n / 2) + (n0 / 2 + nl);
-      static_cast<bf16_t*>(a.out)[o] = from_float<bf16_t>((sum / (1.0f + expf(-sum))) * partner);
+      static_cast<bf16_t*>(a.out)[o] = from_float<bf16_t>(silu_quick(sum) * partner);
     } else {
       const RopeKvArgs& r = a.rope;
       const int d = r.head_dim;

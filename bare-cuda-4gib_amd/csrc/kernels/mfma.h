@@ -26,6 +26,13 @@ __device__ inline floatx16 mfma_32x32x16(uint4 a, uint4 b, floatx16 acc) {
                                                  acc, 0, 0, 0);
 }
 
+// x / (1 + e^-x) for the bfloat16 products' SwiGLU epilogues, by the hardware's 2^x and reciprocal (each good to a unit
+// in the last place of a float; the result is rounded to bfloat16).  expf and a true division are an eighth of the
+// tiled kernel's epilogue, and that a sixth of a wide gate-up product's time.
+__device__ inline float silu_quick(float x) {
+  return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * -1.4426950408889634f));
+}
+
 __device__ inline uint4 load16(const void* p) { return *reinterpret_cast<const uint4*>(p); }
 __device__ inline uint4 zero16() { return make_uint4(0u, 0u, 0u, 0u); }
 
