@@ -148,6 +148,15 @@ int bc4g_gemm_mfma(const void* a, const void* w, void* out, int epilogue, int m,
 // The output tile (rows, columns) bc4g_gemm_mfma takes for these operands: for the accounting of bytes and for
 // tests that want to meet every tile.  Launches nothing.
 int bc4g_gemm_mfma_tile(const void* a, const void* w, int m, int n, int k, int* rows, int* cols);
+// The q|k|v product of many rows with rotation and cache write in its epilogue, as bc4g_gemm_skinny_qkv for few (k a
+// multiple of 64, operands on 16-byte boundaries): w [n, k] holds n_heads query, n_kv_heads key and as many value heads of
+// head_dim (a multiple of 16), every head's rows in blocks of eight dimensions followed by their rotation partners.  out
+// [m, n_heads * head_dim] bfloat16 receives the rotated queries; keys go rotated, values as they are into the pages that
+// slot_map [m] names, in the cache's layout (write_kv 0: nowhere).  table [m, head_dim / 2, 2]: cosine and sine
+// of every row's position and pair (bc4g_rope_table; null: nothing is rotated).
+int bc4g_gemm_mfma_qkv(const void* a, const void* w, void* out, const float* table, const int32_t* slot_map, void* k_cache,
+                       void* v_cache, int m, int n, int k, int n_heads, int n_kv_heads, int head_dim, int page_tokens,
+                       int write_kv, void* stream);
 }
 
 extern "C" {

@@ -36,7 +36,19 @@ constexpr int kXcds = 8;
 
 // kSwigluBf16: every 16 rows of w are eight gate rows and the eight up rows of the same outputs;
 // out [m, n / 2] = silu(gate) * up.  A gate and its up lie eight columns apart in the product.
-enum Epilogue : int { kStoreBf16 = 0, kStoreF32 = 1, kAccumF32 = 2, kSwigluBf16 = 3 };
+// kRopeKvBf16: w holds query, key and value heads with every head's rows in blocks of 16 (eight dimensions, then their
+// rotation partners, which so lie eight columns apart in the product): queries are stored rotated, keys go rotated
+// into their pages, values into theirs (operands straight into LDS only).
+enum Epilogue : int { kStoreBf16 = 0, kStoreF32 = 1, kAccumF32 = 2, kSwigluBf16 = 3, kRopeKvBf16 = 4 };
+
+struct RopeKvArgs {
+  const float2* table;        // [m, head_dim / 2] (cos, sin) of every row's position and pair (null: no rotation)
+  const int32_t* slot_map;    // [m] page * page_tokens + offset
+  bf16_t* k_cache;            // [pages, n_kv, page_tokens, d], or every [page_tokens, d] in fragment order
+  bf16_t* v_cache;            // [pages, n_kv, d, page_tokens], or likewise
+  int n_heads, n_kv_heads, head_dim, page_tokens, write_kv;
+  int fragment_order;         // how the cache's pages are laid out (cache_fragment_order)
+};
 
 // Which tile a workgroup takes.  Workgroups are dealt to the 8 XCDs in turn, each with an L2 of its
 // own: consecutive logical ids stay on one XCD and walk the output in bands of kBand rows of tiles,
@@ -112,6 +124,93 @@ __device__ inline void store_patch(const float* patch, void* __restrict__ out, i
           else static_cast<float*>(out)[o + e] += v[e];
         }
       }
+    }
+  }
+}
+
+// The q|k|v epilogue: THREADS threads take ROWS x COLS floats (stride COLS + 4) from LDS, four neighbouring columns a
+// thread -- half a block's eight dimensions, or half of their partners -- rotate them with what lies eight columns
+// away in the patch, and store queries to out [m, n_heads * head_dim], keys and values into their pages.
+template <int THREADS, int ROWS, int COLS>
+__device__ inline void store_patch_rope(const float* patch, bf16_t* __restrict__ out, int m, int n, long m0, long n0, int tid,
+                                        const RopeKvArgs& ra) {
+  constexpr int kStride = COLS + 4;
+  const int d = ra.head_dim;
+  if (ra.fragment_order && n0 >= static_cast<long>(ra.n_heads + ra.n_kv_heads) * d) {
+    // A patch of value columns only, for a cache in fragment order, where four consecutive tokens of one dimension
+    // lie side by side: a thread takes one column of four rows, and where those four tokens' places are four in a
+    // row from a multiple of four on (a prompt portion's usually are) it stores them at once.
+    static_assert(ROWS % 4 == 0, "rows in fours");
+    for (int c = tid; c < (ROWS / 4) * COLS; c += THREADS) {
+      const int col = c % COLS, row = (c / COLS) * 4;
+      const long gm = m0 + row, gn = n0 + col;
+      if (gm >= m || gn >= n) continue;
+      const int head = static_cast<int>(gn / d) - ra.n_heads - ra.n_kv_heads, dim = static_cast<int>(gn % d);
+      const int rows = static_cast<int>(min(4L, m - gm));
+      int slot[4];
+      uint16_t bits[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        slot[e] = e < rows ? ra.slot_map[gm + e] : -1;
+        bits[e] = bf16_bits_from_float(patch[(row + e) * kStride + col]);
+      }
+      if (rows == 4 && slot[0] % 4 == 0 && slot[1] == slot[0] + 1 && slot[2] == slot[0] + 2 && slot[3] == slot[0] + 3) {
+        const long page = slot[0] / ra.page_tokens;
+        const int off = slot[0] % ra.page_tokens;
+        bf16_t* region = ra.v_cache + (page * ra.n_kv_heads + head) * static_cast<long>(d) * ra.page_tokens;
+        uint2 pk;
+        pk.x = static_cast<uint32_t>(bits[0]) | (static_cast<uint32_t>(bits[1]) << 16);
+        pk.y = static_cast<uint32_t>(bits[2]) | (static_cast<uint32_t>(bits[3]) << 16);
+        *reinterpret_cast<uint2*>(region + frag_v_offset(off, dim, d)) = pk;
+      } else {
+        for (int e = 0; e < rows; ++e) {
+          const long page = slot[e] / ra.page_tokens;
+          const int off = slot[e] % ra.page_tokens;
+          bf16_t* region = ra.v_cache + (page * ra.n_kv_heads + head) * static_cast<long>(d) * ra.page_tokens;
+          region[frag_v_offset(off, dim, d)].bits = bits[e];
+        }
+      }
+    }
+    return;
+  }
+  for (int c = tid; c < ROWS * (COLS / 4); c += THREADS) {
+    const int row = c / (COLS / 4), col = (c % (COLS / 4)) * 4;
+    const long gm = m0 + row, gn = n0 + col;
+    if (gm >= m || gn >= n) continue;
+    const int head = static_cast<int>(gn / d), dim = static_cast<int>(gn % d);
+    const bool is_q = head < ra.n_heads, is_v = head >= ra.n_heads + ra.n_kv_heads;
+    if (!is_q && !ra.write_kv) continue;
+    floatx4 v = *reinterpret_cast<const floatx4*>(patch + row * kStride + col);
+    if (ra.table != nullptr && !is_v) {
+      const bool first = dim % 16 < 8;                       // the pairs' first halves; their partners lie 8 further
+      const floatx4 other = *reinterpret_cast<const floatx4*>(patch + row * kStride + (first ? col + 8 : col - 8));
+      const float2* cs = ra.table + gm * (d / 2) + (dim / 16) * 8 + dim % 8;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float2 a = cs[e];
+        v[e] = first ? v[e] * a.x - other[e] * a.y : v[e] * a.x + other[e] * a.y;
+      }
+    }
+    uint2 pk;
+    pk.x = static_cast<uint32_t>(bf16_bits_from_float(v[0])) | (static_cast<uint32_t>(bf16_bits_from_float(v[1])) << 16);
+    pk.y = static_cast<uint32_t>(bf16_bits_from_float(v[2])) | (static_cast<uint32_t>(bf16_bits_from_float(v[3])) << 16);
+    if (is_q) {
+      *reinterpret_cast<uint2*>(out + gm * (static_cast<long>(ra.n_heads) * d) + gn) = pk;
+      continue;
+    }
+    const int slot = ra.slot_map[gm];
+    const long page = slot / ra.page_tokens;
+    const int off = slot % ra.page_tokens;
+    if (!is_v) {      // keys: [page][kv head][token][dim], or in fragment order: eight dimensions of 16 tokens together
+      bf16_t* region = ra.k_cache + (page * ra.n_kv_heads + (head - ra.n_heads)) * ra.page_tokens * d;
+      bf16_t* dst = ra.fragment_order ? region + frag_k_offset(off, dim, d) : region + static_cast<long>(off) * d + dim;
+      *reinterpret_cast<uint2*>(dst) = pk;
+    } else {          // values are kept transposed: [page][kv head][dim][token], or in fragment order
+      bf16_t* region = ra.v_cache + (page * ra.n_kv_heads + (head - ra.n_heads - ra.n_kv_heads)) * static_cast<long>(d) * ra.page_tokens;
+      bf16_t* dst = ra.fragment_order ? region + frag_v_offset(off, dim, d) : region + static_cast<long>(dim) * ra.page_tokens + off;
+      const long step = ra.fragment_order ? 4 : ra.page_tokens;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) dst[e * step] = from_float<bf16_t>(v[e]);
     }
   }
 }
@@ -316,7 +415,7 @@ struct DirectShape {
 template <int EPI, int WM, int WN, int TM, int TN, int BK, int STAGES, int MINWG>
 __global__ __launch_bounds__(64 * WM * WN, MINWG) void gemm_mfma_direct_kernel(
     const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, void* __restrict__ out, int m, int n, int k, int m_blocks,
-    int n_blocks) {
+    int n_blocks, const RopeKvArgs ra) {
   typedef DirectShape<WM, WN, TM, TN, BK, STAGES> S;
   constexpr int RA = S::kRowsA, RW = S::kRowsW, RB = S::kRowBytes, NW = S::kWaves;
   constexpr int kGroupRows = 1024 / RB;                    // rows a wave-wide load covers
@@ -429,12 +528,15 @@ __global__ __launch_bounds__(64 * WM * WN, MINWG) void gemm_mfma_direct_kernel(
     for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) patch[(8 * (r / 4) + 4 * (lane / 32) + r % 4) * kStride + j * 32 + lane % 32] = acc[i][j][r];
-    store_patch<EPI, kWave, 32, 32 * TN>(patch, out, m, n, m0 + (wm * TM + i) * 32, n0 + wn * TN * 32, lane);
+    if constexpr (EPI == kRopeKvBf16)
+      store_patch_rope<kWave, 32, 32 * TN>(patch, static_cast<bf16_t*>(out), m, n, m0 + (wm * TM + i) * 32, n0 + wn * TN * 32, lane, ra);
+    else
+      store_patch<EPI, kWave, 32, 32 * TN>(patch, out, m, n, m0 + (wm * TM + i) * 32, n0 + wn * TN * 32, lane);
   }
 }
 
 template <int EPI, int WM, int WN, int TM, int TN, int BK, int STAGES, int MINWG>
-int launch_direct(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, int k, hipStream_t s) {
+int launch_direct(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, int k, hipStream_t s, const RopeKvArgs& ra) {
   typedef DirectShape<WM, WN, TM, TN, BK, STAGES> S;
   auto kernel = gemm_mfma_direct_kernel<EPI, WM, WN, TM, TN, BK, STAGES, MINWG>;
   static bool raised = false;   // per instantiation: allow more than the default dynamic LDS
@@ -446,7 +548,7 @@ int launch_direct(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, i
   }
   const long m_blocks = (m + S::kRowsA - 1) / S::kRowsA, n_blocks = (n + S::kRowsW - 1) / S::kRowsW;
   kernel<<<dim3(static_cast<unsigned>(m_blocks * n_blocks)), dim3(S::kThreads), S::kLdsBytes, s>>>(
-      ap, wp, out, m, n, k, static_cast<int>(m_blocks), static_cast<int>(n_blocks));
+      ap, wp, out, m, n, k, static_cast<int>(m_blocks), static_cast<int>(n_blocks), ra);
   return 0;
 }
 
@@ -479,13 +581,14 @@ int direct_form(int m, int n, int k) {
 }
 
 template <int EPI>
-int launch_direct_form(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, int k, hipStream_t s) {
+int launch_direct_form(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, int k, hipStream_t s,
+                       const RopeKvArgs& ra = RopeKvArgs{}) {
   switch (direct_form(m, n, k)) {
-    case 0: return launch_direct<EPI, 4, 4, 2, 2, 64, 2, 1>(ap, wp, out, m, n, k, s);
-    case 1: return launch_direct<EPI, 4, 2, 2, 3, 64, 2, 1>(ap, wp, out, m, n, k, s);
-    case 2: return launch_direct<EPI, 4, 2, 2, 2, 64, 2, 1>(ap, wp, out, m, n, k, s);
-    case 3: return launch_direct<EPI, 2, 2, 2, 1, 64, 2, 4>(ap, wp, out, m, n, k, s);
-    default: return launch_direct<EPI, 2, 2, 1, 1, 64, 4, 2>(ap, wp, out, m, n, k, s);
+    case 0: return launch_direct<EPI, 4, 4, 2, 2, 64, 2, 1>(ap, wp, out, m, n, k, s, ra);
+    case 1: return launch_direct<EPI, 4, 2, 2, 3, 64, 2, 1>(ap, wp, out, m, n, k, s, ra);
+    case 2: return launch_direct<EPI, 4, 2, 2, 2, 64, 2, 1>(ap, wp, out, m, n, k, s, ra);
+    case 3: return launch_direct<EPI, 2, 2, 2, 1, 64, 2, 4>(ap, wp, out, m, n, k, s, ra);
+    default: return launch_direct<EPI, 2, 2, 1, 1, 64, 4, 2>(ap, wp, out, m, n, k, s, ra);
   }
 }
 
@@ -530,6 +633,33 @@ extern "C" int bc4g_gemm_mfma(const void* a, const void* w, void* out, int epilo
   }
   if (e) return e;
   return check_launch("gemm_mfma");
+}
+
+extern "C" int bc4g_gemm_mfma_qkv(const void* a, const void* w, void* out, const float* table, const int32_t* slot_map,
+                                  void* k_cache, void* v_cache, int m, int n, int k, int n_heads, int n_kv_heads,
+                                  int head_dim, int page_tokens, int write_kv, void* stream) {
+  BC4G_REQUIRE(m > 0 && n > 0 && k > 0 && direct_operands(a, w, k),
+               "gemm_mfma_qkv: K=%d must be a multiple of 64 and the operands on 16-byte boundaries (M=%d N=%d)", k, m, n);
+  BC4G_REQUIRE(n_heads > 0 && n_kv_heads > 0 && head_dim > 0 && head_dim % 16 == 0 &&
+                   static_cast<long>(n_heads + 2 * n_kv_heads) * head_dim == n,
+               "gemm_mfma_qkv: %d + 2 x %d heads of %d (a multiple of 16) are not %d columns", n_heads, n_kv_heads, head_dim, n);
+  BC4G_REQUIRE(!write_kv || (page_tokens > 0 && k_cache && v_cache && slot_map), "gemm_mfma_qkv: cache write asked for without a cache");
+  BC4G_REQUIRE(((m + 63L) / 64) * ((n + 63L) / 64) <= 2147483647L, "gemm_mfma_qkv: too many tiles");
+  RopeKvArgs ra{};
+  ra.table = reinterpret_cast<const float2*>(table);
+  ra.slot_map = slot_map;
+  ra.k_cache = static_cast<bf16_t*>(k_cache);
+  ra.v_cache = static_cast<bf16_t*>(v_cache);
+  ra.n_heads = n_heads;
+  ra.n_kv_heads = n_kv_heads;
+  ra.head_dim = head_dim;
+  ra.page_tokens = page_tokens;
+  ra.write_kv = write_kv ? 1 : 0;
+  ra.fragment_order = write_kv && cache_fragment_order(true, head_dim, page_tokens) ? 1 : 0;
+  if (int e = launch_direct_form<kRopeKvBf16>(static_cast<const bf16_t*>(a), static_cast<const bf16_t*>(w), out, m, n, k,
+                                              static_cast<hipStream_t>(stream), ra))
+    return e;
+  return check_launch("gemm_mfma_qkv");
 }
 
 extern "C" int bc4g_gemm_mfma_tile(const void* a, const void* w, int m, int n, int k, int* rows, int* cols) {

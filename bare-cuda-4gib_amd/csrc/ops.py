@@ -599,6 +599,46 @@ def gemm_qkv_rope(x: torch.Tensor, g: Optional[torch.Tensor], eps: float, w,
     return q
 
 
+TILED_QKV_ROPE = True               # (off: the product, then a kernel that rotates and writes the cache)
+
+
+def gemm_qkv_rope_tiled_supported(x: torch.Tensor, w, head_dim: int, rotary_dim: int) -> bool:
+    """Whether the tiled kernel takes the q|k|v product of these (many) rows with rotation and cache write in its
+    epilogue: bfloat16, operands straight into LDS, heads in blocks of 16, the whole head rotated or none of it."""
+    w, _ = _weight(w)
+    return (TILED_QKV_ROPE and x.is_cuda and _fast_operands(x, w) and not streams_weights(x.shape[0], w.shape[0], w.shape[1])
+            and x.shape[1] % 64 == 0 and x.is_contiguous() and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
+            and head_dim % 16 == 0 and rotary_dim in (0, head_dim))
+
+
+def gemm_qkv_rope_tiled(x: torch.Tensor, w, table: Optional[torch.Tensor], slot_map: Optional[torch.Tensor],
+                        k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor], n_heads: int, n_kv_heads: int,
+                        head_dim: int, write_kv: bool = True) -> torch.Tensor:
+    """The q|k|v product of a prompt portion with rotary positions (``table``: rope_table() of the rows' positions;
+    None: no rotation) and the cache write in its epilogue (w in the reordered head layout).  Returns the rotated
+    queries [M, heads * head_dim]."""
+    w, _ = _weight(w)
+    _dev("gemm_qkv_rope_tiled", x, w, table, slot_map, k_cache, v_cache)
+    m, k = x.shape
+    n = (n_heads + 2 * n_kv_heads) * head_dim
+    if tuple(w.shape) != (n, k):
+        raise KernelError(f"gemm_qkv_rope_tiled: weight must be [{n}, {k}], got {tuple(w.shape)}")
+    if table is not None and (table.dtype != torch.float32 or tuple(table.shape) != (m, head_dim // 2, 2)
+                              or not table.is_contiguous()):
+        raise KernelError(f"gemm_qkv_rope_tiled: the table must be float32 [{m}, {head_dim // 2}, 2], "
+                          f"got {table.dtype} {tuple(table.shape)}")
+    page_tokens = 0
+    if write_kv:
+        _check_cache("gemm_qkv_rope_tiled", k_cache, v_cache, n_kv_heads, head_dim, torch.bfloat16)
+        _i32("gemm_qkv_rope_tiled", "slot_map", slot_map, m)
+        page_tokens = k_cache.shape[2]
+    q = torch.empty((m, n_heads * head_dim), dtype=torch.bfloat16, device=x.device)
+    library.call("bc4g_gemm_mfma_qkv", _ptr(x), _ptr(w), _ptr(q), _ptr(table), _ptr(slot_map), _ptr(k_cache), _ptr(v_cache),
+                 m, n, k, n_heads, n_kv_heads, head_dim, page_tokens, 1 if write_kv else 0, _stream(),
+                 cost=_tiled_cost(m, n, k, 2))
+    return q
+
+
 def attention_mfma_supported(qkv: torch.Tensor, k_cache: torch.Tensor, head_dim: int) -> bool:
     return (qkv.dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= 256
             and k_cache.shape[2] % 16 == 0)

@@ -124,6 +124,8 @@ class CausalAttention(Part):
         q = None
         if self.block_pairs and fused is not None:
             q = self._fused_qkv(h, ctx, slot_map, k_cache, v_cache, rotary_dim, theta, writes)
+        if q is None and self.block_pairs and fused is not None:
+            q = self._tiled_qkv(h, ctx, slot_map, k_cache, v_cache, rotary_dim, theta, writes)
         if q is None:
             q = linear(h, self.w_qkv, out_dtype=self.act_dtype)
             if fused is None:
@@ -143,6 +145,18 @@ class CausalAttention(Part):
         o = ops.attention(q, cache.k, cache.v, ctx.block_tables[cache.group], ctx, (arrays, notes) if notes else None,
                           self.num_heads, self.num_kv_heads, self.head_dim, self.window, self.scale)
         linear(o, self.w_o, accumulate_into=residual, ctx=ctx)
+
+    def _tiled_qkv(self, h, ctx, slot_map, k_cache, v_cache, rotary_dim, theta, writes):
+        """The q|k|v product of many rows (a prompt portion) with rotation and cache write in the tiled kernel's
+        epilogue, the angles from the step's table; None where that kernel does not take the operands."""
+        x = h.tensor() if isinstance(h, Normed) else h
+        if not ops.gemm_qkv_rope_tiled_supported(x, self.w_qkv, self.head_dim, rotary_dim):
+            return None
+        table = None
+        if rotary_dim > 0:
+            table = ctx.shared(("rope_table", rotary_dim, theta), lambda: ops.rope_table(ctx.positions, rotary_dim, theta))
+        return ops.gemm_qkv_rope_tiled(x, self.w_qkv, table, slot_map, k_cache, v_cache, self.num_heads, self.num_kv_heads,
+                                       self.head_dim, write_kv=writes)
 
     def _fused_qkv(self, h, ctx, slot_map, k_cache, v_cache, rotary_dim, theta, writes):
         """The q|k|v product with rotation and cache write in its epilogue, where a kernel takes

@@ -673,6 +673,73 @@ def test_qkv_product_with_rotation_and_cache_write(ops, nh, nkv, d, m, normed, r
         close(buf.view(m, nh + 2 * nkv, d)[:, :nh], q.view(m, nh, d), 1e-2, 2e-2, "unfused queries")
 
 
+@pytest.mark.parametrize("nh,nkv,d,m,k,page", [(4, 2, 16, 200, 64, 16), (6, 2, 48, 333, 128, 16), (32, 4, 64, 2048 - 20, 192, 64),
+                                               (24, 8, 128, 2048 - 20, 192, 32), (32, 8, 128, 4096 - 236, 192, 64)])
+@pytest.mark.parametrize("rotate", [True, False])
+def test_tiled_qkv_product_with_rotation_and_cache_write(ops, nh, nkv, d, m, k, page, rotate):
+    """The same for the many rows of a prompt portion, in the tiled kernel's epilogue (tiles of 64 x 64 up to 256 x 256
+    by the shapes): queries rotated, keys rotated into the pages the slot map names, values into theirs, nothing else
+    touched -- against the plain product and rotation, and against the unfused pair of kernels."""
+    if torch.cuda.get_device_properties(0).multi_processor_count != 256:
+        pytest.skip("the shapes are chosen for 256 CUs")
+    theta = 500.0
+    order = block_order(d)
+    pages = -(-m // page) + 3                                     # (room for the rows in a row from the second page on)
+    w = bf(rnd((nh + 2 * nkv) * d, k, seed=33, scale=0.3))
+    wp = w.view(nh + 2 * nkv, d, k)[:, order, :].reshape(-1, k).contiguous()        # reordered rows
+    positions = [3 + 5 * i for i in range(m)]
+    slots = random.Random(2).sample(range(pages * page), m)
+    x = bf(rnd(m, k, seed=34))
+    xin = x.to(DEV)
+    assert ops.gemm_qkv_rope_tiled_supported(xin, wp.to(DEV), d, d if rotate else 0)
+    qkv = (x.double() @ w.double().T).view(m, nh + 2 * nkv, d)
+    pos = torch.tensor(positions)
+    q_want = P.rope(qkv[:, :nh], pos, theta) if rotate else qkv[:, :nh]
+    k_want = P.rope(qkv[:, nh:nh + nkv], pos, theta) if rotate else qkv[:, nh:nh + nkv]
+    v_want = qkv[:, nh + nkv:]
+    dev = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    kc = torch.full((pages, nkv, page, d), -7.5, dtype=torch.bfloat16, device=DEV)
+    vc = torch.full((pages, nkv, d, page), -7.5, dtype=torch.bfloat16, device=DEV)
+    table = ops.rope_table(dev(positions), d, theta) if rotate else None
+    q = ops.gemm_qkv_rope_tiled(xin, wp.to(DEV), table, dev(slots), kc, vc, nh, nkv, d)
+    assert tuple(q.shape) == (m, nh * d)
+    tol = dict(rtol=2e-2, atol=3e-2)
+    close(q.view(m, nh, d), q_want[:, :, order], what="q", **tol)
+    kc_c, vc_c = (c.cpu().double() for c in ops.cache_to_plain(kc, vc))   # by token and dimension
+    at = torch.tensor(slots)
+    close(kc_c[at // page, :, at % page, :], k_want[:, :, order], what="keys", **tol)
+    close(vc_c[at // page, :, :, at % page], v_want[:, :, order], what="values", **tol)
+    seen = torch.zeros(pages, page, dtype=torch.bool)
+    seen[at // page, at % page] = True
+    assert bool((kc_c.permute(0, 2, 1, 3)[~seen] == -7.5).all()) and bool((vc_c.permute(0, 3, 1, 2)[~seen] == -7.5).all()), "spill"
+    # the unfused pair: the product rounded to bfloat16 before it is rotated (either half of a pair is off by up to
+    # 2^-9 of itself there, and the rotation mixes the two), then rounded once more
+    kc2, vc2 = torch.full_like(kc, -7.5), torch.full_like(vc, -7.5)
+    buf = ops.gemm_fast(xin, wp.to(DEV), torch.bfloat16)
+    ops.rope_kv_write_blocks(buf, table, dev(slots), kc2, vc2, nh, nkv, d)
+    kc2, vc2 = ops.cache_to_plain(kc2, vc2)
+    twice = 2.0 ** -7 * float(qkv.abs().max())
+    close(kc2, kc_c, 1e-2, twice, "unfused keys")
+    close(vc2, vc_c, 1e-2, twice, "unfused values")
+    close(buf.view(m, nh + 2 * nkv, d)[:, :nh], q.view(m, nh, d), 1e-2, twice, "unfused queries")
+    # without the cache (a layer that reads another layer's): queries only
+    q_only = ops.gemm_qkv_rope_tiled(xin, wp.to(DEV), table, None, None, None, nh, nkv, d, write_kv=False)
+    assert torch.equal(q_only, q)
+    # a prompt portion's tokens lie one after the other in their pages (four tokens of a value dimension are then
+    # stored at once, where the four begin at a multiple of four): from the first place of a page, and from its fourth
+    for first in (page, page + 3):
+        run = [first + i for i in range(m)]
+        kc3, vc3 = torch.full_like(kc, -7.5), torch.full_like(vc, -7.5)
+        assert torch.equal(ops.gemm_qkv_rope_tiled(xin, wp.to(DEV), table, dev(run), kc3, vc3, nh, nkv, d), q)
+        kc3, vc3 = (c.cpu().double() for c in ops.cache_to_plain(kc3, vc3))
+        to = torch.tensor(run)
+        assert torch.equal(kc3[to // page, :, to % page, :], kc_c[at // page, :, at % page, :]), "the same keys, elsewhere"
+        assert torch.equal(vc3[to // page, :, :, to % page], vc_c[at // page, :, :, at % page]), "the same values, elsewhere"
+        free = torch.ones(pages, page, dtype=torch.bool)
+        free[to // page, to % page] = False
+        assert bool((kc3.permute(0, 2, 1, 3)[free] == -7.5).all()) and bool((vc3.permute(0, 3, 1, 2)[free] == -7.5).all()), "spill"
+
+
 @pytest.mark.parametrize("m", [1, 5, 8, 9, 16, 33, 64, 100])
 @pytest.mark.parametrize("width,k,gdt", [(96, 40, torch.bfloat16), (2048, 256, torch.bfloat16), (200, 72, torch.float32)])
 def test_adding_product_prepares_the_next_norm(ops, m, width, k, gdt):
