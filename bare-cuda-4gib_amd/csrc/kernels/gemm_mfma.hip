@@ -73,26 +73,48 @@ template <int EPI, int THREADS, int ROWS, int COLS>
 __device__ inline void store_patch(const float* patch, void* __restrict__ out, int m, int n, long m0, long n0, int tid) {
   constexpr int kStride = COLS + 4;
   if constexpr (EPI == kSwigluBf16) {
+    // (a block of 16 columns -- eight gates, then their eight ups -- a thread: eight outputs, stored at once)
     const long n_out = n / 2;
-    for (int c = tid; c < ROWS * (COLS / 8); c += THREADS) {
-      const int row = c / (COLS / 8), q = c % (COLS / 8);
-      const int col = (q / 2) * 16 + (q % 2) * 4;
+    for (int c = tid; c < ROWS * (COLS / 16); c += THREADS) {
+      const int row = c / (COLS / 16), col = (c % (COLS / 16)) * 16;
       const long gm = m0 + row, gn = n0 + col;
       if (gm >= m || gn >= n) continue;
       const float* src = patch + row * kStride + col;
-      float v[4];
+      const floatx4 g0 = *reinterpret_cast<const floatx4*>(src), g1 = *reinterpret_cast<const floatx4*>(src + 4);
+      const floatx4 u0 = *reinterpret_cast<const floatx4*>(src + 8), u1 = *reinterpret_cast<const floatx4*>(src + 12);
+      float v[8];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) v[e] = silu_quick(src[e]) * src[e + 8];
-      bf16_t* dst = static_cast<bf16_t*>(out) + gm * n_out + (gn / 16) * 8 + gn % 16;
-      if (n_out % 4 == 0) {
-        uint2 pk;
+      for (int e = 0; e < 4; ++e) {
+        v[e] = silu_quick(g0[e]) * u0[e];
+        v[4 + e] = silu_quick(g1[e]) * u1[e];
+      }
+      bf16_t* dst = static_cast<bf16_t*>(out) + gm * n_out + (gn / 16) * 8;
+      if (n_out % 8 == 0) {
+        uint4 pk;
         pk.x = static_cast<uint32_t>(bf16_bits_from_float(v[0])) | (static_cast<uint32_t>(bf16_bits_from_float(v[1])) << 16);
         pk.y = static_cast<uint32_t>(bf16_bits_from_float(v[2])) | (static_cast<uint32_t>(bf16_bits_from_float(v[3])) << 16);
-        *reinterpret_cast<uint2*>(dst) = pk;
+        pk.z = static_cast<uint32_t>(bf16_bits_from_float(v[4])) | (static_cast<uint32_t>(bf16_bits_from_float(v[5])) << 16);
+        pk.w = static_cast<uint32_t>(bf16_bits_from_float(v[6])) | (static_cast<uint32_t>(bf16_bits_from_float(v[7])) << 16);
+        *reinterpret_cast<uint4*>(dst) = pk;
       } else {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) dst[e] = from_float<bf16_t>(v[e]);
+        for (int e = 0; e < 8; ++e) dst[e] = from_float<bf16_t>(v[e]);
       }
+    }
+  } else if (EPI == kStoreBf16 && n % 8 == 0) {
+    // (eight columns a thread, stored at once: 16-byte stores where 8-byte ones were, 108 -> 102 us for a wide product)
+    for (int c = tid; c < ROWS * (COLS / 8); c += THREADS) {
+      const int row = c / (COLS / 8), col = (c % (COLS / 8)) * 8;
+      const long gm = m0 + row, gn = n0 + col;
+      if (gm >= m || gn >= n) continue;
+      const floatx4 v0 = *reinterpret_cast<const floatx4*>(patch + row * kStride + col);
+      const floatx4 v1 = *reinterpret_cast<const floatx4*>(patch + row * kStride + col + 4);
+      uint4 pk;
+      pk.x = static_cast<uint32_t>(bf16_bits_from_float(v0[0])) | (static_cast<uint32_t>(bf16_bits_from_float(v0[1])) << 16);
+      pk.y = static_cast<uint32_t>(bf16_bits_from_float(v0[2])) | (static_cast<uint32_t>(bf16_bits_from_float(v0[3])) << 16);
+      pk.z = static_cast<uint32_t>(bf16_bits_from_float(v1[0])) | (static_cast<uint32_t>(bf16_bits_from_float(v1[1])) << 16);
+      pk.w = static_cast<uint32_t>(bf16_bits_from_float(v1[2])) | (static_cast<uint32_t>(bf16_bits_from_float(v1[3])) << 16);
+      *reinterpret_cast<uint4*>(static_cast<bf16_t*>(out) + gm * n + gn) = pk;
     }
   } else {
     const bool vec = n % 4 == 0;
@@ -128,9 +150,9 @@ __device__ inline void store_patch(const float* patch, void* __restrict__ out, i
   }
 }
 
-// The q|k|v epilogue: THREADS threads take ROWS x COLS floats (stride COLS + 4) from LDS, four neighbouring columns a
-// thread -- half a block's eight dimensions, or half of their partners -- rotate them with what lies eight columns
-// away in the patch, and store queries to out [m, n_heads * head_dim], keys and values into their pages.
+// The q|k|v epilogue: THREADS threads take ROWS x COLS floats (stride COLS + 4) from LDS, eight neighbouring columns a
+// thread -- a block's eight dimensions, or their eight partners -- rotate them with what lies eight columns away in
+// the patch, and store queries to out [m, n_heads * head_dim], keys and values into their pages.
 template <int THREADS, int ROWS, int COLS>
 __device__ inline void store_patch_rope(const float* patch, bf16_t* __restrict__ out, int m, int n, long m0, long n0, int tid,
                                         const RopeKvArgs& ra) {
@@ -173,29 +195,40 @@ __device__ inline void store_patch_rope(const float* patch, bf16_t* __restrict__
     }
     return;
   }
-  for (int c = tid; c < ROWS * (COLS / 4); c += THREADS) {
-    const int row = c / (COLS / 4), col = (c % (COLS / 4)) * 4;
+  for (int c = tid; c < ROWS * (COLS / 8); c += THREADS) {
+    const int row = c / (COLS / 8), col = (c % (COLS / 8)) * 8;
     const long gm = m0 + row, gn = n0 + col;
     if (gm >= m || gn >= n) continue;
     const int head = static_cast<int>(gn / d), dim = static_cast<int>(gn % d);
     const bool is_q = head < ra.n_heads, is_v = head >= ra.n_heads + ra.n_kv_heads;
     if (!is_q && !ra.write_kv) continue;
-    floatx4 v = *reinterpret_cast<const floatx4*>(patch + row * kStride + col);
+    float v[8];
+    {
+      const floatx4 v0 = *reinterpret_cast<const floatx4*>(patch + row * kStride + col);
+      const floatx4 v1 = *reinterpret_cast<const floatx4*>(patch + row * kStride + col + 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = v0[e], v[4 + e] = v1[e];
+    }
     if (ra.table != nullptr && !is_v) {
-      const bool first = dim % 16 < 8;                       // the pairs' first halves; their partners lie 8 further
-      const floatx4 other = *reinterpret_cast<const floatx4*>(patch + row * kStride + (first ? col + 8 : col - 8));
-      const float2* cs = ra.table + gm * (d / 2) + (dim / 16) * 8 + dim % 8;
+      const bool first = dim % 16 < 8;                       // a block's eight first halves of pairs; their partners lie 8 further
+      const float* partner = patch + row * kStride + (first ? col + 8 : col - 8);
+      const floatx4 o0 = *reinterpret_cast<const floatx4*>(partner), o1 = *reinterpret_cast<const floatx4*>(partner + 4);
+      const floatx4* cs = reinterpret_cast<const floatx4*>(ra.table + gm * (d / 2) + (dim / 16) * 8);   // (cos, sin) of two pairs each
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const float2 a = cs[e];
-        v[e] = first ? v[e] * a.x - other[e] * a.y : v[e] * a.x + other[e] * a.y;
+        const floatx4 a = cs[e];
+        const float p0 = e < 2 ? o0[2 * e] : o1[2 * e - 4], p1 = e < 2 ? o0[2 * e + 1] : o1[2 * e - 3];
+        v[2 * e] = first ? v[2 * e] * a[0] - p0 * a[1] : v[2 * e] * a[0] + p0 * a[1];
+        v[2 * e + 1] = first ? v[2 * e + 1] * a[2] - p1 * a[3] : v[2 * e + 1] * a[2] + p1 * a[3];
       }
     }
-    uint2 pk;
+    uint4 pk;
     pk.x = static_cast<uint32_t>(bf16_bits_from_float(v[0])) | (static_cast<uint32_t>(bf16_bits_from_float(v[1])) << 16);
     pk.y = static_cast<uint32_t>(bf16_bits_from_float(v[2])) | (static_cast<uint32_t>(bf16_bits_from_float(v[3])) << 16);
+    pk.z = static_cast<uint32_t>(bf16_bits_from_float(v[4])) | (static_cast<uint32_t>(bf16_bits_from_float(v[5])) << 16);
+    pk.w = static_cast<uint32_t>(bf16_bits_from_float(v[6])) | (static_cast<uint32_t>(bf16_bits_from_float(v[7])) << 16);
     if (is_q) {
-      *reinterpret_cast<uint2*>(out + gm * (static_cast<long>(ra.n_heads) * d) + gn) = pk;
+      *reinterpret_cast<uint4*>(out + gm * (static_cast<long>(ra.n_heads) * d) + gn) = pk;
       continue;
     }
     const int slot = ra.slot_map[gm];
@@ -204,13 +237,13 @@ __device__ inline void store_patch_rope(const float* patch, bf16_t* __restrict__
     if (!is_v) {      // keys: [page][kv head][token][dim], or in fragment order: eight dimensions of 16 tokens together
       bf16_t* region = ra.k_cache + (page * ra.n_kv_heads + (head - ra.n_heads)) * ra.page_tokens * d;
       bf16_t* dst = ra.fragment_order ? region + frag_k_offset(off, dim, d) : region + static_cast<long>(off) * d + dim;
-      *reinterpret_cast<uint2*>(dst) = pk;
+      *reinterpret_cast<uint4*>(dst) = pk;
     } else {          // values are kept transposed: [page][kv head][dim][token], or in fragment order
       bf16_t* region = ra.v_cache + (page * ra.n_kv_heads + (head - ra.n_heads - ra.n_kv_heads)) * static_cast<long>(d) * ra.page_tokens;
       bf16_t* dst = ra.fragment_order ? region + frag_v_offset(off, dim, d) : region + static_cast<long>(dim) * ra.page_tokens + off;
       const long step = ra.fragment_order ? 4 : ra.page_tokens;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) dst[e * step] = from_float<bf16_t>(v[e]);
+      for (int e = 0; e < 8; ++e) dst[e * step] = from_float<bf16_t>(v[e]);
     }
   }
 }
