@@ -240,6 +240,37 @@ __global__ __launch_bounds__(kThreads, (XMODE != kPlain || (MT == 1 && U == 2)) 
     uint4 w[U];
     uint4 x[kNormed ? 1 : MT][kNormed ? 1 : U];
   };
+  // A batch that lies whole inside the wave's part of k can be loaded without a condition anywhere (rows past m read
+  // the last row: their results are never stored).  The compiler counts outstanding loads by instruction: where a load
+  // may be skipped it cannot know how many were issued after the ones it waits for and waits for all of them, and a
+  // copy from one set of registers to the other waits for the load it copies -- every batch then waits for the batch
+  // asked for just before it.  With 32 rows a workgroup and more, whole batches are loaded so and multiplied from the
+  // registers they were loaded into, two a turn (64 rows: the down projection of 5,632 10.9 -> 9.0 us, the others
+  // 2-4 % less); with 16 rows the plain loop is the faster one (4.2 against 4.7 us for a 2,048 x 2,048 block of weights).
+  constexpr bool kPingPong = MT >= 2;
+  const int last_row_offset = (m - 1) * k;              // (m <= 64 rows: an int)
+  int turn_offset[kTurned ? MT * U : 1];
+  if constexpr (kTurned) {
+#pragma unroll
+    for (int i = 0; i < MT * U; ++i) turn_offset[i] = min((turn_row + i * kRowsPerLoad) * k, last_row_offset) + turn_piece * 8;
+  }
+  const bf16_t* xptr_any[MT];                           // (the row itself, or the last row for rows past m)
+#pragma unroll
+  for (int t = 0; t < MT; ++t) xptr_any[t] = (kNormed || xrow_ok[t]) ? xptr[t] : static_cast<const bf16_t*>(a.x) + last_row_offset;
+  auto load_whole = [&](Batch& b, int k0) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      b.w[u] = load16(wblock + static_cast<long>(k0 / 32 + u) * (kWave * 8) + wlane);
+      if constexpr (!kNormed && !kTurned) {
+#pragma unroll
+        for (int t = 0; t < MT; ++t) b.x[t][u] = load16(xptr_any[t] + k0 + 32 * u + 8 * grp);
+      }
+    }
+    if constexpr (kTurned) {
+#pragma unroll
+      for (int i = 0; i < MT * U; ++i) b.x[i / U][i % U] = load16(static_cast<const bf16_t*>(a.x) + turn_offset[i] + k0);
+    }
+  };
   auto load = [&](Batch& b, int k0) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -366,11 +397,20 @@ __global__ __launch_bounds__(kThreads, (XMODE != kPlain || (MT == 1 && U == 2)) 
     sum_parts();
   }
 
-  for (int k0 = k_begin; k0 < k_end; k0 += kStep) {
-    const bool more = k0 + kStep < k_end;
-    if (more) load(nxt, k0 + kStep);
+  int k0 = k_begin;
+  while (kPingPong && k0 + 3 * kStep <= k_end) {
+    load_whole(nxt, k0 + kStep);
     compute(cur, k0);
-    if (more) cur = nxt;
+    load_whole(cur, k0 + 2 * kStep);
+    compute(nxt, k0 + kStep);
+    k0 += 2 * kStep;
+  }
+  for (; k0 < k_end; k0 += kStep) {
+    const int next = k0 + kStep;
+    if (kPingPong && next + kStep <= k_end) load_whole(nxt, next);
+    else if (next < k_end) load(nxt, next);
+    compute(cur, k0);
+    if (next < k_end) cur = nxt;
   }
 
   if constexpr (kTurned) __syncthreads();               // the partial sums take the buffers' place
