@@ -198,8 +198,9 @@ int bc4g_gemm_skinny_prenormed(const void* x, const float* ssq_parts, int ssq_bl
 extern "C" {
 // What the device delivers to a kernel that does nothing else (probes.hip): bc4g_probe_read reads
 // `bytes` of device memory once (sixteen 16-byte loads of a thread in flight); bc4g_probe_mfma runs
-// iters x 4 back-to-back 32x32x16 bfloat16 MFMAs in every one of its workgroups' four waves
-// (workgroups * 4 * iters * 4 * 32768 operations).  The caller times them.
+// iters x 16 back-to-back 32x32x16 bfloat16 MFMAs in every one of its workgroups' four waves
+// (workgroups * 4 * iters * 16 * 32768 operations) on the caller's operands, 12 * 256 * 16 bytes of bfloat16:
+// the rate depends on them (the clock follows the power that toggling operands draw).  The caller times them.
 int bc4g_probe_read(const void* p, long bytes, float* sink, int workgroups, void* stream);
-int bc4g_probe_mfma(int iters, float* sink, int workgroups, void* stream);
+int bc4g_probe_mfma(const void* operands, int iters, float* sink, int workgroups, void* stream);
 }

@@ -23,21 +23,29 @@ __global__ __launch_bounds__(256) void probe_read_kernel(const uint4* __restrict
   if (acc == 0x12345678u) sink[0] = 1.f;      // (keeps the loads alive; never true for the data the host fills in)
 }
 
-// Four independent chains of 32x32x16 bfloat16 MFMAs per wave, nothing else in the loop.
-__global__ __launch_bounds__(256) void probe_mfma_kernel(int iters, float* sink) {
-  bf16x8 a, b;
-  for (int i = 0; i < 8; ++i) {
-    a[i] = static_cast<__bf16>(threadIdx.x * 0.001f + i);
-    b[i] = static_cast<__bf16>(i * 0.5f);
-  }
-  floatx16 c0 = {}, c1 = {}, c2 = {}, c3 = {};
+// Eight independent chains of 32x32x16 bfloat16 MFMAs per wave (2 x 4 blocks from two and four fragments, two slices
+// of k), nothing else in the loop.  The operands come from memory, 12 fragments of 256 lanes x 16 bytes: what the
+// matrix cores sustain depends on them -- the chip lowers its clock with the power that toggling operands draw (zeros
+// and ones run at 2.1-2.2 GHz, normally distributed values at 1.7).
+__global__ __launch_bounds__(256) void probe_mfma_kernel(const uint4* operands, int iters, float* sink) {
+  uint4 a[2][2], b[4][2];
+  for (int i = 0; i < 2; ++i)
+    for (int s = 0; s < 2; ++s) a[i][s] = operands[(i * 2 + s) * 256 + threadIdx.x];
+  for (int j = 0; j < 4; ++j)
+    for (int s = 0; s < 2; ++s) b[j][s] = operands[(4 + j * 2 + s) * 256 + threadIdx.x];
+  floatx16 c[2][4] = {};
   for (int it = 0; it < iters; ++it) {
-    c0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c0, 0, 0, 0);
-    c1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c1, 0, 0, 0);
-    c2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c2, 0, 0, 0);
-    c3 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c3, 0, 0, 0);
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) c[i][j] = mfma_32x32x16(a[i][s], b[j][s], c[i][j]);
   }
-  sink[blockIdx.x * 256 + threadIdx.x] = c0[0] + c1[1] + c2[2] + c3[3];
+  float total = 0.f;
+  for (int i = 0; i < 2; ++i)
+    for (int j = 0; j < 4; ++j) total += c[i][j][threadIdx.x % 16];
+  sink[blockIdx.x * 256 + threadIdx.x] = total;
 }
 
 }  // namespace
@@ -51,9 +59,10 @@ extern "C" int bc4g_probe_read(const void* p, long bytes, float* sink, int workg
   return check_launch("probe_read");
 }
 
-// sink: float [workgroups * 256].  Operations of one launch: workgroups * 4 waves * iters * 4 * 2 * 32 * 32 * 16.
-extern "C" int bc4g_probe_mfma(int iters, float* sink, int workgroups, void* stream) {
-  BC4G_REQUIRE(sink && iters > 0 && workgroups > 0, "probe_mfma: a sink, a count and a grid are needed");
-  probe_mfma_kernel<<<workgroups, 256, 0, static_cast<hipStream_t>(stream)>>>(iters, sink);
+// operands: 12 * 256 * 16 bytes of bfloat16; sink: float [workgroups * 256].  Operations of one launch:
+// workgroups * 4 waves * iters * 16 * 2 * 32 * 32 * 16.
+extern "C" int bc4g_probe_mfma(const void* operands, int iters, float* sink, int workgroups, void* stream) {
+  BC4G_REQUIRE(operands && sink && iters > 0 && workgroups > 0, "probe_mfma: operands, a sink, a count and a grid are needed");
+  probe_mfma_kernel<<<workgroups, 256, 0, static_cast<hipStream_t>(stream)>>>(static_cast<const uint4*>(operands), iters, sink);
   return check_launch("probe_mfma");
 }

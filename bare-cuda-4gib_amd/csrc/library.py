@@ -28,7 +28,7 @@ _SIGNATURES = {
     "bc4g_sample": [_P, _P, _P, _P, _I, _I, _P],
     "bc4g_argmax_static": [_P, _P, _I, _I, _P],
     "bc4g_probe_read": [_P, c_long, _P, _I, _P],
-    "bc4g_probe_mfma": [_I, _P, _I, _P],
+    "bc4g_probe_mfma": [_P, _I, _P, _I, _P],
     "bc4g_gemm_skinny": [_P, _P, _P, _I, _I, _I, _I, _P],
     "bc4g_gemm_mfma": [_P, _P, _P, _I, _I, _I, _I, _P],
     "bc4g_gemm_mfma_tile": [_P, _P, _I, _I, _I, _P, _P],

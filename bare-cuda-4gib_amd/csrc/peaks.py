@@ -1,7 +1,10 @@
 """What this GPU delivers to a kernel that does nothing else, measured: memory bandwidth for a kernel
 that only reads, and the rate of back-to-back matrix-core instructions.  The published peaks (8 TB/s,
 2.5 PFLOP/s dense bfloat16) are what the benchmark's fractions are stated against; these are what a
-kernel on this machine can come to, and the benchmark programs state their results against both."""
+kernel on this machine can come to, and the benchmark programs state their results against both.
+The matrix cores' rate depends on their operands: the chip lowers its clock with the power that toggling
+operands draw, so it is measured twice -- on normally distributed values, like the benchmark's weights and
+activations (about 1.8 PFLOP/s), and on ones (about 2.3)."""
 from __future__ import annotations
 
 from typing import Dict
@@ -29,7 +32,8 @@ def _timed(fn, runs: int) -> float:
 
 def measured_peaks(device="cuda:0", read_bytes: int = 4 << 30, runs: int = 5) -> Dict[str, float]:
     """{"hbm_gbs": GB/s a read-only kernel reaches over a buffer far larger than the caches,
-    "bf16_tflops": TFLOP/s of nothing but 32x32x16 bfloat16 MFMAs} -- measured once per process and device."""
+    "bf16_tflops": TFLOP/s of nothing but 32x32x16 bfloat16 MFMAs on normally distributed operands,
+    "bf16_tflops_ones": the same on ones} -- measured once per process and device."""
     dev = torch.device(device)
     index = dev.index if dev.index is not None else torch.cuda.current_device()
     if index in _cache:
@@ -45,10 +49,13 @@ def measured_peaks(device="cuda:0", read_bytes: int = 4 << 30, runs: int = 5) ->
         read()
         hbm = read_bytes / (_timed(read, runs) * 1e-3) / 1e9
         del buf
-        iters, groups = 20000, cus * 4
-        mfma = lambda: library.call("bc4g_probe_mfma", iters, sink.data_ptr(), groups, _stream())
-        library.call("bc4g_probe_mfma", 100, sink.data_ptr(), groups, _stream())
-        flops = groups * 4 * iters * 4 * 2.0 * 32 * 32 * 16
-        tflops = flops / (_timed(mfma, max(2, runs // 2)) * 1e-3) / 1e12
-    _cache[index] = {"hbm_gbs": round(hbm, 1), "bf16_tflops": round(tflops, 1)}
+        iters, groups = 20000, cus                          # a workgroup of four waves a CU: a wave a SIMD
+        flops = groups * 4 * iters * 16 * 2.0 * 32 * 32 * 16
+        rates = {}
+        for name, operands in (("bf16_tflops", torch.randn(12 * 256 * 8, device=dev).bfloat16()),
+                               ("bf16_tflops_ones", torch.ones(12 * 256 * 8, device=dev).bfloat16())):
+            mfma = lambda: library.call("bc4g_probe_mfma", operands.data_ptr(), iters, sink.data_ptr(), groups, _stream())
+            library.call("bc4g_probe_mfma", operands.data_ptr(), 100, sink.data_ptr(), groups, _stream())
+            rates[name] = round(flops / (_timed(mfma, max(2, runs // 2)) * 1e-3) / 1e12, 1)
+    _cache[index] = {"hbm_gbs": round(hbm, 1), **rates}
     return _cache[index]
