@@ -137,11 +137,13 @@ def test_gemm_mfma(ops, m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k,tile", [(4096 - 236, 4096 - 244, 192, (256, 256)), (2048 - 20, 6144 - 12, 192, (256, 192)),
+                                        (4096 - 20, 6144 - 12, 64, (256, 192)), (4096 - 20, 6144 - 12, 128, (256, 192)),
                                         (2048 - 20, 4096 - 12, 192, (256, 128)), (2048 - 20, 2048 - 12, 1024, (128, 64))])
 def test_gemm_mfma_every_tile_agrees_bit_for_bit(ops, m, n, k, tile):
     """Five tiles for the operands that go straight into LDS, chosen by the output's shape.  All add over k in
     the same order: a row's result is the same bits whichever tile the number of rows selects (the first 300 rows
-    alone take the smallest), with edges in both directions, for every epilogue."""
+    alone take the smallest), with edges in both directions, for every epilogue.  The 256 x 192 tile's waves take
+    turns half a step apart: one and two steps of k are its shortest walks."""
     if torch.cuda.get_device_properties(0).multi_processor_count != 256:
         pytest.skip("the shapes are chosen for 256 CUs")
     assert ops.tiled_tile(m, n, k) == tile and ops.tiled_tile(300, n, k) == (64, 64)
