@@ -244,10 +244,12 @@ __global__ __launch_bounds__(kThreads, (XMODE != kPlain || (MT == 1 && U == 2)) 
   // the last row: their results are never stored).  The compiler counts outstanding loads by instruction: where a load
   // may be skipped it cannot know how many were issued after the ones it waits for and waits for all of them, and a
   // copy from one set of registers to the other waits for the load it copies -- every batch then waits for the batch
-  // asked for just before it.  With 32 rows a workgroup and more, whole batches are loaded so and multiplied from the
-  // registers they were loaded into, two a turn (64 rows: the down projection of 5,632 10.9 -> 9.0 us, the others
-  // 2-4 % less); with 16 rows the plain loop is the faster one (4.2 against 4.7 us for a 2,048 x 2,048 block of weights).
-  constexpr bool kPingPong = MT >= 2;
+  // asked for just before it.  With 32 rows a workgroup, whole batches are loaded so and multiplied from the
+  // registers they were loaded into, two a turn (64 rows as two workgroups of 32: the down projection of 5,632
+  // 10.9 -> 9.0 us, the others 2-4 % less); with 16 rows the plain loop is the faster one (4.2 against 4.7 us for a
+  // 2,048 x 2,048 block of weights), and with 48 and 64 rows a workgroup the second set of registers does not fit the
+  // 128 a wave has (spilled, the q|k|v product of 64 rows and 4,096 columns took 127 instead of 44 us).
+  constexpr bool kPingPong = MT == 2;
   const int last_row_offset = (m - 1) * k;              // (m <= 64 rows: an int)
   int turn_offset[kTurned ? MT * U : 1];
   if constexpr (kTurned) {
