@@ -22,7 +22,6 @@
 //
 // Workgroups are numbered so that those sharing rows of a and of w run on the same XCD at the same
 // time (tile_of).
-#include <type_traits>
 #include <math.h>
 
 #include "api.h"
@@ -417,9 +416,6 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_staged_kernel(
 // all LDS cycles were conflicts).  A wave-wide load covers 1024 / (BK * 2) rows; which segment a lane
 // brings follows from where its 16 bytes land.
 //
-// TURNS (the 256 x 192 tile): the eight waves are two groups that take turns at the matrix cores and at LDS; see the
-// loop.  With eight waves of 128 x 64 for a 256 x 256 tile it is as fast as the sixteen waves of 64 x 64 and no faster.
-//
 // WM x WN waves take TM x TN MFMA blocks of 32 x 32 each.  An output element is added up over k in
 // ascending order, as in the form above: the same bits whichever form the shape selects.
 // k must be a multiple of BK; rows beyond m or n are read from the last row and not stored.
@@ -430,14 +426,6 @@ __device__ inline void wait_for_stage(int later) {
   } else {
     if (later >= MAX) wait_loads<PER * MAX>();
     else wait_for_stage<PER, MAX - 1>(later);
-  }
-}
-
-template <int I, int N, class F>
-__device__ inline void static_for(F&& f) {
-  if constexpr (I < N) {
-    f(std::integral_constant<int, I>{});
-    static_for<I + 1, N>(f);
   }
 }
 
@@ -457,7 +445,7 @@ struct DirectShape {
   static_assert(kRowBytes == 128 || kRowBytes == 256, "rows of 128 or 256 bytes (the slot rule)");
 };
 
-template <int EPI, int WM, int WN, int TM, int TN, int BK, int STAGES, int MINWG, bool TURNS = false>
+template <int EPI, int WM, int WN, int TM, int TN, int BK, int STAGES, int MINWG>
 __global__ __launch_bounds__(64 * WM * WN, MINWG) void gemm_mfma_direct_kernel(
     const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, void* __restrict__ out, int m, int n, int k, int m_blocks,
     int n_blocks, const RopeKvArgs ra) {
@@ -482,8 +470,7 @@ __global__ __launch_bounds__(64 * WM * WN, MINWG) void gemm_mfma_direct_kernel(
   unsigned dst[PER];
 #pragma unroll
   for (int i = 0; i < PER; ++i) {
-    // (TURNS: a wave's groups lie side by side in LDS, so that one setting of the LDS address serves eight loads)
-    int g = TURNS ? wave * PER + i : wave + NW * i;
+    int g = wave + NW * i;
     if (g >= GA + GW) g = GA + GW - 1;
     const bool of_a = g < GA;
     const int trow = (of_a ? g : g - GA) * kGroupRows + lr;
@@ -494,26 +481,11 @@ __global__ __launch_bounds__(64 * WM * WN, MINWG) void gemm_mfma_direct_kernel(
     src[i] = reinterpret_cast<const unsigned char*>((of_a ? a : w) + row * k) + seg * 16;
     dst[i] = (of_a ? 0 : RA * RB) + (of_a ? g : g - GA) * 1024;
   }
-  static_assert(!TURNS || ((GA + GW) % NW == 0 && PER <= 8), "every wave the same number of groups, eight at most");
-  // TURNS: a wave's groups lie side by side in LDS; the LDS address is set once for the loads that follow (to the wave's
-  // fifth group, which the instructions' offsets of -4 .. 3 KB turn into the eight)
-  auto ask_from = [&](int step) {
-    set_lds_base(__builtin_amdgcn_readfirstlane(lds_base + (step % STAGES) * S::kStageBytes + dst[0] + 4096));
-  };
-  auto ask_one = [&](int step, auto at) {
-    constexpr int i = decltype(at)::value;
-    load_to_lds_16_at<i * 1024 - 4096>(src[i] + static_cast<size_t>(step) * RB);
-  };
   auto ask = [&](int step) {
     const unsigned base = lds_base + (step % STAGES) * S::kStageBytes;
-    if constexpr (TURNS) {
-      ask_from(step);
-      static_for<0, PER>([&](auto at) { ask_one(step, at); });
-    } else {
 #pragma unroll
-      for (int i = 0; i < PER; ++i)
-        load_to_lds_16(src[i] + static_cast<size_t>(step) * RB, __builtin_amdgcn_readfirstlane(base + dst[i]));
-    }
+    for (int i = 0; i < PER; ++i)
+      load_to_lds_16(src[i] + static_cast<size_t>(step) * RB, __builtin_amdgcn_readfirstlane(base + dst[i]));
   };
 
   floatx16 acc[TM][TN];
@@ -553,85 +525,30 @@ __global__ __launch_bounds__(64 * WM * WN, MINWG) void gemm_mfma_direct_kernel(
     for (int j = 0; j < TN; ++j) fw[set][j] = *reinterpret_cast<const uint4*>(stage + woff[j] + ((s ^ wswz[j]) * 16));
   };
 
-  if constexpr (TURNS) {
-    // Two waves a SIMD that take turns: while one multiplies a whole step from registers, the other reads its fragments
-    // of a step from LDS -- the matrix cores always have a wave that does nothing else.  The waves are two groups (a
-    // SIMD's two waves are wave w and w + kWaves / 2) whose turns are half a step apart, kept so by the barriers between
-    // the turns: in turn 2t the first group reads step t while the second multiplies step t - 1; in turn 2t + 1 the
-    // first multiplies step t and the second reads it.  Step t + 1 is asked for in turn 2t (its buffer was last read in
-    // turn 2t - 1) and waited for before the barrier that ends turn 2t + 1.  A load costs the wave that asks for it 50
-    // to 100 clocks (the CU's path takes a wave-wide load every 19 clocks; when all waves ask at once, each is held for
-    // most of a turn): the first group asks after its reads, the second between its matrix instructions, one load
-    // after every third.
-    static_assert(STAGES == 2 && NW % 2 == 0, "two buffers, two groups of waves");
-    constexpr int kSlicesAll = BK / 16;
-    uint4 ra_[kSlicesAll][TM], rw_[kSlicesAll][TN];
-    const bool second = wave >= NW / 2;
-    auto read_step = [&](int t) {
-      const unsigned char* stage = direct_lds + (t % 2) * S::kStageBytes;
+  for (int t = 0; t < nk; ++t) {
+    // step t has landed once only the steps asked for after it are outstanding
+    wait_for_stage<PER, STAGES - 2>(min(nk - 1, t + STAGES - 2) - t);
+    lds_barrier();          // everybody's part of step t is there, and nobody reads step t - 1 any more
+    if (t + STAGES - 1 < nk) ask(t + STAGES - 1);
+    const unsigned char* stage = direct_lds + (t % STAGES) * S::kStageBytes;
+    read_fragments(0, stage, 0);
+    __builtin_amdgcn_sched_group_barrier(0x100, TM + TN, 0);
 #pragma unroll
-      for (int ks = 0; ks < kSlicesAll; ++ks) {
-        const int sl = ks * 2 + fhalf;
-#pragma unroll
-        for (int i = 0; i < TM; ++i) ra_[ks][i] = *reinterpret_cast<const uint4*>(stage + aoff[i] + ((sl ^ aswz[i]) * 16));
-#pragma unroll
-        for (int j = 0; j < TN; ++j) rw_[ks][j] = *reinterpret_cast<const uint4*>(stage + woff[j] + ((sl ^ wswz[j]) * 16));
+    for (int ks = 0; ks < kSlices; ++ks) {
+      // the next slice's fragments are asked for before this slice's MFMAs, which hide the wait (the
+      // order is pinned: left alone, the compiler moves the reads down to where their registers come free)
+      if (ks + 1 < kSlices) {
+        read_fragments((ks + 1) % 2, stage, ks + 1);
+        __builtin_amdgcn_sched_group_barrier(0x100, TM + TN, 0);
       }
-    };
-    constexpr int kEvery = 3;
-    static_assert(kSlicesAll * TM * TN >= kEvery * PER, "a place for every load among the matrix instructions");
-    auto multiply_step = [&](bool asking, int step) {
-      if (asking) ask_from(step);
-      static_for<0, kSlicesAll * TM * TN>([&](auto at) {
-        constexpr int x = decltype(at)::value, ks = x / (TM * TN), i = x / TN % TM, j = x % TN;
-        acc[i][j] = mfma_32x32x16(ra_[ks][i], rw_[ks][j], acc[i][j]);
-        if constexpr (x % kEvery == kEvery - 1 && x / kEvery < PER) {
-          if (asking) ask_one(step, std::integral_constant<int, x / kEvery>{});
-        }
-      });
-    };
-    wait_loads<0>();
-    lds_barrier();                                  // step 0 is there
-    if (second) {                                   // turn 0 of the second group: nothing to multiply yet
-      if (1 < nk) ask(1);
-      lds_barrier();
-    }
-    for (int t = 0; t < nk; ++t) {
-      read_step(t);
-      if (!second && t + 1 < nk) ask(t + 1);
-      if (second) wait_loads<0>();
-      lds_barrier();
-      multiply_step(second && t + 2 < nk, t + 2);
-      if (!second) wait_loads<0>();
-      lds_barrier();
-    }
-    if (!second) lds_barrier();                     // (the second group's last turn)
-  } else {
-    for (int t = 0; t < nk; ++t) {
-      // step t has landed once only the steps asked for after it are outstanding
-      wait_for_stage<PER, STAGES - 2>(min(nk - 1, t + STAGES - 2) - t);
-      lds_barrier();          // everybody's part of step t is there, and nobody reads step t - 1 any more
-      if (t + STAGES - 1 < nk) ask(t + STAGES - 1);
-      const unsigned char* stage = direct_lds + (t % STAGES) * S::kStageBytes;
-      read_fragments(0, stage, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, TM + TN, 0);
 #pragma unroll
-      for (int ks = 0; ks < kSlices; ++ks) {
-        // the next slice's fragments are asked for before this slice's MFMAs, which hide the wait (the
-        // order is pinned: left alone, the compiler moves the reads down to where their registers come free)
-        if (ks + 1 < kSlices) {
-          read_fragments((ks + 1) % 2, stage, ks + 1);
-          __builtin_amdgcn_sched_group_barrier(0x100, TM + TN, 0);
-        }
+      for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-          for (int j = 0; j < TN; ++j) acc[i][j] = mfma_32x32x16(fa[ks % 2][i], fw[ks % 2][j], acc[i][j]);
-        __builtin_amdgcn_sched_group_barrier(0x008, TM * TN, 0);
-      }
+        for (int j = 0; j < TN; ++j) acc[i][j] = mfma_32x32x16(fa[ks % 2][i], fw[ks % 2][j], acc[i][j]);
+      __builtin_amdgcn_sched_group_barrier(0x008, TM * TN, 0);
     }
-    lds_barrier();          // the last step has been read: LDS is free for the output
   }
+  lds_barrier();            // the last step has been read: LDS is free for the output
 
   // The tile goes out through LDS so that a thread stores four neighbouring columns of a row at once:
   // every wave for itself, 32 rows of its part at a time through a patch of its own (no barrier).
@@ -651,10 +568,10 @@ __global__ __launch_bounds__(64 * WM * WN, MINWG) void gemm_mfma_direct_kernel(
   }
 }
 
-template <int EPI, int WM, int WN, int TM, int TN, int BK, int STAGES, int MINWG, bool TURNS = false>
+template <int EPI, int WM, int WN, int TM, int TN, int BK, int STAGES, int MINWG>
 int launch_direct(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, int k, hipStream_t s, const RopeKvArgs& ra) {
   typedef DirectShape<WM, WN, TM, TN, BK, STAGES> S;
-  auto kernel = gemm_mfma_direct_kernel<EPI, WM, WN, TM, TN, BK, STAGES, MINWG, TURNS>;
+  auto kernel = gemm_mfma_direct_kernel<EPI, WM, WN, TM, TN, BK, STAGES, MINWG>;
   static bool raised = false;   // per instantiation: allow more than the default dynamic LDS
   if (!raised) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -701,7 +618,7 @@ int launch_direct_form(const bf16_t* ap, const bf16_t* wp, void* out, int m, int
                        const RopeKvArgs& ra = RopeKvArgs{}) {
   switch (direct_form(m, n, k)) {
     case 0: return launch_direct<EPI, 4, 4, 2, 2, 64, 2, 1>(ap, wp, out, m, n, k, s, ra);
-    case 1: return launch_direct<EPI, 4, 2, 2, 3, 64, 2, 1, true>(ap, wp, out, m, n, k, s, ra);
+    case 1: return launch_direct<EPI, 4, 2, 2, 3, 64, 2, 1>(ap, wp, out, m, n, k, s, ra);
     case 2: return launch_direct<EPI, 4, 2, 2, 2, 64, 2, 1>(ap, wp, out, m, n, k, s, ra);
     case 3: return launch_direct<EPI, 2, 2, 2, 1, 64, 2, 4>(ap, wp, out, m, n, k, s, ra);
     default: return launch_direct<EPI, 2, 2, 1, 1, 64, 4, 2>(ap, wp, out, m, n, k, s, ra);

@@ -74,13 +74,6 @@ __device__ inline void load_to_lds_16_at(const void* wave_base, unsigned lane_of
   asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" ::"v"(lane_offset), "s"(wave_base), "n"(OFFSET) : "memory");
 }
 
-// (each lane with an address of its own)
-template <int OFFSET>
-__device__ inline void load_to_lds_16_at(const void* global) {
-  static_assert(OFFSET >= -4096 && OFFSET <= 4095, "the instruction's offset field");
-  asm volatile("global_load_lds_dwordx4 %0, off offset:%1" ::"v"(static_cast<const char*>(global) - OFFSET), "n"(OFFSET) : "memory");
-}
-
 // Waits until at most N of the wave's memory operations are outstanding (they finish in order).
 template <int N>
 __device__ inline void wait_loads() {
