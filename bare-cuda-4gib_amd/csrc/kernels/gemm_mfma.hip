@@ -6,7 +6,7 @@
 // and feeds 32x32x16 MFMAs.  Two forms:
 //  - gemm_mfma_direct_kernel: the operand tiles go from memory into LDS without passing registers
 //    (k a multiple of 64, operands on 16-byte boundaries).  Tiles of 256 x 256, 256 x 192,
-//    256 x 128, 128 x 64 or 64 x 64, whichever lets the busiest CU finish first.
+//    256 x 128, 128 x 128 or 64 x 64, whichever lets the busiest CU finish first.
 //  - gemm_mfma_staged_kernel: through registers, 128 x 128 tiles; any k that is a multiple of 8.
 // Every output element is accumulated over k in ascending order in both, whatever the number of
 // rows and the tile: the same bits whichever form and tile a shape selects.
@@ -16,7 +16,7 @@
 // of a tile's time, with the matrix cores busy 40-50 % of it -- a step's loads, fragment reads and
 // MFMAs overlap only so far between two barriers, although LDS (no bank conflicts, a third of its
 // cycles in use) and memory (a ring of three stages is no faster than one of two) both have room;
-// the small tiles are bound by what all CUs pull from L2 together (19 TB/s for 128 x 64); the rest
+// a tile of 128 x 64 was bound by what all CUs pull from L2 together (19 TB/s); the rest
 // is the stores after the loop, which all CUs issue at the same time.  More waves a CU (this form
 // spends no registers on staging) and larger tiles (less traffic per FLOP) are what helped.
 //
@@ -590,13 +590,22 @@ int launch_direct(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, i
 // faster than its k-steps follow each other when nothing else hides their latency (microseconds a step,
 // measured on shapes with fewer tiles than CUs: the small tile with four stages is for those).  A
 // function of (m, n, k) alone; every tile adds over k in the same order.
+// The rates are measured with the weights coming from memory, as they do inside a model (the caches filled
+// with other data before each run, then the activations and the output touched): a loop over one product
+// finds its weights in the 256 MB cache before memory and flatters the small tiles and the short rings --
+// 128 x 64 with two stages sustains 3.2 TFLOP/s a CU in such a loop and 2.2-2.4 behind a layer's other
+// kernels.  So the tiles that leave room in LDS keep more steps in flight: 128 x 128 (eight waves of 64 x 32,
+// four stages) took the place of 128 x 64 with two stages and four workgroups a CU, which no shape selects any
+// more (a product takes 20-29 % less time where it was selected: 2,048 x 2,048 x 5,632 85 -> 65 us), and 256 x 128
+// has three stages (5-18 % less than with two).  Five stages for 128 x 128, three for 128 x 64 (then two
+// workgroups a CU) and 128 x 128 with four waves of 64 x 64 were no better or worse.
 struct DirectForm {
   int rows, cols;
   double tflops_a_cu, us_a_step;
 };
 constexpr int kDirectForms = 5;
 constexpr DirectForm kDirectForm[kDirectForms] = {
-    {256, 256, 4.45, 0.5}, {256, 192, 3.9, 0.5}, {256, 128, 3.7, 0.5}, {128, 64, 3.2, 0.5}, {64, 64, 2.2, 0.28}};
+    {256, 256, 4.45, 0.5}, {256, 192, 3.9, 0.5}, {256, 128, 3.8, 0.5}, {128, 128, 3.1, 0.5}, {64, 64, 2.2, 0.28}};
 
 int direct_form(int m, int n, int k) {
   int best = 0;
@@ -619,8 +628,8 @@ int launch_direct_form(const bf16_t* ap, const bf16_t* wp, void* out, int m, int
   switch (direct_form(m, n, k)) {
     case 0: return launch_direct<EPI, 4, 4, 2, 2, 64, 2, 1>(ap, wp, out, m, n, k, s, ra);
     case 1: return launch_direct<EPI, 4, 2, 2, 3, 64, 2, 1>(ap, wp, out, m, n, k, s, ra);
-    case 2: return launch_direct<EPI, 4, 2, 2, 2, 64, 2, 1>(ap, wp, out, m, n, k, s, ra);
-    case 3: return launch_direct<EPI, 2, 2, 2, 1, 64, 2, 4>(ap, wp, out, m, n, k, s, ra);
+    case 2: return launch_direct<EPI, 4, 2, 2, 2, 64, 3, 1>(ap, wp, out, m, n, k, s, ra);
+    case 3: return launch_direct<EPI, 2, 4, 2, 1, 64, 4, 1>(ap, wp, out, m, n, k, s, ra);
     default: return launch_direct<EPI, 2, 2, 1, 1, 64, 4, 2>(ap, wp, out, m, n, k, s, ra);
   }
 }

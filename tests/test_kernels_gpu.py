@@ -138,7 +138,7 @@ def test_gemm_mfma(ops, m, n, k):
 
 @pytest.mark.parametrize("m,n,k,tile", [(4096 - 236, 4096 - 244, 192, (256, 256)), (2048 - 20, 6144 - 12, 192, (256, 192)),
                                         (4096 - 20, 6144 - 12, 64, (256, 192)), (4096 - 20, 6144 - 12, 128, (256, 192)),
-                                        (2048 - 20, 4096 - 12, 192, (256, 128)), (2048 - 20, 2048 - 12, 1024, (128, 64))])
+                                        (2048 - 20, 4096 - 12, 192, (256, 128)), (2048 - 20, 2048 - 12, 1024, (128, 128))])
 def test_gemm_mfma_every_tile_agrees_bit_for_bit(ops, m, n, k, tile):
     """Five tiles for the operands that go straight into LDS, chosen by the output's shape.  All add over k in
     the same order: a row's result is the same bits whichever tile the number of rows selects (the first 300 rows
