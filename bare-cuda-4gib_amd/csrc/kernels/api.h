@@ -145,9 +145,9 @@ extern "C" {
 // bfloat16 a [m, k] times bfloat16 w [n, k] transposed on the matrix cores, any m.
 // epilogue: 0 store bfloat16; 1 store float32; 2 add into float32; 3 SwiGLU as in bc4g_gemm_skinny.
 int bc4g_gemm_mfma(const void* a, const void* w, void* out, int epilogue, int m, int n, int k, void* stream);
-// The output tile (rows, columns) bc4g_gemm_mfma takes for these operands: for the accounting of bytes and for
-// tests that want to meet every tile.  Launches nothing.
-int bc4g_gemm_mfma_tile(const void* a, const void* w, int m, int n, int k, int* rows, int* cols);
+// The output tile (rows, columns) bc4g_gemm_mfma (qkv 0) or bc4g_gemm_mfma_qkv (qkv 1) takes for these operands: for
+// the accounting of bytes and for tests that want to meet every tile.  Launches nothing.
+int bc4g_gemm_mfma_tile(const void* a, const void* w, int m, int n, int k, int qkv, int* rows, int* cols);
 // The q|k|v product of many rows with rotation and cache write in its epilogue, as bc4g_gemm_skinny_qkv for few (k a
 // multiple of 64, operands on 16-byte boundaries): w [n, k] holds n_heads query, n_kv_heads key and as many value heads of
 // head_dim (a multiple of 16), every head's rows in blocks of eight dimensions followed by their rotation partners.  out

@@ -6,7 +6,7 @@
 // and feeds 32x32x16 MFMAs.  Two forms:
 //  - gemm_mfma_direct_kernel: the operand tiles go from memory into LDS without passing registers
 //    (k a multiple of 64, operands on 16-byte boundaries).  Tiles of 256 x 256, 256 x 192,
-//    256 x 128, 128 x 128 or 64 x 64, whichever lets the busiest CU finish first.
+//    256 x 128, 128 x 128 or 64 x 64 (and 128 x 64 for q|k|v), whichever lets the busiest CU finish first.
 //  - gemm_mfma_staged_kernel: through registers, 128 x 128 tiles; any k that is a multiple of 8.
 // Every output element is accumulated over k in ascending order in both, whatever the number of
 // rows and the tile: the same bits whichever form and tile a shape selects.
@@ -596,21 +596,24 @@ int launch_direct(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, i
 // 128 x 64 with two stages sustains 3.2 TFLOP/s a CU in such a loop and 2.2-2.4 behind a layer's other
 // kernels.  So the tiles that leave room in LDS keep more steps in flight: 128 x 128 (eight waves of 64 x 32,
 // four stages) took the place of 128 x 64 with two stages and four workgroups a CU, which no shape selects any
-// more (a product takes 20-29 % less time where it was selected: 2,048 x 2,048 x 5,632 85 -> 65 us), and 256 x 128
+// more but the q|k|v product (a product takes 20-29 % less time where it was selected: 2,048 x 2,048 x 5,632 85 -> 65 us), and 256 x 128
 // has three stages (5-18 % less than with two).  Five stages for 128 x 128, three for 128 x 64 (then two
 // workgroups a CU) and 128 x 128 with four waves of 64 x 64 were no better or worse.
 struct DirectForm {
   int rows, cols;
   double tflops_a_cu, us_a_step;
 };
-constexpr int kDirectForms = 5;
+// The last, 128 x 64 with two stages and four workgroups a CU, is for the q|k|v epilogue alone: what comes after the
+// loop is long there (rotation, three destinations), and several workgroups a CU run it beside each other's loops
+// (a 2,048-token TinyLlama prompt 1 % faster with it than with 160 tiles of 256 x 128, both libraries in one process).
+constexpr int kDirectForms = 6;
 constexpr DirectForm kDirectForm[kDirectForms] = {
-    {256, 256, 4.45, 0.5}, {256, 192, 3.9, 0.5}, {256, 128, 3.8, 0.5}, {128, 128, 3.1, 0.5}, {64, 64, 2.2, 0.28}};
+    {256, 256, 4.45, 0.5}, {256, 192, 3.9, 0.5}, {256, 128, 3.8, 0.5}, {128, 128, 3.1, 0.5}, {64, 64, 2.2, 0.28}, {128, 64, 2.9, 0.5}};
 
-int direct_form(int m, int n, int k) {
+int direct_form(int m, int n, int k, bool long_epilogue) {
   int best = 0;
   double best_time = 0.0;
-  for (int f = 0; f < kDirectForms; ++f) {
+  for (int f = 0; f < (long_epilogue ? kDirectForms : kDirectForms - 1); ++f) {
     const DirectForm& form = kDirectForm[f];
     const long tiles = static_cast<long>((m + form.rows - 1) / form.rows) * ((n + form.cols - 1) / form.cols);
     const long turns = (tiles + compute_units() - 1) / compute_units();
@@ -625,11 +628,12 @@ int direct_form(int m, int n, int k) {
 template <int EPI>
 int launch_direct_form(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, int k, hipStream_t s,
                        const RopeKvArgs& ra = RopeKvArgs{}) {
-  switch (direct_form(m, n, k)) {
+  switch (direct_form(m, n, k, EPI == kRopeKvBf16)) {
     case 0: return launch_direct<EPI, 4, 4, 2, 2, 64, 2, 1>(ap, wp, out, m, n, k, s, ra);
     case 1: return launch_direct<EPI, 4, 2, 2, 3, 64, 2, 1>(ap, wp, out, m, n, k, s, ra);
     case 2: return launch_direct<EPI, 4, 2, 2, 2, 64, 3, 1>(ap, wp, out, m, n, k, s, ra);
     case 3: return launch_direct<EPI, 2, 4, 2, 1, 64, 4, 1>(ap, wp, out, m, n, k, s, ra);
+    case 5: return launch_direct<EPI, 2, 2, 2, 1, 64, 2, 4>(ap, wp, out, m, n, k, s, ra);
     default: return launch_direct<EPI, 2, 2, 1, 1, 64, 4, 2>(ap, wp, out, m, n, k, s, ra);
   }
 }
@@ -704,10 +708,10 @@ extern "C" int bc4g_gemm_mfma_qkv(const void* a, const void* w, void* out, const
   return check_launch("gemm_mfma_qkv");
 }
 
-extern "C" int bc4g_gemm_mfma_tile(const void* a, const void* w, int m, int n, int k, int* rows, int* cols) {
+extern "C" int bc4g_gemm_mfma_tile(const void* a, const void* w, int m, int n, int k, int qkv, int* rows, int* cols) {
   BC4G_REQUIRE(rows != nullptr && cols != nullptr && m > 0 && n > 0 && k > 0, "gemm_mfma_tile: sizes and two places for the answer");
   if (direct_operands(a, w, k)) {
-    const DirectForm& form = kDirectForm[direct_form(m, n, k)];
+    const DirectForm& form = kDirectForm[direct_form(m, n, k, qkv != 0)];
     *rows = form.rows, *cols = form.cols;
   } else {
     *rows = kBM, *cols = kBN;

@@ -31,7 +31,7 @@ _SIGNATURES = {
     "bc4g_probe_mfma": [_P, _I, _P, _I, _P],
     "bc4g_gemm_skinny": [_P, _P, _P, _I, _I, _I, _I, _P],
     "bc4g_gemm_mfma": [_P, _P, _P, _I, _I, _I, _I, _P],
-    "bc4g_gemm_mfma_tile": [_P, _P, _I, _I, _I, _P, _P],
+    "bc4g_gemm_mfma_tile": [_P, _P, _I, _I, _I, _I, _P, _P],
     "bc4g_gemm_skinny_normed": [_P, _P, _P, _I, _F, _P, _P, _I, _I, _I, _I, _P],
     "bc4g_attention_mfma": [_P, _I, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _P, _I, _P, _I, _P, _P],
     "bc4g_gemm_mfma_qkv": [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P],

@@ -67,18 +67,18 @@ def _skinny_cost(m: int, n: int, k: int, in_bytes: int, out_bytes: float):
     return _gemm_cost(m, n, k, in_bytes, 2, out_bytes, x_readers=-(-n // 16))
 
 
-def tiled_tile(m: int, n: int, k: int, a_ptr: int = 0, w_ptr: int = 0) -> Tuple[int, int]:
+def tiled_tile(m: int, n: int, k: int, a_ptr: int = 0, w_ptr: int = 0, qkv: bool = False) -> Tuple[int, int]:
     """(rows, columns) of the output tile the tiled matrix-core kernel takes for an [m, k] x [n, k]^T product of
-    operands at these addresses (0: well aligned)."""
+    operands at these addresses (0: well aligned); ``qkv``: the product with rotation and cache write after it."""
     rows, cols = ctypes.c_int(0), ctypes.c_int(0)
-    library.call("bc4g_gemm_mfma_tile", a_ptr or None, w_ptr or None, m, n, k, ctypes.byref(rows), ctypes.byref(cols),
-                 launches=False)
+    library.call("bc4g_gemm_mfma_tile", a_ptr or None, w_ptr or None, m, n, k, int(qkv), ctypes.byref(rows),
+                 ctypes.byref(cols), launches=False)
     return rows.value, cols.value
 
 
-def _tiled_cost(m: int, n: int, k: int, out_bytes: float):
+def _tiled_cost(m: int, n: int, k: int, out_bytes: float, qkv: bool = False):
     def cost():                                    # asked for by the profiler only: the tile is looked up then
-        rows, cols = tiled_tile(m, n, k)
+        rows, cols = tiled_tile(m, n, k, qkv=qkv)
         return _gemm_cost(m, n, k, 2, 2, out_bytes, x_readers=-(-n // cols), w_readers=-(-m // rows))()
     return cost
 
@@ -635,7 +635,7 @@ def gemm_qkv_rope_tiled(x: torch.Tensor, w, table: Optional[torch.Tensor], slot_
     q = torch.empty((m, n_heads * head_dim), dtype=torch.bfloat16, device=x.device)
     library.call("bc4g_gemm_mfma_qkv", _ptr(x), _ptr(w), _ptr(q), _ptr(table), _ptr(slot_map), _ptr(k_cache), _ptr(v_cache),
                  m, n, k, n_heads, n_kv_heads, head_dim, page_tokens, 1 if write_kv else 0, _stream(),
-                 cost=_tiled_cost(m, n, k, 2))
+                 cost=_tiled_cost(m, n, k, 2, qkv=True))
     return q
 
 
