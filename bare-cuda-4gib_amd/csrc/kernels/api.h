@@ -22,6 +22,11 @@ int bc4g_embed_gather(const void* table, int table_dtype, const int32_t* ids, fl
 // x is the float residual stream; out has out_dtype; w has w_dtype.
 int bc4g_rmsnorm(const float* x, const int32_t* rows, const void* w, int w_dtype, void* out,
                  int out_dtype, int n_rows, int hidden, float eps, void* stream);
+// The same for a stream whose last addition is still in parts [n_parts, n_rows, hidden] (float32, as
+// bc4g_gemm_mfma_parts leaves them): x += parts[0] + parts[1] + ... in that order, written back, then out = its norm
+// (bfloat16).  hidden a multiple of 8, at most 8192.
+int bc4g_rmsnorm_sum(float* x, const float* parts, int n_parts, const void* w, int w_dtype, void* out, int out_dtype,
+                     int n_rows, int hidden, float eps, void* stream);
 
 // out[m, n] (+)= sum_k a[m, k] * w[n, k]        (gemm_tiled.cuh:36-96, plain float FMA)
 // accumulate != 0 adds into a float `out` (the residual stream).
@@ -145,6 +150,10 @@ extern "C" {
 // bfloat16 a [m, k] times bfloat16 w [n, k] transposed on the matrix cores, any m.
 // epilogue: 0 store bfloat16; 1 store float32; 2 add into float32; 3 SwiGLU as in bc4g_gemm_skinny.
 int bc4g_gemm_mfma(const void* a, const void* w, void* out, int epilogue, int m, int n, int k, void* stream);
+// The same product with k cut into k_parts equal parts (each a multiple of 64), part p's sums stored as float32 in
+// parts [k_parts, m, n]: for few rows and a long k, where one workgroup per 64 x 64 tile would walk all of k alone.
+// Whoever reads the parts adds them up in order (bc4g_rmsnorm_sum).
+int bc4g_gemm_mfma_parts(const void* a, const void* w, float* parts, int m, int n, int k, int k_parts, void* stream);
 // The output tile (rows, columns) bc4g_gemm_mfma (qkv 0) or bc4g_gemm_mfma_qkv (qkv 1) takes for these operands: for
 // the accounting of bytes and for tests that want to meet every tile.  Launches nothing.
 int bc4g_gemm_mfma_tile(const void* a, const void* w, int m, int n, int k, int qkv, int* rows, int* cols);

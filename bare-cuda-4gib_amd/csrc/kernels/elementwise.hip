@@ -93,6 +93,63 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const float* __restri
   }
 }
 
+// The same for a stream whose last addition is still in parts: x += parts[0] + parts[1] + ... (in that order, every
+// part [n_rows, hidden] floats), x written back, then its norm -- what follows a product whose k was cut over
+// workgroups (bc4g_gemm_mfma_parts).
+template <typename TW, typename TO, int CHUNKS>
+__global__ __launch_bounds__(256) void rmsnorm_sum_rows_kernel(float* __restrict__ x, const float* __restrict__ parts, int n_parts,
+                                                               const TW* __restrict__ w, TO* __restrict__ out, int n_rows,
+                                                               int hidden, float eps) {
+  __shared__ float scratch[16];
+  const size_t at = static_cast<size_t>(blockIdx.x) * hidden, part_stride = static_cast<size_t>(n_rows) * hidden;
+  float* xr = x + at;
+  TO* orow = out + at;
+  float v[CHUNKS][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c) {
+    const int i = (c * 256 + threadIdx.x) * 8;
+    if (i < hidden) {
+      float4 a = *reinterpret_cast<const float4*>(xr + i), b = *reinterpret_cast<const float4*>(xr + i + 4);
+      for (int p = 0; p < n_parts; ++p) {
+        const float* pr = parts + p * part_stride + at + i;
+        const float4 pa = *reinterpret_cast<const float4*>(pr), pb = *reinterpret_cast<const float4*>(pr + 4);
+        a.x += pa.x; a.y += pa.y; a.z += pa.z; a.w += pa.w;
+        b.x += pb.x; b.y += pb.y; b.z += pb.z; b.w += pb.w;
+      }
+      *reinterpret_cast<float4*>(xr + i) = a;
+      *reinterpret_cast<float4*>(xr + i + 4) = b;
+      v[c][0] = a.x; v[c][1] = a.y; v[c][2] = a.z; v[c][3] = a.w;
+      v[c][4] = b.x; v[c][5] = b.y; v[c][6] = b.z; v[c][7] = b.w;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[c][e] = 0.f;
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss += v[c][e] * v[c][e];
+  }
+  const float mean_sq = block_sum(ss, scratch) / static_cast<float>(hidden);
+  const float scale = 1.0f / sqrtf(mean_sq + eps);
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c) {
+    const int i = (c * 256 + threadIdx.x) * 8;
+    if (i >= hidden) continue;
+    float y[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) y[e] = v[c][e] * scale * to_float(w[i + e]);
+    if constexpr (sizeof(TO) == 2) {
+      uint32_t pk[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        pk[e] = static_cast<uint32_t>(bf16_bits_from_float(y[2 * e])) | (static_cast<uint32_t>(bf16_bits_from_float(y[2 * e + 1])) << 16);
+      *reinterpret_cast<uint4*>(orow + i) = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) orow[i + e] = from_float<TO>(y[e]);
+    }
+  }
+}
+
 // ---- SwiGLU ----------------------------------------------------------------
 // interleaved 0: a row of gu holds the gate values, then the up values.  1: blocks of 16 -- eight
 // gate values followed by the eight up values of the same outputs (the layout the fused
@@ -522,6 +579,28 @@ extern "C" int bc4g_rmsnorm(const float* x, const int32_t* rows, const void* w, 
   else return fail("rmsnorm: unknown dtypes w=%d out=%d", w_dtype, out_dtype);
 #undef BC4G_RMS
   return check_launch("rmsnorm");
+}
+
+extern "C" int bc4g_rmsnorm_sum(float* x, const float* parts, int n_parts, const void* w, int w_dtype, void* out,
+                                int out_dtype, int n_rows, int hidden, float eps, void* stream) {
+  BC4G_REQUIRE(n_rows >= 0 && hidden > 0 && hidden % 8 == 0 && hidden <= 8192 && n_parts >= 1 && n_parts <= 16,
+               "rmsnorm_sum: rows=%d of H=%d (a multiple of 8, at most 8192) in %d parts (1 to 16)", n_rows, hidden, n_parts);
+  if (n_rows == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int chunks = (hidden + 2047) / 2048;
+#define BC4G_RMS_SUM(TW, TO)                                                                                              \
+  do {                                                                                                                    \
+    const TW* wp = static_cast<const TW*>(w);                                                                             \
+    TO* op = static_cast<TO*>(out);                                                                                       \
+    if (chunks == 1) rmsnorm_sum_rows_kernel<TW, TO, 1><<<n_rows, 256, 0, s>>>(x, parts, n_parts, wp, op, n_rows, hidden, eps);      \
+    else if (chunks == 2) rmsnorm_sum_rows_kernel<TW, TO, 2><<<n_rows, 256, 0, s>>>(x, parts, n_parts, wp, op, n_rows, hidden, eps); \
+    else rmsnorm_sum_rows_kernel<TW, TO, 4><<<n_rows, 256, 0, s>>>(x, parts, n_parts, wp, op, n_rows, hidden, eps);                  \
+  } while (0)
+  if (w_dtype == kF32 && out_dtype == kBF16) BC4G_RMS_SUM(float, bf16_t);
+  else if (w_dtype == kBF16 && out_dtype == kBF16) BC4G_RMS_SUM(bf16_t, bf16_t);
+  else return fail("rmsnorm_sum: unknown dtypes w=%d out=%d (the output is bfloat16)", w_dtype, out_dtype);
+#undef BC4G_RMS_SUM
+  return check_launch("rmsnorm_sum");
 }
 
 extern "C" int bc4g_swiglu(const void* gu, void* out, int dtype, int n_tokens, int inter, int interleaved,

@@ -462,6 +462,11 @@ __global__ __launch_bounds__(64 * WM * WN, MINWG) void gemm_mfma_direct_kernel(
   int bm, bn;
   tile_of(blockIdx.x, m_blocks, n_blocks, bm, bn);
   const long m0 = static_cast<long>(bm) * RA, n0 = static_cast<long>(bn) * RW;
+  // gridDim.y > 1: k is cut into that many equal parts (each whole steps), and part y's sums go to an output of
+  // its own, out + y * m * n (the plain store epilogues only: whoever reads them adds the parts up in order)
+  const int nk = k / BK / static_cast<int>(gridDim.y);
+  const size_t k_first = static_cast<size_t>(blockIdx.y) * nk * RB;       // in bytes of a row
+  if constexpr (EPI == kStoreF32) out = static_cast<float*>(out) + static_cast<size_t>(blockIdx.y) * m * n;
 
   // the groups of rows this wave brings every step (a spare turn repeats the last group: the same
   // bytes to the same place), and which of a row's segments this lane's 16 bytes are
@@ -478,7 +483,7 @@ __global__ __launch_bounds__(64 * WM * WN, MINWG) void gemm_mfma_direct_kernel(
     long row = (of_a ? m0 : n0) + trow;
     const long last = (of_a ? m : n) - 1;
     if (row > last) row = last;
-    src[i] = reinterpret_cast<const unsigned char*>((of_a ? a : w) + row * k) + seg * 16;
+    src[i] = reinterpret_cast<const unsigned char*>((of_a ? a : w) + row * k) + k_first + seg * 16;
     dst[i] = (of_a ? 0 : RA * RB) + (of_a ? g : g - GA) * 1024;
   }
   auto ask = [&](int step) {
@@ -496,7 +501,6 @@ __global__ __launch_bounds__(64 * WM * WN, MINWG) void gemm_mfma_direct_kernel(
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  const int nk = k / BK;
 #pragma unroll
   for (int s = 0; s < STAGES - 1; ++s)
     if (s < nk) ask(s);
@@ -569,7 +573,8 @@ __global__ __launch_bounds__(64 * WM * WN, MINWG) void gemm_mfma_direct_kernel(
 }
 
 template <int EPI, int WM, int WN, int TM, int TN, int BK, int STAGES, int MINWG>
-int launch_direct(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, int k, hipStream_t s, const RopeKvArgs& ra) {
+int launch_direct(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, int k, hipStream_t s, const RopeKvArgs& ra,
+                  int k_parts = 1) {
   typedef DirectShape<WM, WN, TM, TN, BK, STAGES> S;
   auto kernel = gemm_mfma_direct_kernel<EPI, WM, WN, TM, TN, BK, STAGES, MINWG>;
   static bool raised = false;   // per instantiation: allow more than the default dynamic LDS
@@ -580,7 +585,7 @@ int launch_direct(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, i
     raised = true;
   }
   const long m_blocks = (m + S::kRowsA - 1) / S::kRowsA, n_blocks = (n + S::kRowsW - 1) / S::kRowsW;
-  kernel<<<dim3(static_cast<unsigned>(m_blocks * n_blocks)), dim3(S::kThreads), S::kLdsBytes, s>>>(
+  kernel<<<dim3(static_cast<unsigned>(m_blocks * n_blocks), static_cast<unsigned>(k_parts)), dim3(S::kThreads), S::kLdsBytes, s>>>(
       ap, wp, out, m, n, k, static_cast<int>(m_blocks), static_cast<int>(n_blocks), ra);
   return 0;
 }
@@ -679,6 +684,17 @@ extern "C" int bc4g_gemm_mfma(const void* a, const void* w, void* out, int epilo
   }
   if (e) return e;
   return check_launch("gemm_mfma");
+}
+
+extern "C" int bc4g_gemm_mfma_parts(const void* a, const void* w, float* parts, int m, int n, int k, int k_parts, void* stream) {
+  BC4G_REQUIRE(m > 0 && n > 0 && k > 0 && k_parts >= 1 && k_parts <= 16 && k % (64 * k_parts) == 0 && direct_operands(a, w, k),
+               "gemm_mfma_parts: K=%d must be %d times a multiple of 64 and the operands on 16-byte boundaries (M=%d N=%d)", k,
+               k_parts, m, n);
+  BC4G_REQUIRE(((m + 63L) / 64) * ((n + 63L) / 64) <= 2147483647L, "gemm_mfma_parts: too many tiles");
+  if (int e = launch_direct<kStoreF32, 2, 2, 1, 1, 64, 4, 2>(static_cast<const bf16_t*>(a), static_cast<const bf16_t*>(w), parts, m, n,
+                                                               k, static_cast<hipStream_t>(stream), RopeKvArgs{}, k_parts))
+    return e;
+  return check_launch("gemm_mfma_parts");
 }
 
 extern "C" int bc4g_gemm_mfma_qkv(const void* a, const void* w, void* out, const float* table, const int32_t* slot_map,

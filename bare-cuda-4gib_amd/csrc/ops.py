@@ -496,6 +496,71 @@ class Prenormed:
         self.xb, self.parts, self.eps = xb, parts, float(eps)
 
 
+class Finished:
+    """The RMSNorm after a product that added into the residual stream, already computed by that product's
+    second kernel (gemm_parts_accumulate_norm): ``tensor`` [m, width] in bfloat16."""
+
+    def __init__(self, tensor: torch.Tensor):
+        self.tensor = tensor
+
+
+PARTS_MIN_ROWS, PARTS_MAX_ROWS = 33, 128   # rows for which an adding product's k may be cut over workgroups
+PARTS_MIN_STEPS = 4                         # k-steps of 64 a part keeps at least
+PARTS_WORKGROUPS = 256                      # as many parts (2, 4 or 8) as bring the 64 x 64 tiles to this many
+PARTS_MIN_WEIGHT = 1 << 24                  # up to 64 rows: only for weights of at least this many elements.
+                                            # Measured in the model, a decode step with the output and down products
+                                            # so against the weight-streaming kernel (and the norm after it prepared or
+                                            # run): TinyLlama's widths (2,048 x 2,048 and 2,048 x 5,632) 1.355 -> 1.40 ms
+                                            # at 64 rows, 1.27 -> 1.32 at 48, but 2.15 -> 1.90 at 96 and 2.33 -> 2.06 at
+                                            # 128 (where the weights are streamed twice); Llama-3-8B's (4,096 x 4,096
+                                            # and 4,096 x 14,336) 6.04 -> 5.44 ms at 64 rows, 9.70 -> 8.05 at 128.
+
+
+def parts_of_k(m: int, n: int, k: int) -> int:
+    """Into how many parts gemm_parts_accumulate_norm cuts k (1: it does not take the product)."""
+    if not (PARTS_MIN_ROWS <= m <= PARTS_MAX_ROWS) or k % 64 or n % 8 or n > 8192:
+        return 1
+    if m <= SKINNY_MAX_ROWS and n * k < PARTS_MIN_WEIGHT:
+        return 1
+    tiles = -(-m // 64) * -(-n // 64)
+    best = 1
+    for parts in (2, 4, 8):
+        if k % (64 * parts) == 0 and k // (64 * parts) >= PARTS_MIN_STEPS and tiles * parts <= PARTS_WORKGROUPS:
+            best = parts
+    return best
+
+
+def gemm_parts_supported(a: torch.Tensor, w, residual: torch.Tensor, g: torch.Tensor) -> bool:
+    """Whether gemm_parts_accumulate_norm takes these operands: bfloat16, 33 to 128 rows, a k that several
+    workgroups can share, a plain RMSNorm after it."""
+    w, _ = _weight(w)
+    return (_fast_operands(a, w) and residual.dtype == torch.float32 and residual.is_contiguous()
+            and tuple(residual.shape) == (a.shape[0], w.shape[0]) and g.dtype in _CODE and tuple(g.shape) == (w.shape[0],)
+            and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0 and parts_of_k(a.shape[0], w.shape[0], w.shape[1]) > 1)
+
+
+def gemm_parts_accumulate_norm(a: torch.Tensor, w, residual: torch.Tensor, g: torch.Tensor, eps: float) -> Finished:
+    """residual += a w^T and the RMSNorm (scale g, eps) of the result, in two kernels: the tiled product with k cut
+    into parts over workgroups, each part's sums stored apart; then one that adds the parts to the residual in
+    order and norms it.  For a few dozen rows and a square or long weight, where a 64 x 64 tile's workgroup
+    would walk all of k alone and the weight-streaming kernel's workgroups all read all of x."""
+    w, _ = _weight(w)
+    _dev("gemm_parts_accumulate_norm", a, w, residual, g)
+    m, k = a.shape
+    n = w.shape[0]
+    n_parts = parts_of_k(m, n, k)
+    if n_parts < 2 or not gemm_parts_supported(a, w, residual, g):
+        raise KernelError(f"gemm_parts_accumulate_norm: not for [{m}, {k}] x [{n}, {k}]^T")
+    parts = torch.empty((n_parts, m, n), dtype=torch.float32, device=a.device)
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
+    library.call("bc4g_gemm_mfma_parts", _ptr(a), _ptr(w), _ptr(parts), m, n, k, n_parts, _stream(),
+                 cost=_gemm_cost(m, n, k, 2, 2, 4 * n_parts, x_readers=-(-n // 64), w_readers=-(-m // 64)))
+    library.call("bc4g_rmsnorm_sum", _ptr(residual), _ptr(parts), n_parts, _ptr(g), _code(g, "rmsnorm_sum"), _ptr(out),
+                 _code(out, "rmsnorm_sum"), m, n, float(eps), _stream(),
+                 cost=lambda: (3.0 * m * n + n_parts * m * n, m * n * (4 * n_parts + 8 + 2) + n * g.element_size()))
+    return Finished(out)
+
+
 def gemm_emit_supported(a: torch.Tensor, w, residual: torch.Tensor, g: torch.Tensor) -> bool:
     """Whether the adding product of these operands can prepare the next RMSNorm: the
     weight-streaming kernel serves it (bfloat16, few rows: streams_weights)."""

@@ -62,9 +62,12 @@ class StepContext:
     # the block around the part; by the model: the norm the next schedule entry begins with).  A product
     # that adds into the stream may then prepare that norm and leave the result in ``prepared`` under
     # id(norm part); the block hands it to the norm's consumer.  Nothing prepared outlives the entry
-    # after the one that made it.
+    # after the one that made it.  What is prepared is the finished norm, which serves every reader, or -- only
+    # if the reader takes that (``..._takes_parts``) -- the parts of one that a product can finish.
     norm_after: Any = None
+    norm_after_takes_parts: bool = False
     next_entry_norm: Any = None
+    next_entry_takes_parts: bool = False
     prepared: Dict[int, Any] = dataclasses.field(default_factory=dict)
 
     def cache(self, stream: Optional[Hashable]):

@@ -169,9 +169,11 @@ class Model:
                 ctx.prepared[id(first)] = kept
             following = self.layers[self.schedule[i + 1].layer] if i + 1 < len(self.schedule) else None
             ctx.next_entry_norm = following.first_norm(ctx.n_tokens) if hasattr(following, "first_norm") else None
+            takes = getattr(following, "first_norm_takes_parts", None)
+            ctx.next_entry_takes_parts = bool(takes(ctx.n_tokens)) if takes is not None else False
             layer.forward(x, ctx, ctx.cache(e.cache), e.writes)
         ctx.prepared.clear()
-        ctx.next_entry_norm = None
+        ctx.next_entry_norm, ctx.next_entry_takes_parts = None, False
         if ctx.n_logits == 0:
             return None
         norm, head = self.final_norm.part, self.head.part

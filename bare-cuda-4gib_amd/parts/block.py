@@ -1,6 +1,7 @@
 """How a layer's parts are arranged around the residual stream."""
 from __future__ import annotations
 
+from ..csrc import ops
 from .base import Part, register_part
 from .lazy import Normed
 
@@ -21,17 +22,21 @@ class PreNormBlock(Part):
         # Each part is told which norm reads the stream after it, so that its last product can
         # prepare that norm: the feed-forward's after the mixer, the next entry's first after the
         # feed-forward.
-        after = ctx.next_entry_norm
-        ctx.norm_after = self.ffn_norm if self._wants_prepared(self.ffn, x.shape[0]) else None
+        # (A finished norm serves every reader; the parts of one only a reader that says so.)
+        after, after_takes_parts = ctx.next_entry_norm, ctx.next_entry_takes_parts
+        ctx.norm_after, ctx.norm_after_takes_parts = self.ffn_norm, self._wants_prepared(self.ffn, x.shape[0])
         self.mixer.forward(self._normed(self.mixer, self.mixer_norm, x, ctx), ctx, cache, x, writes)
-        ctx.norm_after = after
+        ctx.norm_after, ctx.norm_after_takes_parts = after, after_takes_parts
         self.ffn.forward(self._normed(self.ffn, self.ffn_norm, x, ctx), ctx, x)
-        ctx.norm_after = None
+        ctx.norm_after, ctx.norm_after_takes_parts = None, False
 
     def first_norm(self, n_rows: int):
-        """The norm this block begins with, if the entry before should prepare it for a step of
-        ``n_rows`` rows (else None)."""
-        return self.mixer_norm if self._wants_prepared(self.mixer, n_rows) else None
+        """The norm this block begins with, which the entry before may prepare."""
+        return self.mixer_norm
+
+    def first_norm_takes_parts(self, n_rows: int) -> bool:
+        """Whether its reader takes the parts of a prepared norm (ops.Prenormed) for a step of ``n_rows`` rows."""
+        return self._wants_prepared(self.mixer, n_rows)
 
     @staticmethod
     def _wants_prepared(part, n_rows: int) -> bool:
@@ -46,6 +51,8 @@ class PreNormBlock(Part):
         norm not yet computed, so that the part's first product can absorb it (or take what the
         product before has prepared for it)."""
         pre = ctx.prepared.pop(id(norm), None)
+        if isinstance(pre, ops.Finished):
+            return Normed(x, norm, ctx, done=pre.tensor) if getattr(part, "accepts_lazy_norm", False) else pre.tensor
         if getattr(part, "accepts_lazy_norm", False):
             return Normed(x, norm, ctx, pre=pre)
         return norm.forward(x, ctx)

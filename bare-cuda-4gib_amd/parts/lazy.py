@@ -15,12 +15,12 @@ import torch
 
 class Normed:
     def __init__(self, x: torch.Tensor, norm, ctx=None, rows: Optional[torch.Tensor] = None,
-                 n_rows: Optional[int] = None, pre=None):
+                 n_rows: Optional[int] = None, pre=None, done: Optional[torch.Tensor] = None):
         self.x, self.norm, self.ctx, self.rows = x, norm, ctx, rows
         # what the product that last added into x left for this norm (ops.Prenormed), if anything
         self.pre = pre if rows is None else None
         self.n_rows = x.shape[0] if rows is None and n_rows is None else (n_rows if n_rows is not None else rows.numel())
-        self._tensor: Optional[torch.Tensor] = None
+        self._tensor: Optional[torch.Tensor] = done      # (``done``: the product before has computed the norm already)
 
     def tensor(self) -> torch.Tensor:
         if self._tensor is None:

@@ -35,7 +35,9 @@ def linear(x: Union[torch.Tensor, Normed], w, out_dtype: Optional[torch.dtype] =
     """x [M, K] times w [N, K] transposed (w a tensor or an ops.StreamedWeight).  With
     ``accumulate_into`` (the float32 residual stream) the product is added to it in place; with
     ``ctx`` too, and a norm named there as the next reader of the stream (``ctx.norm_after``), the
-    product prepares that norm where its kernel can and leaves the result in ``ctx.prepared``."""
+    product prepares that norm where its kernel can and leaves the result in ``ctx.prepared``: the norm
+    itself (ops.Finished: a few dozen rows, k cut over workgroups) or, if the norm's reader takes that
+    (``ctx.norm_after_takes_parts``), the parts of it a product can finish (ops.Prenormed)."""
     if isinstance(x, Normed):
         if accumulate_into is None and out_dtype in (torch.bfloat16, torch.float32):
             epi = ops.EPI_STORE_BF16 if out_dtype == torch.bfloat16 else ops.EPI_STORE_F32
@@ -48,7 +50,10 @@ def linear(x: Union[torch.Tensor, Normed], w, out_dtype: Optional[torch.dtype] =
     if accumulate_into is not None and ctx is not None and ctx.norm_after is not None:
         norm = ctx.norm_after
         scale = norm.fusable() if hasattr(norm, "fusable") else None
-        if scale is not None and ops.gemm_emit_supported(x, w, accumulate_into, scale[0]):
+        if scale is not None and ops.gemm_parts_supported(x, w, accumulate_into, scale[0]):
+            ctx.prepared[id(norm)] = ops.gemm_parts_accumulate_norm(x, w, accumulate_into, scale[0], scale[1])
+            return accumulate_into
+        if scale is not None and ctx.norm_after_takes_parts and ops.gemm_emit_supported(x, w, accumulate_into, scale[0]):
             ctx.prepared[id(norm)] = ops.gemm_accumulate_emit(x, w, accumulate_into, scale[0], scale[1])
             return accumulate_into
     fast = ops.gemm_fast(x, w, out_dtype, accumulate_into)

@@ -61,6 +61,27 @@ def test_rmsnorm(ops, wdt, odt):
     close(got, short.double() / math.sqrt(13.5), 1e-6, 1e-6, "rmsnorm eps")
 
 
+@pytest.mark.parametrize("m,n,k", [(65, 2048, 2048), (33, 4096, 5632), (128, 4096, 4096), (100, 1000, 1024), (64, 8192, 2048)])
+def test_adding_product_in_parts_of_k_with_the_norm_after_it(ops, m, n, k):
+    """A few dozen rows: the product's k cut over workgroups, the parts added to the residual in order by the kernel
+    that norms it -- against the definition, and the residual against the product that adds at once."""
+    assert ops.parts_of_k(m, n, k) > 1 and ops.parts_of_k(32, n, k) == 1 and ops.parts_of_k(129, n, k) == 1
+    a, w = bf(rnd(m, k, seed=80)), bf(rnd(n, k, seed=81, scale=0.3))
+    base, g = rnd(m, n, seed=82).float(), (1.0 + 0.1 * rnd(n, seed=83)).bfloat16()
+    resid = base.clone().to(DEV)
+    assert ops.gemm_parts_supported(a.to(DEV), w.to(DEV), resid, g.to(DEV))
+    done = ops.gemm_parts_accumulate_norm(a.to(DEV), w.to(DEV), resid, g.to(DEV), 1e-5)
+    want = base.double() + a.double() @ w.double().T
+    close(resid, want, 1e-4, 1e-4 * math.sqrt(k), "residual")
+    at_once = base.clone().to(DEV)
+    ops.gemm_fast(a.to(DEV), w.to(DEV), accumulate_into=at_once)
+    close(resid, at_once.double().cpu(), 1e-5, 1e-5 * math.sqrt(k), "residual, against the product that adds at once")
+    # the norm is of the residual as the kernel holds it: the same bits as the norm kernel's of what it wrote back
+    assert torch.equal(done.tensor, ops.rmsnorm(resid, g.to(DEV), 1e-5, torch.bfloat16))
+    close(done.tensor, P.rmsnorm(want, g.double(), 1e-5), 8e-3, 2e-3, "norm")
+    assert not ops.gemm_parts_supported(a.float().to(DEV), w.to(DEV), resid, g.to(DEV))
+
+
 @pytest.mark.parametrize("m,n,k", [(17, 130, 300), (1, 130, 300), (150, 61, 48), (64, 64, 64), (3, 5, 7)])
 def test_gemm_generic(ops, m, n, k):
     a, w = rnd(m, k, seed=4), rnd(n, k, seed=5)
