@@ -148,26 +148,26 @@ def test_tinyllama_widths_greedy_ids_in_32_bit(tinyllama):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_tinyllama_widths_steps_of_65_to_128_rows(tinyllama, dtype):
-    """Steps of 80, 120 and 66 rows (two or three tokens of many requests): in bfloat16 the output and down products
+def test_tinyllama_widths_steps_of_65_to_256_rows(tinyllama, dtype):
+    """Steps of 80, 120, 200 and 66 rows (a few tokens of many requests): in bfloat16 the output and down products
     of such steps cut k over workgroups and the kernel that adds the parts up norms the stream for the next product."""
     from bare_cuda_4gib_amd.csrc import ops
     from bare_cuda_4gib_amd.engine import Executor, StepEntry, load_model
     folder, _, plain, _ = tinyllama(dtype)
     model, _ = load_model(folder, dtype, "cuda:0")
-    assert ops.parts_of_k(80, 2048, 2048) > 1 and ops.parts_of_k(120, 2048, 5632) > 1
+    assert ops.parts_of_k(80, 2048, 2048) > 1 and ops.parts_of_k(120, 2048, 5632) > 1 and ops.parts_of_k(200, 2048, 5632) > 1
     n = 40
-    prompts = [helpers.random_ids(12 + (3 * i) % 5, 32000, 1500 + i) for i in range(n)]
-    want = [plain_rows(plain, ids, range(len(ids) - 7, len(ids))) for ids in prompts]
+    prompts = [helpers.random_ids(17 + (3 * i) % 5, 32000, 1500 + i) for i in range(n)]
+    want = [plain_rows(plain, ids, range(len(ids) - 12, len(ids))) for ids in prompts]
     ex = Executor(model, num_pages=n, max_requests=n, max_tokens=64, page_tokens=64, max_batch_tokens=1024, poison=True)
     ex.cache.shuffle_free_pages(5)
     for i in range(n):
         ex.admit(i)
     for lo in range(0, n, 20):
-        ex.step([StepEntry(i, prompts[i][:-7], []) for i in range(lo, lo + 20)])
+        ex.step([StepEntry(i, prompts[i][:-12], []) for i in range(lo, lo + 20)])
     tol = TOL[dtype]
-    done = 7
-    for per, who in ((2, range(n)), (3, range(n)), (2, range(7, n))):          # 80, 120 and 66 rows
+    done = 12
+    for per, who in ((2, range(n)), (3, range(n)), (5, range(n)), (2, range(7, n))):          # 80, 120, 200 and 66 rows
         entries = [StepEntry(i, prompts[i][len(prompts[i]) - done:len(prompts[i]) - done + per], list(range(per))) for i in who]
         got = ex.step(entries).float().cpu().numpy()
         row = 0
