@@ -352,13 +352,15 @@ def _weight(w):
 
 
 SKINNY_MAX_ROWS = 64
-SKINNY_PASSES_ROWS = 128            # up to here the weights are streamed once per 64 rows rather than tiled, unless
+SKINNY_PASSES_ROWS = 64             # up to here the weights are streamed rather than tiled (beyond 64 rows they would be
+                                    # streamed once per 64 rows: a decode step of 65 to 128 rows is 2-3 % longer so at
+                                    # TinyLlama's widths and 8-10 % at Llama-3-8B's, measured in the model), unless
 SKINNY_PASSES_MAX_N = 8192          # the output is at least this wide, and then only below SKINNY_WIDE_ROWS rows.
 SKINNY_WIDE_ROWS = 32               # With one or two rows of tiles a product is as long as its chain of k-steps,
                                     # which the streaming kernel's eight waves cut into eight -- but a wide output
                                     # has tiles enough for every CU (64 x 64 ones, four stages), while every one of
                                     # the streaming kernel's many workgroups reads all the rows of x (measured,
-                                    # streamed against tiled, us: 128 rows 2048 x 5632 20 / 27, 4096 x 14336 66 / 64;
+                                    # streamed against tiled in a loop over one product, us:
                                     # 64 rows 11264 x 2048 16.9 / 12.3, 28672 x 4096 59 / 37, 32000 x 2048 37 / 22,
                                     # 6144 x 4096 19.4 / 19.6; 32 rows 11264 x 2048 12.7 / 12.4; 16 rows 9.3 / 12.2)
 
@@ -382,8 +384,8 @@ def gemm_fast(a: torch.Tensor, w, out_dtype=None,
               accumulate_into: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
     """The matrix-core product where a kernel takes these operands (bfloat16, k a multiple of
     8), else None (the caller then uses the plain float kernel).  Up to 64 rows the weights
-    are streamed once (a decode step), up to 128 once per 64 rows; a wide output goes to the tiled
-    kernel from 32 rows on, everything from 129."""
+    are streamed once (a decode step); a wide output goes to the tiled kernel from 32 rows on,
+    everything from 65."""
     w, packed = _weight(w)
     if not _fast_operands(a, w):
         return None

@@ -61,7 +61,7 @@ def test_norms_prepared_by_the_product_before(folders, monkeypatch, name, varian
     attention begins with (and, from 64 rows on, the feed-forward's): the path is taken -- the
     preparing kernel runs once a layer and step, none where no layer follows -- and the logits are
     those of the path without it up to rounding, and the plain implementation's, for decoded tokens
-    alone, for 70 rows in a step (both norms prepared) and for portions beside decoded tokens."""
+    alone, for 64 rows in a step (both norms prepared) and for portions beside decoded tokens."""
     from bare_cuda_4gib_amd.csrc import ops
     from bare_cuda_4gib_amd.engine import Executor, load_model
     from bare_cuda_4gib_amd.parts.attention import CausalAttention
@@ -78,7 +78,7 @@ def test_norms_prepared_by_the_product_before(folders, monkeypatch, name, varian
         e = {"id": rid, "tokens": requests[rid][at[rid]:at[rid] + n], "want": list(range(n)), "_start": at[rid]}
         at[rid] += n
         return e
-    plan = [[("r0", 70)], [("r0", 1)], [("r0", 1), ("r1", 18)], [("r0", 1), ("r1", 1), ("r2", 9)], [("r0", 1), ("r1", 1)], [("r0", 1)]]
+    plan = [[("r0", 64)], [("r0", 1)], [("r0", 1), ("r1", 18)], [("r0", 1), ("r1", 1), ("r2", 9)], [("r0", 1), ("r1", 1)], [("r0", 1)]]
     steps = [{"step": i, "entries": [entry(rid, n) for rid, n in group], "end": []} for i, group in enumerate(plan)]
     steps, where = helpers._finish(steps)
     calls = []

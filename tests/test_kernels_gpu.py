@@ -137,7 +137,7 @@ def test_gemm_swiglu(ops, m, inter, k):
           "interleaved: the activation sees the float sums")
 
 
-@pytest.mark.parametrize("m,n,k", [(65, 130, 304), (150, 257, 64), (300, 128, 2048), (128, 384, 96), (129, 61, 8),
+@pytest.mark.parametrize("m,n,k", [(65, 130, 304), (70, 130, 304), (150, 257, 64), (300, 128, 2048), (128, 384, 96), (129, 61, 8),
                                    (200, 384, 96)])
 def test_gemm_mfma(ops, m, n, k):
     a, w = bf(rnd(m, k, seed=12)), bf(rnd(n, k, seed=13))
@@ -151,8 +151,8 @@ def test_gemm_mfma(ops, m, n, k):
     ops.gemm_fast(a.to(DEV), w.to(DEV), accumulate_into=acc)
     close(acc, want + base.double(), 1e-4, 1e-4 * scale, "mfma accumulate")
     # rows do not depend on M (while the same kind of kernel serves them: up to SKINNY_PASSES_ROWS rows the
-    # weights are streamed in passes of 64 rows, beyond that the output is tiled)
-    part = m - 3 if m - 3 > ops.SKINNY_PASSES_ROWS else min(m, 40)
+    # weights are streamed, beyond that the output is tiled)
+    part = max(m - 3, ops.SKINNY_PASSES_ROWS + 1) if m > ops.SKINNY_PASSES_ROWS else min(m, 40)
     fewer = ops.gemm_fast(a[:part].contiguous().to(DEV), w.to(DEV), torch.float32)
     assert torch.equal(fewer, got[:part])
     assert ops.gemm_fast(a.float().to(DEV), w.to(DEV)) is None                      # float operands: not taken
@@ -766,7 +766,7 @@ def test_tiled_qkv_product_with_rotation_and_cache_write(ops, nh, nkv, d, m, k, 
         assert bool((kc3.permute(0, 2, 1, 3)[free] == -7.5).all()) and bool((vc3.permute(0, 3, 1, 2)[free] == -7.5).all()), "spill"
 
 
-@pytest.mark.parametrize("m", [1, 5, 8, 9, 16, 33, 64, 100])
+@pytest.mark.parametrize("m", [1, 5, 8, 9, 16, 33, 64])
 @pytest.mark.parametrize("width,k,gdt", [(96, 40, torch.bfloat16), (2048, 256, torch.bfloat16), (200, 72, torch.float32)])
 def test_adding_product_prepares_the_next_norm(ops, m, width, k, gdt):
     """The product that adds into the residual stream also leaves bfloat16(new residual * g) and, per
