@@ -356,7 +356,9 @@ SKINNY_PASSES_ROWS = 64             # up to here the weights are streamed rather
                                     # streamed once per 64 rows: a decode step of 65 to 128 rows is 2-3 % longer so at
                                     # TinyLlama's widths and 8-10 % at Llama-3-8B's, measured in the model), unless
 SKINNY_PASSES_MAX_N = 8192          # the output is at least this wide, and then only below SKINNY_WIDE_ROWS rows.
-SKINNY_WIDE_ROWS = 32               # With one or two rows of tiles a product is as long as its chain of k-steps,
+SKINNY_WIDE_ROWS = 24               # (a decode step of 24 to 31 rows with the wide outputs tiled: 1-2 % shorter at TinyLlama's
+                                    # widths, 4-7 % at Llama-3-8B's, 1 % at Llama-2-7B's, where 17 to 20 rows are 1-3 % longer so)
+                                    # With one or two rows of tiles a product is as long as its chain of k-steps,
                                     # which the streaming kernel's eight waves cut into eight -- but a wide output
                                     # has tiles enough for every CU (64 x 64 ones, four stages), while every one of
                                     # the streaming kernel's many workgroups reads all the rows of x (measured,
@@ -384,7 +386,7 @@ def gemm_fast(a: torch.Tensor, w, out_dtype=None,
               accumulate_into: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
     """The matrix-core product where a kernel takes these operands (bfloat16, k a multiple of
     8), else None (the caller then uses the plain float kernel).  Up to 64 rows the weights
-    are streamed once (a decode step); a wide output goes to the tiled kernel from 32 rows on,
+    are streamed once (a decode step); a wide output goes to the tiled kernel from 24 rows on,
     everything from 65."""
     w, packed = _weight(w)
     if not _fast_operands(a, w):

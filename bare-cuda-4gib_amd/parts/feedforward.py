@@ -54,7 +54,7 @@ class SwiGLU(Part):
         against 1.072 ms at 16 rows, 1.269 against 1.252 at 32, 1.558 against 1.565 at 64)."""
         if not self.interleaved:
             return False
-        # (a wide gate-up product of 32 rows and more goes to the tiled kernel, which reads a finished norm)
+        # (a wide gate-up product of 24 rows and more goes to the tiled kernel, which reads a finished norm)
         return 5 <= n_rows <= ops.NORMED_MAX_ROWS or (n_rows >= 64 and ops.streams_weights(n_rows, *self.w_gu.shape))
 
     def forward(self, h, ctx, residual) -> None:
