@@ -508,8 +508,10 @@ class Finished:
         self.tensor = tensor
 
 
-PARTS_MIN_ROWS, PARTS_MAX_ROWS = 33, 256   # rows for which an adding product's k may be cut over workgroups (a prompt of
-                                            # 256 tokens at TinyLlama's widths 2.42 -> 2.21 ms, of 192 2.36 -> 2.20)
+PARTS_MIN_ROWS, PARTS_MAX_ROWS = 10, 256   # rows for which an adding product's k may be cut over workgroups (a prompt of
+                                            # 256 tokens at TinyLlama's widths 2.42 -> 2.21 ms, of 192 2.36 -> 2.20; a decode
+                                            # step at the Llama-3-8B shape 4.11 -> 3.89 ms at 12 rows, 4.60 -> 4.31 at 32,
+                                            # the same at 9 and 3.53 -> 3.71 at 8, where the norm is fused into the products)
 PARTS_MIN_STEPS = 4                         # k-steps of 64 a part keeps at least
 PARTS_WORKGROUPS = 256                      # as many parts (2, 4 or 8) as bring the 64 x 64 tiles to this many
 PARTS_MIN_WEIGHT = 1 << 24                  # up to 64 rows: only for weights of at least this many elements.
@@ -536,7 +538,7 @@ def parts_of_k(m: int, n: int, k: int) -> int:
 
 
 def gemm_parts_supported(a: torch.Tensor, w, residual: torch.Tensor, g: torch.Tensor) -> bool:
-    """Whether gemm_parts_accumulate_norm takes these operands: bfloat16, 33 to 256 rows, a k that several
+    """Whether gemm_parts_accumulate_norm takes these operands: bfloat16, 10 to 256 rows, a k that several
     workgroups can share, a plain RMSNorm after it."""
     w, _ = _weight(w)
     return (_fast_operands(a, w) and residual.dtype == torch.float32 and residual.is_contiguous()

@@ -36,7 +36,7 @@ def linear(x: Union[torch.Tensor, Normed], w, out_dtype: Optional[torch.dtype] =
     ``accumulate_into`` (the float32 residual stream) the product is added to it in place; with
     ``ctx`` too, and a norm named there as the next reader of the stream (``ctx.norm_after``), the
     product prepares that norm where its kernel can and leaves the result in ``ctx.prepared``: the norm
-    itself (ops.Finished: 33 to 256 rows, k cut over workgroups) or, if the norm's reader takes that
+    itself (ops.Finished: 10 to 256 rows, k cut over workgroups) or, if the norm's reader takes that
     (``ctx.norm_after_takes_parts``), the parts of it a product can finish (ops.Prenormed)."""
     if isinstance(x, Normed):
         if accumulate_into is None and out_dtype in (torch.bfloat16, torch.float32):
