@@ -209,3 +209,41 @@ def test_one_layer_at_llama3_8b_widths(tmp_path_factory, dtype):
         got = helpers.replay_in_process(ex, steps)
         helpers.compare_with_plain(got, where, rows, label=f"Llama-3-8B widths, {label}, {dtype}", **TOL[dtype])
         assert ex.cache.pages_in_use() == 0
+
+
+def test_decode_batch_of_16_at_llama3_8b_widths_in_a_captured_graph(tmp_path_factory):
+    """Sixteen requests decoded together at the widest shape: from 10 rows on its output and down products cut k over
+    workgroups and the kernel that adds the parts up norms the stream.  The steps replayed from a captured graph give
+    the bits of the steps launched one kernel at a time, and the plain implementation's logits."""
+    from bare_cuda_4gib_amd.csrc import ops
+    from bare_cuda_4gib_amd.engine import Executor, StepEntry, load_model
+    from bare_cuda_4gib_amd.weights import write_random_model
+    folder = os.path.join(str(tmp_path_factory.getbasetemp()), "llama3_8b_widths")
+    if not os.path.exists(os.path.join(folder, "model.safetensors")):
+        write_random_model(LLAMA3_8B_WIDTHS, 41, folder, "bfloat16", norm_std=0.1, scales={"lm_head.weight": 0.125})
+    assert ops.parts_of_k(16, 4096, 4096) > 1 and ops.parts_of_k(16, 4096, 14336) > 1
+    n, tail = 16, 4
+    prompts = [helpers.random_ids(6 + i % 5 + tail, 128256, 1700 + i) for i in range(n)]
+    plain = PlainLlama(folder)
+    want = [plain_rows(plain, ids, range(len(ids) - tail, len(ids))) for ids in prompts]
+    del plain
+    model, _ = load_model(folder, "bfloat16", "cuda:0")
+    runs = {}
+    for graphs in (False, True):
+        ex = Executor(model, num_pages=n, max_requests=n, max_tokens=64, page_tokens=64, poison=True)
+        ex.use_graphs = ex.use_graphs and graphs
+        assert ex.use_graphs == graphs
+        for i in range(n):
+            ex.admit(i)
+        ex.step([StepEntry(i, prompts[i][:-tail], []) for i in range(n)])
+        runs[graphs] = [ex.step([StepEntry(i, [prompts[i][len(prompts[i]) - tail + t]], [0]) for i in range(n)]).float().cpu()
+                        for t in range(tail)]
+    tol = TOL["bfloat16"]
+    for t in range(tail):
+        assert torch.equal(runs[True][t], runs[False][t]), f"decoded token {t}: the graph's replay and the plain launches differ"
+        got = runs[True][t].numpy()
+        for i in range(n):
+            w = want[i][len(prompts[i]) - tail + t]
+            err = np.abs(got[i] - w)
+            assert np.all(err <= tol["atol"] + tol["rtol"] * np.abs(w)), f"request {i}, token {t}: off by {float(err.max()):.3g}"
+
