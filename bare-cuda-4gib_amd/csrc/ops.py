@@ -543,7 +543,8 @@ def gemm_parts_supported(a: torch.Tensor, w, residual: torch.Tensor, g: torch.Te
     w, _ = _weight(w)
     return (_fast_operands(a, w) and residual.dtype == torch.float32 and residual.is_contiguous()
             and tuple(residual.shape) == (a.shape[0], w.shape[0]) and g.dtype in _CODE and tuple(g.shape) == (w.shape[0],)
-            and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0 and parts_of_k(a.shape[0], w.shape[0], w.shape[1]) > 1)
+            and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0 and residual.data_ptr() % 16 == 0 and a.is_contiguous()
+            and w.is_contiguous() and parts_of_k(a.shape[0], w.shape[0], w.shape[1]) > 1)
 
 
 def gemm_parts_accumulate_norm(a: torch.Tensor, w, residual: torch.Tensor, g: torch.Tensor, eps: float) -> Finished:
