@@ -627,11 +627,18 @@ def gemm_prenormed(pre: Prenormed, w, epilogue: int) -> torch.Tensor:
     return out
 
 
+QKV_WIDE_ROWS = 48      # rows from which a q|k|v output of 8,192 columns and more (every query head with keys of its own) goes
+                        # to the tiled kernel like other wide outputs (a decode step at the Llama-2-7B shape 7.91 -> 7.69 ms
+                        # at 64 rows, 6.77 -> 6.70 at 48, 5.12 -> 5.17 at 24)
+
+
 def gemm_qkv_rope_supported(x: torch.Tensor, n_rows: int, normed: bool, w, head_dim: int,
                             rotary_dim: int) -> bool:
     """Whether the q|k|v product of these rows can rotate and write the cache in its epilogue."""
     w, _ = _weight(w)
     rows_ok = _normed_rows_fit(n_rows, x.shape[1]) if normed else n_rows <= SKINNY_MAX_ROWS
+    if not normed and n_rows >= QKV_WIDE_ROWS and not streams_weights(n_rows, w.shape[0], x.shape[1]):
+        return False                  # a wide q|k|v output: the tiled kernel's epilogue does the same
     return (x.is_cuda and w.dtype == torch.bfloat16 and x.shape[1] % 8 == 0 and 0 < n_rows and rows_ok
             and head_dim % 16 == 0 and rotary_dim in (0, head_dim)
             and x.dtype == (torch.float32 if normed else torch.bfloat16))
