@@ -700,11 +700,12 @@ def test_qkv_product_with_rotation_and_cache_write(ops, nh, nkv, d, m, normed, r
 @pytest.mark.parametrize("nh,nkv,d,m,k,page", [(4, 2, 16, 200, 64, 16), (6, 2, 48, 333, 128, 16), (32, 4, 64, 2048 - 20, 192, 64),
                                                (24, 8, 128, 2048 - 20, 192, 32), (32, 8, 128, 4096 - 236, 192, 64),
                                                (16, 8, 128, 4096 - 236, 192, 64), (16, 8, 128, 2048 - 20, 192, 64),
-                                               (8, 4, 128, 2048 - 20, 1024, 64), (32, 4, 64, 2048 - 20, 1024, 64)])
+                                               (8, 4, 128, 2048 - 20, 1024, 64), (32, 4, 64, 2048 - 20, 1024, 64),
+                                               (64, 32, 64, 56, 192, 64)])
 @pytest.mark.parametrize("rotate", [True, False])
 def test_tiled_qkv_product_with_rotation_and_cache_write(ops, nh, nkv, d, m, k, page, rotate):
     """The same for the many rows of a prompt portion, in the tiled kernel's epilogue (every tile, 64 x 64 up to
-    256 x 256, by the shapes; the last four 256 x 256, 256 x 128, 128 x 128 and 128 x 64): queries rotated, keys rotated into the pages the slot map names, values into theirs, nothing else
+    256 x 256, by the shapes; the last five 256 x 256, 256 x 128, 128 x 128, 128 x 64 and a wide output of few rows): queries rotated, keys rotated into the pages the slot map names, values into theirs, nothing else
     touched -- against the plain product and rotation, and against the unfused pair of kernels."""
     if torch.cuda.get_device_properties(0).multi_processor_count != 256:
         pytest.skip("the shapes are chosen for 256 CUs")
