@@ -741,6 +741,8 @@ ATTENTION_MAX_SPLITS = 64
 ATTENTION_PROMPT_GROUPS = 512     # workgroups a prompt step should bring where the caller cuts every walk alike
 ATTENTION_SLOTS = 512             # workgroups of the prompt form the GPU holds at a time (two a CU: the kernel's registers)
 ATTENTION_MAX_PROMPT_SPLITS = 8
+ATTENTION_SHARE_SLACK = 1.5       # a part of a prompt's walk may be this much longer than an even share of all tiles
+                                  # (2,048-token prompts in the model: 1.25 to 2 within 1 %, 1 and 3 are 2-5 % longer)
 ATTENTION_MIN_WALK = 4            # 32-key tiles a part of a prompt's keys should hold at least
 ATTENTION_APART_CONTEXT = 256     # cached tokens from which on a single-tile request beside prompt portions gets a
                                   # launch of the decode form for itself
@@ -839,7 +841,7 @@ def prompt_work_list(batch, piece_starts, piece: int, head_blocks: int, window: 
     Under the causal mask a piece's walk over the keys is as long as its position: walks of 1 to 64 tiles of
     32 keys in a 2,048-token prompt.  A workgroup takes about as long as its walk (1.6-1.9 us a tile, with a
     second workgroup beside it on the CU or without, plus 6 us before and after), and a CU holds two at a
-    time.  So the walks are cut into parts of at most a quarter more than an even share of all tiles per place
+    time.  So the walks are cut into parts of at most half more than an even share of all tiles per place
     (eight parts at most: every part of a row leaves float partial outputs), and the list starts with the
     longest: what is short fills in behind them (list scheduling).  Measured against every walk in two parts
     in the grid's own order, attention and merge: head size 64, 2,048 tokens 69 -> 57 us, 4,096 212 -> 180, 8,192
@@ -853,7 +855,7 @@ def prompt_work_list(batch, piece_starts, piece: int, head_blocks: int, window: 
             lo = max(0, first - window + 1) if window > 0 else 0
             pieces.append((last // 32 - lo // 32 + 1, piece_starts[s] + j, start[s] + j * piece, min(new, (j + 1) * piece) - j * piece))
     share = sum(p[0] for p in pieces) * head_blocks / ATTENTION_SLOTS
-    longest = max(ATTENTION_MIN_WALK, -(-5 * share // 4))
+    longest = max(ATTENTION_MIN_WALK, math.ceil(ATTENTION_SHARE_SLACK * share))
     items, row_parts, most = [], [1] * batch.n_tokens, 1
     for tiles, index, row, rows in pieces:
         parts = int(max(1, min(ATTENTION_MAX_PROMPT_SPLITS, -(-tiles // longest))))

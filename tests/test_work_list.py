@@ -65,11 +65,11 @@ def test_every_part_of_every_piece_once_and_the_longest_first(seed):
 
 def test_a_long_prompt_alone_is_cut_by_an_even_share():
     """2,048 tokens, 32-token pieces, four head blocks: 8,320 key tiles over 512 places are 16.25 each; parts hold
-    at most a quarter more (21), so the last piece's 64 tiles go in four parts and the first 21 pieces in one."""
+    at most half more (25), so the last piece's 64 tiles go in three parts and the first 25 pieces in one."""
     batch = batch_of([(0, 2048)])
     items, row_parts, most = ops.prompt_work_list(batch, [0, 64], 32, 4, 0)
-    assert most == 4 and row_parts[0] == 1 and row_parts[21 * 32 - 1] == 1 and row_parts[21 * 32] == 2 and row_parts[-1] == 4
-    assert len(items) == 21 + 21 * 2 + 21 * 3 + 4                      # pieces 0-20, 21-41, 42-62, 63
+    assert most == 3 and row_parts[0] == 1 and row_parts[25 * 32 - 1] == 1 and row_parts[25 * 32] == 2 and row_parts[-1] == 3
+    assert len(items) == 25 + 25 * 2 + 14 * 3                          # pieces 0-24, 25-49, 50-63
     # a short prompt is cut down to the least walk, a very long one not at all
     assert ops.prompt_work_list(batch_of([(0, 512)]), [0, 16], 32, 4, 0)[2] == 4
     assert ops.prompt_work_list(batch_of([(0, 8192)]), [0, 256], 32, 4, 0)[2] == 1
