@@ -413,14 +413,18 @@ __global__ void argmax_pick_kernel(const float* __restrict__ part_v, const int32
 // ---- temperature sampling --------------------------------------------------
 // The law: weights w_i = exp((l_i - max) / T) in float, summed in double; the token is the first i,
 // in vocabulary order, at which u * total - (w_0 + ... + w_i) turns negative.  One workgroup a row.
-// The vocabulary is cut into groups of 64 consecutive tokens (64 * per_lane beyond 262,144 tokens,
-// so that the groups' sums fit LDS): a wave takes a group at a time, a lane a token, so every pass
-// over the row reads whole cache lines; the groups' sums, a running sum over them (one wave, 64
-// groups a step) and a last look inside the one group where the target is crossed find the token.
+// The vocabulary is cut into groups of 512 consecutive tokens, a lane holding eight in a row (more
+// beyond 2,097,152 tokens, so that the groups' sums fit LDS): a lane sums its own tokens in order
+// without a word to its neighbours (sums of doubles across lanes go through the LDS crossbar, which
+// sixteen waves share), a wave then a group; every pass over the row reads whole cache lines.  The
+// groups' sums, a running sum over them (one wave, 64 groups a step) and a last look inside the one
+// group where the target is crossed find the token.
 // (Sums in another order than the host's one-by-one walk: a boundary may move by one token when u
 // falls within rounding of it.)
-constexpr int kSampleThreads = 512;
+constexpr int kSampleThreads = 1024;
 constexpr int kSampleMaxGroups = 4096;
+constexpr int kSamplePerLane = 8;           // consecutive tokens a lane holds of a group
+constexpr int kSampleAhead = 4;             // loads of 16 bytes (pairs of them in the second pass) a thread has in flight
 
 __device__ inline double wave_sum_f64(double v) {
 #pragma unroll
@@ -442,32 +446,58 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(const float* __r
                                                                const double* __restrict__ u, int32_t* __restrict__ out,
                                                                int vocab) {
   __shared__ double group_sum[kSampleMaxGroups];      // then: the running sum up to and with each group
-  __shared__ float best_v[kSampleThreads];
-  __shared__ int best_i[kSampleThreads];
-  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   constexpr int kWaves = kSampleThreads / kWave;
+  __shared__ float best_v[kWaves];
+  __shared__ int best_i[kWaves];
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const float* row = logits + static_cast<size_t>(blockIdx.x) * vocab;
 
   // the maximum and where it stands first
   float v = -FLT_MAX;
   int idx = vocab;
-  for (int i = threadIdx.x; i < vocab; i += kSampleThreads) better(v, idx, row[i], i);
-  best_v[threadIdx.x] = v;
-  best_i[threadIdx.x] = idx;
-  __syncthreads();
-  for (int h = kSampleThreads / 2; h > 0; h >>= 1) {
-    if (threadIdx.x < h) better(best_v[threadIdx.x], best_i[threadIdx.x], best_v[threadIdx.x + h], best_i[threadIdx.x + h]);
-    __syncthreads();
+  const bool by_four = vocab % 4 == 0;      // then every row starts on 16 bytes and no group of four straddles its end
+  if (by_four) {
+    const float4* row4 = reinterpret_cast<const float4*>(row);
+    const int n4 = vocab / 4;
+    for (int at = threadIdx.x; at < n4; at += kSampleAhead * kSampleThreads) {
+      float4 t[kSampleAhead];               // the loads first, so that they are in flight together
+#pragma unroll
+      for (int j = 0; j < kSampleAhead; ++j) {
+        const int i4 = at + j * kSampleThreads;
+        t[j] = i4 < n4 ? row4[i4] : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+#pragma unroll
+      for (int j = 0; j < kSampleAhead; ++j) {
+        const int i4 = at + j * kSampleThreads;
+        if (i4 < n4) {
+          better(v, idx, t[j].x, 4 * i4);
+          better(v, idx, t[j].y, 4 * i4 + 1);
+          better(v, idx, t[j].z, 4 * i4 + 2);
+          better(v, idx, t[j].w, 4 * i4 + 3);
+        }
+      }
+    }
+  } else {
+    for (int at = threadIdx.x; at < vocab; at += kSampleThreads) better(v, idx, row[at], at);
   }
-  const float row_max = best_v[0];
-  const int arg = best_i[0] < vocab ? best_i[0] : 0;
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) better(v, idx, __shfl_xor(v, off, kWave), __shfl_xor(idx, off, kWave));
+  if (lane == 0) {
+    best_v[wave] = v;
+    best_i[wave] = idx;
+  }
+  __syncthreads();
+  float row_max = best_v[0];
+  int best = best_i[0];
+  for (int w = 1; w < kWaves; ++w) better(row_max, best, best_v[w], best_i[w]);
+  const int arg = best < vocab ? best : 0;
   const float temp = temperature[blockIdx.x];
   if (!(temp > 0.f)) {
     if (threadIdx.x == 0) out[blockIdx.x] = arg;
     return;
   }
   const float inv_t = 1.0f / temp;
-  const int per_lane = (vocab + kWave * kSampleMaxGroups - 1) / (kWave * kSampleMaxGroups);   // 1 for usual vocabularies
+  const int per_lane = max(kSamplePerLane, (vocab + kWave * kSampleMaxGroups - 1) / (kWave * kSampleMaxGroups));
   const int group_size = kWave * per_lane;
   const int n_groups = (vocab + group_size - 1) / group_size;
   auto lane_weight_sum = [&](int g) {      // this lane's tokens of group g, in order
@@ -479,9 +509,40 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(const float* __r
     }
     return s;
   };
-  for (int g = wave; g < n_groups; g += kWaves) {
-    const double s = wave_sum_f64(lane_weight_sum(g));
-    if (lane == 0) group_sum[g] = s;
+  if (by_four && per_lane == kSamplePerLane) {        // a wave's groups at once: their loads are in flight together
+    static_assert(kSamplePerLane == 8, "two loads of four a lane");
+    for (int g0 = wave; g0 < n_groups; g0 += kWaves * kSampleAhead) {
+      float4 t[kSampleAhead][2];
+#pragma unroll
+      for (int j = 0; j < kSampleAhead; ++j) {
+        const int first = (g0 + j * kWaves) * group_size + lane * kSamplePerLane;
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+          t[j][h] = first + 4 * h < vocab ? *reinterpret_cast<const float4*>(row + first + 4 * h) : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+#pragma unroll
+      for (int j = 0; j < kSampleAhead; ++j) {
+        const int g = g0 + j * kWaves;
+        const int first = g * group_size + lane * kSamplePerLane;
+        double s = 0.0;                     // the order of lane_weight_sum: the look inside a group sums the same
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          if (first + 4 * h < vocab) {
+            s += static_cast<double>(expf((t[j][h].x - row_max) * inv_t));
+            s += static_cast<double>(expf((t[j][h].y - row_max) * inv_t));
+            s += static_cast<double>(expf((t[j][h].z - row_max) * inv_t));
+            s += static_cast<double>(expf((t[j][h].w - row_max) * inv_t));
+          }
+        }
+        s = wave_sum_f64(s);
+        if (lane == 0 && g < n_groups) group_sum[g] = s;
+      }
+    }
+  } else {
+    for (int g = wave; g < n_groups; g += kWaves) {
+      const double s = wave_sum_f64(lane_weight_sum(g));
+      if (lane == 0) group_sum[g] = s;
+    }
   }
   __syncthreads();
   if (wave != 0) return;

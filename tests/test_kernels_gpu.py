@@ -587,11 +587,12 @@ def test_argmax_ties_and_sampling(ops):
             assert abs(got[i] - want) == 1 and edge < 1e-3 * cum[-1], (i, got[i], want)
 
 
-@pytest.mark.parametrize("vocab", [97, 1000, 128256, 300001])
+@pytest.mark.parametrize("vocab", [97, 1000, 1028, 128256, 300001, 2100003])
 def test_sampling_follows_the_law_at_other_vocabularies(ops, vocab):
     """The device's draw against the host's walk through the vocabulary for the same uniform numbers:
-    vocabularies that are no multiple of the 64-token groups, one as large as Llama 3's, and one beyond
-    262,144 tokens (a lane then takes several tokens of a group); u near 0 and near 1 reach the ends."""
+    vocabularies that are no multiple of the 512-token groups (with and without a row start on 16 bytes: the
+    kernel reads by four where it can), one as large as Llama 3's, and one beyond 2,097,152 tokens (a lane
+    then takes more than eight tokens of a group); u near 0 and near 1 reach the ends."""
     from bare_cuda_4gib_amd.sampling import SamplingParams, sample_token
     row = rnd(1, vocab, seed=21, scale=2.0).float()
     us = [0.0, 1e-12, 0.25, 0.5, 0.731, 0.999999, 0.9999999999]
