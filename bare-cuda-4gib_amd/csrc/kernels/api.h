@@ -154,6 +154,12 @@ int bc4g_gemm_mfma(const void* a, const void* w, void* out, int epilogue, int m,
 // parts [k_parts, m, n]: for few rows and a long k, where one workgroup per 64 x 64 tile would walk all of k alone.
 // Whoever reads the parts adds them up in order (bc4g_rmsnorm_sum).
 int bc4g_gemm_mfma_parts(const void* a, const void* w, float* parts, int m, int n, int k, int k_parts, void* stream);
+// The SwiGLU product (epilogue 3) of rows that lack their RMSNorm's common factor: a = bfloat16(residual * g) [m, k] and
+// the parts of the rows' sums of squares as bc4g_gemm_skinny_emit leaves them (ssq_parts [ssq_blocks][ssq_stride]); every
+// row's sums are multiplied by 1 / sqrt(sum of squares / k + eps) before the activation, the parts added in the order
+// of bc4g_gemm_skinny_prenormed.  k a multiple of 64, n of 16, operands on 16-byte boundaries; any m.
+int bc4g_gemm_mfma_swiglu_scaled(const void* a, const float* ssq_parts, int ssq_blocks, int ssq_stride, float eps,
+                                 const void* w, void* out, int m, int n, int k, void* stream);
 // The output tile (rows, columns) bc4g_gemm_mfma (qkv 0) or bc4g_gemm_mfma_qkv (qkv 1) takes for these operands: for
 // the accounting of bytes and for tests that want to meet every tile.  Launches nothing.
 int bc4g_gemm_mfma_tile(const void* a, const void* w, int m, int n, int k, int qkv, int* rows, int* cols);

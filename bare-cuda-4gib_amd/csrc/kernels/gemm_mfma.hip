@@ -39,7 +39,24 @@ constexpr int kXcds = 8;
 // kRopeKvBf16: w holds query, key and value heads with every head's rows in blocks of 16 (eight dimensions, then their
 // rotation partners, which so lie eight columns apart in the product): queries are stored rotated, keys go rotated
 // into their pages, values into theirs (operands straight into LDS only).
-enum Epilogue : int { kStoreBf16 = 0, kStoreF32 = 1, kAccumF32 = 2, kSwigluBf16 = 3, kRopeKvBf16 = 4 };
+// kSwigluScaledBf16: the same for rows of a that lack their RMSNorm's common factor (a = bfloat16(residual * g), as the
+// product that last added to the residual left it, with every row's sum of squares in parts): a row's sums are
+// multiplied by 1 / sqrt(sum of squares / k + eps) before the activation (operands straight into LDS only).
+enum Epilogue : int { kStoreBf16 = 0, kStoreF32 = 1, kAccumF32 = 2, kSwigluBf16 = 3, kRopeKvBf16 = 4, kSwigluScaledBf16 = 5 };
+
+constexpr int kPartSums = 8;  // chains a row's parts are added in: chain j takes parts j, j + 8, ... in ascending order, and the
+                              // chains are added in order of j -- the order of the weight-streaming kernel, so the same factor
+struct RowScaleArgs {
+  const float* parts;         // [blocks][stride]: block b's share of every row's sum of squares
+  int blocks, stride;
+  float eps;
+};
+// a patch's rows' sums in LDS ([kPartSums][stride], from the patch's first row on) and what finishes them
+struct RowScale {
+  const float* sums = nullptr;
+  int stride = 0;
+  float inv_k = 0.f, eps = 0.f;
+};
 
 struct RopeKvArgs {
   const float2* table;        // [m, head_dim / 2] (cos, sin) of every row's position and pair (null: no rotation)
@@ -70,9 +87,10 @@ __device__ inline void tile_of(int block, int m_blocks, int n_blocks, int& bm, i
 
 // Stores ROWS x COLS floats (stride COLS + 4) from LDS with the epilogue, THREADS threads together.
 template <int EPI, int THREADS, int ROWS, int COLS>
-__device__ inline void store_patch(const float* patch, void* __restrict__ out, int m, int n, long m0, long n0, int tid) {
+__device__ inline void store_patch(const float* patch, void* __restrict__ out, int m, int n, long m0, long n0, int tid,
+                                   const RowScale& rs = RowScale{}) {
   constexpr int kStride = COLS + 4;
-  if constexpr (EPI == kSwigluBf16) {
+  if constexpr (EPI == kSwigluBf16 || EPI == kSwigluScaledBf16) {
     // (a block of 16 columns -- eight gates, then their eight ups -- a thread: eight outputs, stored at once)
     const long n_out = n / 2;
     for (int c = tid; c < ROWS * (COLS / 16); c += THREADS) {
@@ -82,11 +100,18 @@ __device__ inline void store_patch(const float* patch, void* __restrict__ out, i
       const float* src = patch + row * kStride + col;
       const floatx4 g0 = *reinterpret_cast<const floatx4*>(src), g1 = *reinterpret_cast<const floatx4*>(src + 4);
       const floatx4 u0 = *reinterpret_cast<const floatx4*>(src + 8), u1 = *reinterpret_cast<const floatx4*>(src + 12);
+      float scale = 1.f;
+      if constexpr (EPI == kSwigluScaledBf16) {
+        float ssq = 0.f;
+#pragma unroll
+        for (int j = 0; j < kPartSums; ++j) ssq += rs.sums[j * rs.stride + row];
+        scale = 1.0f / sqrtf(ssq * rs.inv_k + rs.eps);
+      }
       float v[8];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        v[e] = silu_quick(g0[e]) * u0[e];
-        v[4 + e] = silu_quick(g1[e]) * u1[e];
+        v[e] = silu_quick(g0[e] * scale) * (u0[e] * scale);
+        v[4 + e] = silu_quick(g1[e] * scale) * (u1[e] * scale);
       }
       bf16_t* dst = static_cast<bf16_t*>(out) + gm * n_out + (gn / 16) * 8;
       if (n_out % 8 == 0) {
@@ -448,7 +473,7 @@ struct DirectShape {
 template <int EPI, int WM, int WN, int TM, int TN, int BK, int STAGES, int MINWG>
 __global__ __launch_bounds__(64 * WM * WN, MINWG) void gemm_mfma_direct_kernel(
     const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, void* __restrict__ out, int m, int n, int k, int m_blocks,
-    int n_blocks, const RopeKvArgs ra) {
+    int n_blocks, const RopeKvArgs ra, const RowScaleArgs rows) {
   typedef DirectShape<WM, WN, TM, TN, BK, STAGES> S;
   constexpr int RA = S::kRowsA, RW = S::kRowsW, RB = S::kRowBytes, NW = S::kWaves;
   constexpr int kGroupRows = 1024 / RB;                    // rows a wave-wide load covers
@@ -504,6 +529,30 @@ __global__ __launch_bounds__(64 * WM * WN, MINWG) void gemm_mfma_direct_kernel(
 #pragma unroll
   for (int s = 0; s < STAGES - 1; ++s)
     if (s < nk) ask(s);
+
+  // kSwigluScaledBf16: the tile's rows' sums of squares from their parts, a chain a thread (its loads all in flight
+  // together), beside the first operands' way into LDS.  (The compiler's wait for these loads knows nothing of the
+  // operands asked for before them and so waits for those too: loads return in the order asked.  By the loop's own
+  // waits, which count the operands' loads alone, these are done.)
+  __shared__ float part_sum[EPI == kSwigluScaledBf16 ? kPartSums * RA : 1];
+  if constexpr (EPI == kSwigluScaledBf16) {
+    for (int slot = tid; slot < kPartSums * RA; slot += S::kThreads) {
+      const int row = slot % RA, chain = slot / RA;
+      float ss = 0.f;
+      if (m0 + row < m) {
+        const float* p = rows.parts + m0 + row;
+        int b = chain;
+        for (; b + 3 * kPartSums < rows.blocks; b += 4 * kPartSums) {
+          const float p0 = p[static_cast<long>(b) * rows.stride], p1 = p[static_cast<long>(b + kPartSums) * rows.stride];
+          const float p2 = p[static_cast<long>(b + 2 * kPartSums) * rows.stride];
+          const float p3 = p[static_cast<long>(b + 3 * kPartSums) * rows.stride];
+          ss = (((ss + p0) + p1) + p2) + p3;
+        }
+        for (; b < rows.blocks; b += kPartSums) ss += p[static_cast<long>(b) * rows.stride];
+      }
+      part_sum[slot] = ss;
+    }
+  }
 
   const int frow = lane % 32, fhalf = lane / 32;
   int aoff[TM], woff[TN], aswz[TM], wswz[TN];
@@ -567,6 +616,9 @@ __global__ __launch_bounds__(64 * WM * WN, MINWG) void gemm_mfma_direct_kernel(
       for (int r = 0; r < 16; ++r) patch[(8 * (r / 4) + 4 * (lane / 32) + r % 4) * kStride + j * 32 + lane % 32] = acc[i][j][r];
     if constexpr (EPI == kRopeKvBf16)
       store_patch_rope<kWave, 32, 32 * TN>(patch, static_cast<bf16_t*>(out), m, n, m0 + (wm * TM + i) * 32, n0 + wn * TN * 32, lane, ra);
+    else if constexpr (EPI == kSwigluScaledBf16)
+      store_patch<EPI, kWave, 32, 32 * TN>(patch, out, m, n, m0 + (wm * TM + i) * 32, n0 + wn * TN * 32, lane,
+                                           RowScale{part_sum + (wm * TM + i) * 32, RA, 1.0f / static_cast<float>(k), rows.eps});
     else
       store_patch<EPI, kWave, 32, 32 * TN>(patch, out, m, n, m0 + (wm * TM + i) * 32, n0 + wn * TN * 32, lane);
   }
@@ -574,7 +626,7 @@ __global__ __launch_bounds__(64 * WM * WN, MINWG) void gemm_mfma_direct_kernel(
 
 template <int EPI, int WM, int WN, int TM, int TN, int BK, int STAGES, int MINWG>
 int launch_direct(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, int k, hipStream_t s, const RopeKvArgs& ra,
-                  int k_parts = 1) {
+                  int k_parts = 1, const RowScaleArgs& rows = RowScaleArgs{}) {
   typedef DirectShape<WM, WN, TM, TN, BK, STAGES> S;
   auto kernel = gemm_mfma_direct_kernel<EPI, WM, WN, TM, TN, BK, STAGES, MINWG>;
   static bool raised = false;   // per instantiation: allow more than the default dynamic LDS
@@ -586,7 +638,7 @@ int launch_direct(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, i
   }
   const long m_blocks = (m + S::kRowsA - 1) / S::kRowsA, n_blocks = (n + S::kRowsW - 1) / S::kRowsW;
   kernel<<<dim3(static_cast<unsigned>(m_blocks * n_blocks), static_cast<unsigned>(k_parts)), dim3(S::kThreads), S::kLdsBytes, s>>>(
-      ap, wp, out, m, n, k, static_cast<int>(m_blocks), static_cast<int>(n_blocks), ra);
+      ap, wp, out, m, n, k, static_cast<int>(m_blocks), static_cast<int>(n_blocks), ra, rows);
   return 0;
 }
 
@@ -632,14 +684,14 @@ int direct_form(int m, int n, int k, bool long_epilogue) {
 
 template <int EPI>
 int launch_direct_form(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, int k, hipStream_t s,
-                       const RopeKvArgs& ra = RopeKvArgs{}) {
+                       const RopeKvArgs& ra = RopeKvArgs{}, const RowScaleArgs& rows = RowScaleArgs{}) {
   switch (direct_form(m, n, k, EPI == kRopeKvBf16)) {
-    case 0: return launch_direct<EPI, 4, 4, 2, 2, 64, 2, 1>(ap, wp, out, m, n, k, s, ra);
-    case 1: return launch_direct<EPI, 4, 2, 2, 3, 64, 2, 1>(ap, wp, out, m, n, k, s, ra);
-    case 2: return launch_direct<EPI, 4, 2, 2, 2, 64, 3, 1>(ap, wp, out, m, n, k, s, ra);
-    case 3: return launch_direct<EPI, 2, 4, 2, 1, 64, 4, 1>(ap, wp, out, m, n, k, s, ra);
-    case 5: return launch_direct<EPI, 2, 2, 2, 1, 64, 2, 4>(ap, wp, out, m, n, k, s, ra);
-    default: return launch_direct<EPI, 2, 2, 1, 1, 64, 4, 2>(ap, wp, out, m, n, k, s, ra);
+    case 0: return launch_direct<EPI, 4, 4, 2, 2, 64, 2, 1>(ap, wp, out, m, n, k, s, ra, 1, rows);
+    case 1: return launch_direct<EPI, 4, 2, 2, 3, 64, 2, 1>(ap, wp, out, m, n, k, s, ra, 1, rows);
+    case 2: return launch_direct<EPI, 4, 2, 2, 2, 64, 3, 1>(ap, wp, out, m, n, k, s, ra, 1, rows);
+    case 3: return launch_direct<EPI, 2, 4, 2, 1, 64, 4, 1>(ap, wp, out, m, n, k, s, ra, 1, rows);
+    case 5: return launch_direct<EPI, 2, 2, 2, 1, 64, 2, 4>(ap, wp, out, m, n, k, s, ra, 1, rows);
+    default: return launch_direct<EPI, 2, 2, 1, 1, 64, 4, 2>(ap, wp, out, m, n, k, s, ra, 1, rows);
   }
 }
 
@@ -684,6 +736,21 @@ extern "C" int bc4g_gemm_mfma(const void* a, const void* w, void* out, int epilo
   }
   if (e) return e;
   return check_launch("gemm_mfma");
+}
+
+extern "C" int bc4g_gemm_mfma_swiglu_scaled(const void* a, const float* ssq_parts, int ssq_blocks, int ssq_stride, float eps,
+                                            const void* w, void* out, int m, int n, int k, void* stream) {
+  BC4G_REQUIRE(m >= 0 && n > 0 && n % 16 == 0 && k > 0 && direct_operands(a, w, k),
+               "gemm_mfma_swiglu_scaled: K=%d must be a multiple of 64, N=%d one of 16 and the operands on 16-byte boundaries (M=%d)", k, n, m);
+  BC4G_REQUIRE(ssq_parts != nullptr && ssq_blocks > 0 && ssq_stride >= m && eps >= 0.f,
+               "gemm_mfma_swiglu_scaled: the sums of squares need %d parts of at least %d rows, and eps must not be negative", ssq_blocks, m);
+  if (m == 0) return 0;
+  BC4G_REQUIRE(((m + 63L) / 64) * ((n + 63L) / 64) <= 2147483647L, "gemm_mfma_swiglu_scaled: too many tiles");
+  if (int e = launch_direct_form<kSwigluScaledBf16>(static_cast<const bf16_t*>(a), static_cast<const bf16_t*>(w), out, m, n, k,
+                                                     static_cast<hipStream_t>(stream), RopeKvArgs{},
+                                                     RowScaleArgs{ssq_parts, ssq_blocks, ssq_stride, eps}))
+    return e;
+  return check_launch("gemm_mfma_swiglu_scaled");
 }
 
 extern "C" int bc4g_gemm_mfma_parts(const void* a, const void* w, float* parts, int m, int n, int k, int k_parts, void* stream) {

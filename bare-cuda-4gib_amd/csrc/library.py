@@ -20,6 +20,7 @@ _SIGNATURES = {
     "bc4g_rmsnorm": [_P, _P, _P, _I, _P, _I, _I, _I, _F, _P],
     "bc4g_rmsnorm_sum": [_P, _P, _I, _P, _I, _P, _I, _I, _I, _F, _P],
     "bc4g_gemm_mfma_parts": [_P, _P, _P, _I, _I, _I, _I, _P],
+    "bc4g_gemm_mfma_swiglu_scaled": [_P, _P, _I, _I, _F, _P, _P, _I, _I, _I, _P],
     "bc4g_gemm_generic": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _P],
     "bc4g_swiglu": [_P, _P, _I, _I, _I, _I, _P],
     "bc4g_rope_table": [_P, _P, _I, _I, _F, _P],

@@ -598,9 +598,21 @@ def gemm_accumulate_emit(a: torch.Tensor, w, residual: torch.Tensor, g: torch.Te
     return Prenormed(xb, parts, eps)
 
 
-def gemm_prenormed_supported(pre: Prenormed, w) -> bool:
+TILED_PRENORMED = True
+
+
+def tiled_takes_prenormed(n_rows: int, n: int, k: int) -> bool:
+    """Whether a SwiGLU product of these sizes that goes to the tiled kernel can finish a prepared norm there."""
+    return TILED_PRENORMED and not streams_weights(n_rows, n, k) and k % 64 == 0 and n % 16 == 0
+
+
+def gemm_prenormed_supported(pre: Prenormed, w, epilogue: Optional[int] = None) -> bool:
     w, _ = _weight(w)
-    return _fast_operands(pre.xb, w) and streams_weights(pre.xb.shape[0], w.shape[0], w.shape[1])
+    if not _fast_operands(pre.xb, w):
+        return False
+    m, (n, k) = pre.xb.shape[0], w.shape
+    return streams_weights(m, n, k) or (epilogue == EPI_SWIGLU and tiled_takes_prenormed(m, n, k)
+                                        and _ptr(pre.xb) % 16 == 0 and _ptr(w) % 16 == 0)
 
 
 def gemm_prenormed(pre: Prenormed, w, epilogue: int) -> torch.Tensor:
@@ -619,6 +631,12 @@ def gemm_prenormed(pre: Prenormed, w, epilogue: int) -> torch.Tensor:
         out = torch.empty((m, n), dtype=torch.float32, device=w.device)
     else:
         raise KernelError(f"gemm_prenormed: epilogue {epilogue} is not supported")
+    if not streams_weights(m, n, k):
+        if epilogue != EPI_SWIGLU:
+            raise KernelError("gemm_prenormed: the tiled kernel finishes a prepared norm in its SwiGLU epilogue only")
+        library.call("bc4g_gemm_mfma_swiglu_scaled", _ptr(pre.xb), _ptr(pre.parts), pre.parts.shape[0], pre.parts.shape[1], pre.eps,
+                     _ptr(w), _ptr(out), m, n, k, _stream(), cost=_tiled_cost(m, n, k, 1))
+        return out
     for r0 in range(0, m, SKINNY_MAX_ROWS):
         rows = min(SKINNY_MAX_ROWS, m - r0)
         library.call("bc4g_gemm_skinny_prenormed", _ptr(pre.xb[r0:]), _ptr(pre.parts[:, r0:]), pre.parts.shape[0], m,

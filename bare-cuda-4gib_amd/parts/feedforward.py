@@ -51,10 +51,15 @@ class SwiGLU(Part):
         1.020 -> 0.990 ms at 8 rows, no difference at 4, 0.918 -> 0.948 at one).  From 9 rows on the
         fused norm is out of reach and the choice is a norm kernel of its own: that is the faster way
         up to 63 rows, because every workgroup of the product has to add up the prepared parts (1.085
-        against 1.072 ms at 16 rows, 1.269 against 1.252 at 32, 1.558 against 1.565 at 64)."""
+        against 1.072 ms at 16 rows, 1.269 against 1.252 at 32, 1.558 against 1.565 at 64).  Those are
+        the weight-streaming kernel's figures: a wide gate-up product of 24 to 64 rows goes to the tiled
+        kernel, which adds the parts up once a tile of 64 rows while its first operands are on their way
+        and puts the rows' factors into its epilogue -- the norm's kernel goes (1.212 -> 1.197 ms at
+        32 rows, 1.361 -> 1.345 at 64)."""
         if not self.interleaved:
             return False
-        # (a wide gate-up product of 24 rows and more goes to the tiled kernel, which reads a finished norm)
+        if n_rows <= ops.SKINNY_MAX_ROWS and ops.tiled_takes_prenormed(n_rows, *self.w_gu.shape):
+            return True
         return 5 <= n_rows <= ops.NORMED_MAX_ROWS or (n_rows >= 64 and ops.streams_weights(n_rows, *self.w_gu.shape))
 
     def forward(self, h, ctx, residual) -> None:

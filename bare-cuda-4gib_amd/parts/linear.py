@@ -25,7 +25,7 @@ def _fused_norm(x: Normed, w, epilogue: int) -> Optional[torch.Tensor]:
 
 def _prepared_norm(x: Normed, w, epilogue: int) -> Optional[torch.Tensor]:
     """The product from what the product before left for this norm, where there is such a thing."""
-    if x.pre is None or x._tensor is not None or not ops.gemm_prenormed_supported(x.pre, w):
+    if x.pre is None or x._tensor is not None or not ops.gemm_prenormed_supported(x.pre, w, epilogue):
         return None
     return ops.gemm_prenormed(x.pre, w, epilogue)
 

@@ -768,6 +768,36 @@ def test_tiled_qkv_product_with_rotation_and_cache_write(ops, nh, nkv, d, m, k, 
         assert bool((kc3.permute(0, 2, 1, 3)[free] == -7.5).all()) and bool((vc3.permute(0, 3, 1, 2)[free] == -7.5).all()), "spill"
 
 
+@pytest.mark.parametrize("m,width,n2", [(24, 128, 8192), (37, 320, 8208), (64, 2048, 11264), (50, 192, 9008)])
+def test_tiled_swiglu_finishes_a_prepared_norm(ops, m, width, n2):
+    """A wide gate-up product of 24 to 64 rows goes to the tiled kernel, which takes what the adding product before it
+    left (bfloat16(residual * g) and the parts of the rows' sums of squares) and puts every row's factor into its
+    epilogue: equal to SwiGLU of rmsnorm(residual) w^T up to rounding, and to what the weight-streaming kernel makes
+    of the same operands (rows whose sizes differ a hundredfold show a factor taken from the wrong row), in
+    tiles that hang over the rows and the columns, and with other things having been in the parts' memory."""
+    k = 64
+    a, w = bf(rnd(m, k, seed=80)), bf(rnd(width, k, seed=81, scale=0.3))
+    g = bf(1.0 + 0.2 * rnd(width, seed=82))
+    base = rnd(m, width, seed=83, scale=2.0).float()
+    base *= torch.tensor([100.0 if r % 3 == 1 else (0.01 if r % 3 == 2 else 1.0) for r in range(m)]).unsqueeze(1)
+    res = base.clone().to(DEV)
+    torch.full((4096,), 1e30, device=DEV)                     # (freed at once: what the next allocations may find)
+    pre = ops.gemm_accumulate_emit(a.to(DEV), w.to(DEV), res, g.to(DEV), 1e-5)
+    r = res.cpu()
+    hb = pre.xb.cpu().double() / torch.sqrt((r.double() ** 2).mean(-1, keepdim=True) + 1e-5)
+    w2 = bf(rnd(n2, width, seed=84, scale=0.3))
+    wi = interleave8(w2[:n2 // 2], w2[n2 // 2:]).to(DEV)
+    assert not ops.streams_weights(m, n2, width) and ops.gemm_prenormed_supported(pre, wi, ops.EPI_SWIGLU)
+    assert not ops.gemm_prenormed_supported(pre, wi, ops.EPI_STORE_BF16)
+    got = ops.gemm_prenormed(pre, wi, ops.EPI_SWIGLU)
+    gu = hb @ w2.double().T
+    close(got, P.swiglu(gu[:, :n2 // 2], gu[:, n2 // 2:]), 8e-3, 3e-2, "prenormed, SwiGLU, tiled")
+    # the weight-streaming kernel on the first 23 rows of the same operands: the same factor from the same parts
+    few = ops.Prenormed(pre.xb[:23].contiguous(), pre.parts[:, :23].contiguous(), pre.eps)
+    assert ops.streams_weights(23, n2, width)
+    close(got[:23], ops.gemm_prenormed(few, wi, ops.EPI_SWIGLU), 8e-3, 1e-3, "against the weight-streaming kernel")
+
+
 @pytest.mark.parametrize("m", [1, 5, 8, 9, 16, 33, 64])
 @pytest.mark.parametrize("width,k,gdt", [(96, 40, torch.bfloat16), (2048, 256, torch.bfloat16), (200, 72, torch.float32)])
 def test_adding_product_prepares_the_next_norm(ops, m, width, k, gdt):
