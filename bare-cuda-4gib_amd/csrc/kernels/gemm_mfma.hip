@@ -536,19 +536,23 @@ __global__ __launch_bounds__(64 * WM * WN, MINWG) void gemm_mfma_direct_kernel(
   // waits, which count the operands' loads alone, these are done.)
   __shared__ float part_sum[EPI == kSwigluScaledBf16 ? kPartSums * RA : 1];
   if constexpr (EPI == kSwigluScaledBf16) {
-    for (int slot = tid; slot < kPartSums * RA; slot += S::kThreads) {
-      const int row = slot % RA, chain = slot / RA;
+    static_assert(kPartSums * RA % S::kThreads == 0, "whole chains a thread");
+    constexpr int kAhead = 16;              // parts of a chain asked for together: one way to memory and back for 128 parts
+#pragma unroll
+    for (int turn = 0; turn < kPartSums * RA / S::kThreads; ++turn) {
+      const int slot = turn * S::kThreads + tid, row = slot % RA, chain = slot / RA;
+      const bool live = m0 + row < m;
+      const float* p = rows.parts + (live ? m0 + row : 0);
       float ss = 0.f;
-      if (m0 + row < m) {
-        const float* p = rows.parts + m0 + row;
-        int b = chain;
-        for (; b + 3 * kPartSums < rows.blocks; b += 4 * kPartSums) {
-          const float p0 = p[static_cast<long>(b) * rows.stride], p1 = p[static_cast<long>(b + kPartSums) * rows.stride];
-          const float p2 = p[static_cast<long>(b + 2 * kPartSums) * rows.stride];
-          const float p3 = p[static_cast<long>(b + 3 * kPartSums) * rows.stride];
-          ss = (((ss + p0) + p1) + p2) + p3;
+      for (int b0 = chain; b0 < rows.blocks; b0 += kAhead * kPartSums) {
+        float part[kAhead];
+#pragma unroll
+        for (int i = 0; i < kAhead; ++i) {
+          const int b = b0 + i * kPartSums;
+          part[i] = live && b < rows.blocks ? p[static_cast<long>(b) * rows.stride] : 0.f;
         }
-        for (; b < rows.blocks; b += kPartSums) ss += p[static_cast<long>(b) * rows.stride];
+#pragma unroll
+        for (int i = 0; i < kAhead; ++i) ss += part[i];          // (in ascending order; a part that is not there adds 0)
       }
       part_sum[slot] = ss;
     }
