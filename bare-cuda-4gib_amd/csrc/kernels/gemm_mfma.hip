@@ -534,10 +534,33 @@ __global__ __launch_bounds__(64 * WM * WN, MINWG) void gemm_mfma_direct_kernel(
   // together), beside the first operands' way into LDS.  (The compiler's wait for these loads knows nothing of the
   // operands asked for before them and so waits for those too: loads return in the order asked.  By the loop's own
   // waits, which count the operands' loads alone, these are done.)
-  __shared__ float part_sum[EPI == kSwigluScaledBf16 ? kPartSums * RA : 1];
+  __shared__ __align__(16) float part_sum[EPI == kSwigluScaledBf16 ? kPartSums * RA : 4];
   if constexpr (EPI == kSwigluScaledBf16) {
-    static_assert(kPartSums * RA % S::kThreads == 0, "whole chains a thread");
+    static_assert(kPartSums * RA % S::kThreads == 0 && kPartSums * RA / 4 <= S::kThreads, "whole chains a thread");
     constexpr int kAhead = 16;              // parts of a chain asked for together: one way to memory and back for 128 parts
+    // Four rows a thread where the parts' rows allow loads of 16 bytes (a tile begins at a multiple of 64 rows): a CU
+    // takes a wave's load every 19 clocks or so, whatever its width, and a row a thread was 128 of them a tile of 64
+    // rows and 128 parts -- a microsecond, with the operands' loads waiting among them.
+    if (rows.stride % 4 == 0 && reinterpret_cast<uintptr_t>(rows.parts) % 16 == 0) {
+      if (tid < kPartSums * RA / 4) {
+        const int row = (tid % (RA / 4)) * 4, chain = tid / (RA / 4);
+        const bool live = m0 + row < m;     // (then all four are within the stride, which is no less than m)
+        const float* p = rows.parts + (live ? m0 + row : 0);
+        floatx4 ss = {0.f, 0.f, 0.f, 0.f};
+        for (int b0 = chain; b0 < rows.blocks; b0 += kAhead * kPartSums) {
+          floatx4 part[kAhead];
+#pragma unroll
+          for (int i = 0; i < kAhead; ++i) {
+            const int b = b0 + i * kPartSums;
+            part[i] = live && b < rows.blocks ? *reinterpret_cast<const floatx4*>(p + static_cast<long>(b) * rows.stride)
+                                              : floatx4{0.f, 0.f, 0.f, 0.f};
+          }
+#pragma unroll
+          for (int i = 0; i < kAhead; ++i) ss += part[i];        // (in ascending order; a part that is not there adds 0)
+        }
+        *reinterpret_cast<floatx4*>(part_sum + chain * RA + row) = ss;
+      }
+    } else
 #pragma unroll
     for (int turn = 0; turn < kPartSums * RA / S::kThreads; ++turn) {
       const int slot = turn * S::kThreads + tid, row = slot % RA, chain = slot / RA;

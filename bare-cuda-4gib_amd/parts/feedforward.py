@@ -54,8 +54,8 @@ class SwiGLU(Part):
         against 1.072 ms at 16 rows, 1.269 against 1.252 at 32, 1.558 against 1.565 at 64).  Those are
         the weight-streaming kernel's figures: a wide gate-up product of 24 to 64 rows goes to the tiled
         kernel, which adds the parts up once a tile of 64 rows while its first operands are on their way
-        and puts the rows' factors into its epilogue -- the norm's kernel goes (1.212 -> 1.187 ms at
-        32 rows, 1.363 -> 1.333 at 64)."""
+        and puts the rows' factors into its epilogue -- the norm's kernel goes (1.217 -> 1.178 ms at
+        32 rows, 1.368 -> 1.322 at 64)."""
         if not self.interleaved:
             return False
         if n_rows <= ops.SKINNY_MAX_ROWS and ops.tiled_takes_prenormed(n_rows, *self.w_gu.shape):
