@@ -37,6 +37,7 @@
 // residual stream can prepare the RMSNorm that follows (emit): it also stores bfloat16(new residual * g)
 // and, per row, the sum of squares over its 16 columns -- parts that the next product adds up in
 // block order, so the result does not depend on timing.
+#include <type_traits>
 #include <math.h>
 
 #include "api.h"
@@ -203,9 +204,14 @@ __global__ __launch_bounds__(kThreads, (XMODE != kPlain || (MT == 1 && U == 2)) 
   }
 
   // prenormed x: every row's sum of squares from its parts.  Eight threads a row, thread j adding
-  // the parts of blocks j, j + 8, ... in ascending order (its loads all in flight together); the eight
-  // sums meet in LDS and are added in order of j after the product: the order of the additions, and
-  // so the rounding, is the same for every number of rows.  (After the first weights have been asked for.)
+  // the parts of blocks j, j + 8, ... in ascending order; the eight sums meet in LDS and are added in
+  // order of j after the product: the order of the additions, and so the rounding, is the same for
+  // every number of rows.  (After the first weights have been asked for.)  How many parts a thread asks
+  // for together, by what was measured inside a model: sixteen -- one way to memory and back for 128
+  // parts instead of four -- up to 8 rows in the kernels that serve those (four k-steps a turn, and the
+  // SwiGLU product: a decode step at TinyLlama's sizes 1.000 -> 0.983 ms at 8 rows, 0.922 -> 0.917 at
+  // one), four otherwise (with sixteen or eight a step of 16 rows was 0.4-0.8 % longer, and the other
+  // kernels of two k-steps a turn spilled).
   constexpr int kPartSums = 8;
   __shared__ float part_sum[kPartSums][MT * 16];
   const bool prenormed = !kNormed && a.ssq_parts != nullptr;
@@ -215,14 +221,21 @@ __global__ __launch_bounds__(kThreads, (XMODE != kPlain || (MT == 1 && U == 2)) 
       float ss = 0.f;
       if (row < m) {
         const float* p = a.ssq_parts + row;
-        int b = j0;
-        for (; b + 3 * kPartSums < a.ssq_blocks; b += 4 * kPartSums) {
-          const float p0 = p[static_cast<long>(b) * a.ssq_stride], p1 = p[static_cast<long>(b + kPartSums) * a.ssq_stride];
-          const float p2 = p[static_cast<long>(b + 2 * kPartSums) * a.ssq_stride];
-          const float p3 = p[static_cast<long>(b + 3 * kPartSums) * a.ssq_stride];
-          ss = (((ss + p0) + p1) + p2) + p3;
-        }
-        for (; b < a.ssq_blocks; b += kPartSums) ss += p[static_cast<long>(b) * a.ssq_stride];
+        auto chain = [&](auto ahead) {
+          constexpr int kAhead = decltype(ahead)::value;
+          for (int b0 = j0; b0 < a.ssq_blocks; b0 += kAhead * kPartSums) {
+            float part[kAhead];
+#pragma unroll
+            for (int i = 0; i < kAhead; ++i) {
+              const int b = b0 + i * kPartSums;
+              part[i] = b < a.ssq_blocks ? p[static_cast<long>(b) * a.ssq_stride] : 0.f;
+            }
+#pragma unroll
+            for (int i = 0; i < kAhead; ++i) ss += part[i];      // (in ascending order; a part that is not there adds 0)
+          }
+        };
+        if ((U == 4 || EPI == kSwigluBf16) && m <= 8) chain(std::integral_constant<int, 16>{});
+        else chain(std::integral_constant<int, 4>{});
       }
       part_sum[j0][row] = ss;
     }
