@@ -4,10 +4,11 @@ request, and slots for per-request state of fixed size.
 A model's cache *streams* (one per schedule entry that caches, or shared
 between entries) each declare a spec, which says what it keeps and in which
 tensors (see ``specs.py``; the manager knows no spec by name).  Streams that keep
-something per token are put into *groups* by their window: all streams that keep
-every token share one page pool and one block table per request; streams with a
-window of W tokens share another, whose pages are given back once a request's
-window has passed them.  Within a group one page index stands for the same
+something per token are put into *groups* by the rule under which their tokens may
+be given back, which the spec states itself (``group_key``, ``first_kept``): all
+streams that keep every token share one page pool and one block table per request;
+streams with a window of W tokens share another, whose pages are given back once a
+request's window has passed them.  Within a group one page index stands for the same
 ``page_tokens`` tokens in every stream of the group, each stream having tensors
 of its own, ``[pages, *shape of one page]`` (for keys and values:
 ``[pages, kv_heads, page_tokens, head_dim]`` and, transposed,
@@ -85,9 +86,23 @@ def bytes_per_page(specs: Iterable[Any], page_tokens: int, dtype: torch.dtype) -
     return total
 
 
+def _retention(spec):
+    """(group key, first_kept, keeps everything) of a per-token spec: its own statement, or what its
+    ``window`` says (0 or absent: every token is kept)."""
+    window = int(getattr(spec, "window", 0))
+    if hasattr(spec, "first_kept"):
+        key = spec.group_key() if hasattr(spec, "group_key") else ("rule", type(spec).__name__, window)
+        return key, spec.first_kept, key == ("window", 0)
+    if window > 0:
+        return ("window", window), (lambda length: max(0, length - window + 1)), False
+    return ("window", 0), (lambda length: 0), True
+
+
 class _Group:
-    def __init__(self, window: int, num_pages: int):
-        self.window = window
+    def __init__(self, window: int, num_pages: int, first_kept, keeps_all: bool):
+        self.window = window                 # (what the views show; the rule itself is first_kept)
+        self.first_kept = first_kept         # length -> earliest token still read by a query at `length` or later
+        self.keeps_all = keeps_all
         self.pool = PagePool(num_pages)
         self.streams: List[Hashable] = []
 
@@ -123,15 +138,15 @@ class CacheManager:
                 continue
             if getattr(spec, "per_token", None) is True and hasattr(spec, "page_tensors"):
                 window = int(getattr(spec, "window", 0))
-                key = ("window", window)
+                key, first_kept, keeps_all = _retention(spec)
                 group = self.groups.get(key)
                 if group is None:
-                    group = self.groups[key] = _Group(window, num_pages)
+                    group = self.groups[key] = _Group(window, num_pages, first_kept, keeps_all)
                 group.streams.append(sid)
                 tensors = {}
                 for name, entry in spec.page_tensors(page_tokens).items():
                     shape, dt = _shape_and_dtype(entry, dtype)
-                    t = torch.empty((num_pages, *shape), dtype=dt, device=self.device)
+                    t = torch.empty((num_pages + 1, *shape), dtype=dt, device=self.device)   # (+ the scratch page)
                     if poison and t.is_floating_point():
                         t.fill_(float("nan"))
                     tensors[name] = t
@@ -140,19 +155,27 @@ class CacheManager:
                 tensors = {}
                 for name, entry in spec.slot_tensors().items():
                     shape, dt = _shape_and_dtype(entry, dtype)
-                    tensors[name] = torch.zeros((max_requests, *shape), dtype=dt, device=self.device)
+                    tensors[name] = torch.zeros((max_requests + 1, *shape), dtype=dt, device=self.device)  # (+ the scratch slot)
                 self._views[sid] = View(tensors)
             else:
                 raise EngineError(f"cache: stream {sid!r} has a spec that says neither what it keeps per token "
                                   f"(per_token = True, page_tensors) nor per request (per_token = False, slot_tensors): {spec!r}")
         self._requests: Dict[Hashable, _Request] = {}
+        self._peaks: Dict[Tuple[int, int], Dict[Hashable, int]] = {}
         self._free_slots: List[int] = list(range(max_requests - 1, -1, -1))
         # The same bookkeeping as arrays by request slot, for whoever describes a batch of many
         # requests to the device without a Python loop over them: lengths, and every group's block
         # tables as rows of a matrix (-1 where there is no page), kept in step with the lists above.
-        self.lengths_by_slot = np.zeros(max_requests, dtype=np.int32)
+        # One page and one slot beyond those that requests can hold: the *scratch* page (index num_pages, in no
+        # pool) and the scratch slot (index max_requests, never admitted to).  Rows that stand for no request --
+        # the rows that fill a captured decode step up to its graph's size -- write their keys and their state
+        # there and read nothing else.  The arrays by slot have a row for it: no tokens, one page.
+        self.scratch_page, self.scratch_slot = num_pages, max_requests
+        self.lengths_by_slot = np.zeros(max_requests + 1, dtype=np.int32)
         self.tables_by_slot: Dict[Hashable, np.ndarray] = {
-            g: np.full((max_requests, self.max_pages_per_request), -1, dtype=np.int32) for g in self.groups}
+            g: np.full((max_requests + 1, self.max_pages_per_request), -1, dtype=np.int32) for g in self.groups}
+        for t in self.tables_by_slot.values():
+            t[self.scratch_slot, 0] = self.scratch_page
 
     # ---- requests ---------------------------------------------------------
     def has(self, request: Hashable) -> bool:
@@ -270,11 +293,11 @@ class CacheManager:
         r.length += n_new
         self.lengths_by_slot[r.slot] = r.length
         for g, t in r.tables.items():
-            window = self.groups[g].window
-            if window <= 0:
+            group = self.groups[g]
+            if group.keeps_all:
                 continue
-            # the next query sits at position r.length and reads keys from r.length - window + 1
-            first_needed = max(0, r.length - window + 1) // self.page_tokens
+            # the next query sits at position r.length; pages wholly before what it and later ones read go back
+            first_needed = max(0, int(group.first_kept(r.length))) // self.page_tokens
             for idx in range(r.released[g], min(first_needed, len(t))):
                 self._give_back(g, t[idx])
                 t[idx] = -1
@@ -301,6 +324,30 @@ class CacheManager:
         self.lengths_by_slot[r.slot] = 0
         self._free_slots.append(r.slot)
         del self._requests[request]
+
+    def peak_pages(self, total_tokens: int, portion: int) -> Dict[Hashable, int]:
+        """group -> the most pages one request holds at a time while ``total_tokens`` tokens are fed
+        to it in portions of at most ``portion``, however they are cut: a step that begins at length p
+        holds the pages from first_kept(p) to p + its tokens.  Nothing for a model whose streams keep
+        nothing per token."""
+        key = (total_tokens, portion)
+        hit = self._peaks.get(key)
+        if hit is not None:
+            return hit
+        P, out = self.page_tokens, {}
+        for g, group in self.groups.items():
+            if group.keeps_all:
+                out[g] = -(-total_tokens // P)
+                continue
+            most = 0
+            for p in range(0, max(total_tokens, 1)):
+                upto = min(p + max(portion, 1), total_tokens)
+                most = max(most, -(-upto // P) - max(0, int(group.first_kept(p))) // P)
+            out[g] = most
+        if len(self._peaks) > 4096:
+            self._peaks.clear()
+        self._peaks[key] = out
+        return out
 
     def release_all(self) -> None:
         for request in list(self._requests):

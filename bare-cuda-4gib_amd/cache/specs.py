@@ -5,9 +5,13 @@ bookkeeping, and knows no spec by name.  Two kinds:
 
 per token   ``per_token = True``.  ``page_tensors(page_tokens)`` names the tensors of ONE page
             (name -> shape, or name -> (shape, dtype name) for a tensor that is not in the cache's
-            own dtype); the manager allocates ``[num_pages, *shape]`` of each.  ``window`` (0 = keep
-            everything) says how far back a token is ever read again: specs with the same window share
-            a page pool and one block table per request, and pages a window has passed are given back.
+            own dtype); the manager allocates ``[num_pages, *shape]`` of each.  When its tokens may be
+            given back the spec says itself: ``first_kept(length)`` is the earliest token that any
+            query at position ``length`` or later still reads (0: every token is kept), and pages
+            wholly before it go back to their pool; ``group_key()`` names the rule -- specs with equal
+            keys share a page pool and one block table per request.  A spec that has neither is read
+            by its ``window`` (0 or absent = keep everything; W = a query reads the W tokens up to and
+            including its own).
 per request ``per_token = False``.  ``slot_tensors()`` names the tensors of ONE request slot
             (name -> (shape, dtype name)); the manager allocates ``[max_requests, *shape]`` of each and
             zeroes a slot when a request is admitted to it.
@@ -37,6 +41,13 @@ class PagedKV:
     def page_tensors(self, page_tokens: int) -> Dict[str, Tuple[int, ...]]:
         return {"k": (self.num_kv_heads, page_tokens, self.head_dim),
                 "v": (self.num_kv_heads, self.head_dim, page_tokens)}
+
+    def group_key(self):
+        return ("window", self.window)
+
+    def first_kept(self, length: int) -> int:
+        """The query at position ``length`` reads keys from ``length - window + 1`` on."""
+        return max(0, length - self.window + 1) if self.window > 0 else 0
 
 
 @dataclasses.dataclass(frozen=True)

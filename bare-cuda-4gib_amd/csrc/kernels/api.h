@@ -86,19 +86,6 @@ int bc4g_attention_generic(const void* qkv, int q_stride, void* out, int dtype, 
 int bc4g_argmax(const float* logits, int32_t* out, float* part_v, int32_t* part_i, int n_rows, int vocab,
                 void* stream);
 
-// bc4g_argmax without a workspace argument, for callers that cannot allocate device memory: code
-// under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  (No counterpart
-// in the reference, whose argmax keeps its partial results in a buffer the model allocated.)  The slices'
-// bests go through an array of the library's own (512 KiB on every GPU the library runs on, held until
-// the process ends); the call allocates nothing and calls no allocating routine.  At most
-// bc4g_argmax_static_max_rows() = 1024 rows a call; more is refused with an error that says so.  All
-// calls on one GPU share the array, which keeps the last call's contents (nothing in it has to start
-// at zero): calls that overlap on one GPU -- on different streams, or from different threads -- race.
-// The first call on a device asks the runtime for the array's address there; a caller that captures
-// graphs makes one call outside a capture first.
-int bc4g_argmax_static(const float* logits, int32_t* out, int n_rows, int vocab, void* stream);
-int bc4g_argmax_static_max_rows();
-
 // out[r] = first i with cumsum(exp((l - max) / temperature[r]))[i] > u[r] * total, walking the
 // vocabulary in order (engine/src/sampler.cpp:39-61); temperature <= 0 gives the argmax.
 int bc4g_sample(const float* logits, const float* temperature, const double* u, int32_t* out,

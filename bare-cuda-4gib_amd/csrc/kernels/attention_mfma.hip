@@ -32,6 +32,7 @@
 // whatever lies in those places (NaN included) cannot reach the sums.
 #include <math.h>
 
+#include <mutex>
 #include <type_traits>
 
 #include "api.h"
@@ -377,37 +378,27 @@ __global__ __launch_bounds__((WS > 1 ? WS : kWavesPerBlock) * kWave, 2) void att
     bool ok[2];
     locate(ok, kt);
     if constexpr (kWholeChunks) {
-      // the wave's kPieces chunks of 1 KB go side by side: one LDS address for all, in the middle of the stretch
-      constexpr int kMid = kPieces / 2;
-      set_lds_base(__builtin_amdgcn_readfirstlane(tiles_lds + stage * (128 * d) + (wave * kPieces + kMid) * 1024));
-      auto ask_chunk = [&](auto index) {
-        constexpr int r = decltype(index)::value;
+      // the wave's kPieces chunks of 1 KB go side by side: one LDS address for all and one statement for the loads
+      // (what is looked up by a run-time index is chosen here, by selects, before that statement)
+      const void* from[kPieces];
+#pragma unroll
+      for (int r = 0; r < kPieces; ++r) {
         const int seg = chunk_seg[r];
-        const bf16_t* from = (seg >= 2 ? a.v_cache : a.k_cache) + block_at[seg & 1] + chunk_off[r];
-        load_to_lds_16_at<(r - kMid) * 1024>(ok[seg & 1] ? static_cast<const void*>(from) : static_cast<const void*>(kZeroLine),
-                                             lane * 16u);
-      };
-      static_assert(kPieces == 1 || kPieces == 2 || kPieces == 4 || kPieces == 8, "chunks a wave brings");
-      ask_chunk(std::integral_constant<int, 0>{});
-      if constexpr (kPieces >= 2) ask_chunk(std::integral_constant<int, 1>{});
-      if constexpr (kPieces >= 4) {
-        ask_chunk(std::integral_constant<int, 2>{});
-        ask_chunk(std::integral_constant<int, 3>{});
+        const long block = (seg & 1) ? block_at[1] : block_at[0];
+        const bool seen = (seg & 1) ? ok[1] : ok[0];
+        const bf16_t* at = (seg >= 2 ? a.v_cache : a.k_cache) + block + chunk_off[r];
+        from[r] = seen ? static_cast<const void*>(at) : static_cast<const void*>(kZeroLine);
       }
-      if constexpr (kPieces >= 8) {
-        ask_chunk(std::integral_constant<int, 4>{});
-        ask_chunk(std::integral_constant<int, 5>{});
-        ask_chunk(std::integral_constant<int, 6>{});
-        ask_chunk(std::integral_constant<int, 7>{});
-      }
+      load_chunks_to_lds<kPieces>(from, lane * 16u, tiles_lds + stage * (128 * d) + wave * kPieces * 1024);
     } else {
 #pragma unroll
       for (int r = 0; r < kPieces; ++r) {
         if (wave * kWave + 256 * r >= 8 * d) continue;
         const unsigned to = __builtin_amdgcn_readfirstlane(tiles_lds + stage * (128 * d) + (wave * kWave + 256 * r) * 16);
         const int seg = piece_seg[r];
-        const bf16_t* from = (seg >= 2 ? a.v_cache : a.k_cache) + block_at[seg & 1] + piece_off[r];
-        load_to_lds_16(ok[seg & 1] ? static_cast<const void*>(from) : static_cast<const void*>(kZeroLine + lane * 16), to);
+        const bf16_t* from = (seg >= 2 ? a.v_cache : a.k_cache) + ((seg & 1) ? block_at[1] : block_at[0]) + piece_off[r];
+        const bool seen = (seg & 1) ? ok[1] : ok[0];
+        load_to_lds_16(seen ? static_cast<const void*>(from) : static_cast<const void*>(kZeroLine + lane * 16), to);
       }
     }
   };
@@ -779,17 +770,25 @@ using namespace bc4g;
 namespace bc4g {
 namespace {
 template <int DJ, int DB, int QT, int WS>
-void launch_attention(const AttnArgs& a, dim3 grid, dim3 block, size_t lds, hipStream_t s) {
-  static bool raised = false;   // per instantiation: the staged form's ring may need more than the default dynamic LDS
-  if (!raised && lds > 48 * 1024) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(attention_mfma_kernel<DJ, DB, QT, WS, true>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(attention_mfma_kernel<DJ, DB, QT, WS, false>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    raised = true;
+int launch_attention(const AttnArgs& a, dim3 grid, dim3 block, size_t lds, hipStream_t s) {
+  // per instantiation, once: the staged form's ring may need more than the default dynamic LDS
+  static std::once_flag once;
+  static hipError_t raised = hipSuccess;
+  if (lds > 48 * 1024) {
+    std::call_once(once, [] {
+      raised = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_mfma_kernel<DJ, DB, QT, WS, true>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+      if (raised == hipSuccess)
+        raised = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_mfma_kernel<DJ, DB, QT, WS, false>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    });
+    if (raised != hipSuccess)
+      return fail("attention_mfma: cannot raise the dynamic LDS limit to the %zu bytes of the key tiles' ring (%s)", lds,
+                  hipGetErrorString(raised));
   }
   if (a.head_dim == 16 * DB) attention_mfma_kernel<DJ, DB, QT, WS, true><<<grid, block, lds, s>>>(a);
   else attention_mfma_kernel<DJ, DB, QT, WS, false><<<grid, block, lds, s>>>(a);
+  return 0;
 }
 }  // namespace
 }  // namespace bc4g
@@ -861,6 +860,7 @@ extern "C" int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, flo
   BC4G_REQUIRE(form >= 0 && form <= 2, "attention_mfma: unknown form %d", form);
   BC4G_REQUIRE(form != 1 || q_tiles == 1, "attention_mfma: waves share the keys of single query tiles only");
   hipStream_t s = static_cast<hipStream_t>(stream);
+  int status = 0;
   if (form == 2) {
     // four waves' tiles per workgroup (n_tiles counts workgroups), key tiles staged in a ring in LDS
     // (with a work list: heads fastest, so that the items start in the list's order, longest first)
@@ -869,34 +869,35 @@ extern "C" int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, flo
     dim3 block(kWavesPerBlock * kWave);
     const size_t lds = static_cast<size_t>(db <= 8 ? 4 : 2) * 128 * head_dim + 1024 * 4;   // (the kernel's ring of key tiles and its part of the block table)
     if (dj <= 2 && db <= 4) {
-      if (q_tiles == 4) launch_attention<2, 4, 4, 0>(a, grid, block, lds, s);
-      else launch_attention<2, 4, 1, 0>(a, grid, block, lds, s);
+      if (q_tiles == 4) status = launch_attention<2, 4, 4, 0>(a, grid, block, lds, s);
+      else status = launch_attention<2, 4, 1, 0>(a, grid, block, lds, s);
     } else if (dj <= 4 && db <= 8) {
-      if (q_tiles == 2) launch_attention<4, 8, 2, 0>(a, grid, block, lds, s);
-      else launch_attention<4, 8, 1, 0>(a, grid, block, lds, s);
+      if (q_tiles == 2) status = launch_attention<4, 8, 2, 0>(a, grid, block, lds, s);
+      else status = launch_attention<4, 8, 1, 0>(a, grid, block, lds, s);
     } else {
-      launch_attention<8, 16, 1, 0>(a, grid, block, lds, s);
+      status = launch_attention<8, 16, 1, 0>(a, grid, block, lds, s);
     }
   } else if (form == 1) {
     // one workgroup per tile; its waves (8, or 4 for the largest heads) cut the keys between them
     dim3 grid(n_tiles, n_kv_heads * a.n_sub, n_splits);
     auto lds = [&](int ws) { return static_cast<size_t>(ws) * 16 * (head_dim + kMergePad + 2) * sizeof(float); };
-    if (dj <= 2 && db <= 4) launch_attention<2, 4, 1, 8>(a, grid, 8 * kWave, lds(8), s);
-    else if (dj <= 4 && db <= 8) launch_attention<4, 8, 1, 8>(a, grid, 8 * kWave, lds(8), s);
-    else launch_attention<8, 16, 1, 4>(a, grid, 4 * kWave, lds(4), s);
+    if (dj <= 2 && db <= 4) status = launch_attention<2, 4, 1, 8>(a, grid, 8 * kWave, lds(8), s);
+    else if (dj <= 4 && db <= 8) status = launch_attention<4, 8, 1, 8>(a, grid, 8 * kWave, lds(8), s);
+    else status = launch_attention<8, 16, 1, 4>(a, grid, 4 * kWave, lds(4), s);
   } else {
     dim3 grid((n_tiles + kWavesPerBlock - 1) / kWavesPerBlock, n_kv_heads * a.n_sub, n_splits);
     dim3 block(kWavesPerBlock * kWave);
     if (dj <= 2 && db <= 4) {
-      if (q_tiles == 4) launch_attention<2, 4, 4, 1>(a, grid, block, 0, s);
-      else launch_attention<2, 4, 1, 1>(a, grid, block, 0, s);
+      if (q_tiles == 4) status = launch_attention<2, 4, 4, 1>(a, grid, block, 0, s);
+      else status = launch_attention<2, 4, 1, 1>(a, grid, block, 0, s);
     } else if (dj <= 4 && db <= 8) {
-      if (q_tiles == 2) launch_attention<4, 8, 2, 1>(a, grid, block, 0, s);
-      else launch_attention<4, 8, 1, 1>(a, grid, block, 0, s);
+      if (q_tiles == 2) status = launch_attention<4, 8, 2, 1>(a, grid, block, 0, s);
+      else status = launch_attention<4, 8, 1, 1>(a, grid, block, 0, s);
     } else {
-      launch_attention<8, 16, 1, 1>(a, grid, block, 0, s);
+      status = launch_attention<8, 16, 1, 1>(a, grid, block, 0, s);
     }
   }
+  if (status) return status;
   if (int e = check_launch("attention_mfma")) return e;
   if (n_splits > 1) {
     const long rows_heads = static_cast<long>(n_tokens) * n_heads;

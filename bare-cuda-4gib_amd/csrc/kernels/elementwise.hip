@@ -6,6 +6,7 @@
 #include <mutex>
 
 #include "api.h"
+#include "no_alloc.h"
 #include "common.h"
 
 namespace bc4g {
@@ -213,10 +214,20 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const int32_t* __restr
     float b = to_float(base[i1]);
     const bool is_v = head >= n_heads + n_kv_heads;
     if (rotate && !is_v) {
-      const float inv_freq = 1.0f / powf(theta, (2.0f * static_cast<float>(j)) / static_cast<float>(rotary_dim));
-      const float angle = static_cast<float>(positions[token]) * inv_freq;
       float s, c;
-      sincosf(angle, &s, &c);
+      if constexpr (sizeof(T) == sizeof(float)) {
+        // The 32-bit path works the angle out in double: a float angle carries an error of position * 2^-24
+        // (1e-4 rad at position 2,000), which would show in the logits of long prompts as an error that grows with
+        // the position, ten times what the rest of the path leaves, and hide what the path is there to show.
+        const double inv_freq = 1.0 / pow(static_cast<double>(theta), (2.0 * j) / static_cast<double>(rotary_dim));
+        double sd, cd;
+        sincos(static_cast<double>(positions[token]) * inv_freq, &sd, &cd);
+        s = static_cast<float>(sd);
+        c = static_cast<float>(cd);
+      } else {
+        const float inv_freq = 1.0f / powf(theta, (2.0f * static_cast<float>(j)) / static_cast<float>(rotary_dim));
+        sincosf(static_cast<float>(positions[token]) * inv_freq, &s, &c);
+      }
       const float lo = a, hi = b;
       a = lo * c - hi * s;
       b = hi * c + lo * s;
@@ -455,7 +466,9 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(const float* __r
   // the maximum and where it stands first
   float v = -FLT_MAX;
   int idx = vocab;
-  const bool by_four = vocab % 4 == 0;      // then every row starts on 16 bytes and no group of four straddles its end
+  // in fours where every row starts on 16 bytes (the base does and the vocabulary is a multiple of four): no group of
+  // four then straddles a row's end
+  const bool by_four = vocab % 4 == 0 && reinterpret_cast<uintptr_t>(logits) % 16 == 0;
   if (by_four) {
     const float4* row4 = reinterpret_cast<const float4*>(row);
     const int n4 = vocab / 4;

@@ -39,11 +39,12 @@ __device__ inline uint4 zero16() { return make_uint4(0u, 0u, 0u, 0u); }
 // Memory to LDS without passing registers: every lane of the wave brings the 16 bytes at its `global` to
 // lds_address (the same in all lanes) + 16 * lane -- 1 KB of consecutive LDS a wave.
 __device__ inline void load_to_lds_16(const void* global, unsigned lds_address) {
-  // The LDS base of a wave-wide load travels in m0, which the compiler reserves for such uses of its
-  // own and sets right before each (the kernels that call this give it none: no LDS load builtin, no
-  // register array indexed at run time).  The compiler does not know the instruction, so the waits for it are written
-  // by hand (wait_loads).
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(global), "s"(lds_address) : "memory");
+  // The LDS base of a wave-wide load travels in m0, which the compiler also uses for purposes of its own (it
+  // sets it right before each): the statement sets m0 and uses it at once, and says that it clobbers it.  The
+  // compiler does not know the instruction, so the waits for it are written by hand (wait_loads): between asking
+  // and waiting a loop must hold no other vector-memory operation of the wave -- no spill, nothing the compiler
+  // might add -- or the hand-counted waits count the wrong loads.
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(global), "s"(lds_address) : "memory", "m0");
 }
 
 // The same from one base address for the whole wave (in scalar registers) plus each lane's offset in bytes.
@@ -54,24 +55,49 @@ __device__ inline void load_to_lds_16(const void* wave_base, unsigned lane_offse
   const unsigned hi = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(bits >> 32));
   wave_base = reinterpret_cast<const void*>((static_cast<uintptr_t>(hi) << 32) | lo);
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_offset), "s"(wave_base), "s"(lds_address)
-               : "memory");
+               : "memory", "m0");
 }
 
-// The same in two steps, for several loads to one stretch of LDS: the LDS address is set once, and each load adds
-// OFFSET bytes (-4096 .. 4095) to it -- and to its memory address, so the caller takes OFFSET off that one.  (Setting
-// the LDS address anew for every load costs the wave hundreds of clocks a load: the write to m0 waits for the load
-// before it, which still needs the old value.)
-__device__ inline void set_lds_base(unsigned lds_address) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0" ::"s"(lds_address) : "memory");
-}
-template <int OFFSET>
-__device__ inline void load_to_lds_16_at(const void* wave_base, unsigned lane_offset) {
-  static_assert(OFFSET >= -4096 && OFFSET <= 4095, "the instruction's offset field");
-  const uintptr_t bits = reinterpret_cast<uintptr_t>(wave_base) - OFFSET;
-  const unsigned lo = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(bits));
-  const unsigned hi = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(bits >> 32));
-  wave_base = reinterpret_cast<const void*>((static_cast<uintptr_t>(hi) << 32) | lo);
-  asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" ::"v"(lane_offset), "s"(wave_base), "n"(OFFSET) : "memory");
+// Several such loads to one stretch of LDS as ONE statement: N chunks of 1 KB side by side, chunk r from bases[r]
+// (the same in every lane) plus each lane's offset in bytes.  The LDS address is set once, to the chunk in the
+// middle of the stretch, and each load adds its (r - N / 2) * 1024 bytes to it through the instruction's offset
+// field -- and to its memory address, so that much is taken off the base here.  (Setting the LDS address anew for
+// every load costs the wave hundreds of clocks a load: the write to m0 waits for the load before it, which still
+// needs the old value.)  The write to m0 and the loads that rely on it stand in one asm statement that says it
+// clobbers m0, so nothing the compiler makes of the code around them -- indexing a register array at run time
+// writes m0 on this hardware -- can come between them.
+template <int N>
+__device__ inline void load_chunks_to_lds(const void* const (&bases)[N], unsigned lane_offset, unsigned lds_first_chunk) {
+  static_assert(N == 1 || N == 2 || N == 4 || N == 8, "chunks a wave brings");
+  constexpr int kMid = N / 2;
+  const void* b[N];
+#pragma unroll
+  for (int r = 0; r < N; ++r) {
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(bases[r]) - (r - kMid) * 1024;
+    const unsigned lo = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(bits));
+    const unsigned hi = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(bits >> 32));
+    b[r] = reinterpret_cast<const void*>((static_cast<uintptr_t>(hi) << 32) | lo);
+  }
+  const unsigned mid = __builtin_amdgcn_readfirstlane(lds_first_chunk + kMid * 1024);
+#define BC4G_LDS_LOAD(i, op) "global_load_lds_dwordx4 %1, %" #op " offset:" #i "\n\t"
+  if constexpr (N == 1) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t" BC4G_LDS_LOAD(0, 2)
+                 ::"s"(mid), "v"(lane_offset), "s"(b[0]) : "memory", "m0");
+  } else if constexpr (N == 2) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t" BC4G_LDS_LOAD(-1024, 2) BC4G_LDS_LOAD(0, 3)
+                 ::"s"(mid), "v"(lane_offset), "s"(b[0]), "s"(b[1]) : "memory", "m0");
+  } else if constexpr (N == 4) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t" BC4G_LDS_LOAD(-2048, 2) BC4G_LDS_LOAD(-1024, 3) BC4G_LDS_LOAD(0, 4)
+                 BC4G_LDS_LOAD(1024, 5)
+                 ::"s"(mid), "v"(lane_offset), "s"(b[0]), "s"(b[1]), "s"(b[2]), "s"(b[3]) : "memory", "m0");
+  } else {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t" BC4G_LDS_LOAD(-4096, 2) BC4G_LDS_LOAD(-3072, 3) BC4G_LDS_LOAD(-2048, 4)
+                 BC4G_LDS_LOAD(-1024, 5) BC4G_LDS_LOAD(0, 6) BC4G_LDS_LOAD(1024, 7) BC4G_LDS_LOAD(2048, 8)
+                 BC4G_LDS_LOAD(3072, 9)
+                 ::"s"(mid), "v"(lane_offset), "s"(b[0]), "s"(b[1]), "s"(b[2]), "s"(b[3]), "s"(b[4]), "s"(b[5]), "s"(b[6]),
+                 "s"(b[7]) : "memory", "m0");
+  }
+#undef BC4G_LDS_LOAD
 }
 
 // Waits until at most N of the wave's memory operations are outstanding (they finish in order).

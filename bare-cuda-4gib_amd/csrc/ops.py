@@ -8,8 +8,9 @@ library, or on a CPU tensor, they raise.
 from __future__ import annotations
 
 import ctypes
+import dataclasses
 import math
-from typing import Optional, Tuple
+from typing import Dict, Optional, Tuple
 
 import torch
 
@@ -305,7 +306,7 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
 def sample(logits: torch.Tensor, temperature: torch.Tensor, u: torch.Tensor) -> torch.Tensor:
     """One draw per row from softmax(logits / temperature) by inverse CDF with the given
     uniform u in [0, 1); rows with temperature <= 0 get the argmax."""
-    _dev("sample", logits, temperature, u)
+    _dev("sample", logits, temperature, u)          # (contiguous rows: a strided view would be read as if it were dense)
     rows = logits.shape[0]
     if logits.dtype != torch.float32 or logits.dim() != 2:
         raise KernelError("sample: logits must be float32 [rows, vocab]")
@@ -342,6 +343,8 @@ class StreamedWeight:
         self.shape, self.dtype, self.device = rows.shape, rows.dtype, rows.device
         ok = rows.is_cuda and rows.dtype == torch.bfloat16 and rows.dim() == 2 and rows.shape[1] % 8 == 0
         self.packed = pack_weight(rows) if ok else None
+        # which kernel serves this weight at which number of rows: its own table, made from its shape
+        self.plan = plan_for(int(rows.shape[0]), int(rows.shape[1])) if rows.dim() == 2 else None
 
 
 def _weight(w):
@@ -351,27 +354,123 @@ def _weight(w):
     return w, None
 
 
-SKINNY_MAX_ROWS = 64
-SKINNY_PASSES_ROWS = 64             # up to here the weights are streamed rather than tiled (beyond 64 rows they would be
-                                    # streamed once per 64 rows: a decode step of 65 to 128 rows is 2-3 % longer so at
-                                    # TinyLlama's widths and 8-10 % at Llama-3-8B's, measured in the model), unless
-SKINNY_PASSES_MAX_N = 8192          # the output is at least this wide, and then only below SKINNY_WIDE_ROWS rows.
-SKINNY_WIDE_ROWS = 24               # (a decode step of 24 to 31 rows with the wide outputs tiled: 1-2 % shorter at TinyLlama's
-                                    # widths, 4-7 % at Llama-3-8B's, 1 % at Llama-2-7B's, where 17 to 20 rows are 1-3 % longer so)
-                                    # With one or two rows of tiles a product is as long as its chain of k-steps,
-                                    # which the streaming kernel's eight waves cut into eight -- but a wide output
-                                    # has tiles enough for every CU (64 x 64 ones, four stages), while every one of
-                                    # the streaming kernel's many workgroups reads all the rows of x (measured,
-                                    # streamed against tiled in a loop over one product, us:
-                                    # 64 rows 11264 x 2048 16.9 / 12.3, 28672 x 4096 59 / 37, 32000 x 2048 37 / 22,
-                                    # 6144 x 4096 19.4 / 19.6; 32 rows 11264 x 2048 12.7 / 12.4; 16 rows 9.3 / 12.2)
+SKINNY_MAX_ROWS = 64                # rows the weight-streaming kernel takes in one launch
+NORMED_STAGE_BYTES = 96 * 1024      # LDS the fused norm may fill with its rows of bf16(x * g)
+
+
+@dataclasses.dataclass(frozen=True)
+class LinearPlan:
+    """Which kernel serves x W^T at which number of rows, for ONE weight [n, k].  A weight gets its plan when it is
+    bound (StreamedWeight.plan; plan_for(n, k) for a bare tensor), from its own shape and the number of compute
+    units; the ops below and the parts ask the plan and carry no row thresholds of their own, so a model of other
+    widths gets thresholds of its own and a measured plan can take a computed one's place (set_plan).
+
+    The rules a plan is computed by (each measured as a whole decode step at three shapes of this architecture,
+    not as a loop over one product, whose weights would come from the 256 MB cache):
+    - stream_rows.  Up to 64 rows the weight is streamed once by gemm_skinny: with one or two rows of tiles a tiled
+      product is as long as its chain of k-steps, which the streaming kernel's eight waves cut into eight.  But every
+      one of the streaming kernel's workgroups reads all the rows of x, and an output with 64 x 64 tiles enough for
+      every other CU and more (n >= 32 tiles' worth of columns per CU pair: 8,192 on 256 CUs) fills the chip tiled:
+      such a weight goes to the tiled kernel from 24 rows on.
+    - fused_norm_rows.  Up to 8 rows the RMSNorm before the product is fused into the streaming kernel (it takes 16,
+      but every workgroup stages all the rows, and from 9 on a norm kernel of its own is faster), as long as the
+      staged rows fit LDS.
+    - parts_rows.  For 10 to 256 rows a product that adds into the residual stream cuts k over workgroups (64 x 64
+      tiles, the parts added up by a second kernel that norms the stream for the next product): a tile's workgroup
+      would walk all of k alone and the streaming kernel's workgroups all read all of x.  Up to 64 rows only for
+      weights of 2^24 elements and more (for smaller ones the streaming kernel wins there).
+    - qkv_stream_rows.  The product with rotation and cache write in its epilogue stays with the streaming kernel up
+      to 47 rows where the output is wide (every query head with keys of its own), to 64 otherwise.
+    """
+    n: int
+    k: int
+    stream_rows: int
+    fused_norm_rows: int
+    parts_rows: Tuple[int, int]
+    qkv_stream_rows: int
+
+    def streams(self, m: int) -> bool:
+        """Whether the weight-streaming kernel takes a product of m rows."""
+        return m <= self.stream_rows
+
+    def fuses_norm(self, m: int) -> bool:
+        return 0 < m <= self.fused_norm_rows
+
+    def parts(self, m: int) -> int:
+        """Into how many parts an adding product of m rows cuts k over workgroups (1: it does not)."""
+        lo, hi = self.parts_rows
+        if not (lo <= m <= hi):
+            return 1
+        tiles = -(-m // 64) * -(-self.n // 64)
+        best = 1
+        for parts in (2, 4, 8):
+            if self.k % (64 * parts) == 0 and self.k // (64 * parts) >= PARTS_MIN_STEPS and tiles * parts <= PARTS_WORKGROUPS:
+                best = parts
+        return best
+
+    def tiled_finishes_norm(self, m: int) -> bool:
+        """Whether a SwiGLU product of m rows goes to the tiled kernel and can finish a prepared norm there."""
+        return TILED_PRENORMED and not self.streams(m) and self.k % 64 == 0 and self.n % 16 == 0
+
+    def wants_prepared(self, m: int, swiglu: bool = False) -> bool:
+        """Whether a part whose first product is this weight's is better served, at m rows, by a norm that the
+        product before prepared than by fusing the norm or running it.  A q|k|v product reads prepared bfloat16 rows
+        faster than it stages float ones for a fused norm, and beyond the fused norm's rows a prepared norm saves
+        the norm's own kernel: always.  A SwiGLU product has many more workgroups, each of which adds up the
+        prepared parts: with few rows the fused norm costs little; from 5 rows to the fused norm's last, prepared
+        rows beat float rows staged in every workgroup; beyond, up to 63 rows, a norm kernel of its own is the
+        faster way for the streaming kernel -- while the tiled kernel, where the product goes there, adds the parts
+        up once a tile and takes them; at 64 rows and more the streaming kernel takes them too."""
+        if not swiglu:
+            return True
+        if m <= SKINNY_MAX_ROWS and self.tiled_finishes_norm(m):
+            return True
+        return 5 <= m <= self.fused_norm_rows or (m >= 64 and self.streams(m))
+
+
+PARTS_MIN_STEPS = 4                 # k-steps of 64 a part keeps at least
+PARTS_WORKGROUPS = 256              # as many parts (2, 4 or 8) as bring the 64 x 64 tiles to this many
+TILED_PRENORMED = True
+_PLANS: Dict[Tuple[int, int], LinearPlan] = {}
+
+
+def compute_plan(n: int, k: int, cus: int = 256) -> LinearPlan:
+    """The plan of a weight [n, k] by the rules LinearPlan states."""
+    wide = k % 64 == 0 and n >= 32 * cus             # (the tiled kernel's small tiles need k in steps of 64)
+    fused = 0
+    for rows in range(1, 9):
+        if (-(-rows // 4) * 4) * (k + 8) * 2 <= NORMED_STAGE_BYTES:     # rows rounded up to 4, each k + 8 bfloat16
+            fused = rows
+    if k % 64 or n % 8 or n > 8192:
+        parts_rows = (1, 0)
+    else:
+        parts_rows = (10 if n * k >= (1 << 24) else SKINNY_MAX_ROWS + 1, 256)
+    return LinearPlan(n=n, k=k, stream_rows=23 if wide else SKINNY_MAX_ROWS, fused_norm_rows=fused,
+                      parts_rows=parts_rows, qkv_stream_rows=47 if wide else SKINNY_MAX_ROWS)
+
+
+def plan_for(n: int, k: int) -> LinearPlan:
+    """The plan every weight of this shape shares: computed at first sight, or what set_plan put there."""
+    plan = _PLANS.get((n, k))
+    if plan is None:
+        plan = _PLANS[(n, k)] = compute_plan(n, k)
+    return plan
+
+
+def set_plan(plan: LinearPlan) -> None:
+    """Put a plan (a measured one, say) in the place of the computed one for weights of its shape.  Weights bound
+    before keep the plan they were bound with."""
+    _PLANS[(plan.n, plan.k)] = plan
+
+
+def _plan(w) -> LinearPlan:
+    plan = getattr(w, "plan", None)
+    return plan if plan is not None else plan_for(int(w.shape[0]), int(w.shape[1]))
 
 
 def streams_weights(m: int, n: int, k: int) -> bool:
     """Whether the weight-streaming kernel takes a product of m rows, n outputs and this k."""
-    if k % 64 or n < SKINNY_PASSES_MAX_N:       # (the tiled kernel's small tiles need k in steps of 64)
-        return m <= SKINNY_PASSES_ROWS
-    return m < SKINNY_WIDE_ROWS
+    return plan_for(n, k).streams(m)
 
 
 EPI_STORE_BF16, EPI_STORE_F32, EPI_ACCUM_F32, EPI_SWIGLU = 0, 1, 2, 3
@@ -417,22 +516,17 @@ def gemm_fast(a: torch.Tensor, w, out_dtype=None,
     return out
 
 
-NORMED_MAX_ROWS = 8                 # the kernel takes 16; beyond 8 every workgroup's staging of all the rows costs
-                                    # more than a norm kernel of its own (measured: 1.15 against 1.30 ms a step at 16 rows)
-NORMED_STAGE_BYTES = 96 * 1024      # LDS the fused norm may fill with its rows of bf16(x * g)
-
-
-def _normed_rows_fit(n_rows: int, k: int) -> bool:
-    """Whether the rows a fused RMSNorm stages in LDS (rounded up to 4, each k + 8 bfloat16) fit there:
-    8 rows do up to k = 6,136."""
-    return 0 < n_rows <= NORMED_MAX_ROWS and (-(-n_rows // 4) * 4) * (k + 8) * 2 <= NORMED_STAGE_BYTES
+def _normed_rows_fit(n_rows: int, k: int, n: int = 0) -> bool:
+    """Whether an RMSNorm before a product of these rows is fused into the streaming kernel: few rows (the plan's
+    fused_norm_rows: at most 8), which fit LDS rounded up to 4 with k + 8 bfloat16 each (8 rows do up to k = 6,136)."""
+    return plan_for(n or k, k).fuses_norm(n_rows)
 
 
 def gemm_normed_supported(x: torch.Tensor, n_rows: int, g: torch.Tensor, w) -> bool:
     """Whether RMSNorm can be fused into the product: few rows, bfloat16 weights, k a multiple of 8."""
     w, _ = _weight(w)
-    return (x.is_cuda and x.dtype == torch.float32 and w.dtype == torch.bfloat16 and _normed_rows_fit(n_rows, x.shape[1])
-            and x.shape[1] == w.shape[1] and x.shape[1] % 8 == 0 and g.dtype in _CODE)
+    return (x.is_cuda and x.dtype == torch.float32 and w.dtype == torch.bfloat16 and x.shape[1] == w.shape[1]
+            and _normed_rows_fit(n_rows, x.shape[1], w.shape[0]) and x.shape[1] % 8 == 0 and g.dtype in _CODE)
 
 
 def gemm_normed(x: torch.Tensor, rows: Optional[torch.Tensor], n_rows: int, g: torch.Tensor, eps: float,
@@ -508,33 +602,9 @@ class Finished:
         self.tensor = tensor
 
 
-PARTS_MIN_ROWS, PARTS_MAX_ROWS = 10, 256   # rows for which an adding product's k may be cut over workgroups (a prompt of
-                                            # 256 tokens at TinyLlama's widths 2.42 -> 2.21 ms, of 192 2.36 -> 2.20; a decode
-                                            # step at the Llama-3-8B shape 4.11 -> 3.89 ms at 12 rows, 4.60 -> 4.31 at 32,
-                                            # the same at 9 and 3.53 -> 3.71 at 8, where the norm is fused into the products)
-PARTS_MIN_STEPS = 4                         # k-steps of 64 a part keeps at least
-PARTS_WORKGROUPS = 256                      # as many parts (2, 4 or 8) as bring the 64 x 64 tiles to this many
-PARTS_MIN_WEIGHT = 1 << 24                  # up to 64 rows: only for weights of at least this many elements.
-                                            # Measured in the model, a decode step with the output and down products
-                                            # so against the weight-streaming kernel (and the norm after it prepared or
-                                            # run): TinyLlama's widths (2,048 x 2,048 and 2,048 x 5,632) 1.355 -> 1.40 ms
-                                            # at 64 rows, 1.27 -> 1.32 at 48, but 2.15 -> 1.90 at 96 and 2.33 -> 2.06 at
-                                            # 128 (where the weights are streamed twice); Llama-3-8B's (4,096 x 4,096
-                                            # and 4,096 x 14,336) 6.04 -> 5.44 ms at 64 rows, 9.70 -> 8.05 at 128.
-
-
 def parts_of_k(m: int, n: int, k: int) -> int:
     """Into how many parts gemm_parts_accumulate_norm cuts k (1: it does not take the product)."""
-    if not (PARTS_MIN_ROWS <= m <= PARTS_MAX_ROWS) or k % 64 or n % 8 or n > 8192:
-        return 1
-    if m <= SKINNY_MAX_ROWS and n * k < PARTS_MIN_WEIGHT:
-        return 1
-    tiles = -(-m // 64) * -(-n // 64)
-    best = 1
-    for parts in (2, 4, 8):
-        if k % (64 * parts) == 0 and k // (64 * parts) >= PARTS_MIN_STEPS and tiles * parts <= PARTS_WORKGROUPS:
-            best = parts
-    return best
+    return plan_for(n, k).parts(m)
 
 
 def gemm_parts_supported(a: torch.Tensor, w, residual: torch.Tensor, g: torch.Tensor) -> bool:
@@ -598,12 +668,9 @@ def gemm_accumulate_emit(a: torch.Tensor, w, residual: torch.Tensor, g: torch.Te
     return Prenormed(xb, parts, eps)
 
 
-TILED_PRENORMED = True
-
-
 def tiled_takes_prenormed(n_rows: int, n: int, k: int) -> bool:
     """Whether a SwiGLU product of these sizes that goes to the tiled kernel can finish a prepared norm there."""
-    return TILED_PRENORMED and not streams_weights(n_rows, n, k) and k % 64 == 0 and n % 16 == 0
+    return plan_for(n, k).tiled_finishes_norm(n_rows)
 
 
 def gemm_prenormed_supported(pre: Prenormed, w, epilogue: Optional[int] = None) -> bool:
@@ -645,17 +712,13 @@ def gemm_prenormed(pre: Prenormed, w, epilogue: int) -> torch.Tensor:
     return out
 
 
-QKV_WIDE_ROWS = 48      # rows from which a q|k|v output of 8,192 columns and more (every query head with keys of its own) goes
-                        # to the tiled kernel like other wide outputs (a decode step at the Llama-2-7B shape 7.91 -> 7.69 ms
-                        # at 64 rows, 6.77 -> 6.70 at 48, 5.12 -> 5.17 at 24)
-
-
 def gemm_qkv_rope_supported(x: torch.Tensor, n_rows: int, normed: bool, w, head_dim: int,
                             rotary_dim: int) -> bool:
     """Whether the q|k|v product of these rows can rotate and write the cache in its epilogue."""
     w, _ = _weight(w)
-    rows_ok = _normed_rows_fit(n_rows, x.shape[1]) if normed else n_rows <= SKINNY_MAX_ROWS
-    if not normed and n_rows >= QKV_WIDE_ROWS and not streams_weights(n_rows, w.shape[0], x.shape[1]):
+    plan = plan_for(int(w.shape[0]), int(x.shape[1]))
+    rows_ok = plan.fuses_norm(n_rows) if normed else n_rows <= SKINNY_MAX_ROWS
+    if not normed and n_rows > plan.qkv_stream_rows:
         return False                  # a wide q|k|v output: the tiled kernel's epilogue does the same
     return (x.is_cuda and w.dtype == torch.bfloat16 and x.shape[1] % 8 == 0 and 0 < n_rows and rows_ok
             and head_dim % 16 == 0 and rotary_dim in (0, head_dim)

@@ -6,6 +6,7 @@ from typing import Any, Dict, Hashable, List, Optional, Sequence, Tuple
 
 import torch
 
+from ..parts.lazy import NormHandoff
 from .runtime import Runtime
 
 
@@ -58,17 +59,8 @@ class StepContext:
     # the part noted for itself on the host).
     step_data: Dict[Hashable, Tuple[Dict[str, torch.Tensor], Any]] = dataclasses.field(default_factory=dict)
     captured: bool = False               # see HostBatch
-    # The norm that reads the residual stream next, while a part that adds into the stream runs (set by
-    # the block around the part; by the model: the norm the next schedule entry begins with).  A product
-    # that adds into the stream may then prepare that norm and leave the result in ``prepared`` under
-    # id(norm part); the block hands it to the norm's consumer.  Nothing prepared outlives the entry
-    # after the one that made it.  What is prepared is the finished norm, which serves every reader, or -- only
-    # if the reader takes that (``..._takes_parts``) -- the parts of one that a product can finish.
-    norm_after: Any = None
-    norm_after_takes_parts: bool = False
-    next_entry_norm: Any = None
-    next_entry_takes_parts: bool = False
-    prepared: Dict[int, Any] = dataclasses.field(default_factory=dict)
+    # Who reads the residual stream next and what the product before left for that reader: see NormHandoff.
+    handoff: NormHandoff = dataclasses.field(default_factory=NormHandoff)
 
     def cache(self, stream: Optional[Hashable]):
         return None if stream is None else self.cache_views.get(stream)

@@ -26,13 +26,15 @@ from .scheduler import (FINISH_CANCELLED, FINISH_ERROR, Request, Scheduler, Toke
 Event = Tuple[int, int, int, str]
 
 
-def working_memory_estimate(model, max_seqs: int, max_batch_tokens: int, graphs: int) -> int:
-    """Device bytes the engine will take beyond weights and cache while it serves: a step's activations
-    (a few rows of the widest activation per token) and, for every captured decode graph, its own
-    logits [requests, vocab] in float and activations."""
-    per_token = 64 * model.hidden_size                      # residual stream, products' outputs, attention parts
-    step = max(max_batch_tokens, max_seqs) * (per_token + 4 * model.vocab_size // 8)
-    graph = max_seqs * (4 * model.vocab_size + per_token)
+def working_memory_estimate(model, max_seqs: int, max_batch_tokens: int, graphs: int, max_tokens: int = 0,
+                            elem: int = 2) -> int:
+    """Device bytes the engine will take beyond weights and cache while it serves, from what the model's parts
+    state (Model.working_bytes): the largest step -- max_batch_tokens rows, or, where that is 0 and only memory
+    limits a step, as many as one request may bring (max_tokens) -- with logits for every request, and for every
+    captured decode graph its own activations and its logits [requests, vocab] in float."""
+    rows = max(max_batch_tokens or max_tokens, max_seqs)
+    step = model.working_bytes(rows, max_seqs, elem)
+    graph = model.working_bytes(max_seqs, max_seqs, elem)
     return step + graphs * graph
 
 
@@ -67,7 +69,8 @@ class Engine:
             raise EngineError(f"max_tokens {max_tokens} is beyond the model's {self.model.max_seq_len} positions")
         rt = self.model.rt
         if kv_pages <= 0:
-            working = working_memory_estimate(self.model, max_seqs, max_batch_tokens, Executor.MAX_GRAPHS)
+            working = working_memory_estimate(self.model, max_seqs, max_batch_tokens, Executor.MAX_GRAPHS, max_tokens,
+                                              torch.empty((), dtype=rt.act_dtype).element_size())
             kv_pages = fit_kv_pages(self.model, max_tokens, max_seqs, page_tokens, rt.act_dtype, rt.device,
                                     working_bytes=working)
         self.executor = Executor(self.model, num_pages=kv_pages, max_requests=max_seqs,

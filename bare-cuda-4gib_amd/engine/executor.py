@@ -52,14 +52,23 @@ class Executor:
           fixed here (what forward() derives from ctx.max_kv_len is fixed by itself: that is
           max_context while capturing).
     """
-    MAX_GRAPHS = 16       # captured decode graphs kept (each owns its logits and activations); the least
+    MAX_GRAPHS = 32       # captured decode graphs kept (each owns its logits and activations); the least
                           # recently used one goes when another is captured
+    # A captured decode step has one of these numbers of rows: a step of S requests runs in the smallest graph
+    # that holds them, and the rows beyond S stand for no request (they write the cache's scratch page and the
+    # scratch slot, and their logits are dropped).  So the graphs a workload needs are bounded by sizes x context
+    # buckets however its number of live requests wanders.  Up to 8 rows every count has its own graph: there a
+    # row more or less is a kernel form more or less (the norm fused into the products), and a request decoding
+    # alone should not pay for rows it does not have.
+    GRAPH_ROWS = (1, 2, 3, 4, 5, 6, 7, 8, 12, 16, 24, 32, 48, 64, 96, 128, 192, 256, 384, 512, 768, 1024)
 
     def __init__(self, model: Model, *, num_pages: int, max_requests: int, max_tokens: int,
                  page_tokens: int = 64, max_batch_tokens: int = 0, poison: bool = False,
                  use_graphs: bool = True, graph_max_batch: int = 256):
         if model.rt is None:
             raise EngineError("executor: the model has no weights bound")
+        if max_tokens > model.max_seq_len:       # (reference: Model::load, engine/src/model.cpp:429-433)
+            raise EngineError(f"executor: max_tokens {max_tokens} is beyond the model's {model.max_seq_len} positions")
         self.model = model
         self.rt = model.rt
         self.max_batch_tokens = max_batch_tokens
@@ -79,6 +88,7 @@ class Executor:
             and self.rt.device.type == "cuda"
         self.graph_max_batch = graph_max_batch
         self._graphs = collections.OrderedDict()
+        self.captures = 0                 # graphs captured so far (a key captured again after it was dropped counts again)
 
     # ---- requests -----------------------------------------------------------
     def admit(self, request: Hashable) -> int:
@@ -125,10 +135,12 @@ class Executor:
         return total
 
     def _host_arrays(self, entries: Sequence[StepEntry], table_width: int = 0, all_logits: bool = False,
-                     max_kv_bound: int = 0):
+                     max_kv_bound: int = 0, pad_to: int = 0):
         """The batch as one flat int32 array and the layout of its parts.  ``table_width`` 0
         makes block tables as wide as the batch needs; ``all_logits`` asks for every row;
-        ``max_kv_bound`` (a step about to be captured): the context bound the parts are to plan for."""
+        ``max_kv_bound`` (a step about to be captured): the context bound the parts are to plan for;
+        ``pad_to``: the number of requests the batch is filled up to with rows that stand for no request
+        (one token each, nothing cached, the cache's scratch slot and scratch page)."""
         cache, P = self.cache, self.cache.page_tokens
         i32 = np.int32
         token_ids, positions, row_seq, logit_rows = [], [], [], []
@@ -146,7 +158,17 @@ class Executor:
             logit_rows.append(np.arange(base, base + n, dtype=i32) if all_logits
                               else base + np.asarray(e.want, dtype=np.int64).astype(i32))
             max_q, max_kv = max(max_q, n), max(max_kv, ctx_len + n)
-        T, S = seq_start[-1], len(entries)
+        n_real = len(entries)
+        for s in range(n_real, pad_to):
+            base = seq_start[-1]
+            token_ids.append(np.zeros(1, dtype=i32))
+            positions.append(np.zeros(1, dtype=i32))
+            row_seq.append(np.full(1, s, dtype=i32))
+            seq_start.append(base + 1)
+            seq_ctx.append(0)
+            seq_slots.append(cache.scratch_slot)
+            logit_rows.append(np.arange(base, base + 1, dtype=i32) if all_logits else np.zeros(0, dtype=i32))
+        T, S = seq_start[-1], max(n_real, pad_to)
         empty = np.zeros(0, dtype=i32)
         logit_rows = np.concatenate(logit_rows) if logit_rows else empty
         chunks = [np.concatenate(token_ids) if token_ids else empty, np.concatenate(positions) if positions else empty,
@@ -165,12 +187,13 @@ class Executor:
         group_layout = []
         for g in cache.groups:
             tables = [np.asarray(cache.table(g, e.request), dtype=i32) for e in entries]
+            tables += [np.asarray([cache.scratch_page], dtype=i32)] * (S - n_real)
             width = table_width or max(1, max(len(t) for t in tables))
             padded = np.full((S, width), -1, dtype=i32)
             for row, t in zip(padded, tables):
                 row[:len(t)] = t
             chunks.append(padded.reshape(-1))
-            for e, t, where in zip(entries, tables, positions):       # where every new token's key and value go
+            for t, where in zip(tables, positions):                   # where every new token's key and value go
                 chunks.append(t[where // P] * P + where % P if len(where) else empty)
             group_layout.append((g, width))
         host = dict(seq_start=seq_start, seq_ctx=seq_ctx, seq_slots=seq_slots, n_logits=len(logit_rows),
@@ -213,15 +236,26 @@ class Executor:
         return (self.use_graphs and len(entries) <= self.graph_max_batch
                 and all(len(e.tokens) == 1 for e in entries))
 
+    def graph_rows(self, n_requests: int) -> int:
+        """Rows of the captured graph that serves a decode step of ``n_requests`` requests."""
+        for rows in self.GRAPH_ROWS:
+            if rows >= n_requests:
+                return min(rows, max(self.graph_max_batch, n_requests))
+        return n_requests
+
     def _graph_step(self, entries: Sequence[StepEntry], device_tokens: Optional[torch.Tensor] = None) -> torch.Tensor:
         """A step in which every request brings one token, replayed from a HIP graph captured
-        for this batch size and context bucket.  Only the int32 batch description changes
-        between replays; it is copied into the graph's own buffer first.  Logits of every row
-        come back ([S, vocab]); the buffer is the graph's and is overwritten by its next replay."""
+        for a number of rows (graph_rows: at least this step's) and a context bucket.  Only the int32
+        batch description changes between replays; it is copied into the graph's own buffer first.
+        Logits of the requests' rows come back ([requests, vocab]); the buffer is the graph's and is
+        overwritten by its next replay."""
         cache, P = self.cache, self.cache.page_tokens
-        S = len(entries)
+        n_real = len(entries)
+        S = self.graph_rows(n_real)
         width = cache.max_pages_per_request
         slots = cache.slots([e.request for e in entries])
+        if S > n_real:                      # the rows that stand for no request: the scratch slot, nothing cached
+            slots = np.concatenate([slots, np.full(S - n_real, cache.scratch_slot, dtype=np.int32)])
         ctx = cache.lengths_by_slot[slots]
         bucket = 256
         while bucket < int(ctx.max()) + 1:
@@ -230,7 +264,7 @@ class Executor:
         slot = self._graphs.get(key)
         if slot is None:
             flat, layout, group_layout, host = self._host_arrays(entries, table_width=width, all_logits=True,
-                                                                 max_kv_bound=bucket)
+                                                                 max_kv_bound=bucket, pad_to=S)
             slot = self._capture(key, flat, layout, group_layout, host, bucket)
         else:
             self._graphs.move_to_end(key)
@@ -243,7 +277,7 @@ class Executor:
         # loop over the requests; what does not (rows 0..S-1 one per request) is in the buffers since
         # the capture.  The layout is that of _host_arrays.
         at = slot["at"]
-        view[0:S] = [e.tokens[0] for e in entries]
+        view[0:n_real] = [e.tokens[0] for e in entries]
         view[at["positions"]:at["positions"] + S] = ctx
         view[at["seq_ctx"]:at["seq_ctx"] + S] = ctx
         view[at["seq_slots"]:at["seq_slots"] + S] = slots
@@ -265,9 +299,9 @@ class Executor:
         slot["dev"].copy_(buf, non_blocking=True)
         event.record()
         if device_tokens is not None:
-            slot["dev"][:S].copy_(device_tokens)
+            slot["dev"][:n_real].copy_(device_tokens)
         slot["graph"].replay()
-        return slot["logits"]
+        return slot["logits"][:n_real]
 
     def _capture(self, key, flat, layout, group_layout, host, bucket):
         S = key[0]
@@ -304,6 +338,7 @@ class Executor:
         slot = dict(graph=graph, dev=dev, logits=logits, ring=ring, next=0, at=at, rows=np.arange(S),
                     seq_start=list(range(S + 1)))
         self._graphs[key] = slot
+        self.captures += 1
         return slot
 
     def step(self, entries: Sequence[StepEntry], device_tokens: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:

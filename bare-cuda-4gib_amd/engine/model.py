@@ -153,27 +153,27 @@ class Model:
             flops, nbytes = flops + f, nbytes + b
         return flops, nbytes
 
+    def working_bytes(self, rows: int, n_logits: int, elem: int) -> int:
+        """Device bytes a step of ``rows`` rows with logits at ``n_logits`` of them needs beyond weights and cache, as
+        the parts state it: the float residual stream and a normed copy of it, the layer that needs most (one
+        layer's activations are given back before the next runs), and the float logits."""
+        layer = max((part.working_bytes_per_row(elem) for part in self.layers), default=0.0)
+        head = self.final_norm.part.working_bytes_per_row(elem) + self.hidden_size * elem
+        per_row = self.hidden_size * (4 + 4 + elem) + self.embedding.part.working_bytes_per_row(elem) + layer
+        return int(rows * per_row + n_logits * (head + 4 * self.vocab_size))
+
     # ---- forward ------------------------------------------------------------
     def forward(self, ctx: StepContext) -> Optional[torch.Tensor]:
         """Run the batch through every schedule entry; float32 logits at the
         wanted rows ([n_logits, vocab]), or None if none are wanted."""
         x = self.embedding.part.forward(ctx)
-        ctx.prepared.clear()
+        ctx.handoff.end_step()
         for i, e in enumerate(self.schedule):
             layer = self.layers[e.layer]
-            # what the entry before prepared for this entry's first norm stays; nothing else does
-            first = layer.first_norm(ctx.n_tokens) if hasattr(layer, "first_norm") else None
-            kept = ctx.prepared.pop(id(first), None) if first is not None else None
-            ctx.prepared.clear()
-            if kept is not None:
-                ctx.prepared[id(first)] = kept
             following = self.layers[self.schedule[i + 1].layer] if i + 1 < len(self.schedule) else None
-            ctx.next_entry_norm = following.first_norm(ctx.n_tokens) if hasattr(following, "first_norm") else None
-            takes = getattr(following, "first_norm_takes_parts", None)
-            ctx.next_entry_takes_parts = bool(takes(ctx.n_tokens)) if takes is not None else False
+            ctx.handoff.begin_entry(layer, following, ctx.n_tokens)
             layer.forward(x, ctx, ctx.cache(e.cache), e.writes)
-        ctx.prepared.clear()
-        ctx.next_entry_norm, ctx.next_entry_takes_parts = None, False
+        ctx.handoff.end_step()
         if ctx.n_logits == 0:
             return None
         norm, head = self.final_norm.part, self.head.part

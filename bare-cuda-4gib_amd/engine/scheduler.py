@@ -96,13 +96,21 @@ def target_tokens(limits: EngineLimits, prompt_len: int, max_new_tokens: int) ->
     return min(max_new_tokens, limits.max_tokens - prompt_len + 1)
 
 
+def cached_tokens(limits: EngineLimits, prompt_len: int, max_new_tokens: int) -> int:
+    """Tokens of the request that ever reach the cache: the last generated one is never run."""
+    return prompt_len + target_tokens(limits, prompt_len, max_new_tokens) - 1
+
+
 def pages_needed(limits: EngineLimits, prompt_len: int, max_new_tokens: int) -> int:
-    cached = prompt_len + target_tokens(limits, prompt_len, max_new_tokens) - 1
-    return -(-cached // limits.page_tokens)
+    """Pages of a stream that keeps every token (reference: pages_needed, engine/src/scheduler.cpp:36-43)."""
+    return -(-cached_tokens(limits, prompt_len, max_new_tokens) // limits.page_tokens)
 
 
-def check_request(limits: EngineLimits, request: Request) -> str:
-    """Empty if the request can ever run, else why not."""
+def check_request(limits: EngineLimits, request: Request, cache=None, portion: int = 0) -> str:
+    """Empty if the request can ever run, else why not.  What it needs of the page pools the cache
+    manager says (``cache.peak_pages``: per group of streams, by the group's own rule of what is
+    kept -- a windowed group needs its window and a portion, a model without per-token streams
+    nothing); without a cache manager, one stream that keeps every token is assumed."""
     n = len(request.prompt)
     if n == 0:
         return "empty prompt"
@@ -110,9 +118,15 @@ def check_request(limits: EngineLimits, request: Request) -> str:
         return "max_new_tokens must be positive"
     if n > limits.max_tokens:
         return f"prompt has {n} tokens, the engine holds {limits.max_tokens} per sequence"
-    pages = pages_needed(limits, n, request.max_new_tokens)
-    if pages > limits.kv_pages:
-        return f"request needs {pages} KV pages, the pool holds {limits.kv_pages}"
+    if cache is None:
+        pages = pages_needed(limits, n, request.max_new_tokens)
+        if pages > limits.kv_pages:
+            return f"request needs {pages} KV pages, the pool holds {limits.kv_pages}"
+    else:
+        need = cache.peak_pages(cached_tokens(limits, n, request.max_new_tokens), portion or limits.max_tokens)
+        for g, pages in need.items():
+            if pages > cache.groups[g].pool.num_pages:
+                return f"request needs {pages} KV pages, the pool holds {cache.groups[g].pool.num_pages}"
     return check_sampling(request.sampling)
 
 
@@ -143,9 +157,9 @@ class Scheduler:
         self.prefill_chunk = prefill_chunk
         self._clock = clock
         cache = executor.cache
-        pools = [g.pool.num_pages for g in cache.groups.values()]
+        pools = [g.pool.num_pages for g in cache.groups.values()]       # (none: the model keeps nothing per token)
         self.limits = EngineLimits(max_tokens=cache.max_tokens, max_seqs=cache.max_requests,
-                                   kv_pages=min(pools) if pools else 1 << 30, page_tokens=cache.page_tokens)
+                                   kv_pages=min(pools) if pools else 0, page_tokens=cache.page_tokens)
         self.waiting: Deque[_Live] = collections.deque()
         self.running: List[_Live] = []
         self._admissions = 0
@@ -154,7 +168,9 @@ class Scheduler:
 
     # ---- submitting and cancelling ---------------------------------------------
     def check(self, request: Request) -> str:
-        error = check_request(self.limits, request)
+        cache = self.executor.cache
+        error = check_request(self.limits, request, cache if hasattr(cache, "peak_pages") else None,
+                              min(self.prefill_chunk, self.max_batch_tokens))
         if error:
             return error
         if self.vocab_size is not None:

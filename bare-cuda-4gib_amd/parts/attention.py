@@ -109,12 +109,17 @@ class CausalAttention(Part):
         return (flops + 4.0 * pairs * self.num_heads * self.head_dim,
                 nbytes + 2.0 * keys * self.num_kv_heads * self.head_dim * elem)
 
+    def working_bytes_per_row(self, elem: int) -> float:
+        """The products' outputs, the attention output, and the float partial outputs and sums of a row whose
+        keys are cut into parts (as many as a prompt's work list may make)."""
+        q = self.num_heads * self.head_dim
+        return (super().working_bytes_per_row(elem) + q * elem
+                + ops.ATTENTION_MAX_PROMPT_SPLITS * (q + 2 * self.num_heads) * 4)
+
     def wants_prepared_norm(self, n_rows: int) -> bool:
-        """The q|k|v product reads bfloat16 rows faster than it stages float ones for a fused norm
-        (6.1 against 8.7 us at TinyLlama's sizes), and beyond 8 rows a prepared norm saves the
-        norm's own kernel (a decode step: 0.944 -> 0.916 ms at one row, 1.054 -> 1.020 at 8,
-        1.294 -> 1.252 at 32)."""
-        return self.act_dtype == torch.bfloat16
+        """Whether the q|k|v product is better served by a norm that the product before prepared than by fusing
+        the norm or running it: the weight's own plan says (ops.LinearPlan.wants_prepared)."""
+        return self.act_dtype == torch.bfloat16 and self.w_qkv.plan.wants_prepared(n_rows)
 
     def forward(self, h, ctx, cache, residual, writes: bool = True) -> None:
         fused = self.position.fused() if self.position is not None else (0, 1.0)

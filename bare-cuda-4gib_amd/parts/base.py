@@ -72,6 +72,18 @@ class Part:
             flops, nbytes = flops + f, nbytes + b
         return flops, nbytes
 
+    def working_bytes_per_row(self, elem: int) -> float:
+        """Device bytes this part needs for every row of a step while it runs, beyond its weights and the
+        cache (``elem``: bytes of a stored activation): by default the output of every linear map it holds,
+        nested parts included -- an upper bound, since what one product leaves is mostly gone before the
+        part's last product runs.  A part with working memory that its tensors do not show (float partial
+        results, staging) adds it."""
+        total = 0.0
+        for spec in self.weight_specs().values():
+            if spec.kind == "matrix" and len(spec.shape) == 2:
+                total += spec.shape[0] * elem
+        return total + sum(child.working_bytes_per_row(elem) for child in self.children())
+
 
 def register_part(category: str, kind: str, factory: Callable[..., Part], *, replace: bool = False) -> None:
     """Make ``kind`` buildable: ``factory(**params)`` returns the part."""

@@ -19,24 +19,18 @@ class PreNormBlock(Part):
         return [self.mixer_norm, self.mixer, self.ffn_norm, self.ffn]
 
     def forward(self, x, ctx, cache, writes: bool = True) -> None:
-        # Each part is told which norm reads the stream after it, so that its last product can
-        # prepare that norm: the feed-forward's after the mixer, the next entry's first after the
-        # feed-forward.
-        # (A finished norm serves every reader; the parts of one only a reader that says so.)
-        after, after_takes_parts = ctx.next_entry_norm, ctx.next_entry_takes_parts
-        ctx.norm_after, ctx.norm_after_takes_parts = self.ffn_norm, self._wants_prepared(self.ffn, x.shape[0])
-        self.mixer.forward(self._normed(self.mixer, self.mixer_norm, x, ctx), ctx, cache, x, writes)
-        ctx.norm_after, ctx.norm_after_takes_parts = after, after_takes_parts
-        self.ffn.forward(self._normed(self.ffn, self.ffn_norm, x, ctx), ctx, x)
-        ctx.norm_after, ctx.norm_after_takes_parts = None, False
+        # Each part is told which norm reads the stream after it, so that its last product can prepare that
+        # norm: the feed-forward's after the mixer, the next entry's first after the feed-forward.
+        handoff, n = ctx.handoff, x.shape[0]
+        with handoff.reader(self.ffn_norm, self._wants_prepared(self.ffn, n)):
+            self.mixer.forward(self._normed(self.mixer, self.mixer_norm, x, ctx), ctx, cache, x, writes)
+        with handoff.reader(*(handoff.next_entry or (None, False))):
+            self.ffn.forward(self._normed(self.ffn, self.ffn_norm, x, ctx), ctx, x)
 
-    def first_norm(self, n_rows: int):
-        """The norm this block begins with, which the entry before may prepare."""
-        return self.mixer_norm
-
-    def first_norm_takes_parts(self, n_rows: int) -> bool:
-        """Whether its reader takes the parts of a prepared norm (ops.Prenormed) for a step of ``n_rows`` rows."""
-        return self._wants_prepared(self.mixer, n_rows)
+    def first_reader(self, n_rows: int):
+        """(the norm this block begins with, whether its reader takes the parts of a prepared norm for a step of
+        ``n_rows`` rows): what the entry before may prepare."""
+        return self.mixer_norm, self._wants_prepared(self.mixer, n_rows)
 
     @staticmethod
     def _wants_prepared(part, n_rows: int) -> bool:
@@ -50,7 +44,7 @@ class PreNormBlock(Part):
         """The part's input: the norm's result, or -- for a part that says it takes one -- the
         norm not yet computed, so that the part's first product can absorb it (or take what the
         product before has prepared for it)."""
-        pre = ctx.prepared.pop(id(norm), None)
+        pre = ctx.handoff.take(norm)
         if isinstance(pre, ops.Finished):
             return Normed(x, norm, ctx, done=pre.tensor) if getattr(part, "accepts_lazy_norm", False) else pre.tensor
         if getattr(part, "accepts_lazy_norm", False):

@@ -45,22 +45,9 @@ class SwiGLU(Part):
         self.act_dtype = rt.act_dtype
 
     def wants_prepared_norm(self, n_rows: int) -> bool:
-        """From 5 to 8 rows and from 64 on.  With fewer rows the norm fused into the gate-up product
-        costs little (few float rows to stage); from 5 on reading prepared bfloat16 rows beats staging
-        float ones in every one of the product's many workgroups (a decode step at TinyLlama's sizes:
-        1.020 -> 0.990 ms at 8 rows, no difference at 4, 0.918 -> 0.948 at one).  From 9 rows on the
-        fused norm is out of reach and the choice is a norm kernel of its own: that is the faster way
-        up to 63 rows, because every workgroup of the product has to add up the prepared parts (1.085
-        against 1.072 ms at 16 rows, 1.269 against 1.252 at 32, 1.558 against 1.565 at 64).  Those are
-        the weight-streaming kernel's figures: a wide gate-up product of 24 to 64 rows goes to the tiled
-        kernel, which adds the parts up once a tile of 64 rows while its first operands are on their way
-        and puts the rows' factors into its epilogue -- the norm's kernel goes (1.217 -> 1.178 ms at
-        32 rows, 1.368 -> 1.322 at 64)."""
-        if not self.interleaved:
-            return False
-        if n_rows <= ops.SKINNY_MAX_ROWS and ops.tiled_takes_prenormed(n_rows, *self.w_gu.shape):
-            return True
-        return 5 <= n_rows <= ops.NORMED_MAX_ROWS or (n_rows >= 64 and ops.streams_weights(n_rows, *self.w_gu.shape))
+        """Whether the gate-up product, at this many rows, is better served by a norm that the product before
+        prepared than by fusing the norm or running it: the weight's own plan says (ops.LinearPlan.wants_prepared)."""
+        return self.interleaved and self.w_gu.plan.wants_prepared(n_rows, swiglu=True)
 
     def forward(self, h, ctx, residual) -> None:
         act = linear_swiglu(h, self.w_gu, self.interleaved)

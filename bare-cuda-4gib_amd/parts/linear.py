@@ -34,10 +34,11 @@ def linear(x: Union[torch.Tensor, Normed], w, out_dtype: Optional[torch.dtype] =
            accumulate_into: Optional[torch.Tensor] = None, ctx=None) -> torch.Tensor:
     """x [M, K] times w [N, K] transposed (w a tensor or an ops.StreamedWeight).  With
     ``accumulate_into`` (the float32 residual stream) the product is added to it in place; with
-    ``ctx`` too, and a norm named there as the next reader of the stream (``ctx.norm_after``), the
-    product prepares that norm where its kernel can and leaves the result in ``ctx.prepared``: the norm
-    itself (ops.Finished: 10 to 256 rows, k cut over workgroups) or, if the norm's reader takes that
-    (``ctx.norm_after_takes_parts``), the parts of it a product can finish (ops.Prenormed)."""
+    ``ctx`` too, and a norm named as the next reader of the stream (``ctx.handoff.reading_next``), the
+    product prepares that norm where its kernel can and leaves the result with the handoff: the norm
+    itself (ops.Finished) where the product cuts k over workgroups anyway -- the kernel that adds the parts
+    up norms the stream on its way, which serves every reader -- or else, if the reader takes that, the parts
+    of the norm that a product can finish (ops.Prenormed)."""
     if isinstance(x, Normed):
         if accumulate_into is None and out_dtype in (torch.bfloat16, torch.float32):
             epi = ops.EPI_STORE_BF16 if out_dtype == torch.bfloat16 else ops.EPI_STORE_F32
@@ -47,14 +48,15 @@ def linear(x: Union[torch.Tensor, Normed], w, out_dtype: Optional[torch.dtype] =
             if fused is not None:
                 return fused
         x = x.tensor()
-    if accumulate_into is not None and ctx is not None and ctx.norm_after is not None:
-        norm = ctx.norm_after
+    reading = ctx.handoff.reading_next if ctx is not None and accumulate_into is not None else None
+    if reading is not None:
+        norm, takes_parts = reading
         scale = norm.fusable() if hasattr(norm, "fusable") else None
         if scale is not None and ops.gemm_parts_supported(x, w, accumulate_into, scale[0]):
-            ctx.prepared[id(norm)] = ops.gemm_parts_accumulate_norm(x, w, accumulate_into, scale[0], scale[1])
+            ctx.handoff.leave(norm, ops.gemm_parts_accumulate_norm(x, w, accumulate_into, scale[0], scale[1]))
             return accumulate_into
-        if scale is not None and ctx.norm_after_takes_parts and ops.gemm_emit_supported(x, w, accumulate_into, scale[0]):
-            ctx.prepared[id(norm)] = ops.gemm_accumulate_emit(x, w, accumulate_into, scale[0], scale[1])
+        if scale is not None and takes_parts and ops.gemm_emit_supported(x, w, accumulate_into, scale[0]):
+            ctx.handoff.leave(norm, ops.gemm_accumulate_emit(x, w, accumulate_into, scale[0], scale[1]))
             return accumulate_into
     fast = ops.gemm_fast(x, w, out_dtype, accumulate_into)
     if fast is not None:

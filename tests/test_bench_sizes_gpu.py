@@ -247,3 +247,175 @@ def test_decode_batch_of_16_at_llama3_8b_widths_in_a_captured_graph(tmp_path_fac
             err = np.abs(got[i] - w)
             assert np.all(err <= tol["atol"] + tol["rtol"] * np.abs(w)), f"request {i}, token {t}: off by {float(err.max()):.3g}"
 
+
+
+# --- the regime the benchmark times: a 2,048-token prompt, and 64 requests decoded together at 1,000 to 2,000
+# tokens of context from captured graphs ------------------------------------------------------------------------
+# One folder in bfloat16 serves both precisions (the 32-bit path widens its values), so the plain implementation
+# walks each of the two 2,048-token sequences once: at these sizes that is most of the tests' time.
+
+@pytest.fixture(scope="module")
+def long_context(tmp_path_factory):
+    from bare_cuda_4gib_amd.weights import write_random_model
+    folder = write_random_model(TINYLLAMA_WIDTHS, 37, str(tmp_path_factory.mktemp("tinyllama_long") / "model"), "bfloat16",
+                                norm_std=0.1, scales={"lm_head.weight": 0.25})
+    plain = PlainLlama(folder)
+    bases = {name: helpers.random_ids(2048, 32000, seed) for name, seed in (("a", 2048), ("b", 2049))}
+    hidden = {name: plain.hidden_states(ids) for name, ids in bases.items()}
+    norm, head = plain.w["model.norm.weight"], plain.w["lm_head.weight"]
+    eps = plain.eps
+    del plain
+
+    def rows(name, positions):
+        positions = sorted(set(positions))
+        out = (P.rmsnorm(hidden[name][torch.tensor(positions)], norm, eps) @ head.T).numpy()
+        return {p: out[i] for i, p in enumerate(positions)}
+    return folder, bases, rows
+
+
+def _check_rows(got, want, tol, label):
+    for row, w in zip(got, want):
+        err = np.abs(row - w)
+        assert np.all(np.isfinite(row)), f"{label}: non-finite logits"
+        assert np.sqrt(np.mean(err * err)) <= tol["row_rms"] * np.sqrt(np.mean(w * w)), f"{label}: the row's errors are too large as a whole"
+        bound = tol["atol"] + tol["rtol"] * np.abs(w)
+        assert np.all(err <= bound), f"{label}: logit {int(np.argmax(err - bound))} off by {float(err.max()):.3g}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_tinyllama_widths_prompt_of_2048_tokens_whole_and_in_portions(long_context, dtype):
+    """What the benchmark's prefill times: one prompt of 2,048 tokens in one step (in bfloat16: the attention work
+    list with the long walks cut into parts, the largest tiles of the tiled product, its q|k|v epilogue over 2,048
+    rows) and in four portions of 512, logits at sixteen places -- the first tokens, both sides of a page's edge,
+    of a portion's edge, of the middle, and the last -- against the plain implementation (the reference holds
+    its model to its oracle over whole prompts, engine/tests/test_forward.cu:42-46)."""
+    from bare_cuda_4gib_amd.engine import Executor, StepEntry, load_model
+    folder, bases, plain_rows_of = long_context
+    ids = bases["a"]
+    places = [0, 1, 31, 32, 63, 64, 255, 256, 511, 512, 1023, 1024, 1535, 1536, 2046, 2047]
+    want = plain_rows_of("a", places)
+    model, _ = load_model(folder, dtype, "cuda:0")
+    for label, portions in (("whole", [2048]), ("portions", [512, 512, 512, 512])):
+        ex = Executor(model, num_pages=32, max_requests=1, max_tokens=2048, page_tokens=64, poison=True)
+        ex.cache.shuffle_free_pages(7)
+        ex.admit("p")
+        done = 0
+        for n in portions:
+            here = [p for p in places if done <= p < done + n]
+            got = ex.step([StepEntry("p", ids[done:done + n], [p - done for p in here])]).float().cpu().numpy()
+            _check_rows(got, [want[p] for p in here], TOL[dtype], f"2,048-token prompt, {label}, tokens {done}..{done + n - 1}, {dtype}")
+            done += n
+        ex.release("p")
+        assert ex.cache.pages_in_use() == 0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_tinyllama_widths_64_requests_decoded_at_1000_and_2000_tokens_of_context(long_context, dtype):
+    """What the benchmark's decode at batch 64 times, at its longest contexts: 64 requests (prefixes of two
+    sequences, neighbours in the batch from different ones) prefilled to about 1,000 tokens and decoded together
+    for four steps (the graph for 64 rows and contexts up to 1,024), then every second one taken on to about 2,030
+    tokens and all 64 decoded for four more steps (contexts of 1,000 and 2,030 side by side in the graph for up to
+    2,048, whose cut of the keys comes from that bound).  Every row against the plain implementation, and the
+    captured graphs' replays bit for bit against the same steps launched kernel by kernel (the reference holds
+    decoding with its cache to the run without, engine/tests/test_kv_cache.cu:216-217)."""
+    from bare_cuda_4gib_amd.engine import Executor, StepEntry, load_model
+    folder, bases, plain_rows_of = long_context
+    model, _ = load_model(folder, dtype, "cuda:0")
+    n = 64
+    base_of = ["a" if i % 2 == 0 else "b" for i in range(n)]
+    first = [960 + (7 * i) % 60 for i in range(n)]                      # 960 .. 1,019 tokens, then four decoded
+    second = {i: 2008 + (5 * i) % 32 for i in range(0, n, 2)}           # 2,008 .. 2,039 tokens, then four decoded
+    need = {"a": set(), "b": set()}
+    for i in range(n):
+        need[base_of[i]].update(range(first[i], first[i] + 4))
+        if i in second:
+            need[base_of[i]].update(range(second[i], second[i] + 4))
+        else:
+            need[base_of[i]].update(range(first[i] + 4, first[i] + 8))
+    want = {name: plain_rows_of(name, need[name]) for name in need}
+    runs = {}
+    for graphs in (True, False):
+        ex = Executor(model, num_pages=n * 32, max_requests=n, max_tokens=2048, page_tokens=64, max_batch_tokens=16384)
+        ex.use_graphs = ex.use_graphs and graphs
+        assert ex.use_graphs == graphs
+        ex.cache.shuffle_free_pages(11)
+        length = {}
+        for lo in range(0, n, 8):
+            for i in range(lo, lo + 8):
+                ex.admit(i)
+            ex.step([StepEntry(i, bases[base_of[i]][:first[i]], []) for i in range(lo, lo + 8)])
+            length.update({i: first[i] for i in range(lo, lo + 8)})
+        out = []
+
+        def decode(steps):
+            for _ in range(steps):
+                logits = ex.step([StepEntry(i, [bases[base_of[i]][length[i]]], [0]) for i in range(n)])
+                out.append(([(base_of[i], length[i]) for i in range(n)], logits.float().cpu().numpy().copy()))
+                for i in range(n):
+                    length[i] += 1
+        decode(4)
+        for lo in range(0, n, 16):                                      # every second request on to about 2,030 tokens
+            group = [i for i in range(lo, lo + 16) if i in second]
+            ex.step([StepEntry(i, bases[base_of[i]][length[i]:second[i]], []) for i in group])
+            length.update({i: second[i] for i in group})
+        decode(4)
+        if graphs:
+            assert sorted(ex._graphs) == [(64, 1024), (64, 2048)], f"graphs captured: {sorted(ex._graphs)}"
+        runs[graphs] = out
+        del ex
+    for step, ((where, got), (_, eager)) in enumerate(zip(runs[True], runs[False])):
+        assert np.array_equal(got, eager), f"decode step {step}: the graph's replay and the same step launched kernel by kernel differ"
+        _check_rows(got, [want[name][pos] for name, pos in where], TOL[dtype],
+                    f"64 requests, decode step {step} (contexts {min(p for _, p in where)}..{max(p for _, p in where)}), {dtype}")
+
+
+def _kernels_of_a_decode_step(model, n_rows):
+    """Names of the library's entry points that one decode step of ``n_rows`` requests calls (steps launched kernel
+    by kernel, the profiler noting every call)."""
+    from bare_cuda_4gib_amd.csrc.profile import profiler
+    from bare_cuda_4gib_amd.engine import Executor, StepEntry
+    ex = Executor(model, num_pages=n_rows, max_requests=n_rows, max_tokens=64, page_tokens=64, use_graphs=False)
+    for i in range(n_rows):
+        ex.admit(i)
+    ex.step([StepEntry(i, [3 + i, 5, 7 + i], []) for i in range(n_rows)])
+    prof = profiler()
+    prof.reset()
+    prof.enable(True)
+    try:
+        ex.step([StepEntry(i, [11 + i], [0]) for i in range(n_rows)])
+    finally:
+        prof.enable(False)
+    names = {s.name: s.calls for s in prof.stats()}
+    prof.reset()
+    return names
+
+
+def test_which_kernels_serve_32_and_64_rows(long_context, tmp_path_factory):
+    """What the weights' plans say is what runs.  At TinyLlama's widths (two layers) the products that add into the
+    stream are streamed and leave the parts of the next norm, which the q|k|v product and -- in the tiled kernel --
+    the wide gate-up product finish: no norm kernel between the layers' products.  At Llama-3-8B's widths the output
+    projection (2^24 elements) cuts k over workgroups and the kernel that adds its parts up leaves the finished norm,
+    so the gate-up product is the plain tiled one: the parts of a norm are never made there, although its reader
+    would take them."""
+    from bare_cuda_4gib_amd.csrc import ops
+    from bare_cuda_4gib_amd.engine import load_model
+    from bare_cuda_4gib_amd.weights import write_random_model
+    folder, _, _ = long_context
+    model, _ = load_model(folder, "bfloat16", "cuda:0")
+    for rows in (32, 64):
+        names = _kernels_of_a_decode_step(model, rows)
+        assert ops.plan_for(2048, 2048).parts(rows) == 1 and ops.plan_for(11264, 2048).tiled_finishes_norm(rows)
+        assert names.get("gemm_skinny_emit") == 3, names          # both output projections and the first layer's down projection
+        assert names.get("gemm_mfma_swiglu_scaled") == 2 and names.get("gemm_skinny_qkv") == 2, names
+        assert names.get("rmsnorm") == 2 and "gemm_mfma_parts" not in names, names   # (the first norm of all, and the last)
+    del model
+    folder = os.path.join(str(tmp_path_factory.getbasetemp()), "llama3_8b_widths")
+    if not os.path.exists(os.path.join(folder, "model.safetensors")):
+        write_random_model(LLAMA3_8B_WIDTHS, 41, folder, "bfloat16", norm_std=0.1, scales={"lm_head.weight": 0.125})
+    model, _ = load_model(folder, "bfloat16", "cuda:0")
+    for rows in (32, 64):
+        names = _kernels_of_a_decode_step(model, rows)
+        assert ops.plan_for(4096, 4096).parts(rows) > 1
+        assert names.get("gemm_mfma_parts") == 1 and names.get("rmsnorm_sum") == 1, names     # the output projection
+        assert "gemm_skinny_emit" not in names and "gemm_mfma_swiglu_scaled" not in names, names
+        assert names.get("gemm_mfma") == 1 + (rows >= 24), names                               # gate-up (and the wide head)

@@ -136,12 +136,19 @@ def test_groups_have_pages_of_their_own_and_windows_give_pages_back():
 def test_state_slots_are_zeroed_at_admission():
     cm = _manager(extra={"s": FixedState((3,), "float32")})
     view = cm.view("s")
-    assert tuple(view.state.shape) == (4, 3)
+    assert tuple(view.state.shape) == (4 + 1, 3)                     # the requests' slots and the scratch slot
     slot = cm.admit("a")
     view.state[slot] += 5.0
     cm.release("a")
     assert cm.admit("b") == slot and torch.equal(view.state[slot], torch.zeros(3))
-    assert cm.view(0).k.shape == (12, 2, 4, 8) and cm.view(0).group == ("window", 0)
+    assert cm.view(0).k.shape == (12 + 1, 2, 4, 8) and cm.view(0).group == ("window", 0)   # the pool's pages and the scratch page
+    # the scratch page is in no pool and the scratch slot is never given to a request
+    assert cm.scratch_page == 12 and cm.scratch_slot == 4
+    assert all(g.pool.num_pages == 12 for g in cm.groups.values())
+    slots = {cm.admit(r) for r in "cde"}
+    assert cm.free_slots == 0 and cm.scratch_slot not in slots | {slot}
+    for g in cm.groups:
+        assert cm.tables_by_slot[g][cm.scratch_slot].tolist()[:2] == [cm.scratch_page, -1] and cm.lengths_by_slot[cm.scratch_slot] == 0
 
 
 @pytest.mark.parametrize("seed", range(5))
@@ -209,10 +216,10 @@ def test_a_spec_says_its_own_storage():
                       page_tokens=4, num_pages=10, max_requests=3, max_tokens=40, dtype=torch.bfloat16, device="cpu",
                       poison=True)
     lat, lat_w, n = cm.view("lat"), cm.view("lat_w"), cm.view("n")
-    assert lat.c.shape == (10, 4, 6) and lat.c.dtype == torch.bfloat16 and lat.scale.dtype == torch.float32
+    assert lat.c.shape == (10 + 1, 4, 6) and lat.c.dtype == torch.bfloat16 and lat.scale.dtype == torch.float32
     assert lat.group == cm.view("kv").group == ("window", 0) and lat_w.group == ("window", 9) and lat_w.window == 9
     assert torch.isnan(lat.c.float()).all() and torch.isnan(lat.scale).all()
-    assert n.hits.shape == (3, 2) and n.hits.dtype == torch.int32 and not n.paged and lat.paged
+    assert n.hits.shape == (3 + 1, 2) and n.hits.dtype == torch.int32 and not n.paged and lat.paged
     with pytest.raises(AttributeError, match="no tensor 'k'"):
         lat.k
     assert bytes_per_page(cm.specs.values(), 4, torch.bfloat16) == 2 * (2 * 4 * 8 * 2) + (4 * 6 * 2 + 4 * 4) + (4 * 3 * 2 + 4 * 4)
@@ -227,3 +234,67 @@ def test_a_spec_says_its_own_storage():
     assert cm.admit("b") == slot and float(n.sum[slot].sum()) == 0.0     # zeroed at admission
     with pytest.raises(EngineError, match="neither"):
         CacheManager({"x": object()}, page_tokens=4, num_pages=2, max_requests=1, max_tokens=8, dtype=torch.float32, device="cpu")
+
+
+def test_a_spec_states_its_own_rule_of_what_is_kept():
+    """A stream whose queries read only the tokens of their own block of eight (a rule that no window
+    expresses) says so itself: the manager gives a page back once first_kept() has passed it, groups
+    the stream by the rule's key, and answers how many pages a request ever holds under it."""
+    import dataclasses
+
+    @dataclasses.dataclass(frozen=True)
+    class BlockLocal:
+        block: int
+        per_token = True
+
+        def page_tensors(self, page_tokens):
+            return {"k": (page_tokens, 2)}
+
+        def group_key(self):
+            return ("block", self.block)
+
+        def first_kept(self, length):
+            return length // self.block * self.block
+
+    cm = CacheManager({"kv": PagedKV(1, 2), "w": PagedKV(1, 2, window=6), "b": BlockLocal(8), "b2": BlockLocal(8)},
+                      page_tokens=4, num_pages=12, max_requests=2, max_tokens=40, dtype=torch.float32, device="cpu")
+    assert set(cm.groups) == {("window", 0), ("window", 6), ("block", 8)}
+    assert cm.groups[("block", 8)].streams == ["b", "b2"] and cm.view("b").group == ("block", 8)
+    cm.admit("a")
+    length = 0
+    for n in (3, 4, 2, 8, 1, 5, 9):
+        cm.reserve([("a", n)])
+        cm.advance("a", n)
+        length += n
+        table = cm.table(("block", 8), "a")
+        first = length // 8 * 8 // 4
+        assert [p >= 0 for p in table] == [i >= first for i in range(len(table))], f"after {length} tokens"
+        _check_invariants(cm, {})
+    cm.release("a")
+    assert cm.pages_in_use() == 0
+    # the most pages a request ever holds, fed in portions of at most 5 tokens up to 32: everything in the group
+    # that keeps all; the window's 6 tokens and a portion, across page edges, in the windowed one; two blocks'
+    # worth at most where a portion straddles a block's end
+    peak = cm.peak_pages(32, 5)
+    assert peak[("window", 0)] == 8
+    assert peak[("window", 6)] == max(-(-min(p + 5, 32) // 4) - max(0, p - 5) // 4 for p in range(32)) == 4
+    assert peak[("block", 8)] == max(-(-min(p + 5, 32) // 4) - p // 8 * 8 // 4 for p in range(32)) == 3
+    assert cm.peak_pages(32, 40)[("window", 6)] == 8 and cm.peak_pages(3, 5) == {("window", 0): 1, ("window", 6): 1, ("block", 8): 1}
+    # and the peak is reached, never passed, by a request so fed
+    for portion in (1, 5, 7):
+        cm.admit("p")
+        most = {g: 0 for g in cm.groups}
+        done = 0
+        while done < 32:
+            n = min(portion, 32 - done)
+            cm.reserve([("p", n)])
+            for g in cm.groups:
+                most[g] = max(most[g], sum(1 for q in cm.table(g, "p") if q >= 0))
+            cm.advance("p", n)
+            done += n
+        cm.release("p")
+        want = cm.peak_pages(32, portion)
+        assert all(most[g] <= want[g] for g in most) and most[("window", 0)] == want[("window", 0)], (portion, most, want)
+    only_state = CacheManager({"s": FixedState((2,))}, page_tokens=4, num_pages=0, max_requests=2, max_tokens=40,
+                              dtype=torch.float32, device="cpu")
+    assert only_state.peak_pages(32, 5) == {}

@@ -76,3 +76,23 @@ def test_description_is_data():
     assert len(spec.layers) == 2 and [e.layer for e in spec.schedule] == [0, 1]
     assert spec.layers[0].mixer.params["num_kv_heads"] == 2 and spec.layers[0].mixer.params["position"].params["theta"] == 10000.0
     assert spec.layers[1].ffn.params["intermediate_size"] == 176 and spec.final_norm.params["eps"] == 1e-5
+
+
+def test_working_memory_is_what_the_parts_state():
+    """What a step needs beyond weights and cache is added up from the parts (each product's output, attention's
+    float partial results), not a constant times the width: it follows the feed-forward's width and the head
+    count, and a step limited by memory alone is sized for the longest portion a request may bring."""
+    from bare_cuda_4gib_amd.engine.engine import working_memory_estimate
+    from bare_cuda_4gib_amd.engine.model import Model
+    cfg = LlamaConfig.from_dict(helpers.TINY_A)
+    model = Model(architecture_for(helpers.TINY_A).describe(cfg))
+    h, q, kv, inter, vocab = 64, 4 * 16, 2 * 16, 176, 256
+    attention = (q + 2 * kv + h) * 2 + q * 2 + 8 * (q + 2 * 4) * 4       # products' outputs, attention's output, parts of cut keys
+    ffn = (2 * inter + h) * 2
+    per_row = h * (4 + 4 + 2) + attention + ffn
+    assert model.working_bytes(10, 3, 2) == 10 * per_row + 3 * (h * 2 + 4 * vocab)
+    wide = Model(architecture_for(helpers.TINY_A).describe(LlamaConfig.from_dict(dict(helpers.TINY_A, intermediate_size=1760))))
+    assert wide.working_bytes(10, 0, 2) - model.working_bytes(10, 0, 2) == 10 * 2 * (1760 - 176) * 2
+    limited = working_memory_estimate(model, max_seqs=4, max_batch_tokens=32, graphs=0)
+    unlimited = working_memory_estimate(model, max_seqs=4, max_batch_tokens=0, graphs=0, max_tokens=128)
+    assert limited == model.working_bytes(32, 4, 2) and unlimited == model.working_bytes(128, 4, 2) > limited

@@ -228,7 +228,7 @@ def test_greedy_generation_through_the_entry_point(folders, name, dtype):
     cfg, _ = helpers.TINY[name]
     folder = folders(name, dtype)
     plain = PlainLlama(folder)
-    prompts = [helpers.random_ids(n, cfg["vocab_size"], 10 + n) for n in (1, 7, 33)]   # BASELINE's workload for A
+    prompts = [helpers.random_ids(n, cfg["vocab_size"], 10 + n) for n in (1, 7, 33)]   # the first tiny configuration's workload
     engine = Engine(folder, max_tokens=64, max_seqs=3, kv_pages=0, dtype=dtype, page_tokens=16, prefill_chunk=16)
     assert engine.vocab_size == cfg["vocab_size"] and engine.max_seqs == 3 and engine.healthy
     together = generate_batch(engine, prompts, 16)
@@ -351,7 +351,7 @@ def test_sampling_and_preemption_on_the_device(folders):
     pool is so small that requests are preempted and recomputed."""
     from bare_cuda_4gib_amd.engine import Engine, generate_batch
     folder = folders("B", "float32", "spread")
-    prompts = [helpers.random_ids(n, 384, 40 + n) for n in (5, 64, 130)]            # BASELINE's workload for B
+    prompts = [helpers.random_ids(n, 384, 40 + n) for n in (5, 64, 130)]            # the second tiny configuration's workload
     def run(kv_pages, which):
         engine = Engine(folder, max_tokens=256, max_seqs=3, kv_pages=kv_pages, dtype="float32", page_tokens=16,
                         prefill_chunk=32, max_batch_tokens=96)

@@ -607,3 +607,109 @@ def test_a_mixer_with_its_own_cache_layout_and_step_geometry_runs_in_captured_gr
     assert CausalMean.calls["prepare_capture"][len(before["prepare_capture"]):] == [(3, 256), (3, 512)]
     assert CausalMean.calls["forward"] - before["forward"] == 4
     assert CausalMean.calls["prepare_step"] - before["prepare_step"] >= tail
+
+
+# --- through the scheduler: a model whose every stream has a window, and one that keeps nothing per token ---
+# The scheduler asks the cache manager what a request may need at most (by each stream's own rule), not how
+# long the request is: the first toy runs requests much longer than its pool, the second with no pages at all.
+
+def register_stack_toy():
+    register_toy()                       # (the running-mean mixer)
+    from bare_cuda_4gib_amd.config import Architecture, ModelConfig, field_from_json, register_architecture
+    from bare_cuda_4gib_amd.config.registry import unregister_architecture
+    from bare_cuda_4gib_amd.engine.spec import LayerSpec, ModelSpec, PartSpec, ScheduleEntry
+
+    @dataclasses.dataclass
+    class StackConfig(ModelConfig):
+        vocab_size: int = field_from_json("vocab_size")
+        hidden_size: int = field_from_json("hidden_size")
+        kinds: str = field_from_json("kinds")          # one letter a layer: w = windowed attention, m = running mean
+        window: int = field_from_json("window")
+
+    def describe(cfg):
+        norm = dict(size=cfg.hidden_size, eps=1e-5)
+        layers = []
+        for i, kind in enumerate(cfg.kinds):
+            p = f"blocks.{i}."
+            if kind == "w":
+                mixer = PartSpec("attention", dict(hidden_size=cfg.hidden_size, num_heads=NH, num_kv_heads=NKV, head_dim=D,
+                                                   window=cfg.window, position=PartSpec("rotary", dict(theta=100.0, dim=D))),
+                                 prefix=p + "attn.")
+            else:
+                mixer = PartSpec("toy_running_mean", dict(hidden_size=cfg.hidden_size), prefix=p)
+            layers.append(LayerSpec("prenorm", mixer, PartSpec("swiglu", dict(hidden_size=cfg.hidden_size, intermediate_size=INTER),
+                                                               prefix=p + "ffn."),
+                                    PartSpec("rmsnorm", dict(norm), prefix=p + "norm1."), PartSpec("rmsnorm", dict(norm), prefix=p + "norm2.")))
+        return ModelSpec(vocab_size=cfg.vocab_size, hidden_size=cfg.hidden_size, max_seq_len=4096,
+                         embedding=PartSpec("embedding", dict(vocab_size=cfg.vocab_size, hidden_size=cfg.hidden_size), prefix="embed."),
+                         layers=layers, schedule=[ScheduleEntry(i, f"c{i}") for i in range(len(layers))],
+                         final_norm=PartSpec("rmsnorm", dict(norm), prefix="final_norm."),
+                         head=PartSpec("lm_head", dict(vocab_size=cfg.vocab_size, hidden_size=cfg.hidden_size), prefix="head."))
+
+    unregister_architecture("ToyStackForTests")
+    register_architecture(Architecture("ToyStackForTests", "toy_stack_for_tests", StackConfig, describe))
+
+
+def plain_stack_logits(folder, ids, kinds, window):
+    from safetensors import safe_open
+    with safe_open(os.path.join(folder, "model.safetensors"), "pt") as f:
+        w = {n: f.get_tensor(n).double() for n in f.keys()}
+    t = len(ids)
+    pos = torch.arange(t)
+    x = w["embed.weight"][torch.tensor(ids)]
+    for i, kind in enumerate(kinds):
+        p = f"blocks.{i}."
+        h = P.rmsnorm(x, w[p + "norm1.weight"], 1e-5)
+        if kind == "w":
+            q = (h @ w[p + "attn.q_proj.weight"].T).view(t, NH, D)
+            k = (h @ w[p + "attn.k_proj.weight"].T).view(t, NKV, D)
+            v = (h @ w[p + "attn.v_proj.weight"].T).view(t, NKV, D)
+            o = P.attention(P.rope(q, pos, 100.0), P.rope(k, pos, 100.0), v, window=window)
+            x = x + o.reshape(t, -1) @ w[p + "attn.o_proj.weight"].T
+        else:
+            mean = torch.cumsum(h, 0) / torch.arange(1, t + 1, dtype=torch.float64)[:, None]
+            x = x + mean @ w[p + "mix.weight"].T
+        h = P.rmsnorm(x, w[p + "norm2.weight"], 1e-5)
+        x = x + P.swiglu(h @ w[p + "ffn.gate_proj.weight"].T, h @ w[p + "ffn.up_proj.weight"].T) @ w[p + "ffn.down_proj.weight"].T
+    return P.rmsnorm(x, w["final_norm.weight"], 1e-5) @ w["head.weight"].T
+
+
+@pytest.mark.parametrize("kinds,pages", [("ww", 8), ("mm", 0)])
+def test_the_scheduler_asks_the_cache_what_a_request_needs(tmp_path, kinds, pages):
+    """Requests of 40 to 150 tokens plus 12 generated, in portions of 32, with three live at a time.  The windowed
+    model (window 24, pages of 16) holds at most five pages a request and runs in a pool of eight, fewer than the
+    eleven that the longest request's tokens alone would take; the model of running means has no pages.  Greedy tokens against the plain
+    implementation of the same toy, followed along the engine's own tokens."""
+    register_stack_toy()
+    from bare_cuda_4gib_amd.engine import Executor, load_model
+    from bare_cuda_4gib_amd.engine.scheduler import Request, Scheduler
+    from bare_cuda_4gib_amd.sampling.device import DevicePicker
+    from bare_cuda_4gib_amd.weights import write_random_model
+    config = dict(architectures=["ToyStackForTests"], vocab_size=VOCAB, hidden_size=H, kinds=kinds, window=WINDOW)
+    folder = write_random_model(config, 33, str(tmp_path / kinds), "float32", std=0.08)
+    model, _ = load_model(folder, "float32")
+    ex = Executor(model, num_pages=pages, max_requests=3, max_tokens=176, page_tokens=16, poison=True)
+    sched = Scheduler(ex, DevicePicker(), max_batch_tokens=64, prefill_chunk=32)
+    if kinds == "ww":
+        assert ex.cache.peak_pages(161, 32) == {("window", WINDOW): 5} and sched.limits.kv_pages == 8
+    else:
+        assert ex.cache.groups == {} and sched.limits.kv_pages == 0
+    prompts = {i: helpers.random_ids(n, VOCAB, 700 + i) for i, n in enumerate([150, 40, 97, 64, 121])}
+    for i, ids in prompts.items():
+        assert sched.check(Request(id=i, prompt=ids, max_new_tokens=12)) == ""
+        sched.submit(Request(id=i, prompt=ids, max_new_tokens=12))
+    out = {i: [] for i in prompts}
+    for _ in range(400):
+        if sched.idle():
+            break
+        for e in sched.step():
+            if e.token >= 0:
+                out[e.id].append(e.token)
+    assert sched.idle() and ex.cache.pages_in_use() == 0 and ex.cache.free_slots == 3
+    assert sched.stats().prefill_tokens >= sum(len(ids) for ids in prompts.values())
+    for i, ids in prompts.items():
+        assert len(out[i]) == 12
+        full = plain_stack_logits(folder, ids + out[i], kinds, WINDOW)
+        for j, tok in enumerate(out[i]):
+            row = full[len(ids) - 1 + j]
+            assert float(row.max() - row[tok]) <= 1e-4, f"request {i}, token {j}: {tok} is not the plain best {int(row.argmax())}"

@@ -150,9 +150,9 @@ def test_gemm_mfma(ops, m, n, k):
     acc = base.clone().to(DEV)
     ops.gemm_fast(a.to(DEV), w.to(DEV), accumulate_into=acc)
     close(acc, want + base.double(), 1e-4, 1e-4 * scale, "mfma accumulate")
-    # rows do not depend on M (while the same kind of kernel serves them: up to SKINNY_PASSES_ROWS rows the
+    # rows do not depend on M (while the same kind of kernel serves them: up to the plan's stream_rows the
     # weights are streamed, beyond that the output is tiled)
-    part = max(m - 3, ops.SKINNY_PASSES_ROWS + 1) if m > ops.SKINNY_PASSES_ROWS else min(m, 40)
+    part = max(m - 3, ops.SKINNY_MAX_ROWS + 1) if m > ops.SKINNY_MAX_ROWS else min(m, 40)
     fewer = ops.gemm_fast(a[:part].contiguous().to(DEV), w.to(DEV), torch.float32)
     assert torch.equal(fewer, got[:part])
     assert ops.gemm_fast(a.float().to(DEV), w.to(DEV)) is None                      # float operands: not taken

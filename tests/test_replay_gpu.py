@@ -37,9 +37,12 @@ def setups(tmp_path_factory):
     return get
 
 
-def _executor(folder, dtype, num_pages, page_tokens, max_tokens):
+def _executor(folder, dtype, num_pages, page_tokens):
+    """An executor whose requests may grow to the model's positions (the longest request of every configuration
+    is as long as, or a little shorter than, that)."""
     from bare_cuda_4gib_amd.engine import Executor, load_model
     model, _ = load_model(folder, dtype, "cuda:0")
+    max_tokens = model.max_seq_len
     ex = Executor(model, num_pages=num_pages, max_requests=6, max_tokens=max_tokens, page_tokens=page_tokens,
                   poison=True)
     ex.cache.shuffle_free_pages(7)
@@ -53,7 +56,7 @@ CASES = [(n, d, v) for v in ("ones", "spread") for n in ("A", "B", "C") for d in
 def test_whole(setups, name, dtype, variant):
     folder, requests, plain = setups(name, dtype, variant)
     steps, where = helpers.trace_whole(requests)
-    ex = _executor(folder, dtype, num_pages=20, page_tokens=16, max_tokens=320)
+    ex = _executor(folder, dtype, num_pages=20, page_tokens=16)
     got = helpers.replay_in_process(ex, steps)
     helpers.compare_with_plain(got, where, plain, label=f"whole {name} {dtype} {variant}", **TOL[dtype])
     assert ex.cache.pages_in_use() == 0
@@ -63,7 +66,7 @@ def test_whole(setups, name, dtype, variant):
 def test_tail_one_by_one(setups, name, dtype, variant):
     folder, requests, plain = setups(name, dtype, variant)
     steps, where = helpers.trace_tail_one_by_one(requests, tail=32)
-    ex = _executor(folder, dtype, num_pages=20, page_tokens=16, max_tokens=320)
+    ex = _executor(folder, dtype, num_pages=20, page_tokens=16)
     got = helpers.replay_in_process(ex, steps)
     helpers.compare_with_plain(got, where, plain, label=f"tail {name} {dtype} {variant}", **TOL[dtype])
 
@@ -72,7 +75,7 @@ def test_tail_one_by_one(setups, name, dtype, variant):
 def test_portions(setups, name, dtype, variant):
     folder, requests, plain = setups(name, dtype, variant)
     steps, where = helpers.trace_portions(requests, seed=3)
-    ex = _executor(folder, dtype, num_pages=20, page_tokens=16, max_tokens=320)
+    ex = _executor(folder, dtype, num_pages=20, page_tokens=16)
     got = helpers.replay_in_process(ex, steps)
     helpers.compare_with_plain(got, where, plain, label=f"portions {name} {dtype} {variant}", **TOL[dtype])
 
@@ -82,7 +85,7 @@ def test_mixed_few_pages(setups, name, dtype, variant):
     folder, requests, plain = setups(name, dtype, variant)
     page = 16
     steps, where, peak = helpers.trace_mixed(requests, seed=11, max_live=4, page_tokens=page)
-    ex = _executor(folder, dtype, num_pages=peak // page, page_tokens=page, max_tokens=320)
+    ex = _executor(folder, dtype, num_pages=peak // page, page_tokens=page)
     got = helpers.replay_in_process(ex, steps)
     helpers.compare_with_plain(got, where, plain, label=f"mixed {name} {dtype} {variant}", **TOL[dtype])
     assert ex.cache.pages_in_use() == 0

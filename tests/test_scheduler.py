@@ -25,8 +25,8 @@ def fake_logits(tokens):
 class FakeExecutor:
     """Keeps a real cache manager (so pages run out for real) and checks that tokens arrive in
     order, each exactly once per (re)computation."""
-    def __init__(self, num_pages=8, page_tokens=4, max_requests=3, max_tokens=32):
-        self.cache = CacheManager({0: PagedKV(1, 2)}, page_tokens=page_tokens, num_pages=num_pages,
+    def __init__(self, num_pages=8, page_tokens=4, max_requests=3, max_tokens=32, streams=None):
+        self.cache = CacheManager(streams if streams is not None else {0: PagedKV(1, 2)}, page_tokens=page_tokens, num_pages=num_pages,
                                   max_requests=max_requests, max_tokens=max_tokens, dtype=torch.float32, device="cpu")
         self.history = {}
         self.batches = []
@@ -298,3 +298,36 @@ def test_running_ahead_leaves_rows_for_the_host_alone():
     sched.submit(Request(id=1, prompt=prompt(6, 2), max_new_tokens=8))
     out, finish = run(sched)
     assert ex.ahead_steps == 0 and len(out[0]) == 8 and out[1] == expected_greedy(prompt(6, 2), 8)
+
+
+def test_a_windowed_model_runs_in_a_pool_smaller_than_its_requests():
+    """Every stream of the model keeps a window of 6 tokens only: a request of 30 tokens needs the window's
+    pages and a portion's, not 30 tokens' worth, and is admitted and run in a pool of 3 pages (12 tokens);
+    what it may need at most is the cache manager's answer, by the stream's own rule."""
+    windowed = {0: PagedKV(1, 2, window=6), 1: PagedKV(1, 2, window=6)}
+    sched, ex = make(num_pages=3, max_tokens=32, prefill_chunk=4, streams=windowed)
+    assert ex.cache.peak_pages(29, 4) == {("window", 6): 3}
+    p = prompt(20, 11)
+    sched.submit(Request(id=0, prompt=p, max_new_tokens=10))
+    out, finish = run(sched)
+    assert out[0] == expected_greedy(p, 10) and finish[0] == "length"
+    assert ex.cache.groups[("window", 6)].pool.high_water_mark == 3 and sched.stats().preemptions == 0
+    # a portion too large for the pool beside the window is still refused, with the pool's size in the message
+    wide, _ = make(num_pages=5, max_tokens=32, prefill_chunk=16, streams=windowed)
+    assert "needs 6 KV pages, the pool holds 5" in wide.check(Request(id=1, prompt=prompt(20, 1), max_new_tokens=10))
+    # beside a stream that keeps everything the request is held to that stream's need
+    both, _ = make(num_pages=5, max_tokens=32, prefill_chunk=4, streams={0: PagedKV(1, 2), 1: PagedKV(1, 2, window=6)})
+    assert "needs 8 KV pages" in both.check(Request(id=2, prompt=prompt(20, 2), max_new_tokens=10))
+
+
+def test_a_model_that_keeps_nothing_per_token_needs_no_pages():
+    from bare_cuda_4gib_amd.cache import FixedState
+    sched, ex = make(num_pages=0, max_tokens=32, streams={0: FixedState((3,))})
+    assert sched.limits.kv_pages == 0 and ex.cache.peak_pages(31, 6) == {}
+    prompts = {i: prompt(n, 20 + i) for i, n in enumerate([9, 3, 14, 2])}
+    for i, p in prompts.items():
+        sched.submit(Request(id=i, prompt=p, max_new_tokens=5))
+    out, finish = run(sched)
+    for i, p in prompts.items():
+        assert out[i] == expected_greedy(p, 5) and finish[i] == "length"
+    assert sched.stats().preemptions == 0 and ex.cache.free_slots == 3
