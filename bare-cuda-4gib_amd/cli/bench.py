@@ -171,7 +171,7 @@ def main(argv=None) -> int:
           + f" | {args.warmup} warmup + {args.runs} measured runs")
     print(f"load       {load_ms:.0f} ms (file read, upload, weight layouts; excluded below)")
     print(f"memory     {(free_before - free_after) / mib:.1f} MiB taken on the device | {engine.model.weight_bytes / mib:.1f} "
-          f"weights ({engine.model.device_weight_bytes / mib:.1f} in the two layouts the kernels read) + "
+          f"weights ({engine.model.device_weight_bytes / mib:.1f} on the device, as the kernels read them) + "
           f"{engine.executor.cache.storage_bytes() / mib:.1f} cache accounted, dtype {args.dtype}")
     print(f"kv pool    {engine.kv_pages} pages of {args.page_tokens} tokens | max batch {engine.max_seqs} at "
           f"{engine.max_tokens} tokens per sequence\n")

@@ -53,7 +53,7 @@ def main(argv=None) -> int:
         cache_mib = engine.executor.cache.storage_bytes() / 2**20
         print(f"[llm] {len(engine.model.layers)} layers, hidden {engine.model.hidden_size}, vocab "
               f"{engine.model.vocab_size} | weights {engine.model.weight_bytes / 2**20:.1f} MiB "
-              f"({engine.model.device_weight_bytes / 2**20:.1f} on the device, in two layouts), cache "
+              f"({engine.model.device_weight_bytes / 2**20:.1f} on the device, as the kernels read them), cache "
               f"{cache_mib:.1f} MiB ({engine.kv_pages} pages, max batch {engine.max_seqs})")
         generated = generate_batch(engine, [prompt], args.tokens, temperature=args.temperature,
                                    top_p=args.top_p, top_k=args.top_k, seed=args.seed)[0]

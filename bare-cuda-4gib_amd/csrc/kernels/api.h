@@ -136,17 +136,22 @@ int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, float* part_o,
 extern "C" {
 // bfloat16 a [m, k] times bfloat16 w [n, k] transposed on the matrix cores, any m.
 // epilogue: 0 store bfloat16; 1 store float32; 2 add into float32; 3 SwiGLU as in bc4g_gemm_skinny.
-int bc4g_gemm_mfma(const void* a, const void* w, void* out, int epilogue, int m, int n, int k, void* stream);
+// w_packed (here and in the three entry points below) 0: w lies by rows, [n, k].  1: w lies in the order of the
+// weight-streaming kernel (bc4g_gemm_skinny: [ceil(n / 16)][k / 32][64 lanes][8]), so that one copy of a weight
+// serves both kernels; k must then be a multiple of 64 and the operands on 16-byte boundaries.  The sums are the
+// same bits either way.
+int bc4g_gemm_mfma(const void* a, const void* w, int w_packed, void* out, int epilogue, int m, int n, int k, void* stream);
 // The same product with k cut into k_parts equal parts (each a multiple of 64), part p's sums stored as float32 in
 // parts [k_parts, m, n]: for few rows and a long k, where one workgroup per 64 x 64 tile would walk all of k alone.
 // Whoever reads the parts adds them up in order (bc4g_rmsnorm_sum).
-int bc4g_gemm_mfma_parts(const void* a, const void* w, float* parts, int m, int n, int k, int k_parts, void* stream);
+int bc4g_gemm_mfma_parts(const void* a, const void* w, int w_packed, float* parts, int m, int n, int k, int k_parts,
+                         void* stream);
 // The SwiGLU product (epilogue 3) of rows that lack their RMSNorm's common factor: a = bfloat16(residual * g) [m, k] and
 // the parts of the rows' sums of squares as bc4g_gemm_skinny_emit leaves them (ssq_parts [ssq_blocks][ssq_stride]); every
 // row's sums are multiplied by 1 / sqrt(sum of squares / k + eps) before the activation, the parts added in the order
 // of bc4g_gemm_skinny_prenormed.  k a multiple of 64, n of 16, operands on 16-byte boundaries; any m.
 int bc4g_gemm_mfma_swiglu_scaled(const void* a, const float* ssq_parts, int ssq_blocks, int ssq_stride, float eps,
-                                 const void* w, void* out, int m, int n, int k, void* stream);
+                                 const void* w, int w_packed, void* out, int m, int n, int k, void* stream);
 // The output tile (rows, columns) bc4g_gemm_mfma (qkv 0) or bc4g_gemm_mfma_qkv (qkv 1) takes for these operands: for
 // the accounting of bytes and for tests that want to meet every tile.  Launches nothing.
 int bc4g_gemm_mfma_tile(const void* a, const void* w, int m, int n, int k, int qkv, int* rows, int* cols);
@@ -156,7 +161,7 @@ int bc4g_gemm_mfma_tile(const void* a, const void* w, int m, int n, int k, int q
 // [m, n_heads * head_dim] bfloat16 receives the rotated queries; keys go rotated, values as they are into the pages that
 // slot_map [m] names, in the cache's layout (write_kv 0: nowhere).  table [m, head_dim / 2, 2]: cosine and sine
 // of every row's position and pair (bc4g_rope_table; null: nothing is rotated).
-int bc4g_gemm_mfma_qkv(const void* a, const void* w, void* out, const float* table, const int32_t* slot_map, void* k_cache,
+int bc4g_gemm_mfma_qkv(const void* a, const void* w, int w_packed, void* out, const float* table, const int32_t* slot_map, void* k_cache,
                        void* v_cache, int m, int n, int k, int n_heads, int n_kv_heads, int head_dim, int page_tokens,
                        int write_kv, void* stream);
 }

@@ -3,26 +3,29 @@
 // of the 32-bit path, and the fallback where the MFMA kernels refuse a size.
 //
 // Each output element is the sum over k in ascending order in one thread, so
-// a row's result does not depend on how many rows the call has.
+// a row's result does not depend on how many rows the call has -- nor on which of the
+// two tile sizes below serves the call: 64 x 64 outputs a block (four by four a thread),
+// or, for up to 16 rows (a decode step), 16 x 16 (one a thread, k staged 64 at a time),
+// which brings sixteen times the blocks to stream the weights of a product with few rows
+// (a decode step of the 32-bit path at TinyLlama's sizes: 43 ms with the large tile alone).
 #include "api.h"
 #include "common.h"
 
 namespace bc4g {
 namespace {
 
-constexpr int kTile = 64;   // output tile per block, both ways
-constexpr int kStepK = 16;  // k per staging step
-constexpr int kPerThread = 4;
+constexpr int kFewRows = 16;   // rows up to which the small tile serves
 
-template <typename TA, typename TW, typename TO, bool kAccumulate>
+template <typename TA, typename TW, typename TO, bool kAccumulate, int kPerThread, int kStepK>
 __global__ __launch_bounds__(256) void gemm_generic_kernel(const TA* __restrict__ a,
                                                            const TW* __restrict__ w,
                                                            TO* __restrict__ out, int m, int n, int k) {
+  constexpr int kTile = 16 * kPerThread;   // output tile per block, both ways
   // k-major tiles, padded so that the 16 threads of a row group hit different banks.
   __shared__ float as[kStepK][kTile + 1];
   __shared__ float ws[kStepK][kTile + 1];
-  const int tx = threadIdx.x % 16;  // columns tx*4 .. tx*4+3
-  const int ty = threadIdx.x / 16;  // rows    ty*4 .. ty*4+3
+  const int tx = threadIdx.x % 16;  // columns tx*kPerThread ..
+  const int ty = threadIdx.x / 16;  // rows    ty*kPerThread ..
   const long m0 = static_cast<long>(blockIdx.y) * kTile;
   const long n0 = static_cast<long>(blockIdx.x) * kTile;
 
@@ -33,9 +36,9 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const TA* __restrict_
     for (int j = 0; j < kPerThread; ++j) acc[i][j] = 0.f;
 
   for (int k0 = 0; k0 < k; k0 += kStepK) {
-    // 64 rows x 16 k = 1024 elements per operand, 4 per thread; k fastest for coalescing.
+    // kTile rows x kStepK k elements per operand, the same number a thread; k fastest for coalescing.
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
+    for (int r = 0; r < kTile * kStepK / 256; ++r) {
       const int e = threadIdx.x + r * 256;
       const int kk = e % kStepK, row = e / kStepK;
       const long gm = m0 + row, gn = n0 + row;
@@ -78,8 +81,12 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const TA* __restrict_
 
 template <typename TA, typename TW, typename TO, bool kAcc>
 void launch(const void* a, const void* w, void* out, int m, int n, int k, hipStream_t s) {
-  dim3 grid(ceil_div(n, kTile), ceil_div(m, kTile));
-  gemm_generic_kernel<TA, TW, TO, kAcc><<<grid, 256, 0, s>>>(
+  if (m <= kFewRows) {
+    gemm_generic_kernel<TA, TW, TO, kAcc, 1, 64><<<dim3(ceil_div(n, 16), 1), 256, 0, s>>>(
+        static_cast<const TA*>(a), static_cast<const TW*>(w), static_cast<TO*>(out), m, n, k);
+    return;
+  }
+  gemm_generic_kernel<TA, TW, TO, kAcc, 4, 16><<<dim3(ceil_div(n, 64), ceil_div(m, 64)), 256, 0, s>>>(
       static_cast<const TA*>(a), static_cast<const TW*>(w), static_cast<TO*>(out), m, n, k);
 }
 
@@ -92,7 +99,7 @@ extern "C" int bc4g_gemm_generic(const void* a, int a_dtype, const void* w, int 
                                  int out_dtype, int accumulate, int m, int n, int k, void* stream) {
   BC4G_REQUIRE(m >= 0 && n > 0 && k > 0, "gemm: bad sizes M=%d N=%d K=%d", m, n, k);
   BC4G_REQUIRE(!accumulate || out_dtype == kF32, "gemm: accumulation needs a float32 output");
-  BC4G_REQUIRE(ceil_div(m, kTile) <= 65535, "gemm: M=%d is beyond the grid limit", m);
+  BC4G_REQUIRE(ceil_div(m, 64) <= 65535, "gemm: M=%d is beyond the grid limit", m);
   if (m == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int key = a_dtype * 100 + w_dtype * 10 + out_dtype;

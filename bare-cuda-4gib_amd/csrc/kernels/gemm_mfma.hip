@@ -473,7 +473,7 @@ struct DirectShape {
 template <int EPI, int WM, int WN, int TM, int TN, int BK, int STAGES, int MINWG>
 __global__ __launch_bounds__(64 * WM * WN, MINWG) void gemm_mfma_direct_kernel(
     const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, void* __restrict__ out, int m, int n, int k, int m_blocks,
-    int n_blocks, const RopeKvArgs ra, const RowScaleArgs rows) {
+    int n_blocks, const RopeKvArgs ra, const RowScaleArgs rows, const int w_packed) {
   typedef DirectShape<WM, WN, TM, TN, BK, STAGES> S;
   constexpr int RA = S::kRowsA, RW = S::kRowsW, RB = S::kRowBytes, NW = S::kWaves;
   constexpr int kGroupRows = 1024 / RB;                    // rows a wave-wide load covers
@@ -491,6 +491,13 @@ __global__ __launch_bounds__(64 * WM * WN, MINWG) void gemm_mfma_direct_kernel(
   // its own, out + y * m * n (the plain store epilogues only: whoever reads them adds the parts up in order)
   const int nk = k / BK / static_cast<int>(gridDim.y);
   const size_t k_first = static_cast<size_t>(blockIdx.y) * nk * RB;       // in bytes of a row
+  // w_packed: the weight comes in the order the weight-streaming kernel reads ([n / 16][k / 32][64 lanes][8]: the
+  // 16 bytes of row r and k 8 c .. 8 c + 7 lie at ((r / 16) * (k / 32) + c / 4) * 1024 + ((c % 4) * 16 + r % 16) * 16),
+  // so that a model keeps every weight once.  A lane still brings the same 16 bytes of the same row to the same
+  // place in LDS; only where they lie in memory differs, and a step of BK moves on by BK / 32 kilobytes.  A
+  // wave-wide load touches whole lines either way: eight rows' 128 bytes by rows, eight segments' 128 bytes
+  // (eight consecutive rows of one segment) packed.
+  constexpr size_t kPackedStep = static_cast<size_t>(BK / 32) * 1024;
   if constexpr (EPI == kStoreF32) out = static_cast<float*>(out) + static_cast<size_t>(blockIdx.y) * m * n;
 
   // the groups of rows this wave brings every step (a spare turn repeats the last group: the same
@@ -498,6 +505,7 @@ __global__ __launch_bounds__(64 * WM * WN, MINWG) void gemm_mfma_direct_kernel(
   const int lr = (lane * 16) / RB, ls = (lane * 16 % RB) / 16;
   const unsigned char* src[PER];
   unsigned dst[PER];
+  size_t step_bytes[PER];
 #pragma unroll
   for (int i = 0; i < PER; ++i) {
     int g = wave + NW * i;
@@ -508,14 +516,21 @@ __global__ __launch_bounds__(64 * WM * WN, MINWG) void gemm_mfma_direct_kernel(
     long row = (of_a ? m0 : n0) + trow;
     const long last = (of_a ? m : n) - 1;
     if (row > last) row = last;
-    src[i] = reinterpret_cast<const unsigned char*>((of_a ? a : w) + row * k) + k_first + seg * 16;
+    if (w_packed && !of_a) {
+      src[i] = reinterpret_cast<const unsigned char*>(w) + (row / 16) * static_cast<size_t>(k / 32) * 1024 +
+               static_cast<size_t>(blockIdx.y) * nk * kPackedStep + (seg / 4) * 1024 + ((seg % 4) * 16 + row % 16) * 16;
+      step_bytes[i] = kPackedStep;
+    } else {
+      src[i] = reinterpret_cast<const unsigned char*>((of_a ? a : w) + row * k) + k_first + seg * 16;
+      step_bytes[i] = RB;
+    }
     dst[i] = (of_a ? 0 : RA * RB) + (of_a ? g : g - GA) * 1024;
   }
   auto ask = [&](int step) {
     const unsigned base = lds_base + (step % STAGES) * S::kStageBytes;
 #pragma unroll
     for (int i = 0; i < PER; ++i)
-      load_to_lds_16(src[i] + static_cast<size_t>(step) * RB, __builtin_amdgcn_readfirstlane(base + dst[i]));
+      load_to_lds_16(src[i] + static_cast<size_t>(step) * step_bytes[i], __builtin_amdgcn_readfirstlane(base + dst[i]));
   };
 
   floatx16 acc[TM][TN];
@@ -653,7 +668,7 @@ __global__ __launch_bounds__(64 * WM * WN, MINWG) void gemm_mfma_direct_kernel(
 
 template <int EPI, int WM, int WN, int TM, int TN, int BK, int STAGES, int MINWG>
 int launch_direct(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, int k, hipStream_t s, const RopeKvArgs& ra,
-                  int k_parts = 1, const RowScaleArgs& rows = RowScaleArgs{}) {
+                  int k_parts = 1, const RowScaleArgs& rows = RowScaleArgs{}, int w_packed = 0) {
   typedef DirectShape<WM, WN, TM, TN, BK, STAGES> S;
   auto kernel = gemm_mfma_direct_kernel<EPI, WM, WN, TM, TN, BK, STAGES, MINWG>;
   static bool raised = false;   // per instantiation: allow more than the default dynamic LDS
@@ -665,7 +680,7 @@ int launch_direct(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, i
   }
   const long m_blocks = (m + S::kRowsA - 1) / S::kRowsA, n_blocks = (n + S::kRowsW - 1) / S::kRowsW;
   kernel<<<dim3(static_cast<unsigned>(m_blocks * n_blocks), static_cast<unsigned>(k_parts)), dim3(S::kThreads), S::kLdsBytes, s>>>(
-      ap, wp, out, m, n, k, static_cast<int>(m_blocks), static_cast<int>(n_blocks), ra, rows);
+      ap, wp, out, m, n, k, static_cast<int>(m_blocks), static_cast<int>(n_blocks), ra, rows, w_packed);
   return 0;
 }
 
@@ -711,14 +726,14 @@ int direct_form(int m, int n, int k, bool long_epilogue) {
 
 template <int EPI>
 int launch_direct_form(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, int k, hipStream_t s,
-                       const RopeKvArgs& ra = RopeKvArgs{}, const RowScaleArgs& rows = RowScaleArgs{}) {
+                       const RopeKvArgs& ra = RopeKvArgs{}, const RowScaleArgs& rows = RowScaleArgs{}, int w_packed = 0) {
   switch (direct_form(m, n, k, EPI == kRopeKvBf16)) {
-    case 0: return launch_direct<EPI, 4, 4, 2, 2, 64, 2, 1>(ap, wp, out, m, n, k, s, ra, 1, rows);
-    case 1: return launch_direct<EPI, 4, 2, 2, 3, 64, 2, 1>(ap, wp, out, m, n, k, s, ra, 1, rows);
-    case 2: return launch_direct<EPI, 4, 2, 2, 2, 64, 3, 1>(ap, wp, out, m, n, k, s, ra, 1, rows);
-    case 3: return launch_direct<EPI, 2, 4, 2, 1, 64, 4, 1>(ap, wp, out, m, n, k, s, ra, 1, rows);
-    case 5: return launch_direct<EPI, 2, 2, 2, 1, 64, 2, 4>(ap, wp, out, m, n, k, s, ra, 1, rows);
-    default: return launch_direct<EPI, 2, 2, 1, 1, 64, 4, 2>(ap, wp, out, m, n, k, s, ra, 1, rows);
+    case 0: return launch_direct<EPI, 4, 4, 2, 2, 64, 2, 1>(ap, wp, out, m, n, k, s, ra, 1, rows, w_packed);
+    case 1: return launch_direct<EPI, 4, 2, 2, 3, 64, 2, 1>(ap, wp, out, m, n, k, s, ra, 1, rows, w_packed);
+    case 2: return launch_direct<EPI, 4, 2, 2, 2, 64, 3, 1>(ap, wp, out, m, n, k, s, ra, 1, rows, w_packed);
+    case 3: return launch_direct<EPI, 2, 4, 2, 1, 64, 4, 1>(ap, wp, out, m, n, k, s, ra, 1, rows, w_packed);
+    case 5: return launch_direct<EPI, 2, 2, 2, 1, 64, 2, 4>(ap, wp, out, m, n, k, s, ra, 1, rows, w_packed);
+    default: return launch_direct<EPI, 2, 2, 1, 1, 64, 4, 2>(ap, wp, out, m, n, k, s, ra, 1, rows, w_packed);
   }
 }
 
@@ -728,8 +743,9 @@ bool direct_operands(const void* ap, const void* wp, int k) {
 }
 
 template <int EPI>
-int launch_tiled(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, int k, hipStream_t s) {
-  if (direct_operands(ap, wp, k)) return launch_direct_form<EPI>(ap, wp, out, m, n, k, s);
+int launch_tiled(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, int k, hipStream_t s, int w_packed) {
+  if (direct_operands(ap, wp, k)) return launch_direct_form<EPI>(ap, wp, out, m, n, k, s, RopeKvArgs{}, RowScaleArgs{}, w_packed);
+  if (w_packed) return fail("gemm_mfma: a packed weight needs k in whole steps of 64 and operands on 16-byte boundaries (K=%d)", k);
   const long m_blocks = (m + kBM - 1) / kBM, n_blocks = (n + kBN - 1) / kBN;
   gemm_mfma_staged_kernel<EPI><<<dim3(static_cast<unsigned>(m_blocks * n_blocks)), dim3(256), 0, s>>>(
       ap, wp, out, m, n, k, static_cast<int>(m_blocks), static_cast<int>(n_blocks));
@@ -741,7 +757,7 @@ int launch_tiled(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, in
 
 using namespace bc4g;
 
-extern "C" int bc4g_gemm_mfma(const void* a, const void* w, void* out, int epilogue, int m, int n, int k,
+extern "C" int bc4g_gemm_mfma(const void* a, const void* w, int w_packed, void* out, int epilogue, int m, int n, int k,
                               void* stream) {
   BC4G_REQUIRE(m >= 0 && n > 0 && k > 0 && k % 8 == 0, "gemm_mfma: K=%d must be a positive multiple of 8 (M=%d N=%d)",
                k, m, n);
@@ -752,12 +768,12 @@ extern "C" int bc4g_gemm_mfma(const void* a, const void* w, void* out, int epilo
   const bf16_t* wp = static_cast<const bf16_t*>(w);
   int e = 0;
   switch (epilogue) {
-    case kStoreBf16: e = launch_tiled<kStoreBf16>(ap, wp, out, m, n, k, s); break;
-    case kStoreF32: e = launch_tiled<kStoreF32>(ap, wp, out, m, n, k, s); break;
-    case kAccumF32: e = launch_tiled<kAccumF32>(ap, wp, out, m, n, k, s); break;
+    case kStoreBf16: e = launch_tiled<kStoreBf16>(ap, wp, out, m, n, k, s, w_packed); break;
+    case kStoreF32: e = launch_tiled<kStoreF32>(ap, wp, out, m, n, k, s, w_packed); break;
+    case kAccumF32: e = launch_tiled<kAccumF32>(ap, wp, out, m, n, k, s, w_packed); break;
     case kSwigluBf16:
       BC4G_REQUIRE(n % 16 == 0, "gemm_mfma: SwiGLU needs blocks of eight gate and eight up rows, N=%d is no multiple of 16", n);
-      e = launch_tiled<kSwigluBf16>(ap, wp, out, m, n, k, s);
+      e = launch_tiled<kSwigluBf16>(ap, wp, out, m, n, k, s, w_packed);
       break;
     default: return fail("gemm_mfma: unknown epilogue %d", epilogue);
   }
@@ -766,7 +782,7 @@ extern "C" int bc4g_gemm_mfma(const void* a, const void* w, void* out, int epilo
 }
 
 extern "C" int bc4g_gemm_mfma_swiglu_scaled(const void* a, const float* ssq_parts, int ssq_blocks, int ssq_stride, float eps,
-                                            const void* w, void* out, int m, int n, int k, void* stream) {
+                                            const void* w, int w_packed, void* out, int m, int n, int k, void* stream) {
   BC4G_REQUIRE(m >= 0 && n > 0 && n % 16 == 0 && k > 0 && direct_operands(a, w, k),
                "gemm_mfma_swiglu_scaled: K=%d must be a multiple of 64, N=%d one of 16 and the operands on 16-byte boundaries (M=%d)", k, n, m);
   BC4G_REQUIRE(ssq_parts != nullptr && ssq_blocks > 0 && ssq_stride >= m && eps >= 0.f,
@@ -775,23 +791,25 @@ extern "C" int bc4g_gemm_mfma_swiglu_scaled(const void* a, const float* ssq_part
   BC4G_REQUIRE(((m + 63L) / 64) * ((n + 63L) / 64) <= 2147483647L, "gemm_mfma_swiglu_scaled: too many tiles");
   if (int e = launch_direct_form<kSwigluScaledBf16>(static_cast<const bf16_t*>(a), static_cast<const bf16_t*>(w), out, m, n, k,
                                                      static_cast<hipStream_t>(stream), RopeKvArgs{},
-                                                     RowScaleArgs{ssq_parts, ssq_blocks, ssq_stride, eps}))
+                                                     RowScaleArgs{ssq_parts, ssq_blocks, ssq_stride, eps}, w_packed))
     return e;
   return check_launch("gemm_mfma_swiglu_scaled");
 }
 
-extern "C" int bc4g_gemm_mfma_parts(const void* a, const void* w, float* parts, int m, int n, int k, int k_parts, void* stream) {
+extern "C" int bc4g_gemm_mfma_parts(const void* a, const void* w, int w_packed, float* parts, int m, int n, int k, int k_parts,
+                                    void* stream) {
   BC4G_REQUIRE(m > 0 && n > 0 && k > 0 && k_parts >= 1 && k_parts <= 16 && k % (64 * k_parts) == 0 && direct_operands(a, w, k),
                "gemm_mfma_parts: K=%d must be %d times a multiple of 64 and the operands on 16-byte boundaries (M=%d N=%d)", k,
                k_parts, m, n);
   BC4G_REQUIRE(((m + 63L) / 64) * ((n + 63L) / 64) <= 2147483647L, "gemm_mfma_parts: too many tiles");
   if (int e = launch_direct<kStoreF32, 2, 2, 1, 1, 64, 4, 2>(static_cast<const bf16_t*>(a), static_cast<const bf16_t*>(w), parts, m, n,
-                                                               k, static_cast<hipStream_t>(stream), RopeKvArgs{}, k_parts))
+                                                               k, static_cast<hipStream_t>(stream), RopeKvArgs{}, k_parts,
+                                                               RowScaleArgs{}, w_packed))
     return e;
   return check_launch("gemm_mfma_parts");
 }
 
-extern "C" int bc4g_gemm_mfma_qkv(const void* a, const void* w, void* out, const float* table, const int32_t* slot_map,
+extern "C" int bc4g_gemm_mfma_qkv(const void* a, const void* w, int w_packed, void* out, const float* table, const int32_t* slot_map,
                                   void* k_cache, void* v_cache, int m, int n, int k, int n_heads, int n_kv_heads,
                                   int head_dim, int page_tokens, int write_kv, void* stream) {
   BC4G_REQUIRE(m > 0 && n > 0 && k > 0 && direct_operands(a, w, k),
@@ -813,7 +831,7 @@ extern "C" int bc4g_gemm_mfma_qkv(const void* a, const void* w, void* out, const
   ra.write_kv = write_kv ? 1 : 0;
   ra.fragment_order = write_kv && cache_fragment_order(true, head_dim, page_tokens) ? 1 : 0;
   if (int e = launch_direct_form<kRopeKvBf16>(static_cast<const bf16_t*>(a), static_cast<const bf16_t*>(w), out, m, n, k,
-                                              static_cast<hipStream_t>(stream), ra))
+                                              static_cast<hipStream_t>(stream), ra, RowScaleArgs{}, w_packed))
     return e;
   return check_launch("gemm_mfma_qkv");
 }

@@ -19,8 +19,8 @@ _SIGNATURES = {
     "bc4g_embed_gather": [_P, _I, _P, _P, _I, _I, _I, _P],
     "bc4g_rmsnorm": [_P, _P, _P, _I, _P, _I, _I, _I, _F, _P],
     "bc4g_rmsnorm_sum": [_P, _P, _I, _P, _I, _P, _I, _I, _I, _F, _P],
-    "bc4g_gemm_mfma_parts": [_P, _P, _P, _I, _I, _I, _I, _P],
-    "bc4g_gemm_mfma_swiglu_scaled": [_P, _P, _I, _I, _F, _P, _P, _I, _I, _I, _P],
+    "bc4g_gemm_mfma_parts": [_P, _P, _I, _P, _I, _I, _I, _I, _P],
+    "bc4g_gemm_mfma_swiglu_scaled": [_P, _P, _I, _I, _F, _P, _I, _P, _I, _I, _I, _P],
     "bc4g_gemm_generic": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _P],
     "bc4g_swiglu": [_P, _P, _I, _I, _I, _I, _P],
     "bc4g_rope_table": [_P, _P, _I, _I, _F, _P],
@@ -33,11 +33,11 @@ _SIGNATURES = {
     "bc4g_probe_read": [_P, c_long, _P, _I, _P],
     "bc4g_probe_mfma": [_P, _I, _P, _I, _P],
     "bc4g_gemm_skinny": [_P, _P, _P, _I, _I, _I, _I, _P],
-    "bc4g_gemm_mfma": [_P, _P, _P, _I, _I, _I, _I, _P],
+    "bc4g_gemm_mfma": [_P, _P, _I, _P, _I, _I, _I, _I, _P],
     "bc4g_gemm_mfma_tile": [_P, _P, _I, _I, _I, _I, _P, _P],
     "bc4g_gemm_skinny_normed": [_P, _P, _P, _I, _F, _P, _P, _I, _I, _I, _I, _P],
     "bc4g_attention_mfma": [_P, _I, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _P, _I, _P, _I, _P, _P],
-    "bc4g_gemm_mfma_qkv": [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P],
+    "bc4g_gemm_mfma_qkv": [_P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P],
     "bc4g_gemm_skinny_qkv": [_P, _P, _I, _F, _P, _I, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P],
     "bc4g_gemm_skinny_emit": [_P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _P],
     "bc4g_gemm_skinny_prenormed": [_P, _P, _I, _I, _F, _P, _P, _I, _I, _I, _I, _P],

@@ -125,7 +125,7 @@ def gemm_generic(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = None
                  accumulate_into: Optional[torch.Tensor] = None) -> torch.Tensor:
     """a [M, K] times w [N, K] transposed, in plain float arithmetic.  With
     ``accumulate_into`` (float32 [M, N]) the product is added to it in place."""
-    w, _ = _weight(w)
+    w = _rows(w)
     _dev("gemm", a, w, accumulate_into)
     if a.dim() != 2 or w.dim() != 2 or a.shape[1] != w.shape[1]:
         raise KernelError(f"gemm: shapes {tuple(a.shape)} x {tuple(w.shape)}^T do not match")
@@ -333,25 +333,80 @@ def pack_weight(w: torch.Tensor) -> torch.Tensor:
     return padded.view(nb, 16, ks, 4, 8).permute(0, 2, 3, 1, 4).contiguous().view(-1)
 
 
-class StreamedWeight:
-    """A linear map's weight in both orders: by rows (for the tiled and the plain kernels) and
-    packed for the weight-streaming kernel.  The second copy costs memory, not traffic: every
-    step reads one of them."""
+def unpack_weight(packed: torch.Tensor, n: int, k: int) -> torch.Tensor:
+    """The [n, k] weight by rows from its packed form (pack_weight's inverse)."""
+    nb, ks = -(-n // 16), -(-k // 32)
+    return packed.view(nb, ks, 4, 16, 8).permute(0, 3, 1, 2, 4).reshape(nb * 16, ks * 32)[:n, :k].contiguous()
 
-    def __init__(self, rows: torch.Tensor):
-        self.rows = rows
+
+class StreamedWeight:
+    """A linear map's weight [n, k] as the kernels read it.  A bfloat16 weight on the device (k a multiple of 8) is
+    kept packed in the weight-streaming kernel's order; where k is whole steps of 64 the tiled kernel reads that
+    same copy, so the weight is held ONCE.  The rows are kept beside it only where a kernel needs them (k no
+    multiple of 64: the tiled kernel's fallback) or where they cost nothing (``keep_rows``: a tensor that someone
+    else holds anyway, the embedding table of a tied head); otherwise ``rows`` makes them from the packed copy when
+    first asked (the plain float kernel for operands the matrix-core kernels refuse) and keeps them from then on.
+    A weight the matrix-core kernels cannot take at all (float32, a CPU tensor) is its rows."""
+
+    def __init__(self, rows: torch.Tensor, keep_rows: Optional[bool] = None):
         self.shape, self.dtype, self.device = rows.shape, rows.dtype, rows.device
         ok = rows.is_cuda and rows.dtype == torch.bfloat16 and rows.dim() == 2 and rows.shape[1] % 8 == 0
         self.packed = pack_weight(rows) if ok else None
+        if keep_rows is None:
+            keep_rows = not (ok and rows.shape[1] % 64 == 0)
+        self._rows = rows if keep_rows or not ok else None
         # which kernel serves this weight at which number of rows: its own table, made from its shape
         self.plan = plan_for(int(rows.shape[0]), int(rows.shape[1])) if rows.dim() == 2 else None
 
+    @property
+    def rows(self) -> torch.Tensor:
+        if self._rows is None:
+            self._rows = unpack_weight(self.packed, self.shape[0], self.shape[1])
+        return self._rows
+
+    @property
+    def holds_rows(self) -> bool:
+        return self._rows is not None
+
+    # what the wrappers ask of an operand before they launch (answered without making the rows)
+    @property
+    def is_cuda(self) -> bool:
+        return self.device.type == "cuda"
+
+    def dim(self) -> int:
+        return len(self.shape)
+
+    def is_contiguous(self) -> bool:
+        return True
+
+    def stride(self):
+        return (self.shape[1], 1)
+
+    def data_ptr(self) -> int:
+        return (self.packed if self._rows is None else self._rows).data_ptr()
+
+    def element_size(self) -> int:
+        return 2 if self.dtype == torch.bfloat16 else 4
+
 
 def _weight(w):
-    """(rows, packed or None) of a weight given as a tensor or a StreamedWeight."""
+    """(the weight as an operand to check -- shape, dtype, device --, its packed copy or None) of a weight given as
+    a tensor or a StreamedWeight."""
     if isinstance(w, StreamedWeight):
-        return w.rows, w.packed
+        return w, w.packed
     return w, None
+
+
+def _rows(w) -> torch.Tensor:
+    return w.rows if isinstance(w, StreamedWeight) else w
+
+
+def _tiled_weight(w, packed):
+    """(address, 1 if packed else 0) of a weight for the tiled kernel: the packed copy where that kernel takes it
+    (a bound weight, k in whole steps of 64), else the rows."""
+    if isinstance(w, StreamedWeight) and packed is not None and w.shape[1] % 64 == 0:
+        return packed.data_ptr(), 1
+    return _rows(w).data_ptr(), 0
 
 
 SKINNY_MAX_ROWS = 64                # rows the weight-streaming kernel takes in one launch
@@ -505,13 +560,13 @@ def gemm_fast(a: torch.Tensor, w, out_dtype=None,
         epi = EPI_STORE_BF16 if out_dtype == torch.bfloat16 else EPI_STORE_F32
     out_bytes = 8 if accumulate_into is not None else out.element_size()
     if streams_weights(m, n, k):
-        packed = packed if packed is not None else pack_weight(w)      # (packing per call: tests only)
+        packed = packed if packed is not None else pack_weight(_rows(w))      # (packing per call: tests only)
         for r0 in range(0, m, SKINNY_MAX_ROWS):                        # the weights once for every 64 rows
             rows = min(SKINNY_MAX_ROWS, m - r0)
             library.call("bc4g_gemm_skinny", _ptr(a[r0:]), _ptr(packed), _ptr(out[r0:]), epi, rows, n, k, _stream(),
                          cost=_skinny_cost(rows, n, k, 2, out_bytes))
     else:
-        library.call("bc4g_gemm_mfma", _ptr(a), _ptr(w), _ptr(out), epi, m, n, k, _stream(),
+        library.call("bc4g_gemm_mfma", _ptr(a), *_tiled_weight(w, packed), _ptr(out), epi, m, n, k, _stream(),
                      cost=_tiled_cost(m, n, k, out_bytes))
     return out
 
@@ -534,7 +589,7 @@ def gemm_normed(x: torch.Tensor, rows: Optional[torch.Tensor], n_rows: int, g: t
     """rmsnorm(x[rows]) W^T with the norm fused into the product (see gemm_skinny.hip): epilogue
     EPI_STORE_BF16, EPI_STORE_F32 or EPI_SWIGLU (w = gate rows then up rows)."""
     w, packed = _weight(w)
-    packed = packed if packed is not None else pack_weight(w)
+    packed = packed if packed is not None else pack_weight(_rows(w))
     _dev("gemm_normed", x, rows, g, w)
     k, n = x.shape[1], w.shape[0]
     if tuple(g.shape) != (k,):
@@ -569,18 +624,18 @@ def gemm_swiglu(a: torch.Tensor, w_gate_up, interleaved: bool = False) -> torch.
         n = rows.shape[0]
         out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=a.device)
         if streams_weights(m, n, k):
-            packed = packed if packed is not None else pack_weight(rows)
+            packed = packed if packed is not None else pack_weight(_rows(rows))
             for r0 in range(0, m, SKINNY_MAX_ROWS):
                 part = min(SKINNY_MAX_ROWS, m - r0)
                 library.call("bc4g_gemm_skinny", _ptr(a[r0:]), _ptr(packed), _ptr(out[r0:]), EPI_SWIGLU, part, n, k,
                              _stream(), cost=_skinny_cost(part, n, k, 2, 1))
         else:
-            library.call("bc4g_gemm_mfma", _ptr(a), _ptr(rows), _ptr(out), EPI_SWIGLU, m, n, k, _stream(),
+            library.call("bc4g_gemm_mfma", _ptr(a), *_tiled_weight(rows, packed), _ptr(out), EPI_SWIGLU, m, n, k, _stream(),
                          cost=_tiled_cost(m, n, k, 1))
         return out
     gu = gemm_fast(a, w_gate_up, a.dtype)
     if gu is None:
-        gu = gemm_generic(a, rows, a.dtype)
+        gu = gemm_generic(a, w_gate_up, a.dtype)
     return swiglu(gu, interleaved)
 
 
@@ -622,7 +677,7 @@ def gemm_parts_accumulate_norm(a: torch.Tensor, w, residual: torch.Tensor, g: to
     into parts over workgroups, each part's sums stored apart; then one that adds the parts to the residual in
     order and norms it.  For a few dozen rows and a square or long weight, where a 64 x 64 tile's workgroup
     would walk all of k alone and the weight-streaming kernel's workgroups all read all of x."""
-    w, _ = _weight(w)
+    w, packed = _weight(w)
     _dev("gemm_parts_accumulate_norm", a, w, residual, g)
     m, k = a.shape
     n = w.shape[0]
@@ -631,7 +686,7 @@ def gemm_parts_accumulate_norm(a: torch.Tensor, w, residual: torch.Tensor, g: to
         raise KernelError(f"gemm_parts_accumulate_norm: not for [{m}, {k}] x [{n}, {k}]^T")
     parts = torch.empty((n_parts, m, n), dtype=torch.float32, device=a.device)
     out = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
-    library.call("bc4g_gemm_mfma_parts", _ptr(a), _ptr(w), _ptr(parts), m, n, k, n_parts, _stream(),
+    library.call("bc4g_gemm_mfma_parts", _ptr(a), *_tiled_weight(w, packed), _ptr(parts), m, n, k, n_parts, _stream(),
                  cost=_gemm_cost(m, n, k, 2, 2, 4 * n_parts, x_readers=-(-n // 64), w_readers=-(-m // 64)))
     library.call("bc4g_rmsnorm_sum", _ptr(residual), _ptr(parts), n_parts, _ptr(g), _code(g, "rmsnorm_sum"), _ptr(out),
                  _code(out, "rmsnorm_sum"), m, n, float(eps), _stream(),
@@ -650,7 +705,7 @@ def gemm_emit_supported(a: torch.Tensor, w, residual: torch.Tensor, g: torch.Ten
 def gemm_accumulate_emit(a: torch.Tensor, w, residual: torch.Tensor, g: torch.Tensor, eps: float) -> Prenormed:
     """residual += a w^T, and the next RMSNorm (scale g, eps) prepared: see Prenormed."""
     w, packed = _weight(w)
-    packed = packed if packed is not None else pack_weight(w)
+    packed = packed if packed is not None else pack_weight(_rows(w))
     _dev("gemm_accumulate_emit", a, w, residual, g)
     m, k = a.shape
     n = w.shape[0]
@@ -686,7 +741,8 @@ def gemm_prenormed(pre: Prenormed, w, epilogue: int) -> torch.Tensor:
     """rmsnorm(residual) w^T from what gemm_accumulate_emit left: epilogue EPI_STORE_BF16,
     EPI_STORE_F32 or EPI_SWIGLU (w in blocks of eight gate and eight up rows)."""
     w, packed = _weight(w)
-    packed = packed if packed is not None else pack_weight(w)
+    tiled_w = _tiled_weight(w, packed)
+    packed = packed if packed is not None else pack_weight(_rows(w))
     _dev("gemm_prenormed", pre.xb, pre.parts, w)
     m, k = pre.xb.shape
     n = w.shape[0]
@@ -702,7 +758,7 @@ def gemm_prenormed(pre: Prenormed, w, epilogue: int) -> torch.Tensor:
         if epilogue != EPI_SWIGLU:
             raise KernelError("gemm_prenormed: the tiled kernel finishes a prepared norm in its SwiGLU epilogue only")
         library.call("bc4g_gemm_mfma_swiglu_scaled", _ptr(pre.xb), _ptr(pre.parts), pre.parts.shape[0], pre.parts.shape[1], pre.eps,
-                     _ptr(w), _ptr(out), m, n, k, _stream(), cost=_tiled_cost(m, n, k, 1))
+                     *tiled_w, _ptr(out), m, n, k, _stream(), cost=_tiled_cost(m, n, k, 1))
         return out
     for r0 in range(0, m, SKINNY_MAX_ROWS):
         rows = min(SKINNY_MAX_ROWS, m - r0)
@@ -734,7 +790,7 @@ def gemm_qkv_rope(x: torch.Tensor, g: Optional[torch.Tensor], eps: float, w,
     and RMSNorm is fused; with ``pre`` (x = pre.xb) the norm was prepared by the product before.
     Returns the rotated queries [M, heads * head_dim]."""
     w, packed = _weight(w)
-    packed = packed if packed is not None else pack_weight(w)
+    packed = packed if packed is not None else pack_weight(_rows(w))
     _dev("gemm_qkv_rope", x, g, w, positions, slot_map, k_cache, v_cache)
     m, k = x.shape
     n = (n_heads + 2 * n_kv_heads) * head_dim
@@ -778,7 +834,7 @@ def gemm_qkv_rope_tiled(x: torch.Tensor, w, table: Optional[torch.Tensor], slot_
     """The q|k|v product of a prompt portion with rotary positions (``table``: rope_table() of the rows' positions;
     None: no rotation) and the cache write in its epilogue (w in the reordered head layout).  Returns the rotated
     queries [M, heads * head_dim]."""
-    w, _ = _weight(w)
+    w, packed = _weight(w)
     _dev("gemm_qkv_rope_tiled", x, w, table, slot_map, k_cache, v_cache)
     m, k = x.shape
     n = (n_heads + 2 * n_kv_heads) * head_dim
@@ -794,7 +850,7 @@ def gemm_qkv_rope_tiled(x: torch.Tensor, w, table: Optional[torch.Tensor], slot_
         _i32("gemm_qkv_rope_tiled", "slot_map", slot_map, m)
         page_tokens = k_cache.shape[2]
     q = torch.empty((m, n_heads * head_dim), dtype=torch.bfloat16, device=x.device)
-    library.call("bc4g_gemm_mfma_qkv", _ptr(x), _ptr(w), _ptr(q), _ptr(table), _ptr(slot_map), _ptr(k_cache), _ptr(v_cache),
+    library.call("bc4g_gemm_mfma_qkv", _ptr(x), *_tiled_weight(w, packed), _ptr(q), _ptr(table), _ptr(slot_map), _ptr(k_cache), _ptr(v_cache),
                  m, n, k, n_heads, n_kv_heads, head_dim, page_tokens, 1 if write_kv else 0, _stream(),
                  cost=_tiled_cost(m, n, k, 2, qkv=True))
     return q

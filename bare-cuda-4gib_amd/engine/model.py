@@ -105,9 +105,11 @@ class Model:
                         raise ConfigError(f"tensor '{name}' was not loaded")
                 mine[local] = t
             b.part.bind(mine, rt)
-        # the tensors as loaded, and what they take on the device once the parts have packed them
-        # (a linear map's weight is kept in two orders, one for each family of kernels)
+        # the tensors as loaded, and what they take on the device once the parts have packed them and what
+        # nobody holds any more has gone (a linear map's weight is kept once, in the order its kernels read)
         self.weight_bytes = sum(t.numel() * t.element_size() for t in placed.values())
+        placed.clear()
+        tensors = mine = None
         self.device_weight_bytes = torch.cuda.memory_allocated(rt.device) - before if cuda else self.weight_bytes
 
     # ---- cache --------------------------------------------------------------

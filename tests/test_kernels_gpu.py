@@ -918,3 +918,66 @@ def test_attention_at_random_batches(ops):
             close(run_mfma(ops, data, window, n_splits, qt, staged=True), want, rtol=2e-2, atol=2e-2, what=what + " staged")
             close(run_mfma(ops, data, window, n_splits, qt), want, rtol=2e-2, atol=2e-2, what=what + " independent")
             close(run_mfma(ops, data, window, n_splits, shared=True), want, rtol=2e-2, atol=2e-2, what=what + " shared")
+
+
+@pytest.mark.parametrize("m,n,k", [(2048, 11264, 2048), (300, 2048, 5632), (2048, 2560, 2048), (96, 2048, 2048), (70, 200, 192),
+                                   (1000, 4096, 4096), (130, 32000, 2048)])
+def test_the_tiled_kernel_reads_the_packed_weight(ops, m, n, k):
+    """A bound weight whose k is whole steps of 64 is held once, packed for the weight-streaming kernel; the tiled
+    kernel reads that copy and gives the bits it gives from the rows -- for every tile form these shapes select, for
+    the store, accumulate and SwiGLU epilogues and with k cut over workgroups -- and the rows are not kept."""
+    torch.manual_seed(n + k)
+    w = (torch.randn(n, k, device=DEV) * 0.05).bfloat16()
+    a = torch.randn(m, k, device=DEV).bfloat16()
+    held = ops.StreamedWeight(w)
+    assert held.packed is not None and not held.holds_rows
+    assert not ops.streams_weights(m, n, k)
+    for dtype in (torch.bfloat16, torch.float32):
+        assert torch.equal(ops.gemm_fast(a, held, dtype), ops.gemm_fast(a, w, dtype))
+    base = torch.randn(m, n, device=DEV)
+    one, two = base.clone(), base.clone()
+    ops.gemm_fast(a, held, accumulate_into=one)
+    ops.gemm_fast(a, w, accumulate_into=two)
+    assert torch.equal(one, two)
+    if n % 16 == 0:
+        assert torch.equal(ops.gemm_swiglu(a, held, True), ops.gemm_swiglu(a, w, True))
+    g = torch.ones(n, device=DEV, dtype=torch.bfloat16)
+    if ops.gemm_parts_supported(a, w, base, g):
+        one, two = base.clone(), base.clone()
+        f1 = ops.gemm_parts_accumulate_norm(a, held, one, g, 1e-5)
+        f2 = ops.gemm_parts_accumulate_norm(a, w, two, g, 1e-5)
+        assert torch.equal(one, two) and torch.equal(f1.tensor, f2.tensor)
+    assert not held.holds_rows
+    assert torch.equal(held.rows, w) and held.holds_rows                 # made from the packed copy when someone asks
+
+
+def test_a_weight_the_tiled_kernel_cannot_read_packed_keeps_its_rows(ops):
+    w = (torch.randn(48, 176, device=DEV) * 0.05).bfloat16()            # k no multiple of 64
+    held = ops.StreamedWeight(w)
+    assert held.packed is not None and held.holds_rows
+    a = torch.randn(100, 176, device=DEV).bfloat16()
+    assert torch.equal(ops.gemm_fast(a, held, torch.float32), ops.gemm_fast(a, w, torch.float32))
+    f32 = ops.StreamedWeight(w.float())
+    assert f32.packed is None and f32.holds_rows
+
+
+@pytest.mark.parametrize("dtypes", [(torch.float32, torch.float32), (torch.bfloat16, torch.float32), (torch.bfloat16, torch.bfloat16)])
+def test_the_plain_product_s_two_tiles_give_the_same_bits(ops, dtypes):
+    """Up to 16 rows the plain float product runs in tiles of 16 x 16 (sixteen times the blocks, for a decode step of
+    the 32-bit path), beyond that in tiles of 64 x 64; every output element is the same sum over k in ascending order
+    in one thread either way, so a row's bits do not depend on how many rows came with it."""
+    ta, tw = dtypes
+    for m, n, k in ((16, 301, 176), (3, 64, 2048), (9, 1000, 88)):
+        torch.manual_seed(m + n + k)
+        a = torch.randn(40, k, device=DEV).to(ta)
+        w = (torch.randn(n, k, device=DEV) * 0.1).to(tw)
+        many = ops.gemm_generic(a, w, torch.float32)                       # 40 rows: the large tile
+        few = ops.gemm_generic(a[:m].contiguous(), w, torch.float32)       # the small one
+        assert torch.equal(few, many[:m])
+        want = a[:m].double() @ w.double().T
+        torch.testing.assert_close(few.double(), want, rtol=1e-4, atol=1e-4 * math.sqrt(k))
+        base = torch.randn(40, n, device=DEV)
+        one, two = base.clone(), base[:m].clone()
+        ops.gemm_generic(a, w, accumulate_into=one)
+        ops.gemm_generic(a[:m].contiguous(), w, accumulate_into=two)
+        assert torch.equal(two, one[:m])
