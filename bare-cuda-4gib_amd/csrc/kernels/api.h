@@ -136,10 +136,11 @@ int bc4g_attention_mfma(const void* qkv, int q_stride, void* out, float* part_o,
 extern "C" {
 // bfloat16 a [m, k] times bfloat16 w [n, k] transposed on the matrix cores, any m.
 // epilogue: 0 store bfloat16; 1 store float32; 2 add into float32; 3 SwiGLU as in bc4g_gemm_skinny.
-// w_packed (here and in the three entry points below) 0: w lies by rows, [n, k].  1: w lies in the order of the
-// weight-streaming kernel (bc4g_gemm_skinny: [ceil(n / 16)][k / 32][64 lanes][8]), so that one copy of a weight
-// serves both kernels; k must then be a multiple of 64 and the operands on 16-byte boundaries.  The sums are the
-// same bits either way.
+// w_packed 1: w lies in the order of the weight-streaming kernel (bc4g_gemm_skinny: [ceil(n / 16)][k / 32][64 lanes][8]),
+// so that one copy of a weight serves both kernels: the kernel with operands straight into LDS reads it (k a multiple
+// of 64, operands on 16-byte boundaries).  0: w lies by rows, [n, k], for the kernel that stages its tiles through
+// registers (any k that is a multiple of 8).  The sums are the same bits either way.  The three entry points below
+// are forms of the first kernel and take the packed weight only.
 int bc4g_gemm_mfma(const void* a, const void* w, int w_packed, void* out, int epilogue, int m, int n, int k, void* stream);
 // The same product with k cut into k_parts equal parts (each a multiple of 64), part p's sums stored as float32 in
 // parts [k_parts, m, n]: for few rows and a long k, where one workgroup per 64 x 64 tile would walk all of k alone.

@@ -473,7 +473,7 @@ struct DirectShape {
 template <int EPI, int WM, int WN, int TM, int TN, int BK, int STAGES, int MINWG>
 __global__ __launch_bounds__(64 * WM * WN, MINWG) void gemm_mfma_direct_kernel(
     const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, void* __restrict__ out, int m, int n, int k, int m_blocks,
-    int n_blocks, const RopeKvArgs ra, const RowScaleArgs rows, const int w_packed) {
+    int n_blocks, const RopeKvArgs ra, const RowScaleArgs rows) {
   typedef DirectShape<WM, WN, TM, TN, BK, STAGES> S;
   constexpr int RA = S::kRowsA, RW = S::kRowsW, RB = S::kRowBytes, NW = S::kWaves;
   constexpr int kGroupRows = 1024 / RB;                    // rows a wave-wide load covers
@@ -491,46 +491,54 @@ __global__ __launch_bounds__(64 * WM * WN, MINWG) void gemm_mfma_direct_kernel(
   // its own, out + y * m * n (the plain store epilogues only: whoever reads them adds the parts up in order)
   const int nk = k / BK / static_cast<int>(gridDim.y);
   const size_t k_first = static_cast<size_t>(blockIdx.y) * nk * RB;       // in bytes of a row
-  // w_packed: the weight comes in the order the weight-streaming kernel reads ([n / 16][k / 32][64 lanes][8]: the
-  // 16 bytes of row r and k 8 c .. 8 c + 7 lie at ((r / 16) * (k / 32) + c / 4) * 1024 + ((c % 4) * 16 + r % 16) * 16),
-  // so that a model keeps every weight once.  A lane still brings the same 16 bytes of the same row to the same
-  // place in LDS; only where they lie in memory differs, and a step of BK moves on by BK / 32 kilobytes.  A
-  // wave-wide load touches whole lines either way: eight rows' 128 bytes by rows, eight segments' 128 bytes
-  // (eight consecutive rows of one segment) packed.
-  constexpr size_t kPackedStep = static_cast<size_t>(BK / 32) * 1024;
   if constexpr (EPI == kStoreF32) out = static_cast<float*>(out) + static_cast<size_t>(blockIdx.y) * m * n;
+  // The weight comes in the order the weight-streaming kernel reads, so that a model keeps every weight once:
+  // [n / 16][k / 32][64 lanes][8] -- blocks of 16 rows x 32 k, 1 KB each, the 16 bytes of row r and k 8 c .. 8 c + 7 at
+  // ((r / 16) * (k / 32) + c / 4) * 1024 + ((c % 4) * 16 + r % 16) * 16 (rows beyond n are zeros).  A wave-wide load
+  // brings one such block, 1 KB of consecutive memory to 1 KB of consecutive LDS, and the weight's part of a stage is
+  // the tile's blocks as they lie in memory, [rows / 16][BK / 32][1 KB]: a fragment read (lane l: row l % 32, k-slot
+  // l / 32) takes 16 consecutive rows' 16 bytes side by side, 256 bytes without a bank conflict, and its address is the
+  // lane's own offset plus a constant for the slice (no key to fold in, as the rows of x need).
+  static_assert(BK % 32 == 0 && RW % 16 == 0, "whole blocks of the packed weight");
+  constexpr int kBlocksK = BK / 32;                              // blocks a row block brings every step
+  constexpr size_t kPackedStep = static_cast<size_t>(kBlocksK) * 1024;
+  static_assert(GW == RW / 16 * kBlocksK, "a wave-wide load of the weight is one block");
+  const long w_row_blocks = (static_cast<long>(n) + 15) / 16;
 
-  // the groups of rows this wave brings every step (a spare turn repeats the last group: the same
-  // bytes to the same place), and which of a row's segments this lane's 16 bytes are
+  // the groups of rows (of x) and the blocks (of w) this wave brings every step (a spare turn repeats the last: the
+  // same bytes to the same place), and which of a row's segments this lane's 16 bytes of x are
   const int lr = (lane * 16) / RB, ls = (lane * 16 % RB) / 16;
   const unsigned char* src[PER];
   unsigned dst[PER];
-  size_t step_bytes[PER];
+  bool piece_of_w[PER];
 #pragma unroll
   for (int i = 0; i < PER; ++i) {
     int g = wave + NW * i;
     if (g >= GA + GW) g = GA + GW - 1;
     const bool of_a = g < GA;
-    const int trow = (of_a ? g : g - GA) * kGroupRows + lr;
-    const int seg = ls ^ slot_key<RB>(trow);
-    long row = (of_a ? m0 : n0) + trow;
-    const long last = (of_a ? m : n) - 1;
-    if (row > last) row = last;
-    if (w_packed && !of_a) {
-      src[i] = reinterpret_cast<const unsigned char*>(w) + (row / 16) * static_cast<size_t>(k / 32) * 1024 +
-               static_cast<size_t>(blockIdx.y) * nk * kPackedStep + (seg / 4) * 1024 + ((seg % 4) * 16 + row % 16) * 16;
-      step_bytes[i] = kPackedStep;
+    if (of_a) {
+      const int trow = g * kGroupRows + lr;
+      const int seg = ls ^ slot_key<RB>(trow);
+      long row = m0 + trow;
+      if (row > m - 1) row = m - 1;
+      src[i] = reinterpret_cast<const unsigned char*>(a + row * k) + k_first + seg * 16;
+      dst[i] = g * 1024;
     } else {
-      src[i] = reinterpret_cast<const unsigned char*>((of_a ? a : w) + row * k) + k_first + seg * 16;
-      step_bytes[i] = RB;
+      const int gw = g - GA;
+      long block = n0 / 16 + gw / kBlocksK;
+      if (block > w_row_blocks - 1) block = w_row_blocks - 1;
+      src[i] = reinterpret_cast<const unsigned char*>(w) +
+               (block * (k / 32) + static_cast<long>(blockIdx.y) * nk * kBlocksK + gw % kBlocksK) * 1024 + lane * 16;
+      dst[i] = RA * RB + gw * 1024;
     }
-    dst[i] = (of_a ? 0 : RA * RB) + (of_a ? g : g - GA) * 1024;
+    piece_of_w[i] = !of_a;                  // (the same in all lanes of the wave)
   }
   auto ask = [&](int step) {
     const unsigned base = lds_base + (step % STAGES) * S::kStageBytes;
+    const size_t at_a = static_cast<size_t>(step) * RB, at_w = static_cast<size_t>(step) * kPackedStep;   // once a step
 #pragma unroll
     for (int i = 0; i < PER; ++i)
-      load_to_lds_16(src[i] + static_cast<size_t>(step) * step_bytes[i], __builtin_amdgcn_readfirstlane(base + dst[i]));
+      load_to_lds_16(src[i] + (piece_of_w[i] ? at_w : at_a), __builtin_amdgcn_readfirstlane(base + dst[i]));
   };
 
   floatx16 acc[TM][TN];
@@ -597,7 +605,7 @@ __global__ __launch_bounds__(64 * WM * WN, MINWG) void gemm_mfma_direct_kernel(
   }
 
   const int frow = lane % 32, fhalf = lane / 32;
-  int aoff[TM], woff[TN], aswz[TM], wswz[TN];
+  int aoff[TM], woff[TN], aswz[TM];
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
     const int r = (wm * TM + i) * 32 + frow;
@@ -606,18 +614,20 @@ __global__ __launch_bounds__(64 * WM * WN, MINWG) void gemm_mfma_direct_kernel(
   }
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
+    // row r's place in its block of 16, in the block row's first block of the stage; k-slot fhalf of a slice's two
     const int r = (wn * TN + j) * 32 + frow;
-    woff[j] = RA * RB + r * RB;
-    wswz[j] = slot_key<RB>(r);
+    woff[j] = RA * RB + (r / 16) * (kBlocksK * 1024) + (r % 16) * 16 + fhalf * 256;
   }
   constexpr int kSlices = BK / 16;
   uint4 fa[2][TM], fw[2][TN];
   auto read_fragments = [&](int set, const unsigned char* stage, int slice) {
     const int s = slice * 2 + fhalf;
+    // the weight's k-slots 2 slice and 2 slice + 1: block (2 slice) / 4 of the row block, 256 bytes a slot in it
+    const int w_slice = (slice / 2) * 1024 + (slice % 2) * 512;
 #pragma unroll
     for (int i = 0; i < TM; ++i) fa[set][i] = *reinterpret_cast<const uint4*>(stage + aoff[i] + ((s ^ aswz[i]) * 16));
 #pragma unroll
-    for (int j = 0; j < TN; ++j) fw[set][j] = *reinterpret_cast<const uint4*>(stage + woff[j] + ((s ^ wswz[j]) * 16));
+    for (int j = 0; j < TN; ++j) fw[set][j] = *reinterpret_cast<const uint4*>(stage + woff[j] + w_slice);
   };
 
   for (int t = 0; t < nk; ++t) {
@@ -668,7 +678,7 @@ __global__ __launch_bounds__(64 * WM * WN, MINWG) void gemm_mfma_direct_kernel(
 
 template <int EPI, int WM, int WN, int TM, int TN, int BK, int STAGES, int MINWG>
 int launch_direct(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, int k, hipStream_t s, const RopeKvArgs& ra,
-                  int k_parts = 1, const RowScaleArgs& rows = RowScaleArgs{}, int w_packed = 0) {
+                  int k_parts = 1, const RowScaleArgs& rows = RowScaleArgs{}) {
   typedef DirectShape<WM, WN, TM, TN, BK, STAGES> S;
   auto kernel = gemm_mfma_direct_kernel<EPI, WM, WN, TM, TN, BK, STAGES, MINWG>;
   static bool raised = false;   // per instantiation: allow more than the default dynamic LDS
@@ -680,7 +690,7 @@ int launch_direct(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, i
   }
   const long m_blocks = (m + S::kRowsA - 1) / S::kRowsA, n_blocks = (n + S::kRowsW - 1) / S::kRowsW;
   kernel<<<dim3(static_cast<unsigned>(m_blocks * n_blocks), static_cast<unsigned>(k_parts)), dim3(S::kThreads), S::kLdsBytes, s>>>(
-      ap, wp, out, m, n, k, static_cast<int>(m_blocks), static_cast<int>(n_blocks), ra, rows, w_packed);
+      ap, wp, out, m, n, k, static_cast<int>(m_blocks), static_cast<int>(n_blocks), ra, rows);
   return 0;
 }
 
@@ -726,14 +736,14 @@ int direct_form(int m, int n, int k, bool long_epilogue) {
 
 template <int EPI>
 int launch_direct_form(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, int k, hipStream_t s,
-                       const RopeKvArgs& ra = RopeKvArgs{}, const RowScaleArgs& rows = RowScaleArgs{}, int w_packed = 0) {
+                       const RopeKvArgs& ra = RopeKvArgs{}, const RowScaleArgs& rows = RowScaleArgs{}) {
   switch (direct_form(m, n, k, EPI == kRopeKvBf16)) {
-    case 0: return launch_direct<EPI, 4, 4, 2, 2, 64, 2, 1>(ap, wp, out, m, n, k, s, ra, 1, rows, w_packed);
-    case 1: return launch_direct<EPI, 4, 2, 2, 3, 64, 2, 1>(ap, wp, out, m, n, k, s, ra, 1, rows, w_packed);
-    case 2: return launch_direct<EPI, 4, 2, 2, 2, 64, 3, 1>(ap, wp, out, m, n, k, s, ra, 1, rows, w_packed);
-    case 3: return launch_direct<EPI, 2, 4, 2, 1, 64, 4, 1>(ap, wp, out, m, n, k, s, ra, 1, rows, w_packed);
-    case 5: return launch_direct<EPI, 2, 2, 2, 1, 64, 2, 4>(ap, wp, out, m, n, k, s, ra, 1, rows, w_packed);
-    default: return launch_direct<EPI, 2, 2, 1, 1, 64, 4, 2>(ap, wp, out, m, n, k, s, ra, 1, rows, w_packed);
+    case 0: return launch_direct<EPI, 4, 4, 2, 2, 64, 2, 1>(ap, wp, out, m, n, k, s, ra, 1, rows);
+    case 1: return launch_direct<EPI, 4, 2, 2, 3, 64, 2, 1>(ap, wp, out, m, n, k, s, ra, 1, rows);
+    case 2: return launch_direct<EPI, 4, 2, 2, 2, 64, 3, 1>(ap, wp, out, m, n, k, s, ra, 1, rows);
+    case 3: return launch_direct<EPI, 2, 4, 2, 1, 64, 4, 1>(ap, wp, out, m, n, k, s, ra, 1, rows);
+    case 5: return launch_direct<EPI, 2, 2, 2, 1, 64, 2, 4>(ap, wp, out, m, n, k, s, ra, 1, rows);
+    default: return launch_direct<EPI, 2, 2, 1, 1, 64, 4, 2>(ap, wp, out, m, n, k, s, ra, 1, rows);
   }
 }
 
@@ -742,10 +752,16 @@ bool direct_operands(const void* ap, const void* wp, int k) {
   return k % 64 == 0 && reinterpret_cast<uintptr_t>(ap) % 16 == 0 && reinterpret_cast<uintptr_t>(wp) % 16 == 0;
 }
 
+// w_packed: the weight in the weight-streaming kernel's order, for the kernel with operands straight into LDS (k in
+// whole steps of 64, operands on 16-byte boundaries); else the weight by rows, for the kernel that stages its tiles
+// through registers (any k that is a multiple of 8).
 template <int EPI>
 int launch_tiled(const bf16_t* ap, const bf16_t* wp, void* out, int m, int n, int k, hipStream_t s, int w_packed) {
-  if (direct_operands(ap, wp, k)) return launch_direct_form<EPI>(ap, wp, out, m, n, k, s, RopeKvArgs{}, RowScaleArgs{}, w_packed);
-  if (w_packed) return fail("gemm_mfma: a packed weight needs k in whole steps of 64 and operands on 16-byte boundaries (K=%d)", k);
+  if (w_packed) {
+    if (!direct_operands(ap, wp, k))
+      return fail("gemm_mfma: a packed weight needs k in whole steps of 64 and operands on 16-byte boundaries (K=%d)", k);
+    return launch_direct_form<EPI>(ap, wp, out, m, n, k, s);
+  }
   const long m_blocks = (m + kBM - 1) / kBM, n_blocks = (n + kBN - 1) / kBN;
   gemm_mfma_staged_kernel<EPI><<<dim3(static_cast<unsigned>(m_blocks * n_blocks)), dim3(256), 0, s>>>(
       ap, wp, out, m, n, k, static_cast<int>(m_blocks), static_cast<int>(n_blocks));
@@ -783,28 +799,28 @@ extern "C" int bc4g_gemm_mfma(const void* a, const void* w, int w_packed, void* 
 
 extern "C" int bc4g_gemm_mfma_swiglu_scaled(const void* a, const float* ssq_parts, int ssq_blocks, int ssq_stride, float eps,
                                             const void* w, int w_packed, void* out, int m, int n, int k, void* stream) {
-  BC4G_REQUIRE(m >= 0 && n > 0 && n % 16 == 0 && k > 0 && direct_operands(a, w, k),
-               "gemm_mfma_swiglu_scaled: K=%d must be a multiple of 64, N=%d one of 16 and the operands on 16-byte boundaries (M=%d)", k, n, m);
+  BC4G_REQUIRE(m >= 0 && n > 0 && n % 16 == 0 && k > 0 && direct_operands(a, w, k) && w_packed,
+               "gemm_mfma_swiglu_scaled: K=%d must be a multiple of 64, N=%d one of 16, the weight packed and the operands on 16-byte boundaries (M=%d)", k, n, m);
   BC4G_REQUIRE(ssq_parts != nullptr && ssq_blocks > 0 && ssq_stride >= m && eps >= 0.f,
                "gemm_mfma_swiglu_scaled: the sums of squares need %d parts of at least %d rows, and eps must not be negative", ssq_blocks, m);
   if (m == 0) return 0;
   BC4G_REQUIRE(((m + 63L) / 64) * ((n + 63L) / 64) <= 2147483647L, "gemm_mfma_swiglu_scaled: too many tiles");
   if (int e = launch_direct_form<kSwigluScaledBf16>(static_cast<const bf16_t*>(a), static_cast<const bf16_t*>(w), out, m, n, k,
                                                      static_cast<hipStream_t>(stream), RopeKvArgs{},
-                                                     RowScaleArgs{ssq_parts, ssq_blocks, ssq_stride, eps}, w_packed))
+                                                     RowScaleArgs{ssq_parts, ssq_blocks, ssq_stride, eps}))
     return e;
   return check_launch("gemm_mfma_swiglu_scaled");
 }
 
 extern "C" int bc4g_gemm_mfma_parts(const void* a, const void* w, int w_packed, float* parts, int m, int n, int k, int k_parts,
                                     void* stream) {
-  BC4G_REQUIRE(m > 0 && n > 0 && k > 0 && k_parts >= 1 && k_parts <= 16 && k % (64 * k_parts) == 0 && direct_operands(a, w, k),
-               "gemm_mfma_parts: K=%d must be %d times a multiple of 64 and the operands on 16-byte boundaries (M=%d N=%d)", k,
-               k_parts, m, n);
+  BC4G_REQUIRE(m > 0 && n > 0 && k > 0 && k_parts >= 1 && k_parts <= 16 && k % (64 * k_parts) == 0 && direct_operands(a, w, k) &&
+                   w_packed,
+               "gemm_mfma_parts: K=%d must be %d times a multiple of 64, the weight packed and the operands on 16-byte boundaries "
+               "(M=%d N=%d)", k, k_parts, m, n);
   BC4G_REQUIRE(((m + 63L) / 64) * ((n + 63L) / 64) <= 2147483647L, "gemm_mfma_parts: too many tiles");
   if (int e = launch_direct<kStoreF32, 2, 2, 1, 1, 64, 4, 2>(static_cast<const bf16_t*>(a), static_cast<const bf16_t*>(w), parts, m, n,
-                                                               k, static_cast<hipStream_t>(stream), RopeKvArgs{}, k_parts,
-                                                               RowScaleArgs{}, w_packed))
+                                                               k, static_cast<hipStream_t>(stream), RopeKvArgs{}, k_parts))
     return e;
   return check_launch("gemm_mfma_parts");
 }
@@ -812,8 +828,8 @@ extern "C" int bc4g_gemm_mfma_parts(const void* a, const void* w, int w_packed, 
 extern "C" int bc4g_gemm_mfma_qkv(const void* a, const void* w, int w_packed, void* out, const float* table, const int32_t* slot_map,
                                   void* k_cache, void* v_cache, int m, int n, int k, int n_heads, int n_kv_heads,
                                   int head_dim, int page_tokens, int write_kv, void* stream) {
-  BC4G_REQUIRE(m > 0 && n > 0 && k > 0 && direct_operands(a, w, k),
-               "gemm_mfma_qkv: K=%d must be a multiple of 64 and the operands on 16-byte boundaries (M=%d N=%d)", k, m, n);
+  BC4G_REQUIRE(m > 0 && n > 0 && k > 0 && direct_operands(a, w, k) && w_packed,
+               "gemm_mfma_qkv: K=%d must be a multiple of 64, the weight packed and the operands on 16-byte boundaries (M=%d N=%d)", k, m, n);
   BC4G_REQUIRE(n_heads > 0 && n_kv_heads > 0 && head_dim > 0 && head_dim % 16 == 0 &&
                    static_cast<long>(n_heads + 2 * n_kv_heads) * head_dim == n,
                "gemm_mfma_qkv: %d + 2 x %d heads of %d (a multiple of 16) are not %d columns", n_heads, n_kv_heads, head_dim, n);
@@ -831,7 +847,7 @@ extern "C" int bc4g_gemm_mfma_qkv(const void* a, const void* w, int w_packed, vo
   ra.write_kv = write_kv ? 1 : 0;
   ra.fragment_order = write_kv && cache_fragment_order(true, head_dim, page_tokens) ? 1 : 0;
   if (int e = launch_direct_form<kRopeKvBf16>(static_cast<const bf16_t*>(a), static_cast<const bf16_t*>(w), out, m, n, k,
-                                              static_cast<hipStream_t>(stream), ra, RowScaleArgs{}, w_packed))
+                                              static_cast<hipStream_t>(stream), ra))
     return e;
   return check_launch("gemm_mfma_qkv");
 }

@@ -401,10 +401,13 @@ def _rows(w) -> torch.Tensor:
     return w.rows if isinstance(w, StreamedWeight) else w
 
 
-def _tiled_weight(w, packed):
-    """(address, 1 if packed else 0) of a weight for the tiled kernel: the packed copy where that kernel takes it
-    (a bound weight, k in whole steps of 64), else the rows."""
-    if isinstance(w, StreamedWeight) and packed is not None and w.shape[1] % 64 == 0:
+def _tiled_weight(w, packed, a: Optional[torch.Tensor] = None):
+    """(address, 1 if packed else 0) of a weight for the tiled kernel: the packed copy for the kernel with operands
+    straight into LDS (k in whole steps of 64, x on a 16-byte boundary; a bare tensor is packed for the call: tests
+    only), else the rows for the kernel that stages its tiles through registers."""
+    if w.shape[1] % 64 == 0 and w.dtype == torch.bfloat16 and (a is None or a.data_ptr() % 16 == 0):
+        if packed is None:
+            packed = pack_weight(_rows(w))        # (given back to the allocator in stream order, after the launch)
         return packed.data_ptr(), 1
     return _rows(w).data_ptr(), 0
 
@@ -566,7 +569,7 @@ def gemm_fast(a: torch.Tensor, w, out_dtype=None,
             library.call("bc4g_gemm_skinny", _ptr(a[r0:]), _ptr(packed), _ptr(out[r0:]), epi, rows, n, k, _stream(),
                          cost=_skinny_cost(rows, n, k, 2, out_bytes))
     else:
-        library.call("bc4g_gemm_mfma", _ptr(a), *_tiled_weight(w, packed), _ptr(out), epi, m, n, k, _stream(),
+        library.call("bc4g_gemm_mfma", _ptr(a), *_tiled_weight(w, packed, a), _ptr(out), epi, m, n, k, _stream(),
                      cost=_tiled_cost(m, n, k, out_bytes))
     return out
 
@@ -630,7 +633,7 @@ def gemm_swiglu(a: torch.Tensor, w_gate_up, interleaved: bool = False) -> torch.
                 library.call("bc4g_gemm_skinny", _ptr(a[r0:]), _ptr(packed), _ptr(out[r0:]), EPI_SWIGLU, part, n, k,
                              _stream(), cost=_skinny_cost(part, n, k, 2, 1))
         else:
-            library.call("bc4g_gemm_mfma", _ptr(a), *_tiled_weight(rows, packed), _ptr(out), EPI_SWIGLU, m, n, k, _stream(),
+            library.call("bc4g_gemm_mfma", _ptr(a), *_tiled_weight(rows, packed, a), _ptr(out), EPI_SWIGLU, m, n, k, _stream(),
                          cost=_tiled_cost(m, n, k, 1))
         return out
     gu = gemm_fast(a, w_gate_up, a.dtype)
