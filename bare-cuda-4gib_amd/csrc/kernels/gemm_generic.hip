@@ -35,18 +35,32 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const TA* __restrict_
 #pragma unroll
     for (int j = 0; j < kPerThread; ++j) acc[i][j] = 0.f;
 
-  for (int k0 = 0; k0 < k; k0 += kStepK) {
-    // kTile rows x kStepK k elements per operand, the same number a thread; k fastest for coalescing.
+  // A step's operands are asked for a step ahead, into registers, so that the way from memory lies beside the step
+  // before's arithmetic instead of before its own: kTile rows x kStepK k elements per operand, the same number a
+  // thread; k fastest for coalescing.
+  constexpr int kLoads = kTile * kStepK / 256;
+  float ar[kLoads], wr[kLoads];
+  auto fetch = [&](int k0) {
 #pragma unroll
-    for (int r = 0; r < kTile * kStepK / 256; ++r) {
+    for (int r = 0; r < kLoads; ++r) {
       const int e = threadIdx.x + r * 256;
       const int kk = e % kStepK, row = e / kStepK;
       const long gm = m0 + row, gn = n0 + row;
       const int gk = k0 + kk;
-      as[kk][row] = (gm < m && gk < k) ? to_float(a[gm * k + gk]) : 0.f;
-      ws[kk][row] = (gn < n && gk < k) ? to_float(w[gn * k + gk]) : 0.f;
+      ar[r] = (gm < m && gk < k) ? to_float(a[gm * k + gk]) : 0.f;
+      wr[r] = (gn < n && gk < k) ? to_float(w[gn * k + gk]) : 0.f;
+    }
+  };
+  fetch(0);
+  for (int k0 = 0; k0 < k; k0 += kStepK) {
+#pragma unroll
+    for (int r = 0; r < kLoads; ++r) {
+      const int e = threadIdx.x + r * 256;
+      as[e % kStepK][e / kStepK] = ar[r];
+      ws[e % kStepK][e / kStepK] = wr[r];
     }
     __syncthreads();
+    if (k0 + kStepK < k) fetch(k0 + kStepK);
 #pragma unroll
     for (int kk = 0; kk < kStepK; ++kk) {
       float av[kPerThread], wv[kPerThread];

@@ -108,3 +108,26 @@ def test_llm_bench_program(tmp_path):
     assert float(by_name["argmax"][10]) == 1.0
     assert run("--prompt", "1,2", "--prompt-len", "4").returncode == 1          # two prompt sources
     assert run("--prompt-len", "4", "--tokens", "1").returncode == 1            # TPOT needs two tokens
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_llm_batch_check_program(tmp_path, dtype):
+    """The program itself on a tiny model with random prompts: eight prompts (the longest the model's positions hold),
+    four decoding at once; in 32-bit every request's ids are identical alone and batched, in bfloat16 a split may only
+    be a near-tie."""
+    import helpers
+    folder = helpers.make_model_dir(tmp_path, "C", dtype, variant="spread")
+    prog = os.path.join(helpers.ROOT, "bin", "llm-batch-check")
+    proc = subprocess.run([sys.executable, prog, "--model", folder, "--tokens", "24", "--batch", "4", "--dtype", dtype,
+                           "--page-tokens", "16"], capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stdout[-2000:] + proc.stderr[-2000:]
+    lines = proc.stdout.strip().splitlines()
+    assert lines[-1] == "PASS: batched decode agrees with decoding alone"
+    assert "8 prompts of 6-301 tokens, 24 new tokens each, 4 decoding at once" in lines[1]
+    verdicts = [l for l in lines if l.startswith("prompt ")]
+    assert len(verdicts) == 8
+    if dtype == "float32":
+        assert all("match, 24 ids identical" in l for l in verdicts), proc.stdout
+    bad = subprocess.run([sys.executable, prog, "--model", str(tmp_path / "none")], capture_output=True, text=True, timeout=300)
+    assert bad.returncode != 0 and "config.json" in bad.stderr
