@@ -433,7 +433,8 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_staged_kernel(
 // slower than two; with fewer tiles than CUs a step is as long as a load takes, and four stages of a
 // 64 x 64 tile halve that: 512 x 2048 x 5632 48 -> 28 us), raising the waves' priority around the MFMAs, 128 x 64 parts for a wave with half the waves.
 //
-// A tile's rows lie in LDS without padding, BK * 2 bytes each; the 16-byte segment s of row r lies in
+// The weight comes packed (the weight-streaming kernel's order) and its blocks are copied as they are: see the
+// kernel.  The rows of x lie in LDS without padding, BK * 2 bytes each; the 16-byte segment s of row r lies in
 // slot s ^ key(r) of its row, key(r) = (r / 2) % 8 for rows of 128 bytes and r % 16 for rows of 256.  A
 // fragment read is served sixteen lanes (rows r .. r + 15, one segment) at a time from 64 banks of
 // four bytes: two rows of 128 bytes share the banks' span, so the eight rows of one parity must lie
@@ -443,7 +444,8 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_staged_kernel(
 //
 // WM x WN waves take TM x TN MFMA blocks of 32 x 32 each.  An output element is added up over k in
 // ascending order, as in the form above: the same bits whichever form the shape selects.
-// k must be a multiple of BK; rows beyond m or n are read from the last row and not stored.
+// k must be a multiple of BK; rows beyond m are read from the last row, blocks beyond n from the last block, and
+// not stored.
 template <int PER, int MAX>
 __device__ inline void wait_for_stage(int later) {
   if constexpr (MAX == 0) {
