@@ -38,7 +38,8 @@ class Executor:
     page_tokens: tokens per cache page.  num_pages: pages in each group's
     pool.  max_requests: requests that can be live at once.  max_tokens: the
     most tokens one request may hold.  max_batch_tokens: the most rows one
-    step may bring (0: no limit but memory).
+    step may bring (0: no limit but memory).  max_tokens beyond the positions the model's configuration
+    gives is refused.
 
     What a part may add to a step (both optional; the executor knows no part by name):
       prepare_step(batch: HostBatch) -> (arrays, notes)   called once a step before anything is launched,
@@ -64,10 +65,13 @@ class Executor:
 
     def __init__(self, model: Model, *, num_pages: int, max_requests: int, max_tokens: int,
                  page_tokens: int = 64, max_batch_tokens: int = 0, poison: bool = False,
-                 use_graphs: bool = True, graph_max_batch: int = 256):
+                 use_graphs: bool = True, graph_max_batch: int = 256, beyond_positions: bool = False):
         if model.rt is None:
             raise EngineError("executor: the model has no weights bound")
-        if max_tokens > model.max_seq_len:       # (reference: Model::load, engine/src/model.cpp:429-433)
+        # (reference: Model::load, engine/src/model.cpp:429-433.  ``beyond_positions``: a program that replays given
+        # ids and serves nobody may say that it wants positions the configuration does not promise -- nothing here
+        # keeps a table of them -- and takes the answers for what they are.)
+        if max_tokens > model.max_seq_len and not beyond_positions:
             raise EngineError(f"executor: max_tokens {max_tokens} is beyond the model's {model.max_seq_len} positions")
         self.model = model
         self.rt = model.rt

@@ -168,7 +168,7 @@ def run_gemm(m, n, k, runs=20):
     from bare_cuda_4gib_amd.csrc import ops
     gen = torch.Generator(device="cuda").manual_seed(4)
     a = torch.randn(m, k, device="cuda", generator=gen).bfloat16()
-    w = (torch.randn(n, k, device="cuda", generator=gen) * 0.02).bfloat16()
+    w = ops.StreamedWeight((torch.randn(n, k, device="cuda", generator=gen) * 0.02).bfloat16())   # as a model holds it
     for _ in range(3):
         ops.gemm_fast(a, w, torch.bfloat16)
     start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)

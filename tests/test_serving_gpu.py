@@ -196,3 +196,5 @@ def test_more_tokens_than_the_model_has_positions_are_refused(folders):
     Executor(model, num_pages=2, max_requests=1, max_tokens=128, page_tokens=64)
     with pytest.raises(EngineError, match="beyond the model's 128 positions"):
         Executor(model, num_pages=3, max_requests=1, max_tokens=129, page_tokens=64)
+    # the replay program alone may ask for more (it feeds given ids and serves nobody)
+    Executor(model, num_pages=3, max_requests=1, max_tokens=129, page_tokens=64, beyond_positions=True)
