@@ -2,7 +2,10 @@
 
 Objects go to ``_build/`` under this folder.  Sources are compiled in parallel
 and a line is printed as each one finishes, so a first call that has to
-compile shows that it is alive.
+compile shows that it is alive.  Where this folder cannot be written and holds
+no library built from the sources beside it (a checkout that belongs to someone
+else), library and objects go to a folder of the user's own under the system's
+temporary folder instead.
 """
 from __future__ import annotations
 
@@ -12,6 +15,7 @@ import os
 import shutil
 import subprocess
 import sys
+import tempfile
 import time
 from typing import List
 
@@ -19,7 +23,7 @@ from ..errors import KernelError
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 SRC_DIR = os.path.join(HERE, "kernels")
-BUILD_DIR = os.path.join(HERE, "_build")
+BUILD_DIR = os.path.join(HERE, "_build")          # (both moved by _settle() below where HERE cannot be written)
 LIB_PATH = os.path.join(HERE, "libbc4g.so")
 
 ARCH = "gfx950"
@@ -59,12 +63,12 @@ def is_built() -> bool:
 _MARKER = b"bc4g-sources-digest:"
 
 
-def built_digest() -> str:
+def built_digest(path: str = "") -> str:
     """The digest of the sources the library file was built from, read from the file itself (it
     carries it behind a marker), without loading it; empty if there is none."""
     import mmap
     try:
-        with open(LIB_PATH, "rb") as fh, mmap.mmap(fh.fileno(), 0, access=mmap.ACCESS_READ) as mm:
+        with open(path or LIB_PATH, "rb") as fh, mmap.mmap(fh.fileno(), 0, access=mmap.ACCESS_READ) as mm:
             at = mm.find(_MARKER)
             if at < 0:
                 return ""
@@ -72,6 +76,24 @@ def built_digest() -> str:
             return raw.split(b"\0", 1)[0].decode("ascii", "replace")
     except (OSError, ValueError):
         return ""
+
+
+def _settle() -> None:
+    """Where the library lives: beside this file, if that folder can be written or already holds a library of
+    these sources; else in a folder that belongs to this user alone (a library that someone else could have put
+    there is not loaded)."""
+    global BUILD_DIR, LIB_PATH
+    if os.access(HERE, os.W_OK) or built_digest(LIB_PATH) == sources_digest():
+        return
+    home = os.path.join(tempfile.gettempdir(), f"bc4g-{os.getuid()}")
+    os.makedirs(home, mode=0o700, exist_ok=True)
+    st = os.stat(home)
+    if st.st_uid != os.getuid() or st.st_mode & 0o022:
+        raise KernelError(f"{HERE} cannot be written, and {home} is not this user's own folder: nowhere to build")
+    BUILD_DIR, LIB_PATH = os.path.join(home, "_build"), os.path.join(home, "libbc4g.so")
+
+
+_settle()
 
 
 def is_stale() -> bool:

@@ -30,3 +30,31 @@ def test_a_stale_library_is_rebuilt_or_refused(monkeypatch):
     with pytest.raises(KernelError, match="digest"):                        # "rebuilt" (here: not really), checked again
         library.load()
     assert calls == [1]
+
+
+def test_where_the_library_lives(monkeypatch, tmp_path):
+    """Beside its sources, where that folder can be written or already holds a library of these sources; else in a
+    folder that belongs to this user alone under the temporary folder -- and never in one that others can write."""
+    import os
+    import tempfile
+    in_tree = (os.path.join(build.HERE, "_build"), os.path.join(build.HERE, "libbc4g.so"))
+    monkeypatch.setattr(build, "BUILD_DIR", in_tree[0])
+    monkeypatch.setattr(build, "LIB_PATH", in_tree[1])
+    monkeypatch.setattr(tempfile, "tempdir", str(tmp_path))
+    monkeypatch.setattr(os, "access", lambda path, mode: True)
+    build._settle()
+    assert (build.BUILD_DIR, build.LIB_PATH) == in_tree
+    monkeypatch.setattr(os, "access", lambda path, mode: False)          # a checkout that belongs to someone else
+    monkeypatch.setattr(build, "built_digest", lambda path="": build.sources_digest())
+    build._settle()                                                      # ... with a library of these sources
+    assert (build.BUILD_DIR, build.LIB_PATH) == in_tree
+    monkeypatch.setattr(build, "built_digest", lambda path="": "")       # ... without
+    build._settle()
+    home = os.path.join(str(tmp_path), f"bc4g-{os.getuid()}")
+    assert build.LIB_PATH == os.path.join(home, "libbc4g.so") and build.BUILD_DIR == os.path.join(home, "_build")
+    assert os.stat(home).st_mode & 0o777 == 0o700
+    monkeypatch.setattr(build, "BUILD_DIR", in_tree[0])
+    monkeypatch.setattr(build, "LIB_PATH", in_tree[1])
+    os.chmod(home, 0o777)
+    with pytest.raises(KernelError, match="nowhere to build"):
+        build._settle()
