@@ -321,7 +321,9 @@ class Executor:
         torch.cuda.synchronize()
         ctx.made.clear()                             # what layers share is made again inside the graph
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
+        # (thread_local: what another thread does on the device meanwhile -- the caller of an engine whose worker
+        # runs this -- neither fails there nor spoils the capture)
+        with torch.cuda.graph(graph, capture_error_mode="thread_local"):
             logits = self.model.forward(ctx)
         ring = []
         for _ in range(4):

@@ -45,7 +45,7 @@ def drain(engine, n_requests):
     out, finish = {}, {}
     while len(finish) < n_requests:
         events = engine.poll()
-        assert events or not engine.scheduler.idle(), "the engine went idle before every request had finished"
+        assert events or not engine.idle(), "the engine went idle before every request had finished"
         for id, tok, idx, fin in events:
             if tok >= 0:
                 assert idx == len(out.setdefault(id, []))
@@ -198,3 +198,92 @@ def test_more_tokens_than_the_model_has_positions_are_refused(folders):
         Executor(model, num_pages=3, max_requests=1, max_tokens=129, page_tokens=64)
     # the replay program alone may ask for more (it feeds given ids and serves nobody)
     Executor(model, num_pages=3, max_requests=1, max_tokens=129, page_tokens=64, beyond_positions=True)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_worker_thread_serves_while_the_callers_do_other_things(folders, dtype):
+    """With a worker of its own the engine is the reference's (engine/src/async_engine.cpp:22-205): any thread
+    submits, tokens are generated while nobody polls, poll waits up to its time-out and no longer, a cancelled
+    request gets its last event and gives its pages back, a failure ends every live request with 'error', and
+    stop joins the worker.  The tokens are those of the engine whose turns the polling thread runs."""
+    import threading
+    import time
+    from bare_cuda_4gib_amd.engine import Engine, generate_batch
+    folder = folders("A", dtype, "spread")
+    vocab = helpers.TINY_A["vocab_size"]
+    prompts = [helpers.random_ids(n, vocab, 70 + n) for n in (3, 40, 17, 64, 9)]
+    args = dict(max_tokens=128, max_seqs=3, dtype=dtype, page_tokens=16, prefill_chunk=32, max_batch_tokens=96)
+    inline = generate_batch(Engine(folder, **args), prompts, 20)
+
+    engine = Engine(folder, worker=True, **args)
+    t0 = time.monotonic()
+    assert engine.poll(60) == [] and 0.05 <= time.monotonic() - t0 < 1.0        # nothing to wait for but the time
+    with engine._in:                                   # all five before the worker's next turn, as before the first poll
+        assert [engine.submit(i, p, 20) for i, p in enumerate(prompts)] == [("ok", "")] * 5
+    assert engine.submit(1, prompts[1], 20)[0] == "invalid"                      # id in use
+    deadline = time.monotonic() + 60
+    while engine._live:                                                          # nobody polls; the worker goes on
+        assert time.monotonic() < deadline, "the worker does not generate by itself"
+        time.sleep(0.01)
+    assert len(engine._outbox) >= 5 * 20
+    out = {i: [] for i in range(5)}
+    finish = {}
+    while len(finish) < 5:
+        events = engine.poll(1000)
+        assert events, "a second without an event"
+        for id, tok, idx, fin in events:
+            if tok >= 0:
+                assert idx == len(out[id])
+                out[id].append(tok)
+            if fin:
+                finish[id] = fin
+    assert [out[i] for i in range(5)] == inline and set(finish.values()) == {"length"}
+    assert engine.idle() and engine.stats()["kv_pages_used"] == 0 and engine.stats()["waiting"] == 0
+
+    # a request from another thread, cancelled while it runs
+    results = []
+    other = threading.Thread(target=lambda: results.append(engine.submit(7, prompts[2], 100)))
+    other.start()
+    other.join()
+    assert results == [("ok", "")]
+    first = engine.poll(5000)
+    assert first and first[0][:1] == (7,) and first[0][3] == ""
+    engine.cancel(7)
+    engine.cancel(99)                                                             # no such request: nothing happens
+    seen = []
+    while not any(e[3] for e in seen):
+        got = engine.poll(5000)
+        assert got, "the cancellation never arrived"
+        seen += got
+    assert seen[-1] == (7, -1, -1, "cancelled") and len(seen) < 100
+    while engine.stats()["kv_pages_used"]:
+        assert time.monotonic() < deadline + 60
+        time.sleep(0.01)
+    assert engine.idle()
+
+    # a failure on the worker's thread
+    assert engine.submit(8, prompts[3], 60)[0] == "ok" and engine.submit(9, prompts[0], 60)[0] == "ok"
+    engine._fail_for_test("injected")
+    seen = []
+    while sum(1 for e in seen if e[3] == "error") < 2:
+        got = engine.poll(5000)
+        assert got, "the failure must surface"
+        seen += got
+    assert [e[:3] for e in seen if e[3] == "error"] == [(8, -1, -1), (9, -1, -1)]
+    assert not engine.healthy and "injected" in engine.failure
+    assert engine.submit(10, [1], 1) == ("unavailable", "engine failed: injected")
+    engine._thread.join(10)
+    assert not engine._thread.is_alive()                                          # the worker ends with the failure
+    engine.stop()
+    assert engine.poll(10_000) == []                                              # stopped: no waiting
+
+    # stop with work in flight
+    engine = Engine(folder, worker=True, **args)
+    assert engine.submit(1, prompts[3], 60)[0] == "ok"
+    assert engine.poll(5000)
+    engine.stop()
+    assert not engine._thread.is_alive() and engine.submit(2, [1], 1) == ("unavailable", "engine is stopped")
+    engine.poll(0)
+    t0 = time.monotonic()
+    assert engine.poll(10_000) == [] and time.monotonic() - t0 < 1.0
+    assert engine.executor.cache.pages_in_use() == 0
