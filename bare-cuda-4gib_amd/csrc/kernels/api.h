@@ -90,6 +90,13 @@ int bc4g_argmax(const float* logits, int32_t* out, float* part_v, int32_t* part_
 // vocabulary in order (engine/src/sampler.cpp:39-61); temperature <= 0 gives the argmax.
 int bc4g_sample(const float* logits, const float* temperature, const double* u, int32_t* out,
                 int n_rows, int vocab, void* stream);
+
+// out[rows[i]] = the token drawn for logits row rows[i] with top_k[i] and top_p[i]: the tokens by falling weight
+// exp((l - max) / temperature[i]), lower id first among equals; the top_k likeliest (0 or >= vocab: all); of those
+// the fewest whose sum reaches top_p of their total (>= 1: all); the first at which u[i] of the kept mass is passed
+// (engine/src/sampler.cpp:63-104).  Not for a row with neither limit: bc4g_sample walks those in the order of the ids.
+int bc4g_sample_filtered(const float* logits, const int32_t* rows, const float* temperature, const double* u,
+                         const int32_t* top_k, const double* top_p, int32_t* out, int n, int vocab, void* stream);
 }
 
 extern "C" {

@@ -29,6 +29,7 @@ _SIGNATURES = {
     "bc4g_attention_generic": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _P],
     "bc4g_argmax": [_P, _P, _P, _P, _I, _I, _P],
     "bc4g_sample": [_P, _P, _P, _P, _I, _I, _P],
+    "bc4g_sample_filtered": [_P, _P, _P, _P, _P, _P, _P, _I, _I, _P],
     "bc4g_argmax_static": [_P, _P, _I, _I, _P],
     "bc4g_probe_read": [_P, c_long, _P, _I, _P],
     "bc4g_probe_mfma": [_P, _I, _P, _I, _P],

@@ -320,6 +320,30 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, u: torch.Tensor) -> 
     return out
 
 
+def sample_filtered(logits: torch.Tensor, out: torch.Tensor, rows: torch.Tensor, temperature: torch.Tensor,
+                    u: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor) -> torch.Tensor:
+    """Top-k / top-p draws for some rows of the logits: for each i, the token of logits row rows[i] by the
+    reference's law for filtered sampling (weights exp((l - max) / T), the tokens by falling weight with the
+    lower id first among equals, the top_k[i] likeliest, of those the fewest that reach top_p[i] of their
+    total, the first at which u[i] of the kept mass is passed) goes into out[rows[i]].  top_k 0 or beyond the
+    vocabulary and top_p 1 are no limits -- but a row with neither limit is not for this kernel: the law
+    without filters walks the tokens in the order of their ids (sample)."""
+    _dev("sample_filtered", logits, out, rows, temperature, u, top_k, top_p)
+    n = rows.numel()
+    if logits.dtype != torch.float32 or logits.dim() != 2:
+        raise KernelError("sample_filtered: logits must be float32 [rows, vocab]")
+    if out.dtype != torch.int32 or out.numel() != logits.shape[0]:
+        raise KernelError("sample_filtered: out must be int32, one for every logits row")
+    for name, t, dtype in (("rows", rows, torch.int32), ("temperature", temperature, torch.float32), ("u", u, torch.float64),
+                           ("top_k", top_k, torch.int32), ("top_p", top_p, torch.float64)):
+        if t.dtype != dtype or t.numel() != n:
+            raise KernelError(f"sample_filtered: {name} must be {dtype} [{n}]")
+    vocab = logits.shape[1]
+    library.call("bc4g_sample_filtered", _ptr(logits), _ptr(rows), _ptr(temperature), _ptr(u), _ptr(top_k), _ptr(top_p),
+                 _ptr(out), n, vocab, _stream(), cost=lambda: (40.0 * n * vocab, n * vocab * 4))
+    return out
+
+
 def pack_weight(w: torch.Tensor) -> torch.Tensor:
     """A [n, k] weight in the fragment order the weight-streaming kernel reads:
     [ceil(n/16)][ceil(k/32)][64 lanes][8], lane l of a k-step holding row l % 16 of the block and

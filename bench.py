@@ -18,7 +18,7 @@ Beside the headline: `--shape` runs the same measurements at the sizes of Llama-
 `--only decode|prefill` runs one part and prints a short line of its own (what the profiles use);
 `--only serve` submits `--requests` requests of mixed lengths to the scheduler and times the whole
 run, prompts in portions of `--chunk` tokens beside the others' decoded tokens (`--new-tokens-spread`:
-the requests end one after the other instead of all together).
+the requests end one after the other instead of all together; `--top-k`, `--top-p`: they sample with these).
 """
 import argparse
 import json
@@ -182,10 +182,10 @@ def run_gemm(m, n, k, runs=20):
             "frac": round(2.0 * m * n * k / us / 1e6 / PEAK_TFLOPS["bf16"], 4)}
 
 
-def run_serve(model, cfg, n_requests, new_tokens, chunk, seed=3, spread=0):
+def run_serve(model, cfg, n_requests, new_tokens, chunk, seed=3, spread=0, top_k=0, top_p=1.0):
     """A mixed batch through the scheduler: n_requests submitted at once, prompt lengths uniform in
     [128, max context - new_tokens], prompts cut into portions of `chunk` tokens beside the decoded
-    tokens of the others, temperature 1.0.  ``spread``: the requests' numbers of new tokens are spaced
+    tokens of the others, temperature 1.0 (with ``top_k`` / ``top_p`` if given).  ``spread``: the requests' numbers of new tokens are spaced
     evenly from new_tokens down to new_tokens - spread, so that they end one after the other and the
     number of decoding requests takes every value on its way down (0: all generate new_tokens and end
     together).  Returns (seconds, scheduler statistics with the decode graphs captured in the timed run)."""
@@ -210,7 +210,7 @@ def run_serve(model, cfg, n_requests, new_tokens, chunk, seed=3, spread=0):
         for i, n in enumerate(lengths):
             prompt = torch.randint(0, cfg.vocab_size, (n,), generator=gen).tolist()
             sched.submit(Request(id=tag * n_requests + i, prompt=prompt, max_new_tokens=new[i],
-                                 sampling=SamplingParams(temperature=1.0, seed=i)))
+                                 sampling=SamplingParams(temperature=1.0, top_p=top_p, top_k=top_k, seed=i)))
 
     def drain():
         made = 0
@@ -229,6 +229,7 @@ def run_serve(model, cfg, n_requests, new_tokens, chunk, seed=3, spread=0):
     dt = time.perf_counter() - t0
     after = sched.stats()
     return dt, dict(requests=n_requests, generated=made, prompt_tokens=sum(lengths), new_tokens_spread=spread,
+                    top_k=top_k, top_p=top_p,
                     steps=after.steps - before.steps, preemptions=after.preemptions - before.preemptions,
                     graphs=len(ex._graphs), graphs_captured_in_the_timed_run=ex.captures - captured)
 
@@ -252,6 +253,8 @@ def main() -> int:
     ap.add_argument("--new-tokens-spread", type=int, default=0,
                     help="--only serve: the requests generate from --new-tokens down to --new-tokens minus this, evenly "
                          "spaced, so they end one after the other (0: all end together)")
+    ap.add_argument("--top-k", type=int, default=0, help="--only serve: the requests sample with this top-k (0: none)")
+    ap.add_argument("--top-p", type=float, default=1.0, help="--only serve: ... and this top-p (1: none)")
     ap.add_argument("--only", choices=["decode", "prefill", "serve", "gemm", "peaks"], default=None,
                     help="run one part only and print its own short line (for profiling); peaks: what a kernel that only "
                          "reads, and one of nothing but matrix-core instructions, reach on this device")
@@ -302,7 +305,8 @@ def main() -> int:
         return 0
 
     if args.only == "serve":
-        dt, st = run_serve(model, cfg, args.requests, args.new_tokens, args.chunk, spread=args.new_tokens_spread)
+        dt, st = run_serve(model, cfg, args.requests, args.new_tokens, args.chunk, spread=args.new_tokens_spread,
+                           top_k=args.top_k, top_p=args.top_p)
         print(json.dumps(dict(only="serve", shape=args.shape, **st, seconds=round(dt, 3),
                               generated_per_s=round(st["generated"] / dt, 1),
                               all_tokens_per_s=round((st["generated"] + st["prompt_tokens"]) / dt, 1))), flush=True)

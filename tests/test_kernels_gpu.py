@@ -612,6 +612,75 @@ def test_sampling_follows_the_law_at_other_vocabularies(ops, vocab):
             assert abs(got[i] - want) == 1 and edge < 1e-6 * cum[-1], (vocab, i, got[i], want)
 
 
+FILTERED_ROWS = {
+    "normal": lambda g, n, v: g.normal(0, 2.0, (n, v)),
+    "ties": lambda g, n, v: np.round(g.normal(0, 1.5, (n, v)) * 2) / 2,          # many tokens share a weight
+    "equal": lambda g, n, v: np.full((n, v), 0.25),                             # all of them do
+    "peaked": lambda g, n, v: g.normal(0, 1.0, (n, v)) + 12.0 * (g.random((n, v)) < 3.0 / v),   # as a model's rows are
+    "wide": lambda g, n, v: g.normal(0, 30.0, (n, v)),                          # weights down to zero
+}
+
+
+@pytest.mark.parametrize("kind", sorted(FILTERED_ROWS))
+@pytest.mark.parametrize("vocab", [7, 1000, 18433, 36864, 36865, 128256])
+def test_filtered_sampling_follows_the_law(ops, vocab, kind):
+    """Top-k, top-p and both on the device against the host's sorted walk (sampling/host.py, the reference's law)
+    for the same uniform numbers, into chosen places of the output: rows whose candidates fit the kernel's list
+    (peaked) and rows whose do not (flat: their patterns in LDS up to 36,864 tokens, worked out again beyond), rows
+    where many or all tokens share a weight (the order of the ids decides), k beyond what one bucket holds, a
+    nucleus of one token, u at both ends.  The same call twice gives the same ids (the sums are integer adds)."""
+    from bare_cuda_4gib_amd.sampling import SamplingParams, sample_token
+    gen = np.random.default_rng(vocab * 7 + len(kind))
+    n = 30
+    logits = FILTERED_ROWS[kind](gen, n + 2, vocab).astype(np.float32)
+    us = gen.random(n)
+    us[0], us[1], us[-1] = 0.0, 1e-12, 1.0 - 2.0 ** -53
+    temps = np.array([(0.7, 1.0, 1.6, 0.05)[i % 4] for i in range(n)], np.float32)
+    ks = np.array([(0, 1 + vocab // 50, 5, 2, 40, vocab - 1, 3)[i % 7] for i in range(n)], np.int32)
+    ps = np.array([(0.9, 0.5, 0.99, 0.1, 1e-6)[(i // 2) % 5] if not 0 < ks[i] < vocab or i % 3 else 1.0 for i in range(n)], np.float64)
+    # (a row with neither limit is not the kernel's: the law without filters walks in the order of the ids)
+    rows = np.array([(i * 7) % (n + 2) for i in range(n)], np.int32)            # some logits rows, in another order
+    assert len(set(rows.tolist())) == n
+    dev = lambda a: torch.from_numpy(a).to(DEV)
+    out = torch.full((n + 2,), -7, dtype=torch.int32, device=DEV)
+    ops.sample_filtered(dev(logits), out, dev(rows), dev(temps), dev(us), dev(ks), dev(ps))
+    again = torch.full((n + 2,), -7, dtype=torch.int32, device=DEV)
+    ops.sample_filtered(dev(logits), again, dev(rows), dev(temps), dev(us), dev(ks), dev(ps))
+    got = out.cpu().numpy()
+    assert np.array_equal(got, again.cpu().numpy())
+    assert sorted(np.nonzero(got == -7)[0].tolist()) == sorted(set(range(n + 2)) - set(rows.tolist()))   # the others untouched
+
+    class Fixed:
+        def __init__(self, u): self.u = u
+        def uniform(self): return self.u
+    for i in range(n):
+        row = logits[rows[i]]
+        params = SamplingParams(temperature=float(temps[i]), top_p=float(ps[i]), top_k=int(ks[i]))
+        want = sample_token(row, params, Fixed(float(us[i])))
+        if got[rows[i]] != want:      # sums in another order may move an edge by one place of the sorted walk
+            w = np.exp((row - row.max()) * (np.float32(1.0) / temps[i])).astype(np.float32).astype(np.float64)
+            order = np.lexsort((np.arange(vocab), -w))
+            at = {int(t): j for j, t in enumerate(order[:max(int(ks[i]), 64) if ks[i] else vocab])}
+            assert int(got[rows[i]]) in at and abs(at[int(got[rows[i]])] - at[want]) == 1, (vocab, kind, i, got[rows[i]], want)
+            cum = np.cumsum(w[order])
+            edge = min(abs(us[i] * c - cum[min(at[int(got[rows[i]])], at[want])]) for c in (cum[-1], cum[len(at) - 1]))
+            assert edge < 1e-9 * cum[-1], (vocab, kind, i, got[rows[i]], want, edge)
+
+
+def test_filtered_sampling_refuses_what_it_cannot_read(ops):
+    logits = torch.zeros(2, 50, device=DEV)
+    good = dict(out=torch.zeros(2, dtype=torch.int32, device=DEV), rows=torch.zeros(1, dtype=torch.int32, device=DEV),
+                temperature=torch.ones(1, device=DEV), u=torch.zeros(1, dtype=torch.float64, device=DEV),
+                top_k=torch.ones(1, dtype=torch.int32, device=DEV), top_p=torch.ones(1, dtype=torch.float64, device=DEV))
+    ops.sample_filtered(logits, **good)
+    for name, bad in (("out", torch.zeros(3, dtype=torch.int32, device=DEV)), ("u", torch.zeros(1, device=DEV)),
+                      ("top_p", torch.ones(2, dtype=torch.float64, device=DEV)), ("top_k", torch.ones(1, device=DEV))):
+        with pytest.raises(Exception, match="sample_filtered"):
+            ops.sample_filtered(logits, **dict(good, **{name: bad}))
+    with pytest.raises(Exception, match="sample_filtered"):
+        ops.sample_filtered(logits.to(torch.bfloat16), **good)
+
+
 @pytest.mark.parametrize("m", [1, 7, 16])
 @pytest.mark.parametrize("n,k", [(130, 304), (2560, 2048), (301, 80)])
 @pytest.mark.parametrize("gdt", [torch.bfloat16, torch.float32])

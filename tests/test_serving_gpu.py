@@ -157,34 +157,41 @@ def test_a_stop_id_met_while_the_next_step_already_runs(folders, dtype):
     assert engine.stats()["kv_pages_used"] == 0
 
 
+@pytest.mark.parametrize("filters", [False, True])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_sampled_tokens_are_the_law_on_the_engine_s_own_logits(folders, dtype):
-    """Temperature 0.8, three requests in one mixed batch: every id the engine draws on the device is, exactly,
-    the id that the host's sampler (the reference's law) draws from the very logits row the step returned,
-    with the request's own generator -- in bfloat16 too, where the logits' tolerance against the plain
-    implementation is wider than a token's share of the running sum and that comparison cannot bite."""
+def test_sampled_tokens_are_the_law_on_the_engine_s_own_logits(folders, dtype, filters):
+    """Three requests in one mixed batch, each with a temperature -- and, with `filters`, one with a top-k, one
+    with a top-p, one with both, which the device draws by the law for filtered rows, the step after running
+    ahead all the same: every id the engine draws on the device is, exactly, the id that the host's sampler (the
+    reference's law) draws from the very logits row the step returned, with the request's own generator -- in
+    bfloat16 too, where the logits' tolerance against the plain implementation is wider than a token's share of
+    the running sum and that comparison cannot bite."""
     from bare_cuda_4gib_amd.engine import Engine
     from bare_cuda_4gib_amd.sampling import MT19937_64, SamplingParams, sample_token
     folder = folders("B", dtype, "spread")
     prompts = [helpers.random_ids(n, 384, 40 + n) for n in (5, 64, 130)]
+    how = [dict(temperature=0.8), dict(temperature=0.8), dict(temperature=0.8)]
+    if filters:
+        how = [dict(temperature=0.8, top_k=7), dict(temperature=1.3, top_p=0.8), dict(temperature=1.0, top_k=40, top_p=0.95)]
     engine = Engine(folder, max_tokens=256, max_seqs=3, kv_pages=0, dtype=dtype, page_tokens=16, prefill_chunk=32,
                     max_batch_tokens=96)
     log = record_steps(engine)
     for i, p in enumerate(prompts):
-        assert engine.submit(i, p, 24, temperature=0.8, seed=4 + i)[0] == "ok"
+        assert engine.submit(i, p, 24, seed=4 + i, **how[i])[0] == "ok"
     out, _ = drain(engine, 3)
+    assert any(s["ahead"] for s in log)                 # steps were launched before the tokens of the last had been read
     rngs = {i: MT19937_64(4 + i) for i in range(3)}
     drawn = {i: [] for i in range(3)}
     for s in log:                                # the steps in order: a request's k-th wanted row gets its generator's k-th number
         for r, (rid, pos) in enumerate(s["rows"]):
             if len(drawn[rid]) < 24:
-                drawn[rid].append(sample_token(s["logits"][r], SamplingParams(temperature=0.8), rngs[rid]))
+                drawn[rid].append(sample_token(s["logits"][r], SamplingParams(**how[rid]), rngs[rid]))
     assert drawn == out
     assert len(set(out[2])) > 3
     # the check bites: another request's generator gives other ids from the same rows
     other = MT19937_64(4 + 2)
     rows_1 = [s["logits"][r] for s in log for r, (rid, _) in enumerate(s["rows"]) if rid == 1][:24]
-    assert [sample_token(row, SamplingParams(temperature=0.8), other) for row in rows_1] != out[1]
+    assert [sample_token(row, SamplingParams(**how[1]), other) for row in rows_1] != out[1]
 
 
 def test_more_tokens_than_the_model_has_positions_are_refused(folders):
