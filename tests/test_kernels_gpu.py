@@ -667,6 +667,29 @@ def test_filtered_sampling_follows_the_law(ops, vocab, kind):
             assert edge < 1e-9 * cum[-1], (vocab, kind, i, got[rows[i]], want, edge)
 
 
+def test_filtered_sampling_beyond_half_a_million_tokens(ops):
+    """Beyond 2^19 tokens a bucket's count no longer fits beside its mantissa sum in one word: the kernel keeps the
+    two apart there.  Rows whose candidates fit the list and rows whose do not."""
+    from bare_cuda_4gib_amd.sampling import SamplingParams, sample_token
+    vocab, n = 600001, 6
+    gen = np.random.default_rng(5)
+    logits = np.concatenate([FILTERED_ROWS["peaked"](gen, n // 2, vocab), FILTERED_ROWS["ties"](gen, n // 2, vocab)]).astype(np.float32)
+    us = np.array([0.0, 0.37, 0.93, 0.5, 0.11, 1.0 - 2.0 ** -53])
+    temps = np.array([1.0, 0.7, 1.3, 1.0, 0.7, 1.3], np.float32)
+    ks = np.array([40, 0, 5, 0, 3000, 40], np.int32)
+    ps = np.array([0.9, 0.5, 1.0, 0.9, 0.99, 0.3], np.float64)
+    dev = lambda a: torch.from_numpy(a).to(DEV)
+    out = torch.full((n,), -7, dtype=torch.int32, device=DEV)
+    ops.sample_filtered(dev(logits), out, torch.arange(n, dtype=torch.int32, device=DEV), dev(temps), dev(us), dev(ks), dev(ps))
+
+    class Fixed:
+        def __init__(self, u): self.u = u
+        def uniform(self): return self.u
+    want = [sample_token(logits[i], SamplingParams(temperature=float(temps[i]), top_p=float(ps[i]), top_k=int(ks[i])),
+                         Fixed(float(us[i]))) for i in range(n)]
+    assert out.tolist() == want
+
+
 def test_filtered_sampling_refuses_what_it_cannot_read(ops):
     logits = torch.zeros(2, 50, device=DEV)
     good = dict(out=torch.zeros(2, dtype=torch.int32, device=DEV), rows=torch.zeros(1, dtype=torch.int32, device=DEV),
