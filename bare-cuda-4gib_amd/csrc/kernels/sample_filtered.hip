@@ -60,7 +60,7 @@ struct Shared {
   unsigned long long msum[kBuckets];
   float red_v[kWaves];
   __align__(16) int wave_cnt[kWaves];
-  // a walk's state: thread 0 writes it between barriers, all read it after
+  // a walk's state: the wave that walks a level's buckets writes it between barriers, all read it after
   unsigned int prefix;         // the digits settled so far
   unsigned int above_count;    // tokens of the universe strictly above the bucket in question
   double above_mass;
