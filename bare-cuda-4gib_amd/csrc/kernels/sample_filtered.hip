@@ -71,6 +71,7 @@ struct Shared {
   long long res_bits;
   int res_ties;
   int res_count;
+  int alone_level;             // (>= 0: the answer is the one token of the bucket settled at this level; its pattern is looked up)
   int hit;
 };
 
@@ -190,6 +191,7 @@ __device__ void walk(Shared& sh, const Row& row, const Prefix& universe, int mod
     sh.above_mass = 0.0;
     sh.done = 0;
     sh.found = 0;
+    sh.alone_level = -1;
   }
   for (int level = 0; level < levels; ++level) {
     for (int i = tid; i < kBuckets; i += kThreads) {
@@ -314,11 +316,27 @@ __device__ void walk(Shared& sh, const Row& row, const Prefix& universe, int mod
             sh.res_bits = settled;
             sh.res_ties = ties_needed(mode, k, target, above_count, above_mass, value_of(settled), count);
           }
+        } else if (count == 1 && levels == 4) {
+          // one token in the bucket: it is the answer, whatever its other digits are
+          sh.done = 1;
+          sh.found = 1;
+          sh.res_ties = 1;
+          sh.alone_level = level;
         }
       }
     }
     __syncthreads();
     if (sh.done) break;
+  }
+  const int alone_level = sh.alone_level;
+  if (alone_level >= 0) {
+    const unsigned int digits = sh.prefix;
+    const bool bounded = universe.bits >= 0;
+    const unsigned int floor_bits = static_cast<unsigned int>(universe.bits);
+    each_token(row, [&](unsigned int b, int) {
+      if ((!bounded || b > floor_bits) && (b >> kShift[alone_level]) == digits) sh.res_bits = b;
+    });
+    __syncthreads();
   }
 }
 
