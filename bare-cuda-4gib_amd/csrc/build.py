@@ -120,6 +120,35 @@ def _compile_one(hipcc: str, name: str, digest: str) -> str:
     return obj
 
 
+TWIN_DIR = os.path.join(HERE, "twin")
+
+
+def twins_path() -> str:
+    """The program of the C++ twin tests, beside the library it is linked against."""
+    return os.path.join(os.path.dirname(LIB_PATH), "bc4g_twins")
+
+
+def build_twins(verbose: bool = True) -> str:
+    """Compile twin/twins.cpp (every kernel family beside a plain C++ twin) against the built library; returns the
+    program's path.  `bc4g_twins [name ...]` runs the tests named (all without names, --list names them) and
+    returns non-zero if one fails; twin/CMakeLists.txt registers the same program with ctest, one test a family."""
+    hipcc = _hipcc()
+    if not is_built():
+        raise KernelError(f"{LIB_PATH} is not built: the twin tests are linked against it")
+    out = twins_path()
+    t0 = time.time()
+    cmd = [hipcc, "--offload-arch=" + ARCH, "-O2", "-std=c++17", "-Wno-unused-command-line-argument", "-I", SRC_DIR,
+           os.path.join(TWIN_DIR, "twins.cpp"), "-o", out + f".tmp{os.getpid()}", "-L", os.path.dirname(LIB_PATH), "-lbc4g",
+           "-Wl,-rpath,$ORIGIN"]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise KernelError(f"hipcc failed on the twin tests:\n{proc.stderr[-4000:]}")
+    os.replace(out + f".tmp{os.getpid()}", out)
+    if verbose:
+        print(f"[bc4g] built {out} in {time.time() - t0:.0f} s", file=sys.stderr, flush=True)
+    return out
+
+
 def build(verbose: bool = True, jobs: int = 0) -> str:
     """Compile every kernel source and link the library; returns its path."""
     hipcc = _hipcc()
