@@ -405,6 +405,82 @@ bool attention_mfma() {
   return ok;
 }
 
+bool qkv_fused() {
+  // The q|k|v product with rotation and cache write in its epilogue -- the tiled kernel for a step of prompt
+  // portions, the weight-streaming one for a step of decoded tokens -- checked through what attention then makes of
+  // the queries it left and the cache it wrote.  Every head's rows of the weight come in blocks of sixteen: eight
+  // dimensions, then their rotation partners; queries, keys, values and so the outputs live in that order.
+  Rng rng(11);
+  const int nh = 4, nkv = 2, d = 32, page = 16, hidden = 128, n = (nh + 2 * nkv) * d;
+  const float theta = 10000.0f;
+  std::vector<int> order(d);                          // place j of a head holds dimension order[j]
+  for (int b = 0; b < d / 16; ++b)
+    for (int t = 0; t < 16; ++t) order[16 * b + t] = t < 8 ? 8 * b + t : d / 2 + 8 * b + (t - 8);
+  const std::vector<bf16> w = as_bf16(normals(rng, static_cast<size_t>(n) * hidden, 0.2f));     // rows: q heads, k heads, v heads
+  std::vector<bf16> reordered(w.size());
+  for (int head = 0; head < nh + 2 * nkv; ++head)
+    for (int j = 0; j < d; ++j)
+      std::copy(w.begin() + (static_cast<size_t>(head) * d + order[j]) * hidden, w.begin() + (static_cast<size_t>(head) * d + order[j] + 1) * hidden,
+                reordered.begin() + (static_cast<size_t>(head) * d + j) * hidden);
+  Dev<bf16> packed(pack_weight(reordered, n, hidden));
+  const std::vector<int> fresh = {40, 23};
+  Paged paged(2, page, 41, rng);
+  const size_t cache = static_cast<size_t>(paged.num_pages) * nkv * page * d;
+  Dev<bf16> kc(cache), vc(cache);
+  Dev<int32_t> dtable(paged.table);
+  std::vector<std::vector<std::vector<double>>> keys(2), values(2);
+  auto step = [&](const std::vector<std::pair<int, int>>& rows, const std::vector<int32_t>& seq_start,
+                  const std::vector<int32_t>& seq_ctx, bool tiled, const char* what) -> bool {
+    const int t = static_cast<int>(rows.size());
+    const std::vector<bf16> x = as_bf16(normals(rng, static_cast<size_t>(t) * hidden));
+    const std::vector<double> product = plain::gemm(widen(x), widen(w), t, n, hidden);
+    std::vector<int32_t> positions, slots, row_seq;
+    std::vector<std::vector<double>> q(t);
+    for (int r = 0; r < t; ++r) {
+      positions.push_back(rows[r].second);
+      slots.push_back(paged.slot(rows[r].first, rows[r].second));
+      row_seq.push_back(rows[r].first);
+      const double* row = &product[static_cast<size_t>(r) * n];
+      q[r].assign(row, row + nh * d);
+      keys[rows[r].first].push_back(std::vector<double>(row + nh * d, row + (nh + nkv) * d));
+      std::vector<double> v(row + (nh + nkv) * d, row + n);
+      for (double& e : v) e = from_bf16(to_bf16(static_cast<float>(e)));           // as the cache holds it
+      values[rows[r].first].push_back(v);
+    }
+    Dev<bf16> dx(x), dq(static_cast<size_t>(t) * nh * d), out(static_cast<size_t>(t) * nh * d);
+    Dev<int32_t> dpos(positions), dslots(slots), dseq(row_seq), dstart(seq_start), dctx(seq_ctx);
+    if (tiled) {
+      Dev<float> table(static_cast<size_t>(t) * d);                                 // [t][d / 2][2]: cosine and sine
+      RUN(bc4g_rope_table(dpos.p, table.p, t, d, theta, kStream));
+      RUN(bc4g_gemm_mfma_qkv(dx.p, packed.p, 1, dq.p, table.p, dslots.p, kc.p, vc.p, t, n, hidden, nh, nkv, d, page, 1, kStream));
+    } else {
+      RUN(bc4g_gemm_skinny_qkv(dx.p, nullptr, 0, 0.0f, nullptr, 0, 0, packed.p, dq.p, dpos.p, dslots.p, kc.p, vc.p, t, hidden,
+                               nh, nkv, d, d, theta, page, 1, kStream));
+    }
+    const int tokens_per_tile = 16 / (nh / nkv);
+    std::vector<int32_t> tile_start = {0};
+    for (size_t s = 0; s + 1 < seq_start.size(); ++s)
+      tile_start.push_back(tile_start.back() + (seq_start[s + 1] - seq_start[s] + tokens_per_tile - 1) / tokens_per_tile);
+    Dev<int32_t> dtiles(tile_start);
+    RUN(bc4g_attention_mfma(dq.p, nh * d, out.p, nullptr, nullptr, kc.p, vc.p, dtable.p, paged.pages_per_seq, dstart.p, dctx.p,
+                            dtiles.p, 2, tile_start.back(), t, nh, nkv, d, page, 0, 1.0f / std::sqrt(static_cast<float>(d)),
+                            tokens_per_tile, 1, tiled ? 0 : 1, 1, nullptr, 0, nullptr, tiled ? 0 : 1, dseq.p, kStream));
+    const std::vector<double> straight = twin_attention(rows, q, keys, values, nh, nkv, d, theta, 0, true);
+    std::vector<double> want(straight.size());
+    for (size_t head = 0; head < straight.size() / d; ++head)
+      for (int j = 0; j < d; ++j) want[head * d + j] = straight[head * d + order[j]];
+    return close(what, widen(out.get()), want, 3e-2, 3e-2);
+  };
+  bool ok = true;
+  std::vector<std::pair<int, int>> rows;
+  for (int s = 0; s < 2; ++s)
+    for (int p = 0; p < fresh[s]; ++p) rows.push_back({s, p});
+  ok &= step(rows, {0, fresh[0], fresh[0] + fresh[1]}, {0, 0}, true, "prompt portions through the tiled product");
+  rows = {{0, fresh[0]}, {1, fresh[1]}};
+  ok &= step(rows, {0, 1, 2}, {fresh[0], fresh[1]}, false, "decoded tokens through the weight-streaming product");
+  return ok;
+}
+
 bool argmax() {
   const int n = 3, vocab = 1000;
   std::vector<float> logits(static_cast<size_t>(n) * vocab, -1.0f);
@@ -497,6 +573,7 @@ const std::vector<std::pair<std::string, std::function<bool()>>>& tests() {
       {"gemm_mfma", gemm_mfma},
       {"attention_generic", attention_generic},
       {"attention_mfma", attention_mfma},
+      {"qkv_fused", qkv_fused},
       {"argmax", argmax},
       {"sampling", sampling},
   };

@@ -11,7 +11,7 @@ import pytest
 from bare_cuda_4gib_amd.csrc import build
 
 FAMILIES = ["embed", "rmsnorm", "swiglu", "gemm_generic", "gemm_skinny", "gemm_skinny_norms", "gemm_mfma",
-            "attention_generic", "attention_mfma", "argmax", "sampling"]
+            "attention_generic", "attention_mfma", "qkv_fused", "argmax", "sampling"]
 
 
 def program() -> str:
