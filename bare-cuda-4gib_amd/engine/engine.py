@@ -76,7 +76,7 @@ class Engine:
     def __init__(self, model_path: str, max_tokens: int = 1024, max_seqs: int = 8, kv_pages: int = 0,
                  max_waiting: int = 64, *, dtype: str = "bfloat16", device: str = "cuda:0",
                  page_tokens: int = 64, max_batch_tokens: int = 2048, prefill_chunk: int = 512,
-                 worker: bool = False):
+                 worker: bool = False, gather_ms: float = 0.0):
         if max_tokens <= 0 or max_seqs <= 0:
             raise EngineError("max_tokens and max_seqs must be positive")
         self.model, self.config = load_model(model_path, dtype, device)
@@ -92,7 +92,7 @@ class Engine:
                                  max_tokens=max_tokens, page_tokens=page_tokens,
                                  max_batch_tokens=max_batch_tokens)
         self.scheduler = Scheduler(self.executor, DevicePicker(), max_batch_tokens=max_batch_tokens,
-                                   prefill_chunk=prefill_chunk, run_ahead=True)
+                                   prefill_chunk=prefill_chunk, run_ahead=True, gather_ms=gather_ms)
         self._max_waiting = max_waiting
         # The inbox: what any thread hands to whoever runs the turns, and the ids not yet finished.
         self._in = threading.Condition()

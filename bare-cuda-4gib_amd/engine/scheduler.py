@@ -90,6 +90,7 @@ class _Live:
         self.rng = MT19937_64(seed_for(request.sampling))
         self.deadline = deadline
         self.admitted_at = -1             # admission counter; the largest is preempted first
+        self.queued_at = 0.0              # when it joined the waiting line (the scheduler's clock)
 
 
 def target_tokens(limits: EngineLimits, prompt_len: int, max_new_tokens: int) -> int:
@@ -140,8 +141,14 @@ class Scheduler:
     """
 
     def __init__(self, executor, picker, *, max_batch_tokens: int = 2048, prefill_chunk: int = 512,
-                 clock=time.monotonic, run_ahead: bool = False):
-        """``run_ahead``: while every running request is decoding and none can be admitted, the next
+                 clock=time.monotonic, run_ahead: bool = False, gather_ms: float = 0.0):
+        """``gather_ms``: while every running request is decoding, a waiting request is admitted only after it has
+        waited this long, and whoever came meanwhile with it: a step that brings a prompt portion cannot be replayed
+        from a captured graph nor run ahead, so where requests come and go all the time (short prompts, long answers)
+        admitting them one by one makes every other step such a step; gathered, they share one.  0 admits at once.
+        Nothing is held back while nothing runs or while a prompt is under way anyway.
+
+        ``run_ahead``: while every running request is decoding and none can be admitted, the next
         step is launched with its tokens taken from what the sampling kernel has just chosen, on
         the device, before the host has read them; the host reads a step's tokens (and emits its
         events) while the next step runs.  The tokens are the same; the events of a step come out
@@ -152,6 +159,7 @@ class Scheduler:
         self.executor = executor
         self.picker = picker
         self.run_ahead = run_ahead
+        self.gather_ms = gather_ms
         self._ahead = None                # (requests, picked): a step whose tokens have not been read yet
         self.max_batch_tokens = max_batch_tokens
         self.prefill_chunk = prefill_chunk
@@ -188,6 +196,7 @@ class Scheduler:
         deadline = self._clock() + request.timeout_ms / 1000.0 if request.timeout_ms > 0 else float("inf")
         live = _Live(request, deadline)
         live.target = target_tokens(self.limits, live.prompt_len, request.max_new_tokens)
+        live.queued_at = self._clock()
         self.waiting.append(live)
 
     def cancel(self, request_id) -> bool:
@@ -245,9 +254,18 @@ class Scheduler:
         self.running.remove(victim)
         self._retire(victim)
         victim.computed = 0
+        victim.queued_at = float("-inf")   # (has waited long enough: back in as soon as it fits)
         self.waiting.appendleft(victim)
         self._totals.preemptions += 1
         return True
+
+    def _gathering(self) -> bool:
+        """Whether those who wait are held back for now, to be admitted together (gather_ms)."""
+        if self.gather_ms <= 0.0 or not self.waiting or not self.running:
+            return False
+        if any(len(r.tokens) - r.computed > 1 for r in self.running):
+            return False                   # a prompt is under way: this step is no decode step anyway
+        return (self._clock() - self.waiting[0].queued_at) * 1000.0 < self.gather_ms
 
     def plan(self) -> List[tuple]:
         """Decide this step's batch: [(live request, number of its next tokens)].  Admits
@@ -277,7 +295,7 @@ class Scheduler:
             preempted = True
         # 3. admit waiting requests in order; one that does not fit blocks those behind it
         #    (not in a step that had to preempt: the pool is full)
-        while not preempted and self.waiting and budget > 0 and cache.free_slots > 0:
+        while not preempted and self.waiting and budget > 0 and cache.free_slots > 0 and not self._gathering():
             r = self.waiting[0]
             n = min(len(r.tokens) - r.computed, self.prefill_chunk, budget)
             self.executor.admit(r.id)
@@ -341,7 +359,7 @@ class Scheduler:
         requests, picked = ahead
         running = {id(r) for r in self.running}
         live = sum(1 for r in requests if id(r) in running)
-        if live != len(self.running) or (self.waiting and self.executor.cache.free_slots > 0):
+        if live != len(self.running) or (self.waiting and self.executor.cache.free_slots > 0 and not self._gathering()):
             return None
         rows = [i for i, r in enumerate(requests) if id(r) in running and r.generated + 1 < r.target]
         if not rows or len(rows) > self.max_batch_tokens:

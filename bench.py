@@ -19,6 +19,8 @@ Beside the headline: `--shape` runs the same measurements at the sizes of Llama-
 `--only serve` submits `--requests` requests of mixed lengths to the scheduler and times the whole
 run, prompts in portions of `--chunk` tokens beside the others' decoded tokens (`--new-tokens-spread`:
 the requests end one after the other instead of all together; `--top-k`, `--top-p`: they sample with these).
+`--only chat` is a closed loop of `--requests` requests with short prompts and long answers that come and go all the
+time (`--gather-ms`: the scheduler gathers those who came for so long before it admits them).
 """
 import argparse
 import json
@@ -234,6 +236,56 @@ def run_serve(model, cfg, n_requests, new_tokens, chunk, seed=3, spread=0, top_k
                     graphs=len(ex._graphs), graphs_captured_in_the_timed_run=ex.captures - captured)
 
 
+def run_chat(model, cfg, concurrency, gather_ms, finished=384, seed=5):
+    """Requests that come and go all the time: `concurrency` requests in flight, each with a prompt of 16 to 64
+    tokens and 64 to 192 new ones at temperature 1.0; whenever one ends the next is submitted (a closed loop), so
+    that new prompts arrive every few steps beside the others' decoded tokens.  ``gather_ms``: the scheduler's
+    wait before it admits those who came (Scheduler(gather_ms=...)).  Times the steps in which `finished` requests
+    end, after as many to warm up.  Returns (seconds, figures)."""
+    import random
+    import torch
+    from bare_cuda_4gib_amd.engine import Executor
+    from bare_cuda_4gib_amd.engine.scheduler import Request, Scheduler
+    from bare_cuda_4gib_amd.sampling.device import DevicePicker
+    from bare_cuda_4gib_amd.sampling.params import SamplingParams
+    ex = Executor(model, num_pages=concurrency * 4, max_requests=concurrency, max_tokens=256, page_tokens=64,
+                  max_batch_tokens=2048)
+    sched = Scheduler(ex, DevicePicker(), max_batch_tokens=2048, prefill_chunk=512, run_ahead=True, gather_ms=gather_ms)
+    rnd = random.Random(seed)
+    gen = torch.Generator().manual_seed(seed)
+    ids = iter(range(1 << 30))
+
+    def arrive():
+        n = rnd.randint(16, 64)
+        i = next(ids)
+        sched.submit(Request(id=i, prompt=torch.randint(0, cfg.vocab_size, (n,), generator=gen).tolist(),
+                             max_new_tokens=rnd.randint(64, 192), sampling=SamplingParams(temperature=1.0, seed=i)))
+
+    def run(until):
+        made = ended = 0
+        while ended < until:
+            for e in sched.step():
+                made += e.token >= 0
+                if e.finish:
+                    ended += 1
+                    arrive()
+        return made
+
+    for _ in range(concurrency):
+        arrive()
+    run(finished)
+    torch.cuda.synchronize()
+    before = sched.stats()
+    t0 = time.perf_counter()
+    made = run(finished)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    after = sched.stats()
+    steps = after.steps - before.steps
+    return dt, dict(concurrency=concurrency, gather_ms=gather_ms, requests_ended=finished, generated=made, steps=steps,
+                    ms_per_step=round(dt / steps * 1e3, 3), preemptions=after.preemptions - before.preemptions)
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -255,7 +307,9 @@ def main() -> int:
                          "spaced, so they end one after the other (0: all end together)")
     ap.add_argument("--top-k", type=int, default=0, help="--only serve: the requests sample with this top-k (0: none)")
     ap.add_argument("--top-p", type=float, default=1.0, help="--only serve: ... and this top-p (1: none)")
-    ap.add_argument("--only", choices=["decode", "prefill", "serve", "gemm", "peaks"], default=None,
+    ap.add_argument("--gather-ms", type=float, default=0.0,
+                    help="--only chat: the scheduler waits this long before it admits those who came while others decode")
+    ap.add_argument("--only", choices=["decode", "prefill", "serve", "chat", "gemm", "peaks"], default=None,
                     help="run one part only and print its own short line (for profiling); peaks: what a kernel that only "
                          "reads, and one of nothing but matrix-core instructions, reach on this device")
     ap.add_argument("--mnk", default="2048,11264,2048",
@@ -302,6 +356,12 @@ def main() -> int:
                           "ms": round(pre_s * 1e3, 3), "frac": round(frac, 4),
                           "frac_of_measured": round(frac * PEAK_TFLOPS[args.dtype] / measured["bf16_tflops"], 4) if args.dtype == "bf16" else None,
                           "tokens_per_s": round(args.prefill_tokens / pre_s, 1)}), flush=True)
+        return 0
+
+    if args.only == "chat":
+        dt, st = run_chat(model, cfg, args.requests, args.gather_ms)
+        print(json.dumps(dict(only="chat", shape=args.shape, **st, seconds=round(dt, 3),
+                              generated_per_s=round(st["generated"] / dt, 1))), flush=True)
         return 0
 
     if args.only == "serve":

@@ -107,7 +107,7 @@ def run(sched, max_steps=500):
 
 
 def make(**kw):
-    sched_kw = {k: kw.pop(k) for k in ("max_batch_tokens", "prefill_chunk", "clock", "run_ahead") if k in kw}
+    sched_kw = {k: kw.pop(k) for k in ("max_batch_tokens", "prefill_chunk", "clock", "run_ahead", "gather_ms") if k in kw}
     ex = FakeExecutor(**kw)
     return Scheduler(ex, HostPicker(), **{"max_batch_tokens": 16, "prefill_chunk": 6, **sched_kw}), ex
 
@@ -331,3 +331,84 @@ def test_a_model_that_keeps_nothing_per_token_needs_no_pages():
     for i, p in prompts.items():
         assert out[i] == expected_greedy(p, 5) and finish[i] == "length"
     assert sched.stats().preemptions == 0 and ex.cache.free_slots == 3
+
+
+@pytest.mark.parametrize("run_ahead", [False, True])
+def test_arrivals_are_gathered_while_others_decode(run_ahead):
+    """gather_ms: a request that arrives while others decode waits until the first of the waiting has waited that
+    long, and goes in together with those that came meanwhile, in one step -- so the steps between stay decode
+    steps (which an engine replays from graphs and runs ahead).  Nothing is held back while nothing runs or while a
+    prompt is under way; a request that lost its pages is not made to wait again; and the tokens are the same."""
+    now = [0.0]
+
+    def build(gather_ms):
+        now[0] = 0.0
+        return make(num_pages=64, max_requests=6, max_tokens=64, clock=lambda: now[0], run_ahead=run_ahead, gather_ms=gather_ms)
+
+    prompts = {i: prompt(3 + i, 50 + i) for i in range(5)}
+
+    def serve(gather_ms):
+        sched, ex = build(gather_ms)
+        out, finish, admitted_in = {}, {}, {}
+        sched.submit(Request(id=0, prompt=prompts[0], max_new_tokens=30))       # nothing runs: in at once
+        arrivals = {3: 1, 4: 2, 9: 3, 20: 4}                                     # step -> request that arrives before it
+        for step in range(200):
+            if step in arrivals:
+                sched.submit(Request(id=arrivals[step], prompt=prompts[arrivals[step]], max_new_tokens=8))
+            if sched.idle():
+                break
+            before = len(ex.batches)
+            for e in sched.step():
+                if e.token >= 0:
+                    out.setdefault(e.id, []).append(e.token)
+                if e.finish:
+                    finish[e.id] = e.finish
+            for batch in ex.batches[before:]:
+                for rid, n in batch:
+                    admitted_in.setdefault(rid, len(ex.batches))
+            now[0] += 0.001                                                      # a millisecond a step
+        assert sched.idle() and len(finish) == 5
+        return out, admitted_in, ex.batches
+
+    plain_out, plain_in, plain_batches = serve(0.0)
+    out, admitted_in, batches = serve(5.0)
+    assert out == plain_out == {i: expected_greedy(prompts[i], 30 if i == 0 else 8) for i in range(5)}
+    assert plain_in[1] < plain_in[2] < plain_in[3]                               # one by one without gathering
+    assert admitted_in[1] == admitted_in[2] and admitted_in[2] < admitted_in[3]  # 1 and 2 together: 2 came while 1 waited
+    assert admitted_in[1] - plain_in[1] >= 4                                     # ... five milliseconds after 1 came
+    mixed = lambda bs: sum(1 for b in bs if any(n > 1 for _, n in b))
+    assert mixed(batches) < mixed(plain_batches)                                 # fewer steps that bring a prompt portion
+
+    # nothing runs: nobody is held back, whatever the clock says
+    sched, ex = build(1000.0)
+    sched.submit(Request(id=7, prompt=prompts[1], max_new_tokens=2))
+    sched.step()
+    assert ex.batches and ex.batches[0] == [(7, len(prompts[1]))]
+    # a long prompt under way: who comes now rides along at once
+    sched, ex = build(1000.0)
+    sched.submit(Request(id=1, prompt=prompt(20, 1), max_new_tokens=2))
+    sched.step()
+    sched.submit(Request(id=2, prompt=prompts[2], max_new_tokens=2))
+    sched.step()
+    assert (2, len(prompts[2])) in ex.batches[1]
+
+
+def test_a_request_that_lost_its_pages_is_not_made_to_wait_again():
+    now = [0.0]
+    sched, ex = make(num_pages=5, page_tokens=4, max_requests=3, max_tokens=20, clock=lambda: now[0], gather_ms=50.0)
+    for i in range(2):
+        sched.submit(Request(id=i, prompt=prompt(7, 80 + i), max_new_tokens=8))
+    out, finish = {}, {}
+    for step in range(300):
+        if sched.idle():
+            break
+        for e in sched.step():
+            if e.token >= 0:
+                out.setdefault(e.id, []).append(e.token)
+            if e.finish:
+                finish[e.id] = e.finish
+        now[0] += 0.001
+    assert sched.idle() and sched.stats().preemptions >= 1
+    assert out == {i: expected_greedy(prompt(7, 80 + i), 8) for i in range(2)}
+    victim_back = [i for i, b in enumerate(ex.batches) if any(rid == 1 and n > 1 for rid, n in b)]
+    assert len(victim_back) >= 2                                                 # its prompt ran twice
