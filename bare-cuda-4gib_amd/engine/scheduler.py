@@ -146,7 +146,9 @@ class Scheduler:
         waited this long, and whoever came meanwhile with it: a step that brings a prompt portion cannot be replayed
         from a captured graph nor run ahead, so where requests come and go all the time (short prompts, long answers)
         admitting them one by one makes every other step such a step; gathered, they share one.  0 admits at once.
-        Nothing is held back while nothing runs or while a prompt is under way anyway.
+        Nothing is held back while nothing runs or while a prompt is under way anyway, nor while requests come so
+        rarely that nobody else is to be expected within the wait (the mean gap between the last arrivals is longer
+        than it): a slot that waits for company that does not come only costs.
 
         ``run_ahead``: while every running request is decoding and none can be admitted, the next
         step is launched with its tokens taken from what the sampling kernel has just chosen, on
@@ -160,6 +162,8 @@ class Scheduler:
         self.picker = picker
         self.run_ahead = run_ahead
         self.gather_ms = gather_ms
+        self._last_arrival = None         # when the last request was submitted, and the running mean of the gaps
+        self._arrival_gap = float("inf")  # between arrivals (seconds; half of it is the newest gap)
         self._ahead = None                # (requests, picked): a step whose tokens have not been read yet
         self.max_batch_tokens = max_batch_tokens
         self.prefill_chunk = prefill_chunk
@@ -197,6 +201,10 @@ class Scheduler:
         live = _Live(request, deadline)
         live.target = target_tokens(self.limits, live.prompt_len, request.max_new_tokens)
         live.queued_at = self._clock()
+        if self._last_arrival is not None:
+            gap = live.queued_at - self._last_arrival
+            self._arrival_gap = gap if self._arrival_gap == float("inf") else 0.5 * (self._arrival_gap + gap)
+        self._last_arrival = live.queued_at
         self.waiting.append(live)
 
     def cancel(self, request_id) -> bool:
@@ -265,6 +273,8 @@ class Scheduler:
             return False
         if any(len(r.tokens) - r.computed > 1 for r in self.running):
             return False                   # a prompt is under way: this step is no decode step anyway
+        if self._arrival_gap * 1000.0 >= self.gather_ms:
+            return False                   # requests come too rarely for company within the wait
         return (self._clock() - self.waiting[0].queued_at) * 1000.0 < self.gather_ms
 
     def plan(self) -> List[tuple]:

@@ -393,6 +393,30 @@ def test_arrivals_are_gathered_while_others_decode(run_ahead):
     assert (2, len(prompts[2])) in ex.batches[1]
 
 
+def test_rare_arrivals_are_not_held_back():
+    """Where requests come further apart than the wait (the running mean of the last gaps), nobody is to be expected
+    for company: the arrival goes in with the next step, as without gathering."""
+    now = [0.0]
+    sched, ex = make(num_pages=64, max_requests=6, max_tokens=64, clock=lambda: now[0], gather_ms=5.0)
+    sched.submit(Request(id=0, prompt=prompt(3, 1), max_new_tokens=60))
+    for step in range(100):
+        if step in (10, 40, 70):                                                  # thirty milliseconds apart
+            sched.submit(Request(id=step, prompt=prompt(4, step), max_new_tokens=3))
+            sched.step()
+            assert (step, 4) in ex.batches[-1], f"the arrival before step {step} was held back"
+        else:
+            sched.step()
+        now[0] += 0.001
+    # ... and once they come in a burst again, they are gathered again
+    burst = {}
+    for i, rid in enumerate((200, 201, 202, 203)):
+        sched.submit(Request(id=rid, prompt=prompt(4, rid), max_new_tokens=3))
+        sched.step()
+        now[0] += 0.001
+        burst[rid] = any(r == rid for r, _ in ex.batches[-1])
+    assert burst[200] and not burst[203]                                          # (by the fourth the mean gap is below the wait)
+
+
 def test_a_request_that_lost_its_pages_is_not_made_to_wait_again():
     now = [0.0]
     sched, ex = make(num_pages=5, page_tokens=4, max_requests=3, max_tokens=20, clock=lambda: now[0], gather_ms=50.0)
