@@ -699,7 +699,8 @@ def gemm_parts_supported(a: torch.Tensor, w, residual: torch.Tensor, g: torch.Te
             and w.is_contiguous() and parts_of_k(a.shape[0], w.shape[0], w.shape[1]) > 1)
 
 
-def gemm_parts_accumulate_norm(a: torch.Tensor, w, residual: torch.Tensor, g: torch.Tensor, eps: float) -> Finished:
+def gemm_parts_accumulate_norm(a: torch.Tensor, w, residual: torch.Tensor, g: torch.Tensor, eps: float,
+                               checked: bool = False) -> Finished:
     """residual += a w^T and the RMSNorm (scale g, eps) of the result, in two kernels: the tiled product with k cut
     into parts over workgroups, each part's sums stored apart; then one that adds the parts to the residual in
     order and norms it.  For a few dozen rows and a square or long weight, where a 64 x 64 tile's workgroup
@@ -709,7 +710,7 @@ def gemm_parts_accumulate_norm(a: torch.Tensor, w, residual: torch.Tensor, g: to
     m, k = a.shape
     n = w.shape[0]
     n_parts = parts_of_k(m, n, k)
-    if n_parts < 2 or not gemm_parts_supported(a, w, residual, g):
+    if n_parts < 2 or not (checked or gemm_parts_supported(a, w, residual, g)):     # (checked: the caller has just asked)
         raise KernelError(f"gemm_parts_accumulate_norm: not for [{m}, {k}] x [{n}, {k}]^T")
     parts = torch.empty((n_parts, m, n), dtype=torch.float32, device=a.device)
     out = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)

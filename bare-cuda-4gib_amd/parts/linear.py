@@ -53,7 +53,7 @@ def linear(x: Union[torch.Tensor, Normed], w, out_dtype: Optional[torch.dtype] =
         norm, takes_parts = reading
         scale = norm.fusable() if hasattr(norm, "fusable") else None
         if scale is not None and ops.gemm_parts_supported(x, w, accumulate_into, scale[0]):
-            ctx.handoff.leave(norm, ops.gemm_parts_accumulate_norm(x, w, accumulate_into, scale[0], scale[1]))
+            ctx.handoff.leave(norm, ops.gemm_parts_accumulate_norm(x, w, accumulate_into, scale[0], scale[1], checked=True))
             return accumulate_into
         if scale is not None and takes_parts and ops.gemm_emit_supported(x, w, accumulate_into, scale[0]):
             ctx.handoff.leave(norm, ops.gemm_accumulate_emit(x, w, accumulate_into, scale[0], scale[1]))
