@@ -359,7 +359,7 @@ def main() -> int:
         return 0
 
     if args.only == "chat":
-        dt, st = run_chat(model, cfg, args.requests, args.gather_ms)
+        dt, st = run_chat(model, cfg, args.requests, args.gather_ms, finished=6 * args.requests)
         print(json.dumps(dict(only="chat", shape=args.shape, **st, seconds=round(dt, 3),
                               generated_per_s=round(st["generated"] / dt, 1))), flush=True)
         return 0
