@@ -207,6 +207,20 @@ bool gemm_skinny_norms() {
   }
   ok &= close("norm prepared by the product before", widen(y.get()), plain::gemm(normed2, widen(w2), m, n2, hidden), 2e-2,
               2e-2 * std::sqrt(static_cast<double>(hidden)) * 0.3);
+  // ... and the tiled SwiGLU product that finishes the same prepared norm (every 16 rows of its weight: eight gate
+  // rows, then the eight up rows of the same outputs)
+  const int n3 = 96;
+  const std::vector<bf16> w3 = as_bf16(normals(rng, static_cast<size_t>(n3) * hidden, 0.3f));
+  Dev<bf16> p3(pack_weight(w3, n3, hidden)), act(static_cast<size_t>(m) * n3 / 2);
+  RUN(bc4g_gemm_mfma_swiglu_scaled(emit_x.p, ssq.p, (hidden + 15) / 16, m, eps, p3.p, 1, act.p, m, n3, hidden, kStream));
+  const std::vector<double> gu = plain::gemm(normed2, widen(w3), m, n3, hidden);
+  std::vector<double> gated;
+  for (int r = 0; r < m; ++r)
+    for (int i = 0; i < n3 / 2; ++i) {
+      const size_t at = static_cast<size_t>(r) * n3 + (i / 8) * 16 + i % 8;
+      gated.push_back(plain::swiglu(gu[at], gu[at + 8]));
+    }
+  ok &= close("SwiGLU over the prepared norm", widen(act.get()), gated, 3e-2, 3e-2 * std::sqrt(static_cast<double>(hidden)) * 0.3);
   return ok;
 }
 
